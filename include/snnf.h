@@ -1,0 +1,148 @@
+/*
+ * snnf.h - C ABI of libsnnf: fused temporal spiking-network operators for AMD MI355X (gfx950).
+ *
+ * One entry point per kernel family of pengjh0111/triton-snn-fusion's Triton layer. Each entry point replaces the
+ * Python launcher (and the Triton kernel behind it) that the reference's runtime/triton_*_backend.py modules call;
+ * the citation above every declaration names that launcher (paths are relative to the reference checkout).
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers of the current HIP device unless the parameter is documented as a host array.
+ *   - `xs` / `residuals` are HOST arrays of T device pointers, one per timestep. A packed [T, ...] tensor is passed as
+ *     base + t * step_stride. Timesteps may alias (the same analog frame repeated T times is detected and computed once).
+ *   - Layouts are the reference's: activations contiguous NCHW per timestep, conv weight OIHW, linear weight [Fout, Fin].
+ *   - dtype codes: SNNF_F32 / SNNF_BF16 / SNNF_F16. Spikes are written as 0/1 in the activation dtype `x_dtype`.
+ *     The membrane potential is held in fp32 on chip for the whole time loop; `v_dtype` is only its dtype in memory
+ *     (v_init / v_out).
+ *   - `v_init == NULL` means a zero initial membrane (the reference's 0-dim v_init). `v_out` may alias `v_init`.
+ *   - LIF update per step (runtime/snn_custom_ops.py:384-409):
+ *         h = v + x            if tau <= 1        else   h = v + (x - v) / tau
+ *         s = (h >= v_threshold)
+ *         v = h - s * v_threshold   if v_reset < 0   else   v = s ? v_reset : h
+ *   - `stream` is a hipStream_t (NULL = the default stream). Calls only enqueue work: they never synchronise and never
+ *     free memory; none allocates device memory (scratch, where needed, is a caller-provided workspace).
+ *   - Return value: SNNF_OK (0) or a negative snnf_status; snnf_status_string() names it and snnf_last_error()
+ *     returns a thread-local detail message for the most recent failure.
+ */
+#ifndef SNNF_H_
+#define SNNF_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SNNF_MAX_T_PER_LAUNCH 16
+
+typedef enum snnf_dtype {
+    SNNF_F32 = 0,
+    SNNF_BF16 = 1,
+    SNNF_F16 = 2
+} snnf_dtype;
+
+typedef enum snnf_status {
+    SNNF_OK = 0,
+    SNNF_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive extent, unknown dtype code */
+    SNNF_ERR_UNSUPPORTED = -2,      /* well-formed request outside what the kernels implement */
+    SNNF_ERR_LAUNCH = -3,           /* hipLaunchKernel / runtime error; see snnf_last_error() */
+    SNNF_ERR_WORKSPACE = -4         /* workspace pointer missing or too small */
+} snnf_status;
+
+/* Library identification; no counterpart in the reference. */
+int snnf_abi_version(void);
+const char* snnf_status_string(int status);
+const char* snnf_last_error(void);
+
+/*
+ * Temporal LIF scan over T steps of `numel` elements.
+ * Replaces run_fused_temporal_lif_state_kernel (kernels/generated_temporal_lif_kernel.py:98-164) as called by
+ * run_triton_fused_temporal_lif_state (runtime/triton_temporal_lif_backend.py:57-117).
+ *   spikes : [T, numel] in x_dtype, timestep stride `spike_step_stride` elements.
+ *   v_out  : [numel] in v_dtype.
+ */
+int snnf_lif_scan(const void* const* xs, int T, int64_t numel, int x_dtype,
+                  const void* v_init, int v_dtype,
+                  void* spikes, int64_t spike_step_stride, void* v_out,
+                  float v_threshold, float v_reset, float tau, void* stream);
+
+/*
+ * Depthwise 3x3 convolution (padding 1, stride 1 or 2) + bias (+ residual) + LIF over T steps.
+ * Replaces run_fused_temporal_general[_residual][_autotuned] with kernel keys depthwise_k3_s1_p1 / depthwise_k3_s2_p1
+ * (kernels/benchmark_conv_lif_temporal_general.py:971-1323, emitter :713-817) as called from
+ * runtime/triton_convlif_backend.py:513-598 and :689-817.
+ *   xs[t]        : [N, C, H, W] x_dtype          weight : [C, 1, 3, 3] w_dtype        bias : [C] w_dtype
+ *   residuals[t] : [N, C, Ho, Wo] x_dtype or residuals == NULL
+ *   spikes       : [T, N, C, Ho, Wo] x_dtype (timestep stride `spike_step_stride` elements), v_out : [N, C, Ho, Wo] v_dtype
+ */
+int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int T,
+                       int N, int C, int H, int W, int stride, int x_dtype,
+                       const void* weight, const void* bias, int w_dtype,
+                       const void* v_init, int v_dtype,
+                       void* spikes, int64_t spike_step_stride, void* v_out,
+                       float v_threshold, float v_reset, float tau, void* stream);
+
+/*
+ * LIF -> global average pool -> Linear, summed over T.
+ *   out_sum[n, k] = sum_t ( fc_weight[k, :] . mean_hw(s_t[n, :, :, :]) + fc_bias[k] )
+ * Replaces run_fused_temporal_lif_avgpool_linear_kernel (kernels/generated_temporal_lif_avgpool_linear_kernel.py:120-209)
+ * as called by run_triton_fused_temporal_lif_avgpool_linear (runtime/triton_temporal_lif_avgpool_linear_backend.py:58-108).
+ *   xs[t] : [N, C, H, W] x_dtype     fc_weight : [K, C] w_dtype     fc_bias : [K] w_dtype or NULL
+ *   out_sum : [N, K] x_dtype         v_out : [N, C, H, W] v_dtype
+ *   workspace : at least snnf_lif_pool_linear_workspace_bytes(N, C) bytes of device memory, 16-byte aligned;
+ *               it holds per-(n, c) spike counts between the two launches and needs no initialisation.
+ */
+size_t snnf_lif_pool_linear_workspace_bytes(int N, int C);
+int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                         const void* v_init, int v_dtype,
+                         const void* fc_weight, const void* fc_bias, int K, int w_dtype,
+                         void* out_sum, void* v_out,
+                         void* workspace, size_t workspace_bytes,
+                         float v_threshold, float v_reset, float tau, void* stream);
+
+/*
+ * Temporal Linear + LIF: for each t, s_t, v = LIF(x_t . W^T + b, v).
+ * Replaces run_fused_temporal_linear_lif_state_kernel (kernels/generated_temporal_linear_lif_kernel.py:205-363) as
+ * called by runtime/triton_temporal_linear_lif_backend.py:185-274.
+ *   xs[t] : [M, Fin] x_dtype (row stride `x_row_stride` elements)   weight : [Fout, Fin] w_dtype   bias : [Fout] w_dtype or NULL
+ *   spikes : [T, M, Fout] x_dtype (timestep stride `spike_step_stride` elements)   v_out : [M, Fout] v_dtype
+ * fp32 operands are rounded to bf16 for the matrix cores (fp32 accumulate); fp16 operands use the fp16 matrix path.
+ */
+int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
+                    const void* weight, const void* bias, int Fout, int w_dtype,
+                    const void* v_init, int v_dtype,
+                    void* spikes, int64_t spike_step_stride, void* v_out,
+                    float v_threshold, float v_reset, float tau, void* stream);
+
+/*
+ * Dense (groups == 1) convolution + bias (+ residual) + LIF over T steps as an implicit GEMM on the matrix cores.
+ * Replaces run_fused_temporal_general[_residual][_autotuned] with kernel keys k1_s1_p0, k3_s1_p1, k3_s2_p1, k5_s1_p2,
+ * k7_s2_p3, k11_s4_p2 (kernels/benchmark_conv_lif_temporal_general.py:971-1323, emitter :561-710) as called from
+ * runtime/triton_convlif_backend.py:331-817. Any square-or-not kernel size, stride and padding is accepted as long as
+ * dilation is 1.
+ *
+ * Two steps: (1) snnf_conv_pack_weight rewrites the OIHW weight (+ bias) into the matrix-core operand order once per
+ * weight tensor; (2) snnf_conv_lif consumes the packed weight on every call. The packed buffer is opaque; its size is
+ * snnf_conv_packed_weight_bytes(). fp32 activations/weights are rounded to bf16 for the matrix cores (fp32
+ * accumulate); fp16 activations use the fp16 matrix path.
+ *   xs[t]        : [N, Cin, H, W] x_dtype
+ *   residuals[t] : [N, Cout, Ho, Wo] x_dtype or residuals == NULL
+ *   spikes       : [T, N, Cout, Ho, Wo] x_dtype (timestep stride `spike_step_stride` elements); v_out : [N, Cout, Ho, Wo] v_dtype
+ */
+size_t snnf_conv_packed_weight_bytes(int Cout, int Cin, int KH, int KW);
+int snnf_conv_pack_weight(const void* weight, const void* bias /* nullable */, int w_dtype,
+                          int Cout, int Cin, int KH, int KW, int x_dtype,
+                          void* packed, size_t packed_bytes, void* stream);
+int snnf_conv_lif(const void* const* xs, const void* const* residuals, int T,
+                  int N, int Cin, int H, int W, int x_dtype,
+                  const void* packed_weight, int Cout, int KH, int KW,
+                  int stride_h, int stride_w, int pad_h, int pad_w,
+                  const void* v_init, int v_dtype,
+                  void* spikes, int64_t spike_step_stride, void* v_out,
+                  float v_threshold, float v_reset, float tau, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SNNF_H_ */

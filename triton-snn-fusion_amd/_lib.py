@@ -1,0 +1,117 @@
+"""ctypes binding of libsnnf.so (the C ABI declared in include/snnf.h).
+
+The library is loaded from triton-snn-fusion_amd/lib/. If it has not been built the loader raises: there is no
+Python or CPU substitute for the HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+from typing import Optional, Sequence
+
+import torch
+
+PKG_DIR = Path(__file__).resolve().parent
+LIB_PATH = PKG_DIR / "lib" / "libsnnf.so"
+
+SNNF_F32, SNNF_BF16, SNNF_F16 = 0, 1, 2
+SNNF_MAX_T_PER_LAUNCH = 16
+
+_DTYPE_CODES = {torch.float32: SNNF_F32, torch.bfloat16: SNNF_BF16, torch.float16: SNNF_F16}
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+_f = ctypes.c_float
+_sz = ctypes.c_size_t
+_pp = ctypes.POINTER(ctypes.c_void_p)
+
+# name -> (restype, argtypes); must list every function declared in include/snnf.h.
+SIGNATURES = {
+    "snnf_abi_version": (_i, []),
+    "snnf_status_string": (ctypes.c_char_p, [_i]),
+    "snnf_last_error": (ctypes.c_char_p, []),
+    "snnf_lif_scan": (_i, [_pp, _i, _i64, _i, _vp, _i, _vp, _i64, _vp, _f, _f, _f, _vp]),
+    "snnf_dwconv3x3_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp,
+                                _f, _f, _f, _vp]),
+    "snnf_lif_pool_linear_workspace_bytes": (_sz, [_i, _i]),
+    "snnf_lif_pool_linear": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _sz,
+                                  _f, _f, _f, _vp]),
+    "snnf_linear_lif": (_i, [_pp, _i, _i, _i, _i64, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _i64, _vp, _f, _f, _f, _vp]),
+    "snnf_conv_packed_weight_bytes": (_sz, [_i, _i, _i, _i]),
+    "snnf_conv_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "snnf_conv_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i64,
+                           _vp, _f, _f, _f, _vp]),
+}
+
+_LIB: Optional[ctypes.CDLL] = None
+
+
+class SnnfError(RuntimeError):
+    """A libsnnf entry point returned a non-zero status."""
+
+    def __init__(self, func: str, status: int, detail: str):
+        super().__init__(detail if detail else f"{func} failed with status {status}")
+        self.func = func
+        self.status = status
+
+
+def library_available() -> bool:
+    return LIB_PATH.exists()
+
+
+def lib() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"libsnnf.so not found at {LIB_PATH}; build it with `python triton-snn-fusion_amd/build.py` "
+                "(the fused SNN operators have no non-HIP implementation)"
+            )
+        handle = ctypes.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError here means header and library disagree
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _LIB = handle
+    return _LIB
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODES[dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported_dtype: libsnnf handles float32, bfloat16 and float16, got {dtype}") from None
+
+
+def check(func: str, status: int) -> None:
+    if status != 0:
+        detail = lib().snnf_last_error().decode("utf-8", "replace")
+        raise SnnfError(func, status, detail)
+
+
+def step_pointers(tensors: Sequence[torch.Tensor]):
+    """Host array of per-timestep device pointers."""
+    arr = (ctypes.c_void_p * len(tensors))()
+    for i, t in enumerate(tensors):
+        arr[i] = t.data_ptr()
+    return arr
+
+
+def packed_step_pointers(x_seq: torch.Tensor):
+    """Per-timestep pointers into a [T, ...] tensor whose steps are individually contiguous."""
+    T = int(x_seq.shape[0])
+    arr = (ctypes.c_void_p * T)()
+    base = x_seq.data_ptr()
+    step = int(x_seq.stride(0)) * x_seq.element_size()
+    for t in range(T):
+        arr[t] = base + t * step
+    return arr
+
+
+def current_stream(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()

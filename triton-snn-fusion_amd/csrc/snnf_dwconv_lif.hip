@@ -1,0 +1,284 @@
+// Depthwise 3x3 (padding 1, stride 1|2) + bias (+ residual) + LIF over T steps.
+//
+// Bound by HBM bandwidth: every activation is read once and every spike written once; the 3x3 halo re-use happens in
+// LDS. A workgroup owns PB consecutive (n, c) planes (or a band of TH output rows of one plane), keeps an fp32 copy of
+// the input band with a zero halo in LDS, and every thread keeps the fp32 membrane of its PX-wide output strips in
+// registers for the whole time loop.
+#include "snnf_common.h"
+
+namespace snnf {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kItems = 2;     // output strips per thread
+constexpr int kColOffset = 4;  // LDS column of input column 0 (keeps 16-byte alignment; column 3 is the left halo)
+
+struct DwGeom {
+    int planes;      // N * C
+    int C, H, W, Ho, Wo;
+    int TH;          // output rows per band
+    int PB;          // planes per workgroup
+    int bands;       // ceil(Ho / TH)
+    int RIN;         // input rows held per plane: (TH - 1) * stride + 3
+    int pitch;       // LDS floats per input row
+    int SW;          // strips per output row = Wo / PX
+    int WV;          // load vectors per input row = W / PX
+};
+
+template <typename XT, int PX>
+__device__ __forceinline__ void load_strip_as_float(const XT* __restrict__ p, float (&out)[PX]) {
+    const Pack<XT, PX> raw = *reinterpret_cast<const Pack<XT, PX>*>(p);
+#pragma unroll
+    for (int i = 0; i < PX; ++i) out[i] = to_float(raw.v[i]);
+}
+
+template <typename XT, typename VT, int STRIDE, int PX>
+__global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, StepPtrs residuals, int has_residual,
+                                                                 int T, DwGeom g, const XT* __restrict__ weight,
+                                                                 const XT* __restrict__ bias,
+                                                                 const VT* __restrict__ v_init,
+                                                                 XT* __restrict__ spikes, int64_t spike_step_stride,
+                                                                 VT* __restrict__ v_out, LifParams lif) {
+    extern __shared__ __align__(16) float tile[];
+    constexpr int IN_COLS = (PX - 1) * STRIDE + 3;
+
+    const int band = blockIdx.x % g.bands;
+    const int plane0 = (blockIdx.x / g.bands) * g.PB;
+    const int planes_here = min(g.PB, g.planes - plane0);
+    const int row0 = band * g.TH;                       // first output row of the band
+    const int rows_here = min(g.TH, g.Ho - row0);
+    const int in_row0 = row0 * STRIDE - 1;              // input row held in LDS row 0
+    const int plane_floats = g.RIN * g.pitch;
+
+    // Zero the whole tile once: halo columns and out-of-image rows stay zero for every timestep.
+    for (int i = threadIdx.x; i < g.PB * plane_floats; i += kThreads) tile[i] = 0.0f;
+
+    // Fixed ownership of output strips for the whole time loop.
+    const int strips_per_plane = rows_here * g.SW;
+    const int strips = planes_here * strips_per_plane;
+    int item_plane[kItems], item_row[kItems], item_col[kItems];
+    bool item_live[kItems];
+    float v[kItems][PX];
+    float w[kItems][9];
+    float b[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int i = threadIdx.x + k * kThreads;
+        item_live[k] = i < strips;
+        const int ii = item_live[k] ? i : 0;
+        item_plane[k] = ii / strips_per_plane;
+        const int rem = ii - item_plane[k] * strips_per_plane;
+        item_row[k] = rem / g.SW;
+        item_col[k] = (rem - item_row[k] * g.SW) * PX;
+        const int c = (plane0 + item_plane[k]) % g.C;
+#pragma unroll
+        for (int j = 0; j < 9; ++j) w[k][j] = to_float(weight[c * 9 + j]);
+        b[k] = to_float(bias[c]);
+        const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
+        if (item_live[k] && v_init != nullptr) {
+            load_strip_as_float<VT, PX>(v_init + o, v[k]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < PX; ++j) v[k][j] = 0.0f;
+        }
+    }
+
+    const int load_vectors = planes_here * g.RIN * g.WV;
+    for (int t = 0; t < T; ++t) {
+        __syncthreads();  // previous step's reads (or the zero fill) are complete
+        const XT* __restrict__ x = static_cast<const XT*>(xs.p[t]);
+        for (int i = threadIdx.x; i < load_vectors; i += kThreads) {
+            const int p = i / (g.RIN * g.WV);
+            const int rem = i - p * (g.RIN * g.WV);
+            const int r = rem / g.WV;
+            const int cv = rem - r * g.WV;
+            const int ih = in_row0 + r;
+            if (ih < 0 || ih >= g.H) continue;
+            float vals[PX];
+            load_strip_as_float<XT, PX>(x + (static_cast<int64_t>(plane0 + p) * g.H + ih) * g.W + cv * PX, vals);
+            float* dst = tile + p * plane_floats + r * g.pitch + kColOffset + cv * PX;
+#pragma unroll
+            for (int j = 0; j < PX; ++j) dst[j] = vals[j];
+        }
+        __syncthreads();
+
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            if (!item_live[k]) continue;
+            const float* src = tile + item_plane[k] * plane_floats + (item_row[k] * STRIDE) * g.pitch +
+                               (kColOffset - 1) + item_col[k] * STRIDE;
+            float acc[PX];
+#pragma unroll
+            for (int j = 0; j < PX; ++j) acc[j] = b[k];
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh) {
+                float in[IN_COLS];
+#pragma unroll
+                for (int j = 0; j < IN_COLS; ++j) in[j] = src[kh * g.pitch + j];
+#pragma unroll
+                for (int j = 0; j < PX; ++j) {
+#pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) acc[j] = fmaf(in[j * STRIDE + kw], w[k][kh * 3 + kw], acc[j]);
+                }
+            }
+            const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
+            if (has_residual) {
+                float res[PX];
+                load_strip_as_float<XT, PX>(static_cast<const XT*>(residuals.p[t]) + o, res);
+#pragma unroll
+                for (int j = 0; j < PX; ++j) acc[j] += res[j];
+            }
+            Pack<XT, PX> out;
+#pragma unroll
+            for (int j = 0; j < PX; ++j) out.v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
+            *reinterpret_cast<Pack<XT, PX>*>(spikes + t * spike_step_stride + o) = out;
+        }
+    }
+
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (!item_live[k]) continue;
+        const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
+        Pack<VT, PX> vo;
+#pragma unroll
+        for (int j = 0; j < PX; ++j) vo.v[j] = from_float<VT>(v[k][j]);
+        *reinterpret_cast<Pack<VT, PX>*>(v_out + o) = vo;
+    }
+}
+
+template <typename XT, typename VT, int STRIDE, int PX>
+int launch(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g, const void* weight, const void* bias,
+           const void* v_init, void* spikes, int64_t spike_step_stride, void* v_out, const LifParams& lif,
+           hipStream_t stream) {
+    g.SW = g.Wo / PX;
+    g.WV = g.W / PX;
+    const int max_strips = kThreads * kItems;
+    const int per_plane = g.Ho * g.SW;
+    if (per_plane >= max_strips) {
+        g.PB = 1;
+        g.TH = max_strips / g.SW;
+        if (g.TH < 1) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: output row of %d pixels is too wide", g.Wo);
+    } else {
+        g.TH = g.Ho;
+        g.PB = max_strips / per_plane;
+        if (g.PB > g.planes) g.PB = g.planes;
+    }
+    g.bands = (g.Ho + g.TH - 1) / g.TH;
+    g.RIN = (g.TH - 1) * STRIDE + 3;
+    g.pitch = ((g.W + kColOffset + 1) + 3) / 4 * 4;
+    size_t lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
+    while (lds > 64 * 1024 && g.PB > 1) {
+        g.PB = (g.PB + 1) / 2;
+        lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
+    }
+    while (lds > 64 * 1024 && g.TH > 1) {
+        g.TH = (g.TH + 1) / 2;
+        g.bands = (g.Ho + g.TH - 1) / g.TH;
+        g.RIN = (g.TH - 1) * STRIDE + 3;
+        lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
+    }
+    if (lds > 64 * 1024) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: input row of %d pixels does not fit LDS", g.W);
+    const int64_t blocks = static_cast<int64_t>((g.planes + g.PB - 1) / g.PB) * g.bands;
+    if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: too many planes");
+    dwconv3x3_lif_kernel<XT, VT, STRIDE, PX><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+        xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
+        static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    return check_launch("snnf_dwconv3x3_lif");
+}
+
+template <typename XT, typename VT, int STRIDE>
+int dispatch_px(int px, const StepPtrs& xs, const StepPtrs& res, int has_res, int T, const DwGeom& g,
+                const void* weight, const void* bias, const void* v_init, void* spikes, int64_t sss, void* v_out,
+                const LifParams& lif, hipStream_t stream) {
+    if (px == 8) return launch<XT, VT, STRIDE, 8>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+    if (px == 4) return launch<XT, VT, STRIDE, 4>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+    return launch<XT, VT, STRIDE, 1>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+}
+
+template <typename XT, typename VT>
+int dispatch_stride(int stride, int px, const StepPtrs& xs, const StepPtrs& res, int has_res, int T, const DwGeom& g,
+                    const void* weight, const void* bias, const void* v_init, void* spikes, int64_t sss, void* v_out,
+                    const LifParams& lif, hipStream_t stream) {
+    if (stride == 1) return dispatch_px<XT, VT, 1>(px, xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+    return dispatch_px<XT, VT, 2>(px, xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+}
+
+}  // namespace
+}  // namespace snnf
+
+extern "C" int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int T, int N, int C, int H, int W,
+                                  int stride, int x_dtype, const void* weight, const void* bias, int w_dtype,
+                                  const void* v_init, int v_dtype, void* spikes, int64_t spike_step_stride, void* v_out,
+                                  float v_threshold, float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    if (xs == nullptr || weight == nullptr || bias == nullptr || spikes == nullptr || v_out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_dwconv3x3_lif: xs, weight, bias, spikes and v_out must be non-null");
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_dwconv3x3_lif: T=%d N=%d C=%d H=%d W=%d", T, N, C, H, W);
+    if (stride != 1 && stride != 2)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: unsupported_stride: 3x3 depthwise supports stride 1 or 2, got %d", stride);
+    if (!valid_dtype(x_dtype) || !valid_dtype(v_dtype) || !valid_dtype(w_dtype))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_dwconv3x3_lif: unknown dtype code");
+    if (w_dtype != x_dtype)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: unsupported_dtype: weight/bias dtype must match x");
+    if (v_dtype != SNNF_F32 && v_dtype != x_dtype)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: unsupported_dtype: membrane dtype must be fp32 or the activation dtype");
+    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: unsupported_tau: tau must be nonzero");
+    if (static_cast<int64_t>(N) * C > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: N*C too large");
+    for (int t = 0; t < T; ++t) {
+        if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_dwconv3x3_lif: xs[%d] is null", t);
+        if (residuals != nullptr && residuals[t] == nullptr)
+            return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_dwconv3x3_lif: residuals[%d] is null", t);
+    }
+
+    DwGeom g = {};
+    g.planes = N * C;
+    g.C = C;
+    g.H = H;
+    g.W = W;
+    g.Ho = (H + 2 - 3) / stride + 1;
+    g.Wo = (W + 2 - 3) / stride + 1;
+    const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
+    const int xsize = dtype_size(x_dtype);
+    const int vsize = dtype_size(v_dtype);
+    hipStream_t hs = as_stream(stream);
+
+    for (int t0 = 0; t0 < T; t0 += SNNF_MAX_T_PER_LAUNCH) {
+        const int tw = (T - t0) < SNNF_MAX_T_PER_LAUNCH ? (T - t0) : SNNF_MAX_T_PER_LAUNCH;
+        StepPtrs xp = {}, rp = {};
+        const void* vi = t0 == 0 ? v_init : v_out;
+        void* sp = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
+        // Widest strip for which every row start of every operand is naturally aligned.
+        int px = 1;
+        for (int cand : {8, 4}) {
+            const size_t xa = static_cast<size_t>(cand) * xsize;
+            const size_t va = static_cast<size_t>(cand) * vsize > 16 ? 16 : static_cast<size_t>(cand) * vsize;
+            bool ok = g.Wo % cand == 0 && g.W % cand == 0 && spike_step_stride % cand == 0 && aligned_to(sp, xa) &&
+                      aligned_to(v_out, va) && (vi == nullptr || aligned_to(vi, va));
+            for (int t = 0; t < tw && ok; ++t) {
+                ok = aligned_to(xs[t0 + t], xa);
+                if (residuals != nullptr) ok = ok && aligned_to(residuals[t0 + t], xa);
+            }
+            if (ok) { px = cand; break; }
+        }
+        for (int t = 0; t < tw; ++t) {
+            xp.p[t] = xs[t0 + t];
+            if (residuals != nullptr) rp.p[t] = residuals[t0 + t];
+        }
+        const int has_res = residuals != nullptr ? 1 : 0;
+        int rc;
+        if (x_dtype == SNNF_F32) {
+            rc = dispatch_stride<float, float>(stride, px, xp, rp, has_res, tw, g, weight, bias, vi, sp, spike_step_stride, v_out, lif, hs);
+        } else if (x_dtype == SNNF_BF16) {
+            rc = v_dtype == SNNF_F32
+                     ? dispatch_stride<bf16_t, float>(stride, px, xp, rp, has_res, tw, g, weight, bias, vi, sp, spike_step_stride, v_out, lif, hs)
+                     : dispatch_stride<bf16_t, bf16_t>(stride, px, xp, rp, has_res, tw, g, weight, bias, vi, sp, spike_step_stride, v_out, lif, hs);
+        } else {
+            rc = v_dtype == SNNF_F32
+                     ? dispatch_stride<f16_t, float>(stride, px, xp, rp, has_res, tw, g, weight, bias, vi, sp, spike_step_stride, v_out, lif, hs)
+                     : dispatch_stride<f16_t, f16_t>(stride, px, xp, rp, has_res, tw, g, weight, bias, vi, sp, spike_step_stride, v_out, lif, hs);
+        }
+        if (rc != SNNF_OK) return rc;
+    }
+    return SNNF_OK;
+}

@@ -1,0 +1,182 @@
+// LIF -> global average pool -> Linear, summed over T (the classifier tail of a spiking network).
+//
+//   out_sum[n, k] = sum_t ( W[k, :] . mean_hw(s_t[n, :, :, :]) + b[k] ) = (W[k, :] . count[n, :]) / HW + T * b[k]
+//
+// where count[n, c] is the number of spikes of plane (n, c) over all T steps: the pooled activations are never
+// materialised per step. Launch 1 streams x once (HBM-bound), keeps the membrane in registers, counts spikes per plane
+// with wave ballots and writes the integer counts to the workspace; launch 2 is a small GEMV over the counts.
+#include "snnf_common.h"
+
+namespace snnf {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kItems = 4;        // neurons per thread in the pooling kernel
+constexpr int kMaxPlanes = 1024;  // planes per workgroup (HW == 1 gives kThreads * kItems planes)
+
+template <typename XT, typename VT>
+__global__ __launch_bounds__(kThreads) void lif_pool_kernel(StepPtrs xs, int T, int planes, int HW, int planes_per_block,
+                                                            const VT* __restrict__ v_init, VT* __restrict__ v_out,
+                                                            int* __restrict__ counts, LifParams lif) {
+    __shared__ int plane_count[kMaxPlanes];
+    const int plane0 = blockIdx.x * planes_per_block;
+    const int planes_here = min(planes_per_block, planes - plane0);
+    const int elems = planes_here * HW;
+    const int64_t base = static_cast<int64_t>(plane0) * HW;
+    for (int i = threadIdx.x; i < planes_here; i += kThreads) plane_count[i] = 0;
+
+    float v[kItems];
+    int plane_of[kItems];
+    int fired_total[kItems];
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int i = threadIdx.x + k * kThreads;
+        plane_of[k] = i < elems ? i / HW : -1;
+        fired_total[k] = 0;
+        v[k] = (i < elems && v_init != nullptr) ? to_float(v_init[base + i]) : 0.0f;
+    }
+    for (int t = 0; t < T; ++t) {
+        const XT* __restrict__ x = static_cast<const XT*>(xs.p[t]) + base;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            const int i = threadIdx.x + k * kThreads;
+            if (i < elems) fired_total[k] += lif_step(to_float(x[i]), v[k], lif) ? 1 : 0;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int i = threadIdx.x + k * kThreads;
+        // Wave-level reduction when the whole wave sits in one plane, LDS atomics otherwise.
+        const int my_plane = plane_of[k];
+        const int lead_plane = __shfl(my_plane, 0);
+        if (__all(my_plane == lead_plane)) {
+            int sum = fired_total[k];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+            if ((threadIdx.x & 63) == 0 && lead_plane >= 0) atomicAdd(&plane_count[lead_plane], sum);
+        } else if (my_plane >= 0 && fired_total[k] != 0) {
+            atomicAdd(&plane_count[my_plane], fired_total[k]);
+        }
+        if (i < elems) v_out[base + i] = from_float<VT>(v[k]);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < planes_here; i += kThreads) counts[plane0 + i] = plane_count[i];
+}
+
+// One workgroup: one sample n, kWavesPerBlock * kRowsPerWave output rows; the sample's spike counts sit in LDS.
+constexpr int kRowsPerWave = 4;
+
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void count_linear_kernel(const int* __restrict__ counts, int C, int K,
+                                                                const XT* __restrict__ W, const XT* __restrict__ bias,
+                                                                XT* __restrict__ out, float inv_hw, float steps) {
+    extern __shared__ float cnt[];
+    const int n = blockIdx.y;
+    for (int c = threadIdx.x; c < C; c += kThreads) cnt[c] = static_cast<float>(counts[n * C + c]);
+    __syncthreads();
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int k0 = (blockIdx.x * (kThreads / 64) + wave) * kRowsPerWave;
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        const int k = k0 + r;
+        if (k >= K) break;
+        const XT* __restrict__ row = W + static_cast<int64_t>(k) * C;
+        float acc = 0.0f;
+        for (int c = lane; c < C; c += 64) acc = fmaf(to_float(row[c]), cnt[c], acc);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+        if (lane == 0) {
+            float o = acc * inv_hw;
+            if (bias != nullptr) o += steps * to_float(bias[k]);
+            out[static_cast<int64_t>(n) * K + k] = from_float<XT>(o);
+        }
+    }
+}
+
+template <typename XT, typename VT>
+int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void* v_out, int* counts,
+        const LifParams& lif, hipStream_t stream) {
+    int ppb = (kThreads * kItems) / HW;
+    if (ppb < 1) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: H*W=%d exceeds %d", HW, kThreads * kItems);
+    if (ppb > kMaxPlanes) ppb = kMaxPlanes;
+    const int blocks = (planes + ppb - 1) / ppb;
+    lif_pool_kernel<XT, VT><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, ppb, static_cast<const VT*>(v_init),
+                                                                  static_cast<VT*>(v_out), counts, lif);
+    return check_launch("snnf_lif_pool_linear(pool)");
+}
+
+}  // namespace
+}  // namespace snnf
+
+extern "C" size_t snnf_lif_pool_linear_workspace_bytes(int N, int C) {
+    if (N < 1 || C < 1) return 0;
+    return static_cast<size_t>(N) * static_cast<size_t>(C) * sizeof(int);
+}
+
+extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                                    const void* v_init, int v_dtype, const void* fc_weight, const void* fc_bias, int K,
+                                    int w_dtype, void* out_sum, void* v_out, void* workspace, size_t workspace_bytes,
+                                    float v_threshold, float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    if (xs == nullptr || fc_weight == nullptr || out_sum == nullptr || v_out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: xs, fc_weight, out_sum and v_out must be non-null");
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: T=%d N=%d C=%d H=%d W=%d K=%d", T, N, C, H, W, K);
+    if (T > SNNF_MAX_T_PER_LAUNCH)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_temporal_length: T=%d exceeds %d", T, SNNF_MAX_T_PER_LAUNCH);
+    if (!valid_dtype(x_dtype) || !valid_dtype(v_dtype) || !valid_dtype(w_dtype))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: unknown dtype code");
+    if (w_dtype != x_dtype)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_dtype: fc_weight/fc_bias dtype must match x");
+    if (v_dtype != SNNF_F32 && v_dtype != x_dtype)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_dtype: membrane dtype must be fp32 or the activation dtype");
+    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_tau: tau must be nonzero");
+    const int64_t planes64 = static_cast<int64_t>(N) * C;
+    const int64_t hw64 = static_cast<int64_t>(H) * W;
+    if (planes64 > 0x7fffffffLL || hw64 > kThreads * kItems)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: N*C=%lld or H*W=%lld too large", (long long)planes64, (long long)hw64);
+    if (N > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: N=%d exceeds 65535", N);
+    if (static_cast<size_t>(C) * sizeof(float) > 64 * 1024)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: C=%d exceeds LDS capacity", C);
+    if (workspace == nullptr || workspace_bytes < snnf_lif_pool_linear_workspace_bytes(N, C) || !aligned_to(workspace, 16))
+        return fail(SNNF_ERR_WORKSPACE, "snnf_lif_pool_linear: workspace of %zu bytes (16-byte aligned) required",
+                    snnf_lif_pool_linear_workspace_bytes(N, C));
+    StepPtrs ptrs = {};
+    for (int t = 0; t < T; ++t) {
+        if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: xs[%d] is null", t);
+        ptrs.p[t] = xs[t];
+    }
+    const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
+    hipStream_t hs = as_stream(stream);
+    int* counts = static_cast<int*>(workspace);
+    const int planes = static_cast<int>(planes64);
+    const int HW = static_cast<int>(hw64);
+
+    int rc;
+    if (x_dtype == SNNF_F32) rc = run<float, float>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs);
+    else if (x_dtype == SNNF_BF16)
+        rc = v_dtype == SNNF_F32 ? run<bf16_t, float>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs)
+                                 : run<bf16_t, bf16_t>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs);
+    else
+        rc = v_dtype == SNNF_F32 ? run<f16_t, float>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs)
+                                 : run<f16_t, f16_t>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs);
+    if (rc != SNNF_OK) return rc;
+
+    const int rows_per_block = (kThreads / 64) * kRowsPerWave;
+    const dim3 grid((K + rows_per_block - 1) / rows_per_block, N);
+    const size_t lds = static_cast<size_t>(C) * sizeof(float);
+    const float inv_hw = 1.0f / static_cast<float>(HW);
+    const float steps = static_cast<float>(T);
+    if (x_dtype == SNNF_F32)
+        count_linear_kernel<float><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const float*>(fc_weight),
+                                                               static_cast<const float*>(fc_bias), static_cast<float*>(out_sum), inv_hw, steps);
+    else if (x_dtype == SNNF_BF16)
+        count_linear_kernel<bf16_t><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const bf16_t*>(fc_weight),
+                                                                static_cast<const bf16_t*>(fc_bias), static_cast<bf16_t*>(out_sum), inv_hw, steps);
+    else
+        count_linear_kernel<f16_t><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const f16_t*>(fc_weight),
+                                                               static_cast<const f16_t*>(fc_bias), static_cast<f16_t*>(out_sum), inv_hw, steps);
+    return check_launch("snnf_lif_pool_linear(linear)");
+}

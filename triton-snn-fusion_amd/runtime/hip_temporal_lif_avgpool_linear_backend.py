@@ -1,0 +1,130 @@
+"""LIF -> AvgPool -> Linear backend on libsnnf: drop-in for runtime/triton_temporal_lif_avgpool_linear_backend.py.
+
+Keeps the reference's names (including the deprecated `*_tail` aliases of
+runtime/triton_temporal_lif_avgpool_linear_backend.py:111-115) and accepts the `use_autotune` keyword the reference
+operator layer passes (runtime/snn_custom_ops.py:1695-1707).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import _lib
+
+SUPPORTED_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+MAX_TIMESTEPS = _lib.SNNF_MAX_T_PER_LAUNCH
+MAX_PLANE_ELEMENTS = 1024
+
+
+@dataclass
+class TritonTemporalLIFAvgPoolLinearResult:
+    """Same fields as runtime/triton_temporal_lif_avgpool_linear_backend.py:8-15."""
+
+    out_sum: torch.Tensor
+    v_next: torch.Tensor
+    used_triton: bool
+    kernel_key: str = "temporal_lif_avgpool_linear"
+    fallback_reason: str = ""
+    kernel_diagnostics: Optional[Dict] = None
+
+
+def strict_temporal_lif_avgpool_linear_enabled(strict: bool = False) -> bool:
+    return bool(strict) or os.environ.get("CHRONOS_STRICT_TEMPORAL_LIF_AVGPOOL_LINEAR_TRITON", "0") == "1"
+
+
+def check_temporal_lif_avgpool_linear_support(x_seq, v_init, fc_weight, fc_bias, tau) -> List[str]:
+    """Counterpart of runtime/triton_temporal_lif_avgpool_linear_backend.py:22-55."""
+    if not isinstance(x_seq, torch.Tensor):
+        return ["x_seq must be a tensor"]
+    reasons: List[str] = []
+    if not x_seq.is_cuda:
+        reasons.append("unsupported_device: x_seq is not CUDA")
+    if x_seq.dim() != 5:
+        reasons.append(f"unsupported_rank: x_seq.dim must be 5, got {x_seq.dim()}")
+    if x_seq.dtype not in SUPPORTED_DTYPES:
+        reasons.append(f"unsupported_dtype: x_seq dtype must be float32, bfloat16 or float16, got {x_seq.dtype}")
+    if x_seq.dim() == 5:
+        if not 1 <= int(x_seq.shape[0]) <= MAX_TIMESTEPS:
+            reasons.append(f"unsupported_temporal_length: T must be in 1..{MAX_TIMESTEPS}, got {int(x_seq.shape[0])}")
+        if int(x_seq.shape[3]) * int(x_seq.shape[4]) > MAX_PLANE_ELEMENTS:
+            reasons.append(f"unsupported_shape: H*W must be at most {MAX_PLANE_ELEMENTS}, got {int(x_seq.shape[3]) * int(x_seq.shape[4])}")
+    if not isinstance(v_init, torch.Tensor):
+        reasons.append("v_init must be a tensor")
+    elif v_init.dim() != 0:
+        if x_seq.dim() == 5 and tuple(v_init.shape) != tuple(x_seq.shape[1:]):
+            reasons.append(
+                f"unsupported_membrane_state: v_init shape {tuple(v_init.shape)} does not match {tuple(x_seq.shape[1:])}")
+        if v_init.device != x_seq.device or v_init.dtype not in (x_seq.dtype, torch.float32):
+            reasons.append("unsupported_dtype: v_init device/dtype must match x_seq (or be float32)")
+    if not isinstance(fc_weight, torch.Tensor) or fc_weight.dim() != 2:
+        reasons.append("fc_weight must be a 2D tensor")
+    elif x_seq.dim() == 5:
+        if int(fc_weight.shape[1]) != int(x_seq.shape[2]):
+            reasons.append(f"unsupported_linear: fc in_features {fc_weight.shape[1]} must match channels {x_seq.shape[2]}")
+        if fc_weight.device != x_seq.device or fc_weight.dtype != x_seq.dtype:
+            reasons.append("unsupported_dtype: fc_weight device/dtype must match x_seq")
+    if isinstance(fc_bias, torch.Tensor) and fc_bias.numel() > 0:
+        if isinstance(fc_weight, torch.Tensor) and fc_weight.dim() == 2 and fc_bias.numel() != fc_weight.shape[0]:
+            reasons.append("unsupported_linear: fc_bias shape does not match out_features")
+        if fc_bias.device != x_seq.device or fc_bias.dtype != x_seq.dtype:
+            reasons.append("unsupported_dtype: fc_bias device/dtype must match x_seq")
+    if float(tau) == 0.0:
+        reasons.append("unsupported_tau: tau must be nonzero")
+    return reasons
+
+
+def run_triton_fused_temporal_lif_avgpool_linear(x_seq, v_init, fc_weight, fc_bias, v_threshold: float, v_reset: float,
+                                                 tau: float, detach_reset: bool, strict: bool = False,
+                                                 verbose: bool = False,
+                                                 use_autotune: bool = True) -> TritonTemporalLIFAvgPoolLinearResult:
+    reasons = check_temporal_lif_avgpool_linear_support(x_seq, v_init, fc_weight, fc_bias, tau)
+    strict = strict_temporal_lif_avgpool_linear_enabled(strict)
+    if reasons:
+        if verbose:
+            print(f"[HIP][FALLBACK][temporal_lif_avgpool_linear] {'; '.join(reasons)}")
+        if strict:
+            raise RuntimeError("[HIP][STRICT][temporal_lif_avgpool_linear] " + "; ".join(reasons))
+        raise RuntimeError("; ".join(reasons))
+
+    lib = _lib.lib()
+    x = x_seq if x_seq.is_contiguous() else x_seq.contiguous()
+    T, N, C, H, W = (int(d) for d in x.shape)
+    K = int(fc_weight.shape[0])
+    v_dtype = v_init.dtype if v_init.dtype in (torch.float32, x.dtype) else x.dtype
+    vi = None
+    if v_init.dim() != 0:
+        vi = v_init if v_init.is_contiguous() else v_init.contiguous()
+    w = fc_weight if fc_weight.is_contiguous() else fc_weight.contiguous()
+    b = None
+    if isinstance(fc_bias, torch.Tensor) and fc_bias.numel() > 0:
+        b = fc_bias if fc_bias.is_contiguous() else fc_bias.contiguous()
+    out_sum = torch.empty((N, K), dtype=x.dtype, device=x.device)
+    v_next = torch.empty((N, C, H, W), dtype=v_dtype, device=x.device)
+    ws_bytes = int(lib.snnf_lif_pool_linear_workspace_bytes(N, C))
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    _lib.check("snnf_lif_pool_linear", lib.snnf_lif_pool_linear(
+        _lib.packed_step_pointers(x), T, N, C, H, W, _lib.dtype_code(x.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype),
+        w.data_ptr(), _lib.ptr(b), K, _lib.dtype_code(w.dtype), out_sum.data_ptr(), v_next.data_ptr(),
+        workspace.data_ptr(), ws_bytes, float(v_threshold), float(v_reset), float(tau), _lib.current_stream(x.device)))
+    diagnostics = {
+        "kernel_kind": "standalone_temporal_lif_avgpool_linear",
+        "fuse_organization": "two_stage_fused_pipeline",
+        "stage_0": "lif_recurrence_plus_spike_count_per_plane",
+        "stage_1": "linear_over_time_summed_counts",
+        "intermediate_materialization": "counts[N,C] int32",
+        "compute_dtype": "float16" if x.dtype == torch.float16 else "float32",
+        "T": T,
+        "shape": tuple(x.shape),
+        "classes": K,
+    }
+    return TritonTemporalLIFAvgPoolLinearResult(out_sum, v_next, True, kernel_diagnostics=diagnostics)
+
+
+# Deprecated compatibility aliases (runtime/triton_temporal_lif_avgpool_linear_backend.py:111-115).
+TritonTemporalLIFTailResult = TritonTemporalLIFAvgPoolLinearResult
+strict_temporal_lif_tail_enabled = strict_temporal_lif_avgpool_linear_enabled
+check_temporal_lif_tail_support = check_temporal_lif_avgpool_linear_support
+run_triton_fused_temporal_lif_tail = run_triton_fused_temporal_lif_avgpool_linear
