@@ -1,0 +1,325 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused temporal SNN operators on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mobilenet_block|conv3x3_block|linear_block]
+
+A "step" is one pass of the workload's fused operators over one batch of synthetic spikes that already sit in HBM.
+The default workload is the MobileNet-style block (depthwise Conv3x3+BN+LIF, then pointwise Conv1x1+BN+LIF; T=4, B=32,
+56x56, bf16 activations/weights, fp32 membrane): two fused ConvBN-LIF layers at T=4. One JSON line is printed with the
+whole-step throughput (images*T/s), ms per step / per layer, the roofline of the dominant kernel measured live with
+HIP events, per-operator timings of the other workloads, and the eager PyTorch CPU path timed on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+METRIC = "fused ConvBN-LIF ms/layer @T=4 + end-to-end img/s; % of HBM/MFMA peak"
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="mobilenet_block",
+                    choices=["mobilenet_block", "conv3x3_block", "linear_block"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-operator timings of the other workloads")
+    return ap.parse_args()
+
+
+def _time_gpu(fn, steps: int, warmup: int):
+    """Average milliseconds per call of `fn`, HIP events on the stream the kernels are launched on."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall
+
+
+def _time_graph(fn, steps: int, warmup: int):
+    """Average milliseconds per replay of `fn` captured once into a HIP graph (launch overhead removed)."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+class Prepared:
+    """A workload moved to the device in its storage dtype, with closures for each fused operator."""
+
+    def __init__(self, wl, dtype, device):
+        import torch
+        from triton_snn_fusion_amd.runtime import snn_custom_ops  # noqa: F401  (registers torch.ops.snn_custom)
+        from triton_snn_fusion_amd import workloads as W
+        self.wl = wl
+        self.dtype = dtype
+        self.device = device
+        self.esize = torch.empty((), dtype=dtype).element_size()
+        self.x_seq = wl.x_seq.to(device=device, dtype=dtype)
+        self.xs = [self.x_seq[t] for t in range(wl.T)]
+        self.v0 = torch.zeros((), dtype=torch.float32, device=device)
+        self.lif = wl.lif
+        self.layers = []
+        ops = torch.ops.snn_custom
+        for layer in wl.conv_layers:
+            w = layer.weight.to(device=device, dtype=dtype)
+            b = layer.bias.to(device=device, dtype=dtype)
+            depthwise = layer.groups > 1
+            pointwise = tuple(layer.weight.shape[2:]) == (1, 1)
+            op = (ops.fused_temporal_depthwise_conv_lif_state if depthwise
+                  else ops.fused_temporal_pointwise_conv_lif_state if pointwise else ops.fused_temporal_conv_lif_state)
+            self.layers.append((op, w, b, list(layer.stride), list(layer.padding), layer.groups))
+        if wl.linear_weight is not None:
+            self.lw = wl.linear_weight.to(device=device, dtype=dtype)
+            self.lb = wl.linear_bias.to(device=device, dtype=dtype)
+        self.W = W
+
+    def run_layer(self, index: int, xs):
+        op, w, b, stride, padding, groups = self.layers[index]
+        return op(xs, w, b, self.v0, stride, padding, [1, 1], groups, self.lif[0], self.lif[1], self.lif[2], False)
+
+    def step(self):
+        import torch
+        if self.wl.linear_weight is not None:
+            return torch.ops.snn_custom.fused_temporal_linear_lif_state_packed(
+                self.x_seq, self.lw, self.lb, self.v0, self.lif[0], self.lif[1], self.lif[2], False)
+        xs = self.xs
+        out = None
+        for i in range(len(self.layers)):
+            out = self.run_layer(i, xs)
+            xs = [out[0][t] for t in range(self.wl.T)]
+        return out
+
+    def layer_inputs(self):
+        """Inputs of every conv layer when the block runs end to end (layer i consumes layer i-1's spikes)."""
+        xs = self.xs
+        per_layer = []
+        for i in range(len(self.layers)):
+            per_layer.append(xs)
+            out = self.run_layer(i, xs)
+            xs = [out[0][t] for t in range(self.wl.T)]
+        return per_layer
+
+    def layer_work(self, index: int, xs):
+        """(algorithmic bytes, flops) of conv layer `index`."""
+        _, w, _, stride, padding, groups = self.layers[index]
+        n, cin, h, wd = (int(d) for d in xs[0].shape)
+        cout, _, kh, kw = (int(d) for d in w.shape)
+        ho = (h + 2 * padding[0] - kh) // stride[0] + 1
+        wo = (wd + 2 * padding[1] - kw) // stride[1] + 1
+        T = self.wl.T
+        return (self.W.algorithmic_conv_bytes(T, n, cin, h, wd, cout, ho, wo, kh, kw, groups, self.esize, 4),
+                self.W.conv_flops(T, n, cin, cout, ho, wo, kh, kw, groups))
+
+
+def _roofline(bound: str, work: float, ms: float, traffic=None):
+    if bound == "hbm":
+        achieved = work / (ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = work / (ms * 1e-3) / 1e12
+        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": traffic}
+
+
+def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
+    """Eager fp32 PyTorch-CPU path (the oracle's restatement of the reference's eager ops) on a bounded sample."""
+    import torch
+    from oracle import snn_oracle as O
+    from triton_snn_fusion_amd import workloads as W
+    if wl_name == "mobilenet_block":
+        sample_batch = 4
+        wl = W.mobilenet_block(batch=sample_batch)
+    elif wl_name == "conv3x3_block":
+        sample_batch = 8
+        wl = W.conv3x3_block(batch=sample_batch)
+    else:
+        sample_batch = 64
+        wl = W.linear_block(batch=sample_batch)
+    v0 = torch.tensor(0.0)
+
+    def run():
+        if wl.linear_weight is not None:
+            return O.temporal_linear_lif(wl.x_seq, wl.linear_weight, wl.linear_bias, v0, *wl.lif)
+        xs = [wl.x_seq[t] for t in range(wl.T)]
+        out = None
+        for layer in wl.conv_layers:
+            out = O.temporal_conv_lif(xs, layer.weight, layer.bias, v0, layer.stride, layer.padding, (1, 1),
+                                      layer.groups, *wl.lif)
+            xs = [out[0][t] for t in range(wl.T)]
+        return out
+
+    run()  # warm-up
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 3 or (len(times) < 20 and time.perf_counter() - t_begin < seconds_budget):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    median = times[len(times) // 2]
+    return {
+        "value": round(sample_batch * wl.T / median, 2),
+        "unit": "images*T/s",
+        "cores": int(torch.get_num_threads()),
+        "kind": "port",
+        "sample": f"{wl_name} at batch {sample_batch} (of the GPU run's batch), fp32 eager PyTorch-CPU ops, "
+                  f"median of {len(times)} runs, {median * 1e3:.1f} ms per step",
+        "ms_per_step": round(median * 1e3, 3),
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the operators shard over the batch axis with no "
+              "communication; see DESIGN.md) - run with --gpus 1", file=sys.stderr)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    from triton_snn_fusion_amd import _lib, workloads as W
+    if not _lib.library_available():
+        import importlib
+        importlib.import_module("triton_snn_fusion_amd.build").build_library()
+    from triton_snn_fusion_amd.runtime import snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=True)
+    device = torch.device("cuda:0")
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+
+    wl = getattr(W, args.workload)()
+    prep = Prepared(wl, dtype, device)
+    prep.step()
+    torch.cuda.synchronize()
+
+    ms_step, wall_step = _time_gpu(prep.step, args.steps, args.warmup)
+    value = wl.batch * wl.T / (ms_step * 1e-3)
+    n_layers = max(1, len(prep.layers))
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "images*T/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "ms_per_layer": round(ms_step / n_layers, 4),
+        "host_ms_per_step": round(wall_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic (seed 0, Bernoulli spikes, Kaiming-normal weights, random eval-mode BN folded)",
+        "config": {"workload": args.workload, "T": wl.T, "batch": wl.batch, "membrane": "f32",
+                   "shape": list(wl.x_seq.shape)},
+    }
+
+    # Per-kernel timing, each operator alone on the launch stream.
+    kernels = {}
+    if prep.layers:
+        inputs = prep.layer_inputs()
+        torch.cuda.synchronize()
+        for i, xs in enumerate(inputs):
+            ms, _ = _time_gpu(lambda i=i, xs=xs: prep.run_layer(i, xs), args.steps, max(3, args.warmup // 2))
+            nbytes, flops = prep.layer_work(i, xs)
+            groups = prep.layers[i][5]
+            kind = "depthwise3x3" if groups > 1 else ("pointwise1x1" if tuple(prep.layers[i][1].shape[2:]) == (1, 1) else "conv")
+            kernels[f"layer{i}_{kind}"] = {
+                "ms": round(ms, 4), "algorithmic_bytes": nbytes, "flops": flops,
+                "hbm": _roofline("hbm", nbytes, ms), "mfma": None if groups > 1 else _roofline("mfma", flops, ms),
+            }
+        dominant = max(kernels.items(), key=lambda kv: kv[1]["ms"])
+        ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
+        bound = "mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS and dominant[1]["mfma"] is not None else "hbm"
+        result["roofline"] = dict(dominant[1][bound], kernel=dominant[0])
+    else:
+        T, M, fin, fout = wl.T, wl.batch, int(wl.linear_weight.shape[1]), int(wl.linear_weight.shape[0])
+        nbytes = (T * M * fin + fout * fin + fout) * prep.esize + T * M * fout * prep.esize + M * fout * 4
+        flops = 2 * T * M * fin * fout
+        kernels["linear_lif"] = {"ms": round(ms_step, 4), "algorithmic_bytes": nbytes, "flops": flops,
+                                 "hbm": _roofline("hbm", nbytes, ms_step), "mfma": _roofline("mfma", flops, ms_step)}
+        result["roofline"] = dict(kernels["linear_lif"]["hbm"], kernel="linear_lif")
+    result["kernels"] = kernels
+    try:
+        result["graph_ms_per_step"] = round(_time_graph(prep.step, args.steps, args.warmup), 4)
+    except Exception as exc:  # graph capture is a convenience measurement only
+        result["graph_ms_per_step"] = None
+        result["graph_error"] = str(exc)[:200]
+
+    if not args.no_extra:
+        extra = {}
+        for name in ("conv3x3_block", "linear_block", "mobilenet_block"):
+            if name == args.workload:
+                continue
+            other = Prepared(getattr(W, name)(), dtype if name != "conv3x3_block" else torch.float32, device)
+            other.step()
+            torch.cuda.synchronize()
+            ms, _ = _time_gpu(other.step, args.steps, max(3, args.warmup // 2))
+            entry = {"ms_per_step": round(ms, 4), "images_T_per_s": round(other.wl.batch * other.wl.T / (ms * 1e-3), 1),
+                     "dtype": "f32" if name == "conv3x3_block" else args.dtype}
+            try:
+                entry["graph_ms_per_step"] = round(_time_graph(other.step, args.steps, max(3, args.warmup // 2)), 4)
+            except Exception as exc:
+                entry["graph_error"] = str(exc)[:200]
+            extra[name] = entry
+        result["extra"] = extra
+
+    stats = ops.get_fused_op_call_stats()
+    result["native_calls"] = stats["triton"]
+    result["fallback_calls"] = stats["fallback"]
+    if stats["fallback"] != 0:
+        print(f"bench.py: {stats['fallback']} operator calls did not run on the HIP kernels: {stats['fallback_reasons']}",
+              file=sys.stderr)
+        return 1
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _cpu_baseline(args.workload)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

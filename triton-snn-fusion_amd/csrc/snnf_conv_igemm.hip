@@ -16,6 +16,10 @@
 //     image borders are handled by redirecting the lane to a zero pixel.
 #include "snnf_common.h"
 
+#include <map>
+#include <mutex>
+#include <tuple>
+
 namespace snnf {
 namespace {
 
@@ -25,7 +29,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int kWaves = 4;
 constexpr int kTilePixels = 128;  // output pixels per workgroup: one 32-pixel fragment per wave
 constexpr int kFragBytes = 1024;  // one packed 32(oc) x 16(k) weight fragment
 
@@ -147,8 +150,8 @@ __global__ __launch_bounds__(kThreads) void conv_lif_kernel(StepPtrs xs, StepPtr
     int iw_lo = c0 * g.sw - g.pw;
     if (g.pair_aligned && (iw_lo & 1)) iw_lo -= 1;
     const int tile_bytes = g.NR * g.WT * g.pitch;
-    const int zero_off = TT * tile_bytes;
     const int t_in = g.shared_x ? 1 : TT;
+    const int zero_off = t_in * tile_bytes;
 
     if (tid < g.pitch / 4) reinterpret_cast<uint32_t*>(lds + zero_off)[tid] = 0u;
 
@@ -293,30 +296,8 @@ __global__ __launch_bounds__(kThreads) void conv_lif_kernel(StepPtrs xs, StepPtr
     }
 }
 
-// Chooses the output tile (TH x TW <= 128 pixels) that wastes the fewest lanes, preferring full-width rows.
-void choose_tile(ConvGeom& g) {
-    const int rows = g.N * g.Ho;
-    double best = -1.0;
-    int best_tw = 1;
-    for (int tw = 1; tw <= g.Wo && tw <= kTilePixels; ++tw) {
-        int th = kTilePixels / tw;
-        if (th > rows) th = rows;
-        const int tx = (g.Wo + tw - 1) / tw;
-        const int ty = (rows + th - 1) / th;
-        const double useful = static_cast<double>(rows) * g.Wo;
-        const double issued = static_cast<double>(tx) * ty * kTilePixels;
-        // halo cost: staged input pixels per useful output pixel
-        const double staged = (static_cast<double>(th - 1) * g.sh + g.KH) * ((tw - 1) * g.sw + g.KW) / (static_cast<double>(th) * tw);
-        double score = useful / issued - 0.02 * staged;
-        if (tw == g.Wo) score += 0.03;  // contiguous stores across rows
-        if (score > best) { best = score; best_tw = tw; }
-    }
-    g.TW = best_tw;
-    g.TH = kTilePixels / best_tw;
-    if (g.TH > rows) g.TH = rows;
-    g.tiles_x = (g.Wo + g.TW - 1) / g.TW;
-    g.tiles_y = (rows + g.TH - 1) / g.TH;
-}
+constexpr size_t kMaxLds = 160 * 1024;
+constexpr size_t kPreferredLds = 80 * 1024;  // two workgroups per CU
 
 // Largest number of distinct input rows (global id n * H + ih) any tile row-band touches.
 int max_tile_rows(const ConvGeom& g) {
@@ -333,13 +314,72 @@ int max_tile_rows(const ConvGeom& g) {
     return worst;
 }
 
-constexpr size_t kMaxLds = 160 * 1024;
+// Chooses the output tile (TH x TW <= 128 pixels, TH rows of the flattened (n, oh) space) whose activation tile for
+// `t_in` timesteps fits LDS, wasting the fewest lanes and preferring full-width rows (contiguous stores) and a
+// footprint that lets two workgroups share a CU. Fills TH, TW, tiles_x, tiles_y, NR, WT. Returns the LDS bytes, 0 if
+// no tile fits.
+size_t plan_tile_uncached(ConvGeom& g, int t_in, bool pair_aligned) {
+    const int rows = g.N * g.Ho;
+    double best = -1e30;
+    size_t best_bytes = 0;
+    ConvGeom best_g = g;
+    for (int tw = 1; tw <= g.Wo && tw <= kTilePixels; ++tw) {
+        for (int px = kTilePixels; px >= 32; px >>= 1) {
+            int th = px / tw;
+            if (th < 1) continue;
+            if (th > rows) th = rows;
+            ConvGeom c = g;
+            c.TW = tw;
+            c.TH = th;
+            c.tiles_x = (g.Wo + tw - 1) / tw;
+            c.tiles_y = (rows + th - 1) / th;
+            c.NR = max_tile_rows(c);
+            c.WT = (tw - 1) * g.sw + g.KW + (pair_aligned ? 1 : 0);
+            c.WT = (c.WT + 1) & ~1;
+            const size_t bytes = static_cast<size_t>(t_in) * c.NR * c.WT * c.pitch + c.pitch;
+            if (bytes > kMaxLds) continue;
+            const double useful = static_cast<double>(rows) * g.Wo;
+            const double issued = static_cast<double>(c.tiles_x) * c.tiles_y * kTilePixels;
+            const double staged = static_cast<double>(c.NR) * c.WT / (static_cast<double>(th) * tw);
+            double score = useful / issued - 0.02 * staged;
+            if (tw == g.Wo) score += 0.03;
+            if (bytes > kPreferredLds) score -= 0.05;
+            if (score > best) { best = score; best_g = c; best_bytes = bytes; }
+        }
+    }
+    if (best_bytes != 0) g = best_g;
+    return best_bytes;
+}
+
+
+
+// Planning scans every candidate tile shape, so plans are memoised per problem geometry.
+size_t plan_tile(ConvGeom& g, int t_in, bool pair_aligned) {
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int>;
+    struct Plan { int TH, TW, tiles_x, tiles_y, NR, WT; size_t bytes; };
+    static std::mutex mu;
+    static std::map<Key, Plan> plans;
+    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, t_in, pair_aligned ? 1 : 0);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = plans.find(key);
+        if (it != plans.end()) {
+            const Plan& p = it->second;
+            g.TH = p.TH; g.TW = p.TW; g.tiles_x = p.tiles_x; g.tiles_y = p.tiles_y; g.NR = p.NR; g.WT = p.WT;
+            return p.bytes;
+        }
+    }
+    const size_t bytes = plan_tile_uncached(g, t_in, pair_aligned);
+    std::lock_guard<std::mutex> lock(mu);
+    plans[key] = Plan{g.TH, g.TW, g.tiles_x, g.tiles_y, g.NR, g.WT, bytes};
+    return bytes;
+}
 
 template <typename XT, typename VT, int TT, int NOF>
 int launch(const StepPtrs& xs, const StepPtrs& res, int has_res, ConvGeom g, const void* packed, const void* v_init,
            void* spikes, void* v_out, const LifParams& lif, hipStream_t stream) {
     g.oc_tiles = (g.Cout + 32 * NOF - 1) / (32 * NOF);
-    const size_t lds = static_cast<size_t>(TT) * g.NR * g.WT * g.pitch + g.pitch;
+    const size_t lds = static_cast<size_t>(g.shared_x ? 1 : TT) * g.NR * g.WT * g.pitch + g.pitch;
     if (lds > kMaxLds)
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: activation tile of %zu bytes exceeds LDS (W=%d, kernel %dx%d)", lds, g.W, g.KH, g.KW);
     const int64_t blocks = static_cast<int64_t>(g.tiles_x) * g.tiles_y * g.oc_tiles;
@@ -455,34 +495,47 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.CK = pg.CK; g.nchunks = pg.nchunks; g.npairs = pg.npairs;
     g.groups_log2 = pg.CK == 8 ? 0 : (pg.CK == 16 ? 1 : 2);
     g.pitch = pg.CK * 2 + 16;
-    choose_tile(g);
-    g.NR = max_tile_rows(g);
     const int xsize = dtype_size(x_dtype);
     g.spike_step_stride = spike_step_stride;
     const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
     hipStream_t hs = as_stream(stream);
 
     constexpr int kMaxTT = 4;
-    for (int t0 = 0; t0 < T; t0 += kMaxTT) {
-        const int tw = (T - t0) < kMaxTT ? (T - t0) : kMaxTT;
+    // Timesteps per launch: as many as fit LDS side by side (a shared analog frame needs one tile for any window).
+    bool all_shared = T > 1;
+    bool pair_ok = xsize == 2 && (W % 2 == 0);
+    for (int t = 0; t < T; ++t) {
+        all_shared = all_shared && xs[t] == xs[0];
+        pair_ok = pair_ok && aligned_to(xs[t], 4);
+    }
+    g.pair_aligned = pair_ok ? 1 : 0;
+    int window = T < kMaxTT ? T : kMaxTT;
+    {
+        int w2 = 1;
+        while (w2 < window) w2 *= 2;
+        window = w2;
+    }
+    size_t lds_bytes = 0;
+    while (true) {
+        lds_bytes = plan_tile(g, all_shared ? 1 : window, pair_ok);
+        if (lds_bytes != 0 || window == 1 || all_shared) break;
+        window >>= 1;
+    }
+    if (lds_bytes == 0)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: no activation tile fits LDS (W=%d, kernel %dx%d, stride %dx%d)", W, KH, KW, stride_h, stride_w);
+
+    for (int t0 = 0; t0 < T; t0 += window) {
+        const int tw = (T - t0) < window ? (T - t0) : window;
         int tt = 1;
         while (tt < tw) tt *= 2;
         StepPtrs xp = {}, rp = {};
-        bool pair_ok = xsize == 2 && (W % 2 == 0);
-        bool shared = true;
         for (int t = 0; t < tt; ++t) {
             xp.p[t] = xs[t0 + (t < tw ? t : 0)];  // padded steps repeat step 0 and are never stored
             if (residuals != nullptr) rp.p[t] = residuals[t0 + (t < tw ? t : 0)];
-            pair_ok = pair_ok && aligned_to(xp.p[t], 4);
-            shared = shared && xp.p[t] == xp.p[0];
         }
         ConvGeom gl = g;
         gl.T = tw;
-        gl.shared_x = (shared && tt > 1) ? 1 : 0;
-        gl.pair_aligned = pair_ok ? 1 : 0;
-        // Columns held per tile row; one extra when the first column was moved down to an even index; even count.
-        gl.WT = (g.TW - 1) * g.sw + g.KW + (pair_ok ? 1 : 0);
-        gl.WT = (gl.WT + 1) & ~1;
+        gl.shared_x = (all_shared && tt > 1) ? 1 : 0;
         const void* vi = t0 == 0 ? v_init : v_out;
         void* sp = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
         const int has_res = residuals != nullptr ? 1 : 0;
