@@ -1,0 +1,343 @@
+"""GPU parity tests: every fused operator, called through torch.ops.snn_custom (-> ctypes -> libsnnf C ABI -> HIP
+kernel), against the CPU oracle on the same seeded operands.
+
+Gate (tests/helpers.py:check): membrane within rtol 1e-3 / atol 1e-4; spike mismatches only where the oracle's pre-reset
+membrane is within 1e-3 of the threshold, at a rate <= 1e-4. 16-bit and fp32-on-matrix-core runs are compared with the
+oracle evaluated in fp32 on operands rounded the way the kernel rounds them (bf16 matrix operands, fp32 accumulate).
+"""
+import ctypes
+import json
+import os
+
+import pytest
+import torch
+
+from helpers import DEV, LIF, check, dev, gen, q, spikes, zero_v
+from oracle import snn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16, F16 = torch.float32, torch.bfloat16, torch.float16
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+S = torch.ops.snn_custom
+
+
+def _no_fallback(ops, expected_calls=None):
+    stats = ops.get_fused_op_call_stats()
+    assert stats["fallback"] == 0, stats["fallback_reasons"]
+    if expected_calls is not None:
+        assert stats["triton"] == expected_calls, stats
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Standalone temporal LIF
+# ---------------------------------------------------------------------------------------------------------------
+def test_lif_scan_known_answer_traces_through_the_c_abi(snnf_lib):
+    """tests/golden/lif_kat.json straight through snnf_lif_scan, bit exact (fp32 in, fp32 membrane)."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd import _lib
+    cases = json.load(open(os.path.join(GOLDEN, "lif_kat.json")))["cases"]
+    groups = {}
+    for c in cases:
+        groups.setdefault((c["v_threshold"], c["v_reset"], c["tau"], len(c["x"])), []).append(c)
+    for (v_th, v_reset, tau, T), members in groups.items():
+        x = torch.tensor([m["x"] for m in members], dtype=F32).t().contiguous().to(DEV)       # [T, n]
+        v0 = torch.tensor([m["v0"] for m in members], dtype=F32).to(DEV)
+        n = len(members)
+        out_s = torch.empty(T, n, device=DEV)
+        out_v = torch.empty(n, device=DEV)
+        rc = snnf_lib.snnf_lif_scan(_lib.packed_step_pointers(x), T, n, 0, v0.data_ptr(), 0, out_s.data_ptr(), n,
+                                    out_v.data_ptr(), v_th, v_reset, tau, _lib.current_stream(x.device))
+        assert rc == 0, snnf_lib.snnf_last_error()
+        torch.cuda.synchronize()
+        assert out_s.t().cpu().tolist() == [[float(k) for k in m["spikes"]] for m in members]
+        assert out_v.cpu().tolist() == [m["v"] for m in members]
+
+
+@pytest.mark.parametrize("dtype,vdtype", [(F32, F32), (BF16, F32), (BF16, BF16), (F16, F32), (F16, F16)])
+@pytest.mark.parametrize("T,shape", [(1, (2, 3, 5, 7)), (4, (2, 8, 14, 14)), (8, (1, 16, 7, 7)), (16, (2, 4, 8, 8)), (20, (1, 3, 9, 5))])
+def test_temporal_lif(hip_ops, dtype, vdtype, T, shape):
+    g = gen(100 + T)
+    x = q(torch.randn((T,) + shape, generator=g) * 0.75 + 0.15, dtype)
+    v0 = q(torch.randn(shape, generator=g) * 0.3, vdtype)
+    ref = O.temporal_lif(x, v0, *LIF)
+    s, v = S.fused_temporal_lif_state(dev(x, dtype), dev(v0, vdtype), *LIF, False)
+    assert s.dtype == dtype and v.dtype == vdtype and s.shape == x.shape
+    rep = check(s, v, ref, v_dtype=vdtype, what=f"lif {dtype} {vdtype} T={T}")
+    assert rep["near_threshold_flips"] == 0          # elementwise fp32 math: bit exact
+    _no_fallback(hip_ops, 1)
+
+
+@pytest.mark.parametrize("v_th,v_reset,tau", [(1.0, -1.0, 2.0), (0.5, 0.0, 1.0), (1.0, 0.25, 4.0), (0.75, 0.0, 1.5), (1.0, -1.0, 3.0)])
+def test_temporal_lif_general_neuron_parameters_are_bit_exact(hip_ops, v_th, v_reset, tau):
+    g = gen(7)
+    x = torch.randn((6, 2, 4, 9, 9), generator=g) * 0.9 + 0.3
+    ref = O.temporal_lif(x, torch.tensor(0.0), v_th, v_reset, tau)
+    s, v = S.fused_temporal_lif_state(dev(x, F32), zero_v(), v_th, v_reset, tau, False)
+    assert torch.equal(s.cpu(), ref[0]) and torch.equal(v.cpu(), ref[1])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Depthwise 3x3 + LIF
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,vdtype", [(F32, F32), (BF16, F32), (F16, F16)])
+@pytest.mark.parametrize("stride,N,C,H,W", [(1, 2, 16, 28, 28), (2, 2, 16, 28, 28), (1, 2, 24, 7, 7), (2, 1, 8, 7, 9),
+                                             (1, 1, 8, 56, 56), (2, 1, 4, 112, 112), (1, 3, 5, 9, 11), (1, 1, 2, 96, 160)])
+def test_depthwise_conv_lif(hip_ops, dtype, vdtype, stride, N, C, H, W):
+    g = gen(200 + H)
+    T = 4
+    xs = [spikes((N, C, H, W), 0.3, g) for _ in range(T)]
+    w = q(torch.randn(C, 1, 3, 3, generator=g) * 0.5, dtype)
+    b = q(torch.randn(C, generator=g) * 0.1, dtype)
+    ref = O.temporal_conv_lif(xs, w, b, torch.tensor(0.0), (stride, stride), (1, 1), (1, 1), C, *LIF)
+    s, v = S.fused_temporal_depthwise_conv_lif_state([dev(x, dtype) for x in xs], dev(w, dtype), dev(b, dtype), zero_v(vdtype),
+                                                     [stride, stride], [1, 1], [1, 1], C, *LIF, False)
+    check(s, v, ref, v_dtype=vdtype, what="depthwise")
+    _no_fallback(hip_ops, 1)
+    assert hip_ops.get_fused_op_call_stats()[f"temporal_depthwise_k3_s{stride}_p1"] == 1
+
+
+def test_depthwise_residual_alias_and_membrane_chaining(hip_ops):
+    g = gen(21)
+    N, C, H, W, T = 2, 16, 14, 14, 4
+    xs = [q(torch.randn(N, C, H, W, generator=g), BF16) for _ in range(T)]     # analog inputs
+    rs = [q(torch.randn(N, C, H, W, generator=g) * 0.3, BF16) for _ in range(T)]
+    w, b = q(torch.randn(C, 1, 3, 3, generator=g) * 0.3, BF16), q(torch.randn(C, generator=g) * 0.1, BF16)
+    v0 = torch.randn(N, C, H, W, generator=g) * 0.2
+    ref = O.temporal_conv_lif(xs, w, b, v0, (1, 1), (1, 1), (1, 1), C, *LIF, residuals=rs)
+    dx, dr = [dev(x, BF16) for x in xs], [dev(r, BF16) for r in rs]
+    args = (dev(w, BF16), dev(b, BF16))
+    s, v = S.fused_temporal_conv_add_lif_state_depthwise(dx, dr, *args, dev(v0, F32), [1, 1], [1, 1], [1, 1], C, *LIF, False)
+    check(s, v, ref, what="depthwise residual")
+    # two chained windows of 2 steps == one window of 4 steps, bit for bit
+    s1, v1 = S.fused_temporal_conv_add_lif_state(dx[:2], dr[:2], *args, dev(v0, F32), [1, 1], [1, 1], [1, 1], C, *LIF, False)
+    s2, v2 = S.fused_temporal_conv_add_lif_state(dx[2:], dr[2:], *args, v1, [1, 1], [1, 1], [1, 1], C, *LIF, False)
+    assert torch.equal(torch.cat([s1, s2]), s) and torch.equal(v2, v)
+    # the alias operator name of the reference
+    s3, v3 = S.fused_temporal_conv_lif_state_depthwise(dx, *args, dev(v0, F32), [1, 1], [1, 1], [1, 1], C, *LIF, False)
+    ref3 = O.temporal_conv_lif(xs, w, b, v0, (1, 1), (1, 1), (1, 1), C, *LIF)
+    check(s3, v3, ref3, what="depthwise alias")
+    _no_fallback(hip_ops, 4)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# LIF -> AvgPool -> Linear tail
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+@pytest.mark.parametrize("T,N,C,H,W,K,bias", [(4, 3, 32, 7, 7, 10, True), (4, 4, 512, 1, 1, 10, True), (4, 4, 512, 2, 2, 1000, True),
+                                               (4, 16, 512, 7, 7, 1000, True), (8, 2, 48, 5, 3, 17, False), (1, 1, 8, 32, 32, 3, True)])
+def test_lif_avgpool_linear(hip_ops, dtype, T, N, C, H, W, K, bias):
+    g = gen(300 + C)
+    x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + 0.15, dtype)
+    w = q(torch.randn(K, C, generator=g) * 0.05, dtype)
+    b = q(torch.randn(K, generator=g) * 0.05, dtype) if bias else None
+    ref_out, ref_v, _, _ = O.temporal_lif_avgpool_linear(x, torch.tensor(0.0), w, b, *LIF)
+    fb = dev(b, dtype) if bias else torch.empty(0, device=DEV, dtype=dtype)
+    op = S.fused_temporal_lif_avgpool_linear if T != 8 else S.fused_temporal_lif_tail
+    out, v = op(dev(x, dtype), zero_v(F32), dev(w, dtype), fb, *LIF, False)
+    assert out.dtype == dtype and tuple(out.shape) == (N, K) and v.dtype == F32
+    assert torch.equal(v.cpu(), ref_v)                              # elementwise LIF: exact
+    tol = 1e-4 if dtype == F32 else (8e-3 if dtype == BF16 else 2e-3)   # out_sum is stored in the activation dtype
+    assert torch.allclose(out.float().cpu(), ref_out, rtol=tol, atol=tol), (out.float().cpu() - ref_out).abs().max()
+    _no_fallback(hip_ops, 1)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Temporal Linear + LIF
+# ---------------------------------------------------------------------------------------------------------------
+def _linear_case(seed, T, M, Fin, Fout, dtype, bias=True, p=0.1):
+    g = gen(seed)
+    x = spikes((T, M, Fin), p, g)
+    w = torch.randn(Fout, Fin, generator=g) * (2.0 / Fin) ** 0.5 * 3.0
+    b = torch.randn(Fout, generator=g) * 0.01 if bias else None
+    wq = q(w, BF16 if dtype == F32 else dtype)        # fp32 operands are rounded to bf16 by the kernel
+    bq = None if b is None else q(b, dtype)
+    return x, w if dtype == F32 else wq, b if dtype == F32 else bq, wq, bq if b is not None else None
+
+
+@pytest.mark.parametrize("dtype,vdtype", [(BF16, F32), (F32, F32), (F16, F16), (BF16, BF16)])
+@pytest.mark.parametrize("T,M,Fin,Fout,bias", [(8, 64, 256, 128, True), (3, 5, 100, 37, True), (16, 1, 512, 512, False),
+                                                (4, 16, 1000, 48, True), (20, 3, 64, 16, True), (2, 33, 96, 130, True)])
+def test_linear_lif_packed(hip_ops, dtype, vdtype, T, M, Fin, Fout, bias):
+    x, w_dev, b_dev, w_ref, b_ref = _linear_case(400 + Fin, T, M, Fin, Fout, dtype, bias)
+    ref = O.temporal_linear_lif(x, w_ref, b_ref, torch.tensor(0.0), *LIF)
+    s, v = S.fused_temporal_linear_lif_state_packed(dev(x, dtype), dev(w_dev, dtype), dev(b_dev, dtype), zero_v(vdtype), *LIF, False)
+    assert tuple(s.shape) == (T, M, Fout) and s.dtype == dtype and v.dtype == vdtype
+    check(s, v, ref, v_dtype=vdtype, what="linear packed")
+    _no_fallback(hip_ops, 1)
+
+
+def test_linear_lif_list_out_and_leading_dims_forms_agree(hip_ops):
+    T, M, Fin, Fout = 4, 12, 192, 80
+    x, w_dev, b_dev, w_ref, b_ref = _linear_case(77, T, M, Fin, Fout, BF16)
+    ref = O.temporal_linear_lif(x, w_ref, b_ref, torch.tensor(0.0), *LIF)
+    dx, dw, db = dev(x, BF16), dev(w_dev, BF16), dev(b_dev, BF16)
+    s, v = S.fused_temporal_linear_lif_state_packed(dx, dw, db, zero_v(), *LIF, False)
+    check(s, v, ref, what="linear packed")
+    s_l, v_l = S.fused_temporal_linear_lif_state([dx[t] for t in range(T)], dw, db, zero_v(), *LIF, False)
+    assert torch.equal(s_l, s) and torch.equal(v_l, v)
+    so, vo = torch.empty_like(s), torch.empty_like(v)
+    assert S.fused_temporal_linear_lif_state_packed_out(dx, dw, db, zero_v(), *LIF, False, so, vo) is None
+    assert torch.equal(so, s) and torch.equal(vo, v)
+    s4, v4 = S.fused_temporal_linear_lif_state_packed(dx.reshape(T, 3, 4, Fin), dw, db, zero_v(), *LIF, False)
+    assert tuple(s4.shape) == (T, 3, 4, Fout) and torch.equal(s4.reshape(T, M, Fout), s) and torch.equal(v4.reshape(M, Fout), v)
+    # window chaining through a full-shape fp32 v_init
+    s1, v1 = S.fused_temporal_linear_lif_state_packed(dx[:1], dw, db, zero_v(), *LIF, False)
+    s2, v2 = S.fused_temporal_linear_lif_state_packed(dx[1:], dw, db, v1, *LIF, False)
+    assert torch.equal(torch.cat([s1, s2]), s) and torch.equal(v2, v)
+    _no_fallback(hip_ops, 6)
+    assert hip_ops.get_fused_op_call_stats()["temporal_linear_lif_stack_materialized"] == 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Dense conv (implicit GEMM) + LIF
+# ---------------------------------------------------------------------------------------------------------------
+def _conv_case(seed, T, N, Cin, Cout, H, W, k, dtype, analog=False, p=0.2, gain=2.0):
+    g = gen(seed)
+    if analog:
+        xs = [q(torch.randn(N, Cin, H, W, generator=g), BF16 if dtype == F32 else dtype) for _ in range(T)]
+    else:
+        xs = [spikes((N, Cin, H, W), p, g) for _ in range(T)]
+    w = torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * k * k)) ** 0.5 * gain
+    b = torch.randn(Cout, generator=g) * 0.1
+    w_ref = q(w, BF16 if dtype == F32 else dtype)
+    b_ref = b if dtype == F32 else q(b, dtype)
+    w_dev = w if dtype == F32 else w_ref
+    return xs, w_dev, b_ref, w_ref, b_ref
+
+
+CONV_KEYS = [  # k, stride, pad, Cin, Cout, H, W, analog
+    (1, 1, 0, 32, 64, 12, 12, False),
+    (3, 1, 1, 16, 32, 12, 12, False),
+    (3, 2, 1, 16, 32, 12, 12, False),
+    (3, 2, 1, 8, 16, 7, 7, False),
+    (5, 1, 2, 8, 16, 9, 9, False),
+    (7, 2, 3, 3, 64, 32, 32, True),
+    (11, 4, 2, 3, 64, 63, 63, True),
+    (3, 1, 1, 40, 70, 14, 14, False),
+    (3, 1, 1, 64, 64, 7, 7, False),
+    (3, 1, 1, 3, 64, 32, 32, True),
+    (1, 1, 0, 128, 256, 14, 14, False),
+    (3, 1, 0, 16, 16, 10, 10, False),
+    (1, 2, 0, 64, 128, 14, 14, False),
+]
+
+
+@pytest.mark.parametrize("dtype,vdtype", [(BF16, F32), (F32, F32), (F16, F16)])
+@pytest.mark.parametrize("k,s,p,Cin,Cout,H,W,analog", CONV_KEYS)
+def test_conv_lif_kernel_keys(hip_ops, dtype, vdtype, k, s, p, Cin, Cout, H, W, analog):
+    T, N = 4, 2
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(500 + k * 10 + s, T, N, Cin, Cout, H, W, k, dtype, analog)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, torch.tensor(0.0), (s, s), (p, p), (1, 1), 1, *LIF)
+    op = S.fused_temporal_pointwise_conv_lif_state if (k, s, p) == (1, 1, 0) else S.fused_temporal_conv_lif_state
+    sp, v = op([dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype), zero_v(vdtype), [s, s], [p, p], [1, 1], 1, *LIF, False)
+    assert sp.dtype == dtype and v.dtype == vdtype and tuple(sp.shape) == tuple(ref[0].shape)
+    check(sp, v, ref, v_dtype=vdtype, what=f"conv k{k} s{s} p{p}")
+    _no_fallback(hip_ops, 1)
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 5, 8, 16])
+def test_conv_lif_timestep_counts_and_windows(hip_ops, T):
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(600 + T, T, 2, 32, 48, 10, 10, 3, BF16)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), 1, *LIF)
+    sp, v = S.fused_temporal_conv_lif_state([dev(x, BF16) for x in xs], dev(w_dev, BF16), dev(b_dev, BF16), zero_v(), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+    check(sp, v, ref, what=f"conv T={T}")
+    _no_fallback(hip_ops, 1)
+
+
+def test_conv_residual_chaining_packed_out_single_step_and_batched_tn(hip_ops):
+    T, N, Cin, Cout, H, W = 4, 3, 64, 64, 14, 14
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(31, T, N, Cin, Cout, H, W, 3, BF16)
+    g = gen(32)
+    rs = [q(torch.randn(N, Cout, H, W, generator=g) * 0.3, BF16) for _ in range(T)]
+    v0 = torch.randn(N, Cout, H, W, generator=g) * 0.2
+    dx, dr, dw, db = [dev(x, BF16) for x in xs], [dev(r, BF16) for r in rs], dev(w_dev, BF16), dev(b_dev, BF16)
+    geo = ([1, 1], [1, 1], [1, 1], 1)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (1, 1), (1, 1), (1, 1), 1, *LIF, residuals=rs)
+    s, v = S.fused_temporal_conv_add_lif_state(dx, dr, dw, db, dev(v0, F32), *geo, *LIF, False)
+    check(s, v, ref, what="conv residual")
+    s_tn, v_tn = S.fused_temporal_conv_add_lif_state_batched_tn(dx, dr, dw, db, dev(v0, F32), *geo, *LIF, False)
+    assert torch.equal(s_tn, s.flatten(0, 1)) and torch.equal(v_tn, v)
+    s1, v1 = S.fused_temporal_conv_add_lif_state(dx[:3], dr[:3], dw, db, dev(v0, F32), *geo, *LIF, False)
+    s2, v2 = S.fused_temporal_conv_add_lif_state(dx[3:], dr[3:], dw, db, v1, *geo, *LIF, False)
+    assert torch.equal(torch.cat([s1, s2]), s) and torch.equal(v2, v)
+    # packed input + caller-owned outputs == list form
+    ref_p = O.temporal_conv_lif(xs, w_ref, b_ref, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), 1, *LIF)
+    s_l, v_l = S.fused_temporal_conv_lif_state(dx, dw, db, zero_v(), *geo, *LIF, False)
+    check(s_l, v_l, ref_p, what="conv list")
+    so, vo = torch.empty_like(s_l), torch.empty_like(v_l)
+    assert S.fused_temporal_conv_lif_state_packed_out(torch.stack(dx), dw, db, zero_v(), *geo, *LIF, False, so, vo) is None
+    assert torch.equal(so, s_l) and torch.equal(vo, v_l)
+    s_b, v_b = S.fused_temporal_conv_lif_state_batched_tn(dx, dw, db, zero_v(), *geo, *LIF, False)
+    assert torch.equal(s_b, s_l.flatten(0, 1))
+    # single-step operator == first step of the temporal operator
+    s0, v0_ = S.fused_conv_lif_state(dx[0], dw, db, zero_v(), *geo, *LIF, False)
+    assert torch.equal(s0, s_l[0])
+    _no_fallback(hip_ops, 8)
+
+
+def test_conv_shared_analog_frame_is_convolved_once_and_matches(hip_ops):
+    """Direct encoding: the same analog frame feeds every timestep (the T list entries alias one tensor)."""
+    g = gen(41)
+    x = q(torch.randn(2, 3, 32, 32, generator=g), BF16)
+    w = q(torch.randn(64, 3, 3, 3, generator=g) * 0.4, BF16)
+    b = q(torch.randn(64, generator=g) * 0.1, BF16)
+    ref = O.temporal_conv_lif([x] * 4, w, b, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), 1, *LIF)
+    dx = dev(x, BF16)
+    s, v = S.fused_temporal_conv_lif_state([dx] * 4, dev(w, BF16), dev(b, BF16), zero_v(), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+    check(s, v, ref, what="shared frame")
+    s2, v2 = S.fused_temporal_conv_lif_state([dx.clone() for _ in range(4)], dev(w, BF16), dev(b, BF16), zero_v(), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+    assert torch.equal(s, s2) and torch.equal(v, v2)
+
+
+def test_conv_and_linear_known_answers_exact(hip_ops):
+    """tests/golden/conv_kat.json: exact sums (multiples of 1/8), so bf16 matrix operands must reproduce them bit for
+    bit. An integrate-and-fire neuron (tau <= 1) with an unreachable threshold makes v_out the convolution output."""
+    cases = json.load(open(os.path.join(GOLDEN, "conv_kat.json")))["cases"]
+    calls = 0
+    for c in cases:
+        for dtype in (F32, BF16):
+            if c["kind"] == "conv2d":
+                x = torch.tensor(c["x"]).reshape(c["N"], c["Cin"], c["H"], c["W"])
+                w = torch.tensor(c["w"]).reshape(c["Cout"], c["Cin"] // c["groups"], c["KH"], c["KW"])
+                b = torch.tensor(c["b"])
+                want = torch.tensor(c["out"]).reshape(c["N"], c["Cout"], c["Ho"], c["Wo"])
+                op = S.fused_temporal_depthwise_conv_lif_state if c["groups"] > 1 else S.fused_temporal_conv_lif_state
+                s, v = op([dev(x, dtype)], dev(w, dtype), dev(b, dtype), zero_v(), c["stride"], c["padding"], [1, 1], c["groups"], 1e30, 0.0, 1.0, False)
+            else:
+                x = torch.tensor(c["x"]).reshape(1, c["M"], c["Fin"])
+                w = torch.tensor(c["w"]).reshape(c["Fout"], c["Fin"])
+                b = torch.tensor(c["b"])
+                want = torch.tensor(c["out"]).reshape(c["M"], c["Fout"])
+                s, v = S.fused_temporal_linear_lif_state_packed(dev(x, dtype), dev(w, dtype), dev(b, dtype), zero_v(), 1e30, 0.0, 1.0, False)
+            calls += 1
+            assert torch.equal(v.cpu(), want), (c["kind"], dtype, (v.cpu() - want).abs().max())
+            assert float(s.float().abs().sum()) == 0.0
+    _no_fallback(hip_ops, calls)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Failure handling through the operator layer
+# ---------------------------------------------------------------------------------------------------------------
+def test_unsupported_configurations_fall_back_to_eager_ops_on_the_gpu_and_are_counted(snnf_lib):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd.runtime import snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=False)
+    ops.reset_fused_op_call_stats()
+    try:
+        g = gen(3)
+        xs = [spikes((1, 4, 9, 9), 0.3, g) for _ in range(2)]
+        w, b = torch.randn(4, 4, 3, 3, generator=g), torch.randn(4, generator=g)
+        ref = O.temporal_conv_lif(xs, w, b, torch.tensor(0.0), (1, 1), (2, 2), (2, 2), 1, *LIF)
+        s, v = S.fused_temporal_conv_lif_state([dev(x, F32) for x in xs], dev(w, F32), dev(b, F32), zero_v(), [1, 1], [2, 2], [2, 2], 1, *LIF, False)
+        check(s, v, ref, what="dilated fallback")
+        stats = ops.get_fused_op_call_stats()
+        assert stats["fallback"] == 1 and stats["triton"] == 0
+        assert stats["fallback_reasons"] == {"temporal:unsupported_dilation": 1}
+        ops.configure_fused_op("hip", strict_triton=True)
+        with pytest.raises(RuntimeError, match="unsupported_dilation"):
+            S.fused_temporal_conv_lif_state([dev(x, F32) for x in xs], dev(w, F32), dev(b, F32), zero_v(), [1, 1], [2, 2], [2, 2], 1, *LIF, False)
+    finally:
+        ops.configure_fused_op("torch")

@@ -150,7 +150,7 @@ def check_triton_support(x, weight, bias, v_prev, stride, padding, dilation, gro
         reasons.append(f"unsupported_rank: x.dim must be 4, got {x.dim()}")
     if weight.dim() != 4:
         reasons.append(f"unsupported_rank: weight.dim must be 4, got {weight.dim()}")
-    if reasons:
+    if x.dim() != 4 or weight.dim() != 4:
         return reasons
     groups = int(groups)
     depthwise = int(weight.shape[1]) == 1 and groups == int(x.shape[1]) == int(weight.shape[0]) and groups > 1
@@ -176,7 +176,7 @@ def check_triton_support(x, weight, bias, v_prev, stride, padding, dilation, gro
             reasons.append(f"unsupported_kernel: kernel {k} larger than padded input {tuple(x.shape[2:])}")
     if float(tau) == 0.0:
         reasons.append("unsupported_tau: tau must be nonzero")
-    if not reasons and isinstance(v_prev, torch.Tensor) and v_prev.dim() != 0:
+    if isinstance(v_prev, torch.Tensor) and v_prev.dim() != 0:
         out_shape = _conv2d_output_shape(x, weight, stride, padding, dilation)
         if tuple(v_prev.shape) != tuple(out_shape):
             reasons.append(f"v_prev shape {tuple(v_prev.shape)} does not match conv output shape {out_shape}")

@@ -8,6 +8,8 @@ Workloads (T = timesteps, B = batch):
   linear_block      Linear(2048->1024, bias N(0, 0.01^2)) + LIF, T=8, B=64, Bernoulli(0.1) spikes
   mobilenet_block   depthwise Conv3x3(128) + BN + LIF, then pointwise Conv1x1(128->256) + BN + LIF, T=4, B=32, 56x56,
                     Bernoulli(0.15) spikes
+`gain` (default 1) scales the Kaiming weights: with the plain recipe most layers are nearly silent (spike rates of
+1e-2 down to 1e-7), so the parity tests also run gain 3, where 7-15 % of the neurons fire every step.
 BatchNorm statistics: gamma ~ U(0.8, 1.2), beta ~ N(0, 0.1^2), running_mean ~ N(0, 0.1^2), running_var ~ U(0.5, 1.5),
 eps 1e-5. Conv / linear weights are Kaiming-normal (std = sqrt(2 / fan_in)). LIF: tau 2, v_th 1, hard reset to 0.
 """
@@ -92,26 +94,29 @@ class Workload:
     lif: Tuple[float, float, float] = LIF_DEFAULT
 
 
-def conv3x3_block(seed: int = 0, T: int = 4, batch: int = 8, channels: int = 64, size: int = 32) -> Workload:
+def conv3x3_block(seed: int = 0, T: int = 4, batch: int = 8, channels: int = 64, size: int = 32,
+                  gain: float = 1.0) -> Workload:
     g = _generator(seed)
     x = bernoulli_spikes((T, batch, channels, size, size), 0.2, g)
-    w, b = folded_conv_bn(kaiming_normal((channels, channels, 3, 3), g), g)
+    w, b = folded_conv_bn(kaiming_normal((channels, channels, 3, 3), g) * gain, g)
     return Workload("conv3x3_block", T, batch, x, [ConvLayer(w, b)])
 
 
-def linear_block(seed: int = 0, T: int = 8, batch: int = 64, fin: int = 2048, fout: int = 1024) -> Workload:
+def linear_block(seed: int = 0, T: int = 8, batch: int = 64, fin: int = 2048, fout: int = 1024,
+                 gain: float = 1.0) -> Workload:
     g = _generator(seed)
     x = bernoulli_spikes((T, batch, fin), 0.1, g)
-    w = kaiming_normal((fout, fin), g)
+    w = kaiming_normal((fout, fin), g) * gain
     b = torch.randn(fout, generator=g) * 0.01
     return Workload("linear_block", T, batch, x, linear_weight=w, linear_bias=b)
 
 
-def mobilenet_block(seed: int = 0, T: int = 4, batch: int = 32, cin: int = 128, cout: int = 256, size: int = 56) -> Workload:
+def mobilenet_block(seed: int = 0, T: int = 4, batch: int = 32, cin: int = 128, cout: int = 256, size: int = 56,
+                    gain: float = 1.0) -> Workload:
     g = _generator(seed)
     x = bernoulli_spikes((T, batch, cin, size, size), 0.15, g)
-    dw_w, dw_b = folded_conv_bn(kaiming_normal((cin, 1, 3, 3), g), g)
-    pw_w, pw_b = folded_conv_bn(kaiming_normal((cout, cin, 1, 1), g), g)
+    dw_w, dw_b = folded_conv_bn(kaiming_normal((cin, 1, 3, 3), g) * gain, g)
+    pw_w, pw_b = folded_conv_bn(kaiming_normal((cout, cin, 1, 1), g) * gain, g)
     return Workload("mobilenet_block", T, batch, x,
                     [ConvLayer(dw_w, dw_b, (1, 1), (1, 1), cin), ConvLayer(pw_w, pw_b, (1, 1), (0, 0), 1)])
 
