@@ -122,14 +122,14 @@ int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int64_t x_row_
  * dilation is 1.
  *
  * Two steps: (1) snnf_conv_pack_weight rewrites the OIHW weight (+ bias) into the matrix-core operand order once per
- * weight tensor; (2) snnf_conv_lif consumes the packed weight on every call. The packed buffer is opaque; its size is
- * snnf_conv_packed_weight_bytes(). fp32 activations/weights are rounded to bf16 for the matrix cores (fp32
+ * weight tensor and activation dtype; (2) snnf_conv_lif consumes the packed weight on every call. The packed buffer is
+ * opaque; its size is snnf_conv_packed_weight_bytes(). fp32 activations/weights are rounded to bf16 for the matrix cores (fp32
  * accumulate); fp16 activations use the fp16 matrix path.
  *   xs[t]        : [N, Cin, H, W] x_dtype
  *   residuals[t] : [N, Cout, Ho, Wo] x_dtype or residuals == NULL
  *   spikes       : [T, N, Cout, Ho, Wo] x_dtype (timestep stride `spike_step_stride` elements); v_out : [N, Cout, Ho, Wo] v_dtype
  */
-size_t snnf_conv_packed_weight_bytes(int Cout, int Cin, int KH, int KW);
+size_t snnf_conv_packed_weight_bytes(int Cout, int Cin, int KH, int KW, int x_dtype);
 int snnf_conv_pack_weight(const void* weight, const void* bias /* nullable */, int w_dtype,
                           int Cout, int Cin, int KH, int KW, int x_dtype,
                           void* packed, size_t packed_bytes, void* stream);

@@ -56,11 +56,12 @@ def test_argument_validation_happens_before_any_gpu_work(snnf_lib):
 
 def test_packed_weight_size_is_whole_fragments(snnf_lib):
     # [ceil(Cout/32)][ceil(Cin/CK)][ceil(taps * CK/8 / 2)] fragments of 1 KiB + fp32 bias
-    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3) == 2 * 2 * 18 * 1024 + 64 * 4
-    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 3, 7, 7) == 2 * 1 * 25 * 1024 + 64 * 4
-    assert snnf_lib.snnf_conv_packed_weight_bytes(70, 40, 1, 1) == 3 * 2 * 2 * 1024 + 96 * 4
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 1) == 2 * 2 * 18 * 1024 + 64 * 4
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 0) == 2 * 4 * 9 * 1024 + 64 * 4   # fp32 activations: 16-channel chunks
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 3, 7, 7, 1) == 2 * 1 * 25 * 1024 + 64 * 4
+    assert snnf_lib.snnf_conv_packed_weight_bytes(70, 40, 1, 1, 2) == 3 * 1 * 4 * 1024 + 96 * 4     # pointwise: one 64-channel chunk
     assert snnf_lib.snnf_lif_pool_linear_workspace_bytes(16, 512) == 16 * 512 * 4
-    assert snnf_lib.snnf_conv_packed_weight_bytes(0, 3, 3, 3) == 0
+    assert snnf_lib.snnf_conv_packed_weight_bytes(0, 3, 3, 3, 1) == 0
 
 
 @pytest.mark.parametrize("shape,stride,padding,groups,key", [

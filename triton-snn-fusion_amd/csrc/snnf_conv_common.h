@@ -1,0 +1,99 @@
+// Geometry shared by the weight packer, the tile planner and the implicit-GEMM conv+LIF kernel.
+#pragma once
+
+#include "snnf_common.h"
+
+namespace snnf {
+
+constexpr int kConvThreads = 256;   // 4 waves
+constexpr int kFragBytes = 1024;    // one packed 32(oc) x 16(k) weight fragment: 64 lanes x 16 bytes
+constexpr int kNPF = 2;             // pixel fragments per wave: a lane owns 2 adjacent output pixels
+constexpr int kNOF = 2;             // output-channel fragments per wave (64 channels)
+constexpr int kMaxItems = 8;        // staging items (8 channels x 2 pixels) per thread and channel chunk
+constexpr size_t kMaxLds = 160 * 1024;
+
+// Channels per chunk staged in LDS; fixed by (Cin, taps, activation width) alone so that packing and the kernel agree.
+// Pointwise convolutions take up to 128 channels at a time (no halo re-use to pay for), everything else 32; fp32
+// activations need two prefetch registers per fetch and therefore use chunks of half the size.
+__host__ __device__ inline int chunk_channels(int Cin, int taps, bool wide_activations) {
+    if (Cin <= 8) return 8;
+    if (Cin <= 16) return 16;
+    if (taps > 1) return wide_activations ? 16 : 32;
+    if (Cin <= 32) return 32;
+    if (Cin <= 64 || wide_activations) return 64;
+    return 128;
+}
+
+struct PackGeom {
+    int Cout, Cin, KH, KW;
+    int CK, nchunks, npairs, nocf;
+};
+
+__host__ __device__ inline PackGeom make_pack_geom(int Cout, int Cin, int KH, int KW, bool wide_activations) {
+    PackGeom p;
+    p.Cout = Cout;
+    p.Cin = Cin;
+    p.KH = KH;
+    p.KW = KW;
+    p.CK = chunk_channels(Cin, KH * KW, wide_activations);
+    p.nchunks = (Cin + p.CK - 1) / p.CK;
+    const int slots = KH * KW * (p.CK / 8);
+    p.npairs = (slots + 1) / 2;
+    p.nocf = (Cout + 31) / 32;
+    return p;
+}
+
+// 16-bit elements of the packed weight: [oc fragment][channel chunk][slot pair][lane 0..63][8]; fp32 bias follows.
+// Slot s of a chunk = tap * (CK / 8) + channel group; pair p holds slots 2p (lanes 0-31) and 2p + 1 (lanes 32-63).
+__host__ __device__ inline size_t packed_weight_elems(const PackGeom& p) {
+    return static_cast<size_t>(p.nocf) * p.nchunks * p.npairs * (kFragBytes / 2);
+}
+
+// How activations are fetched from global memory while staging: two adjacent pixels of one channel per fetch.
+enum LoadMode : int {
+    LOAD_PAIR32 = 0,   // 16-bit activations, pixel pairs 4-byte aligned: one dword load
+    LOAD_2X16 = 1,     // 16-bit activations, unaligned: two halfword loads
+    LOAD_2XF32 = 2     // fp32 activations: two dword loads, rounded to bf16 on the way into LDS
+};
+
+// Staging items a thread may hold in flight per chunk: modes that need two registers per fetch get half as many.
+__host__ __device__ constexpr int staging_items(int load_mode) { return load_mode == LOAD_PAIR32 ? kMaxItems : kMaxItems / 2; }
+
+struct ConvGeom {
+    int N, Cin, H, W, Cout, KH, KW, sh, sw, ph, pw, Ho, Wo;
+    int TH, TW;               // output tile: TH rows of the flattened (n, oh) row space x TW columns
+    int tiles_x, tiles_y;     // ceil(Wo / TW), ceil(N * Ho / TH)
+    int wm_log2, wn_log2;     // waves along pixels / along output channels (WM * WN == 4)
+    int oc_tiles;             // ceil(Cout / (WN * 64))
+    int CK, nchunks, npairs, groups_log2;
+    int NR, WT;               // LDS tile: input rows x input columns (per timestep)
+    int pitch;                // bytes per LDS pixel = CK * 2 + 16
+    int T;                    // timesteps stored by this launch (<= TT)
+    int shared_x;             // every timestep reads the same activation tensor: convolve once
+    int vec_store;            // a lane's two pixels are adjacent and aligned in memory
+    int64_t spike_step_stride;
+    int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
+};
+
+struct ConvLaunch {
+    StepPtrs xs;
+    StepPtrs residuals;
+    int has_residual;
+    ConvGeom g;
+    const uint16_t* wpacked;
+    const float* bias;
+    const void* v_init;
+    void* spikes;
+    void* v_out;
+    LifParams lif;
+    int grid;
+    size_t lds_bytes;
+    hipStream_t stream;
+};
+
+// One launcher per activation dtype (each in its own translation unit so they compile in parallel).
+int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode);
+int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode);
+int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode);
+
+}  // namespace snnf

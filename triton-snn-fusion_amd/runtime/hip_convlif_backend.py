@@ -264,7 +264,7 @@ def _packed_weight(weight: torch.Tensor, bias: Optional[torch.Tensor], x_dtype: 
     cout, cin, kh, kw = (int(d) for d in weight.shape)
     w = weight if weight.is_contiguous() else weight.contiguous()
     b = None if bias is None else (bias if bias.is_contiguous() else bias.contiguous())
-    nbytes = int(lib.snnf_conv_packed_weight_bytes(cout, cin, kh, kw))
+    nbytes = int(lib.snnf_conv_packed_weight_bytes(cout, cin, kh, kw, _lib.dtype_code(x_dtype)))
     packed = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
     _lib.check("snnf_conv_pack_weight", lib.snnf_conv_pack_weight(
         w.data_ptr(), _lib.ptr(b), _lib.dtype_code(weight.dtype), cout, cin, kh, kw, _lib.dtype_code(x_dtype),
