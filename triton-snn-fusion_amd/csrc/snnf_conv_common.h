@@ -11,6 +11,8 @@ constexpr int kNPF = 2;             // pixel fragments per wave: a lane owns 2 a
 constexpr int kNOF = 2;             // output-channel fragments per wave (64 channels)
 constexpr int kMaxItems = 8;        // staging items (8 channels x 2 pixels) per thread and channel chunk
 constexpr size_t kMaxLds = 160 * 1024;
+constexpr int kEpiPitch = 68;       // floats per channel row of the epilogue stage (64 pixels + padding)
+constexpr size_t kEpiBytes = 4 * 4 * 8 * kEpiPitch * sizeof(float);  // four waves x (up to 4 steps x 8 channel rows)
 
 // Channels per chunk staged in LDS; fixed by (Cin, taps, activation width) alone so that packing and the kernel agree.
 // Pointwise convolutions take up to 128 channels at a time (no halo re-use to pay for), everything else 32; fp32
@@ -70,9 +72,10 @@ struct ConvGeom {
     int pitch;                // bytes per LDS pixel = CK * 2 + 16
     int T;                    // timesteps stored by this launch (<= TT)
     int shared_x;             // every timestep reads the same activation tensor: convolve once
-    int vec_store;            // a lane's two pixels are adjacent and aligned in memory
+    int vec8;                 // runs of 8 output pixels may be stored as one 16-byte-aligned vector
     int64_t spike_step_stride;
     int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
+    int debug;
 };
 
 struct ConvLaunch {

@@ -45,7 +45,7 @@ struct Plan {
 
 // Picks the wave arrangement (WM x WN) and the output tile (TH rows of the flattened (n, oh) space x TW columns,
 // TH * TW <= WM * 64) that keep the most matrix lanes and CUs busy, under the LDS and staging-slot limits.
-bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool want_pairs, Plan& best_plan) {
+bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool want_vec8, Plan& best_plan) {
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int rows = g0.N * g0.Ho;
     const int groups = 1 << g0.groups_log2;
@@ -59,7 +59,6 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
         const int oc_tiles = (g0.Cout + OT - 1) / OT;
         const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
         for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
-            if (want_pairs && (tw & 1)) continue;
             int th = PT / tw;
             if (th > rows) th = rows;
             ConvGeom c = g0;
@@ -70,7 +69,9 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
             c.NR = max_tile_rows(c);
             c.WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
             c.WT = (c.WT + 1) & ~1;
-            const size_t bytes = static_cast<size_t>(t_in) * c.NR * c.WT * c.pitch + c.pitch;
+            size_t bytes = static_cast<size_t>(t_in) * c.NR * c.WT * c.pitch;
+            if (bytes < kEpiBytes) bytes = kEpiBytes;
+            bytes += c.pitch;
             if (bytes > kMaxLds) continue;
             if (groups * c.NR * (c.WT / 2) > max_spatial_items) continue;
             const double work = static_cast<double>(c.tiles_x) * c.tiles_y * oc_tiles;
@@ -79,7 +80,9 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
             const double fill = work / (waves * cus);
             const double halo = static_cast<double>(c.NR) * c.WT / (static_cast<double>(th) * tw);
             double score = lane_eff * oc_eff * fill / (1.0 + 0.05 * (halo - 1.0)) / (1.0 + 0.1 * (oc_tiles - 1));
-            if (tw == g0.Wo) score *= 1.02;
+            // 16-byte stores need runs of 8 contiguous output pixels: full-width rows or tile widths that are multiples of 8.
+            const bool runs = want_vec8 && ((tw == g0.Wo && (g0.Wo % 8 == 0 || g0.Ho == 1)) || tw % 8 == 0);
+            if (!runs) score *= 0.6;
             if (score > best) {
                 best = score;
                 best_plan = Plan{th, tw, c.tiles_x, c.tiles_y, c.NR, c.WT, wm_log2, wn_log2, oc_tiles, bytes};
@@ -89,12 +92,12 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
     return best > 0.0;
 }
 
-bool plan(const ConvGeom& g, int t_in, int tt, int load_mode, bool want_pairs, Plan& out) {
+bool plan(const ConvGeom& g, int t_in, int tt, int load_mode, bool want_vec8, Plan& out) {
     using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
     static std::mutex mu;
     static std::map<Key, std::pair<bool, Plan>> plans;
     const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, t_in, tt, load_mode,
-                  want_pairs ? 1 : 0);
+                  want_vec8 ? 1 : 0);
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = plans.find(key);
@@ -104,7 +107,7 @@ bool plan(const ConvGeom& g, int t_in, int tt, int load_mode, bool want_pairs, P
         }
     }
     Plan p = {};
-    const bool ok = plan_uncached(g, t_in, tt, load_mode, want_pairs, p);
+    const bool ok = plan_uncached(g, t_in, tt, load_mode, want_vec8, p);
     std::lock_guard<std::mutex> lock(mu);
     plans[key] = std::make_pair(ok, p);
     out = p;
@@ -165,19 +168,19 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.spike_step_stride = spike_step_stride;
     g.v_is_f32 = v_dtype == SNNF_F32 ? 1 : 0;
     const int xsize = dtype_size(x_dtype);
-    const int vsize = dtype_size(v_dtype);
     const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
     hipStream_t hs = as_stream(stream);
 
     constexpr int kMaxTT = 4;
     bool all_shared = T > 1;
     bool pair_aligned = xsize == 2 && (g.W % 2 == 0);
-    bool vec_ok = (g.Wo % 2 == 0) && (spike_step_stride % 2 == 0) && aligned_to(spikes, 2 * xsize) &&
-                  aligned_to(v_out, 2 * vsize) && (v_init == nullptr || aligned_to(v_init, 2 * vsize));
+    // 8 consecutive output pixels start 16-byte aligned whenever their first pixel offset is a multiple of 8.
+    bool vec_ok = ((static_cast<int64_t>(g.Ho) * g.Wo) % 8 == 0) && (spike_step_stride % 8 == 0) && aligned_to(spikes, 16) &&
+                  aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16));
     for (int t = 0; t < T; ++t) {
         all_shared = all_shared && xs[t] == xs[0];
         pair_aligned = pair_aligned && aligned_to(xs[t], 4);
-        if (residuals != nullptr) vec_ok = vec_ok && aligned_to(residuals[t], 2 * xsize);
+        if (residuals != nullptr) vec_ok = vec_ok && aligned_to(residuals[t], 16);
     }
     const int load_mode = xsize == 4 ? LOAD_2XF32 : (pair_aligned ? LOAD_PAIR32 : LOAD_2X16);
 
@@ -200,7 +203,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
                     W, KH, KW, stride_h, stride_w);
     g.TH = pl.TH; g.TW = pl.TW; g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.NR = pl.NR; g.WT = pl.WT;
     g.wm_log2 = pl.wm_log2; g.wn_log2 = pl.wn_log2; g.oc_tiles = pl.oc_tiles;
-    g.vec_store = (vec_ok && (g.TW % 2 == 0)) ? 1 : 0;
+    g.vec8 = vec_ok ? 1 : 0;
 
     const int n_px_tiles = g.tiles_x * g.tiles_y;
     const int work_per_xcd = ((n_px_tiles + 7) / 8) * g.oc_tiles;
@@ -219,6 +222,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         L.has_residual = residuals != nullptr ? 1 : 0;
         L.g = g;
         L.g.T = tw;
+        L.g.debug = getenv("SNNF_DEBUG_CONV") ? atoi(getenv("SNNF_DEBUG_CONV")) : 0;
         L.g.shared_x = (all_shared && window > 1) ? 1 : 0;
         L.wpacked = static_cast<const uint16_t*>(packed_weight);
         L.bias = reinterpret_cast<const float*>(L.wpacked + packed_weight_elems(pg));

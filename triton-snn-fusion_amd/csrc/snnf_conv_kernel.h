@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
     const int groups = 1 << g.groups_log2;
     const int tile_bytes = g.NR * g.WT * g.pitch;
     const int t_in = g.shared_x ? 1 : TT;
-    const int zero_off = t_in * tile_bytes;
+    const int zero_off = max(t_in * tile_bytes, static_cast<int>(kEpiBytes));   // the epilogue stage shares the tile's LDS
     const int total_rows = g.N * g.Ho;
     const int64_t plane = static_cast<int64_t>(g.H) * g.W;
     const int64_t plane_out = static_cast<int64_t>(g.Ho) * g.Wo;
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             const int t = u % TT;
             const int s = u / TT;
             const uint32_t flags = st_meta[s] >> 20;
-            if (t < t_in && (flags & 4)) {
+            if (!(g.debug & 1) && t < t_in && (flags & 4)) {
                 const char* __restrict__ base = static_cast<const char*>(xs.p[t]) + chunk_bytes;  // uniform
                 const int nval = g.Cin - (chunk * g.CK + static_cast<int>((st_meta[s] >> 24) & 31u) * 8);
                 const bool ok0 = flags & 1, ok1 = flags & 2;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
         for (int u = 0; u < MI; ++u) {
             const int t = u % TT;
             const int s = u / TT;
-            if (t < t_in && ((st_meta[s] >> 20) & 4)) {
+            if (!(g.debug & 8) && t < t_in && ((st_meta[s] >> 20) & 4)) {
                 uint32_t e0[8], e1[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             int cg = half & (groups - 1);
             int kh = 0, kw = 0;
             if (half >> g.groups_log2) { kw = 1; if (kw == g.KW) { kw = 0; kh = 1; } }
-            for (int pair = 0; pair < g.npairs; ++pair, ++gp) {
+            for (int pair = 0; pair < ((g.debug & 2) ? 0 : g.npairs); ++pair, ++gp) {
                 if (gp + 1 < total_pairs) {
 #pragma unroll
                     for (int f = 0; f < kNOF; ++f)
@@ -313,80 +313,143 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             }
         }
 
-        // ---- epilogue: bias (+ residual) + LIF over T. Result row i = 8 * (r / 4) + 4 * half + r % 4 of each fragment.
-        // Branch-free neuron: h = v + (x - v * c0) * c1 covers tau <= 1 (c0 = 0, c1 = 1) and power-of-two tau exactly.
-        if (wave_has_work && (pix_valid[0] || pix_valid[1])) {
-            const bool both = pix_valid[0] && pix_valid[1];
-            const bool vec_sp = g.vec_store && both;
-            const bool vec_v = vec_sp && g.v_is_f32;
-            const float c0 = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
-            const float c1 = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
-            const bool ok0 = pix_valid[0], ok1 = pix_valid[1];
-            const int64_t po0 = ok0 ? pix_off[0] : pix_off[1];   // an invalid pixel reads its neighbour and stores nothing
-            const int64_t po1 = ok1 ? pix_off[1] : pix_off[0];
+        // ---- epilogue. Eight channel rows at a time, the accumulators of all T steps are transposed through LDS (the
+        // activation tile is dead by now) to [step][channel row][64 pixels] per wave, so that a lane owns 8 consecutive
+        // pixels of one channel: bias (+ residual) + LIF run on those 8 neurons with the membrane in registers across
+        // the T steps, spikes leave as one 16-byte store per step and the membrane as two. Branch-free neuron:
+        // h = v + (x - v * c0) * c1 covers tau <= 1 (c0 = 0, c1 = 1) and power-of-two tau exactly.
+        __syncthreads();   // every wave is done reading the activation tile
+        if (g.shared_x) {
+#pragma unroll
+            for (int t = 1; t < TT; ++t)
+#pragma unroll
+                for (int f = 0; f < kNOF; ++f)
+#pragma unroll
+                    for (int p = 0; p < kNPF; ++p) acc[t][f][p] = acc[0][f][p];
+        }
+        if (wave_has_work && !(g.debug & 4)) {
+            float* __restrict__ stage = reinterpret_cast<float*>(lds) + wave * (TT * 8 * kEpiPitch);
+            const int rg = lane >> 3;            // channel row of this lane inside a group of 8
+            const int pcx = lane & 7;            // pixel chunk: pixels 8 * pcx .. 8 * pcx + 7 of the wave's 64
+            // Output offsets (elements, inside one channel plane stack) of the chunk's pixels, walked incrementally.
+            int pxoff[8];
+            uint32_t okmask = 0;
+            {
+                const int pix0 = wm * (32 * kNPF) + pcx * 8;
+                int pr = pix0 / g.TW;
+                int pc = pix0 - pr * g.TW;
+                int q = q0 + pr;
+                int n = q / g.Ho;
+                int oh = q - n * g.Ho;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int ow = c0 + pc;
+                    const bool ok = pr < g.TH && q < total_rows && ow < g.Wo;
+                    pxoff[k] = ok ? (n * g.Cout * static_cast<int>(plane_out) + oh * g.Wo + ow) : 0;
+                    okmask |= ok ? (1u << k) : 0u;
+                    if (++pc == g.TW) {
+                        pc = 0; ++pr; ++q;
+                        if (++oh == g.Ho) { oh = 0; ++n; }
+                    }
+                }
+            }
+            const bool fast = g.vec8 && okmask == 0xffu && (pxoff[7] - pxoff[0]) == 7 && (pxoff[0] & 7) == 0;
+            const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
+            const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+            const int po = static_cast<int>(plane_out);
+
 #pragma unroll
             for (int f = 0; f < kNOF; ++f) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int oc = (ocf0 + f) * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-                    if (oc < g.Cout) {
-                        const int64_t oc_off = oc * plane_out;
-                        const float bv = bias[oc];
-                        float v0 = 0.0f, v1 = 0.0f;
+                for (int kq = 0; kq < 4; ++kq) {
+                    // rows of this group: channel (ocf0 + f) * 32 + 8 * kq + [0, 8); lane (j, half) holds rows 4 * half + (r & 3).
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int t = 0; t < TT; ++t)
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) {
+                            const cv_f32x2 two = {acc[t][f][0][kq * 4 + rr], acc[t][f][1][kq * 4 + rr]};
+                            *reinterpret_cast<cv_f32x2*>(stage + (t * 8 + half * 4 + rr) * kEpiPitch + (lane & 31) * 2) = two;
+                        }
+                    __builtin_amdgcn_wave_barrier();
+                    const int oc = (ocf0 + f) * 32 + kq * 8 + rg;
+                    if (oc < g.Cout && okmask != 0) {
+                        const int64_t row_off = static_cast<int64_t>(oc) * po;
+                        const float bvv = bias[oc];
+                        float v[8];
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) v[k] = 0.0f;
                         if (v_init != nullptr) {
-                            if (vec_v) {
-                                const cv_f32x2 vi = *reinterpret_cast<const cv_f32x2*>(static_cast<const float*>(v_init) + po0 + oc_off);
-                                v0 = vi[0];
-                                v1 = vi[1];
-                            } else if (g.v_is_f32) {
-                                v0 = static_cast<const float*>(v_init)[po0 + oc_off];
-                                v1 = static_cast<const float*>(v_init)[po1 + oc_off];
+                            if (fast && g.v_is_f32) {
+                                const float* src = static_cast<const float*>(v_init) + row_off + pxoff[0];
+                                const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
+                                const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) { v[k] = lo.v[k]; v[4 + k] = hi.v[k]; }
                             } else {
-                                v0 = to_float(static_cast<const XT*>(v_init)[po0 + oc_off]);
-                                v1 = to_float(static_cast<const XT*>(v_init)[po1 + oc_off]);
+#pragma unroll
+                                for (int k = 0; k < 8; ++k) {
+                                    if (okmask & (1u << k)) {
+                                        v[k] = g.v_is_f32 ? static_cast<const float*>(v_init)[row_off + pxoff[k]]
+                                                          : to_float(static_cast<const XT*>(v_init)[row_off + pxoff[k]]);
+                                    }
+                                }
                             }
                         }
 #pragma unroll
                         for (int t = 0; t < TT; ++t) {
                             if (t < g.T) {
-                                float x0 = (g.shared_x ? acc[0][f][0][r] : acc[t][f][0][r]) + bv;
-                                float x1 = (g.shared_x ? acc[0][f][1][r] : acc[t][f][1][r]) + bv;
-                                XT* __restrict__ out_t = spikes + t * g.spike_step_stride + oc_off;
+                                const float* __restrict__ srow = stage + (t * 8 + rg) * kEpiPitch + pcx * 8;
+                                const Pack<float, 4> xlo = *reinterpret_cast<const Pack<float, 4>*>(srow);
+                                const Pack<float, 4> xhi = *reinterpret_cast<const Pack<float, 4>*>(srow + 4);
+                                float x[8];
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) { x[k] = xlo.v[k] + bvv; x[4 + k] = xhi.v[k] + bvv; }
+                                XT* __restrict__ out_t = spikes + t * g.spike_step_stride + row_off;
                                 if (has_residual) {
-                                    const XT* __restrict__ res_t = static_cast<const XT*>(residuals.p[t]) + oc_off;
-                                    if (vec_sp) {
-                                        const Pack<XT, 2> res = *reinterpret_cast<const Pack<XT, 2>*>(res_t + po0);
-                                        x0 += to_float(res.v[0]);
-                                        x1 += to_float(res.v[1]);
+                                    const XT* __restrict__ res_t = static_cast<const XT*>(residuals.p[t]) + row_off;
+                                    if (fast) {
+                                        const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + pxoff[0]);
+#pragma unroll
+                                        for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
                                     } else {
-                                        x0 += to_float(res_t[po0]);
-                                        x1 += to_float(res_t[po1]);
+#pragma unroll
+                                        for (int k = 0; k < 8; ++k)
+                                            if (okmask & (1u << k)) x[k] += to_float(res_t[pxoff[k]]);
                                     }
                                 }
-                                const float h0 = v0 + (x0 - v0 * c0) * c1;
-                                const float h1 = v1 + (x1 - v1 * c0) * c1;
-                                const bool s0 = h0 >= lif.v_threshold, s1 = h1 >= lif.v_threshold;
-                                v0 = s0 ? (lif.soft_reset ? h0 - lif.v_threshold : lif.v_reset) : h0;
-                                v1 = s1 ? (lif.soft_reset ? h1 - lif.v_threshold : lif.v_reset) : h1;
-                                if (vec_sp) {
-                                    Pack<XT, 2> sp;
-                                    sp.v[0] = spike_value<XT>(s0);
-                                    sp.v[1] = spike_value<XT>(s1);
-                                    *reinterpret_cast<Pack<XT, 2>*>(out_t + po0) = sp;
+                                Pack<XT, 8> sp;
+#pragma unroll
+                                for (int k = 0; k < 8; ++k) {
+                                    const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
+                                    const bool fired = h >= lif.v_threshold;
+                                    v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                                    sp.v[k] = spike_value<XT>(fired);
+                                }
+                                if (fast) {
+                                    *reinterpret_cast<Pack<XT, 8>*>(out_t + pxoff[0]) = sp;
                                 } else {
-                                    if (ok0) out_t[po0] = spike_value<XT>(s0);
-                                    if (ok1) out_t[po1] = spike_value<XT>(s1);
+#pragma unroll
+                                    for (int k = 0; k < 8; ++k)
+                                        if (okmask & (1u << k)) out_t[pxoff[k]] = sp.v[k];
                                 }
                             }
                         }
-                        if (vec_v) {
-                            *reinterpret_cast<cv_f32x2*>(static_cast<float*>(v_out) + po0 + oc_off) = cv_f32x2{v0, v1};
-                        } else if (g.v_is_f32) {
-                            if (ok0) static_cast<float*>(v_out)[po0 + oc_off] = v0;
-                            if (ok1) static_cast<float*>(v_out)[po1 + oc_off] = v1;
+                        if (fast && g.v_is_f32) {
+                            float* dst = static_cast<float*>(v_out) + row_off + pxoff[0];
+                            Pack<float, 4> lo, hi;
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
+                            *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
+                            *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
                         } else {
-                            if (ok0) static_cast<XT*>(v_out)[po0 + oc_off] = from_float<XT>(v0);
-                            if (ok1) static_cast<XT*>(v_out)[po1 + oc_off] = from_float<XT>(v1);
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) {
+                                if (okmask & (1u << k)) {
+                                    if (g.v_is_f32) static_cast<float*>(v_out)[row_off + pxoff[k]] = v[k];
+                                    else static_cast<XT*>(v_out)[row_off + pxoff[k]] = from_float<XT>(v[k]);
+                                }
+                            }
                         }
                     }
                 }
