@@ -46,16 +46,18 @@ struct Plan {
 // Picks the wave arrangement (WM x WN) and the output tile (TH rows of the flattened (n, oh) space x TW columns,
 // TH * TW <= WM * 64) that keep the most matrix lanes and CUs busy, under the LDS and staging-slot limits.
 bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool want_vec8, Plan& best_plan) {
+    // tt == 0: time-outer kernel (one timestep in LDS, two workgroups per CU, its own staging depth and LDS stage).
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int rows = g0.N * g0.Ho;
     const int groups = 1 << g0.groups_log2;
-    const int max_spatial_items = kConvThreads * (staging_items(load_mode) / tt);
-    const int cus = compute_units();
+    const int max_spatial_items = tt == 0 ? kConvThreads * (load_mode == LOAD_PAIR32 ? 4 : 2)
+                                           : kConvThreads * (staging_items(load_mode) / tt);
+    const int cus = compute_units() * (tt == 0 ? 2 : 1);
     double best = -1.0;
     for (int wn_log2 = 0; wn_log2 <= 2; ++wn_log2) {
         const int wm_log2 = 2 - wn_log2;
         const int PT = (1 << wm_log2) * 32 * kNPF;
-        const int OT = (1 << wn_log2) * 32 * kNOF;
+        const int OT = (1 << wn_log2) * 32 * (tt == 0 ? 1 : kNOF);   // the time-outer kernel gives a wave 32 channels
         const int oc_tiles = (g0.Cout + OT - 1) / OT;
         const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
         for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
@@ -70,9 +72,14 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
             c.WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
             c.WT = (c.WT + 1) & ~1;
             size_t bytes = static_cast<size_t>(t_in) * c.NR * c.WT * c.pitch;
-            if (bytes < kEpiBytes) bytes = kEpiBytes;
-            bytes += c.pitch;
-            if (bytes > kMaxLds) continue;
+            if (tt == 0) {
+                bytes += c.pitch + 4 * 8 * kEpiPitch * sizeof(float);   // zero pixel + per-wave epilogue stage
+                if (bytes * 2 > kMaxLds) continue;                      // two workgroups per CU
+            } else {
+                if (bytes < kEpiBytes) bytes = kEpiBytes;
+                bytes += c.pitch;
+                if (bytes > kMaxLds) continue;
+            }
             if (groups * c.NR * (c.WT / 2) > max_spatial_items) continue;
             const double work = static_cast<double>(c.tiles_x) * c.tiles_y * oc_tiles;
             const double lane_eff = static_cast<double>(rows) * g0.Wo / (static_cast<double>(c.tiles_x) * c.tiles_y * PT);
@@ -184,19 +191,37 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     }
     const int load_mode = xsize == 4 ? LOAD_2XF32 : (pair_aligned ? LOAD_PAIR32 : LOAD_2X16);
 
-    // Timesteps per launch: as many (<= 4) as fit LDS side by side; a shared analog frame needs one tile for any window.
-    int window = T < kMaxTT ? T : kMaxTT;
-    {
+    // Kernel choice. Layers whose arithmetic intensity is far below the matrix-core / HBM ridge (about 300 flop/byte)
+    // run the time-outer kernel (small footprint, two workgroups per CU, membrane resident for any T); the others
+    // accumulate up to 4 timesteps side by side so that each weight fragment load feeds 4x the matrix work.
+    const double flops = 2.0 * (all_shared ? 1 : T) * N * static_cast<double>(Ho_real) * Wo_real * Cout * Cin * KH * KW;
+    const double bytes = static_cast<double>(xsize) * ((all_shared ? 1 : T) * static_cast<double>(N) * Cin * H * W +
+                                                       static_cast<double>(T) * N * Cout * Ho_real * Wo_real) +
+                         4.0 * N * Cout * Ho_real * Wo_real;
+    bool time_outer = all_shared || flops / bytes < 200.0;
+    const char* force = getenv("SNNF_CONV_KERNEL");   // "tout" / "tin": override for experiments
+    if (force != nullptr && force[0] == 't' && force[1] == 'o') time_outer = true;
+    if (force != nullptr && force[0] == 't' && force[1] == 'i') time_outer = false;
+
+    int window = 0;
+    Plan pl = {};
+    bool planned = false;
+    if (time_outer) {
+        planned = plan(g, 1, 0, load_mode, vec_ok, pl);
+        window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
+        if (!planned) time_outer = false;
+    }
+    if (!time_outer) {
+        // Timesteps per launch: as many (<= 4) as fit LDS side by side; a shared analog frame needs one tile for any window.
+        window = T < kMaxTT ? T : kMaxTT;
         int w2 = 1;
         while (w2 < window) w2 *= 2;
         window = w2;
-    }
-    Plan pl = {};
-    bool planned = false;
-    while (true) {
-        planned = plan(g, all_shared ? 1 : window, window, load_mode, vec_ok, pl);
-        if (planned || window == 1) break;
-        window >>= 1;
+        while (true) {
+            planned = plan(g, all_shared ? 1 : window, window, load_mode, vec_ok, pl);
+            if (planned || window == 1) break;
+            window >>= 1;
+        }
     }
     if (!planned)
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: unsupported_shape: no activation tile fits LDS (W=%d, kernel %dx%d, stride %dx%d)",
@@ -208,7 +233,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     const int n_px_tiles = g.tiles_x * g.tiles_y;
     const int work_per_xcd = ((n_px_tiles + 7) / 8) * g.oc_tiles;
     const int cu_per_xcd = (compute_units() + 7) / 8;
-    const int per_cu = (pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1;
+    const int per_cu = time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1);
     int slots = cu_per_xcd * per_cu;
     if (slots > work_per_xcd) slots = work_per_xcd;
 
@@ -223,7 +248,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         L.g = g;
         L.g.T = tw;
         L.g.debug = getenv("SNNF_DEBUG_CONV") ? atoi(getenv("SNNF_DEBUG_CONV")) : 0;
-        L.g.shared_x = (all_shared && window > 1) ? 1 : 0;
+        L.g.shared_x = (all_shared && (window > 1 || time_outer)) ? 1 : 0;
         L.wpacked = static_cast<const uint16_t*>(packed_weight);
         L.bias = reinterpret_cast<const float*>(L.wpacked + packed_weight_elems(pg));
         L.v_init = t0 == 0 ? v_init : v_out;
@@ -234,9 +259,10 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         L.lds_bytes = pl.lds_bytes;
         L.stream = hs;
         int rc;
-        if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, window, load_mode);
-        else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, window, load_mode);
-        else rc = launch_conv_f16(L, window, load_mode);
+        const int tt = time_outer ? 0 : window;
+        if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, load_mode);
+        else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, load_mode);
+        else rc = launch_conv_f16(L, tt, load_mode);
         if (rc != SNNF_OK) return rc;
     }
     return SNNF_OK;
