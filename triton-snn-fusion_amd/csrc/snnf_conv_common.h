@@ -12,6 +12,8 @@ constexpr int kNOF = 2;             // output-channel fragments per wave (64 cha
 constexpr int kMaxItems = 8;        // staging items (8 channels x 2 pixels) per thread and channel chunk
 constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kEpiPitch = 68;       // floats per channel row of the epilogue stage (64 pixels + padding)
+constexpr size_t kToutStageBytes = 4 * 64 * 12 * sizeof(float);   // time-outer kernel: four waves x 64 pixels x (8 rows + padding)
+constexpr size_t kPwStageBytes = 4 * 8 * 68 * sizeof(float);      // pointwise kernel: four waves x 8 channel rows x (64 pixels + padding)
 constexpr size_t kEpiBytes = 4 * 4 * 8 * kEpiPitch * sizeof(float);  // four waves x (up to 4 steps x 8 channel rows)
 
 // Channels per chunk staged in LDS; fixed by (Cin, taps, activation width) alone so that packing and the kernel agree.
@@ -61,6 +63,33 @@ enum LoadMode : int {
 // Staging items a thread may hold in flight per chunk: modes that need two registers per fetch get half as many.
 __host__ __device__ constexpr int staging_items(int load_mode) { return load_mode == LOAD_PAIR32 ? kMaxItems : kMaxItems / 2; }
 
+// Division by a divisor fixed at launch as a multiply-high and a shift (the divisions of the tile walk are otherwise
+// ~40-instruction sequences on the vector unit). Exact for numerators below 2^31.
+struct FastDiv {
+    uint32_t mul;     // 0: the divisor is 1
+    uint32_t shift;
+    uint32_t d;
+};
+
+inline FastDiv make_fast_div(int divisor) {
+    FastDiv f;
+    f.d = static_cast<uint32_t>(divisor < 1 ? 1 : divisor);
+    f.mul = 0;
+    f.shift = 0;
+    if (f.d > 1) {
+        uint32_t lg = 0;
+        while ((1ull << lg) < f.d) ++lg;
+        const uint32_t p = 31 + lg;
+        f.mul = static_cast<uint32_t>(((1ull << p) + f.d - 1) / f.d);
+        f.shift = p - 32;
+    }
+    return f;
+}
+
+__device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
+    return f.mul == 0 ? n : static_cast<int>(__umulhi(static_cast<uint32_t>(n), f.mul) >> f.shift);
+}
+
 struct ConvGeom {
     int N, Cin, H, W, Cout, KH, KW, sh, sw, ph, pw, Ho, Wo;
     int TH, TW;               // output tile: TH rows of the flattened (n, oh) row space x TW columns
@@ -76,6 +105,9 @@ struct ConvGeom {
     int64_t spike_step_stride;
     int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
     int debug;
+    int w_lds;                // time-outer kernels: this workgroup's weight fragments are kept in LDS
+    int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
+    FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
 };
 
 struct ConvLaunch {
@@ -95,6 +127,7 @@ struct ConvLaunch {
 };
 
 // One launcher per activation dtype (each in its own translation unit so they compile in parallel).
+// tt: 1, 2, 4 = timesteps accumulated side by side; 0 = time-outer kernel; -1 = pointwise kernel.
 int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode);

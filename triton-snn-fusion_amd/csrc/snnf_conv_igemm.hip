@@ -73,7 +73,7 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
             c.WT = (c.WT + 1) & ~1;
             size_t bytes = static_cast<size_t>(t_in) * c.NR * c.WT * c.pitch;
             if (tt == 0) {
-                bytes += c.pitch + 4 * 8 * kEpiPitch * sizeof(float);   // zero pixel + per-wave epilogue stage
+                bytes += c.pitch + kToutStageBytes;                      // zero pixel + per-wave epilogue stage
                 if (bytes * 2 > kMaxLds) continue;                      // two workgroups per CU
             } else {
                 if (bytes < kEpiBytes) bytes = kEpiBytes;
@@ -159,7 +159,8 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     ConvGeom g = {};
     g.N = N; g.Cin = Cin; g.Cout = Cout; g.KH = KH; g.KW = KW;
     g.sh = stride_h; g.sw = stride_w; g.ph = pad_h; g.pw = pad_w;
-    if (KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0) {
+    const bool pointwise = KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0;
+    if (pointwise) {
         // A pointwise convolution has no spatial structure: treat each image as one row of H * W pixels.
         g.H = 1; g.W = H * W;
     } else {
@@ -206,7 +207,29 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     int window = 0;
     Plan pl = {};
     bool planned = false;
-    if (time_outer) {
+    bool pw_kernel = false;
+    size_t pw_lds = 0;
+    if (time_outer && pointwise && Cin % 8 == 0 && static_cast<int64_t>(Cout) * g.Wo < (1LL << 30) &&
+        !(force != nullptr && force[0] == 't' && force[1] == 'o')) {
+        // Pointwise kernel: flat tiles of 64 pixels x 128 output channels, no planning needed.
+        pw_kernel = planned = true;
+        window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
+        pl.TH = 1; pl.TW = 64; pl.tiles_x = (g.Wo + 63) / 64; pl.tiles_y = N; pl.NR = 1; pl.WT = 64;
+        pl.wm_log2 = 0; pl.wn_log2 = 2; pl.oc_tiles = (Cout + 127) / 128;
+        const size_t xb = static_cast<size_t>(64) * g.pitch;
+        const size_t wbytes = static_cast<size_t>(4) * g.nchunks * g.npairs * kFragBytes;
+        pw_lds = xb + kPwStageBytes;
+        g.x_bufs = 1;
+        if ((pw_lds + wbytes) * 2 <= kMaxLds) {
+            g.w_lds = 1;
+            pw_lds += wbytes;
+        }
+        if ((pw_lds + xb) * 2 <= kMaxLds) {
+            g.x_bufs = 2;
+            pw_lds += xb;
+        }
+        pl.lds_bytes = pw_lds;
+    } else if (time_outer) {
         planned = plan(g, 1, 0, load_mode, vec_ok, pl);
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
         if (!planned) time_outer = false;
@@ -229,7 +252,20 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.TH = pl.TH; g.TW = pl.TW; g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.NR = pl.NR; g.WT = pl.WT;
     g.wm_log2 = pl.wm_log2; g.wn_log2 = pl.wn_log2; g.oc_tiles = pl.oc_tiles;
     g.vec8 = vec_ok ? 1 : 0;
+    g.d_TW = make_fast_div(g.TW); g.d_Ho = make_fast_div(g.Ho); g.d_H = make_fast_div(g.H);
+    g.d_WTP = make_fast_div(g.WT / 2); g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
+    g.d_tiles_x = make_fast_div(g.tiles_x); g.d_oc_tiles = make_fast_div(g.oc_tiles);
 
+    size_t lds_bytes = pl.lds_bytes;
+    if (time_outer && !pw_kernel) {
+        // Keep the workgroup's weight fragments in LDS when two workgroups per CU still fit: the matrix loop then needs
+        // no global loads at all.
+        const size_t wbytes = (static_cast<size_t>(1) << g.wn_log2) * 1 * g.nchunks * g.npairs * kFragBytes;
+        if ((lds_bytes + wbytes) * 2 <= kMaxLds) {
+            g.w_lds = 1;
+            lds_bytes += wbytes;
+        }
+    }
     const int n_px_tiles = g.tiles_x * g.tiles_y;
     const int work_per_xcd = ((n_px_tiles + 7) / 8) * g.oc_tiles;
     const int cu_per_xcd = (compute_units() + 7) / 8;
@@ -256,10 +292,10 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         L.v_out = v_out;
         L.lif = lif;
         L.grid = slots * 8;
-        L.lds_bytes = pl.lds_bytes;
+        L.lds_bytes = lds_bytes;
         L.stream = hs;
         int rc;
-        const int tt = time_outer ? 0 : window;
+        const int tt = pw_kernel ? -1 : (time_outer ? 0 : window);
         if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, load_mode);
         else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, load_mode);
         else rc = launch_conv_f16(L, tt, load_mode);

@@ -1,0 +1,532 @@
+// Pointwise (1x1, stride 1, no padding) convolution + bias (+ residual) + LIF over T timesteps.
+//
+// A pointwise layer moves far more bytes than it multiplies (its roofline is HBM), and on this machine a wave64
+// vector instruction occupies its SIMD for four cycles, so what decides the speed of this kernel is the number of
+// vector instructions per output and the waits on memory, not the matrix work. Hence:
+//   * an image is one row of P = H * W pixels; a tile is 64 consecutive pixels x 128 output channels (4 waves x 32).
+//     Per-thread staging offsets, LDS addresses of the matrix operands and output offsets are kernel constants; a tile
+//     only contributes a uniform base address, so loads and stores use the scalar-base addressing form.
+//   * The bias enters through the matrix unit (a fragment holding the fp32 bias split into three 16-bit terms times a
+//     fragment of ones), so a timestep starts with one matrix instruction instead of clearing and biasing registers.
+//   * The membrane of the wave's 32 x 64 neurons stays in registers for all T. Timestep pointers are read from the
+//     kernel-argument segment with a scalar load instead of living in 32 scalar registers per table.
+//   * One counter tracks all of a wave's outstanding global loads and stores, in order. The next stage's loads are
+//     issued from a single place in the loop (copies between two sets of load registers would force a wait right after
+//     the loads), and a timestep's spikes wait in registers until the next stage has been taken out of its load
+//     registers, so that the wait for those loads never finds fresh stores in front of it.
+//   * The activation tile is double buffered in LDS when it fits (one workgroup barrier per stage); WL: the weight
+//     fragments of the workgroup's 128 channels stay in LDS, otherwise they stream from L2 one fragment ahead.
+// Requires Cin % 8 == 0 (channel groups of 8 are whole). Operand mapping and the packed weight format are those of
+// snnf_conv_kernel.h.
+#pragma once
+
+#include <type_traits>
+
+#include "snnf_conv_kernel.h"
+
+namespace snnf {
+
+constexpr int kPwStagePitch = 68;                          // floats per channel row of the wave's stage (64 pixels + padding)
+constexpr int kPwStageFloats = 8 * kPwStagePitch;          // 8 channel rows
+static_assert(4 * kPwStageFloats * sizeof(float) == kPwStageBytes, "host and kernel disagree on the stage size");
+constexpr int kPwTile = 64;                                // pixels per tile
+constexpr int kPwSlots = 2;                                // staging items per thread and chunk (128 channels x 64 pixels)
+
+// Entry i of a pointer table passed by value as a kernel argument, read from the kernel-argument segment (explicit
+// arguments start at offset 0 of that segment, in declaration order and naturally aligned).
+typedef const void* pw_cvp;
+__device__ __forceinline__ const void* kernarg_table_entry(int table_offset_bytes, int i) {
+    typedef const __attribute__((address_space(4))) unsigned char* ka_bytes;
+    typedef const __attribute__((address_space(4))) pw_cvp* ka_entry;
+    ka_bytes ka = (ka_bytes)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(ka_entry)(ka + table_offset_bytes + i * 8);
+}
+
+// The two pointer tables MUST be the first two kernel parameters (offsets 0 and sizeof(StepPtrs)).
+template <typename XT, int LM, bool STD, bool WL>
+__global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const StepPtrs xs, const StepPtrs residuals,
+                                                                      const int has_residual, const ConvGeom g,
+                                                                      const uint16_t* __restrict__ wpacked,
+                                                                      const float* __restrict__ bias,
+                                                                      const void* __restrict__ v_init,
+                                                                      XT* __restrict__ spikes, void* __restrict__ v_out,
+                                                                      const LifParams lif) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
+    constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
+    constexpr int SS = kPwSlots;
+    constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
+    constexpr int NG = 4;                          // epilogue row groups (8 channel rows each) of the wave's 32 channels
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int rg = lane >> 3;                      // epilogue view: channel row inside a group of 8
+    const int pcx = lane & 7;                      //                pixels 8 * pcx .. 8 * pcx + 7 of the tile
+
+    const int P = g.W;
+    const int groups = 1 << g.groups_log2;
+    const int x_buf_bytes = kPwTile * g.pitch;
+    const int dbl = g.x_bufs > 1 ? 1 : 0;
+    float* __restrict__ stage = reinterpret_cast<float*>(lds + g.x_bufs * x_buf_bytes) + wave * kPwStageFloats;
+    unsigned char* __restrict__ wlds = lds + g.x_bufs * x_buf_bytes + kPwStageBytes;
+    const int total_pairs = g.nchunks * g.npairs;
+    const int nocf = (g.Cout + 31) >> 5;
+    const int64_t frag_stride_ocf = static_cast<int64_t>(total_pairs) * (kFragBytes / 2);
+    const int steps_with_input = g.shared_x ? 1 : g.T;
+    const int64_t row_bytes = static_cast<int64_t>(P) * ES;           // one channel row of an image
+
+    // ---- kernel constants of the staging: item e = (channel group of 8, pixel pair) of a 64-pixel x CK-channel stage.
+    uint32_t item_src[SS], item_dst[SS];
+    bool item_on[SS];
+#pragma unroll
+    for (int s = 0; s < SS; ++s) {
+        const int e = s * kConvThreads + tid;
+        const int cg = e >> 5, pp = e & 31;
+        item_on[s] = cg < groups;
+        item_src[s] = (static_cast<uint32_t>(cg) * 8u * static_cast<uint32_t>(P) + 2u * pp) * ES;
+        item_dst[s] = static_cast<uint32_t>(2 * pp * g.pitch + cg * 16);
+    }
+    // The 16 bytes of padding behind a pixel's channels are read as a second channel group when a chunk has only one:
+    // keep them zero (staging never writes there).
+    if (tid < kPwTile * g.x_bufs) {
+        const cv_u32x4 zero = {0u, 0u, 0u, 0u};
+        *reinterpret_cast<cv_u32x4*>(lds + (tid >> 6) * x_buf_bytes + (tid & 63) * g.pitch + g.CK * 2) = zero;
+    }
+
+    // The stage in flight: its data, and which of this thread's items lie outside the image or the channels (bit s).
+    uint32_t pre[SS][8][RPE];
+    uint32_t pre_bad = 0;
+    bool pre_whole = true;
+
+    // Loads of stage (step, chunk) of the tile at pixel px0 of image n. Every load is unconditional: items that lie
+    // outside are redirected to the tile's first pixels (always valid) and zeroed on their way into LDS.
+    auto issue_loads = [&](int step, int chunk, int n, int px0) __attribute__((always_inline)) {
+        const char* __restrict__ base = static_cast<const char*>(kernarg_table_entry(0, step)) +
+                                        (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES;
+        const bool whole = px0 + kPwTile <= P && (chunk + 1) * g.CK <= g.Cin;
+        uint32_t src[SS], second[SS];
+        uint32_t bad = 0;
+#pragma unroll
+        for (int s = 0; s < SS; ++s) {
+            src[s] = item_src[s];
+            second[s] = ES;
+        }
+        if (!whole) {
+#pragma unroll
+            for (int s = 0; s < SS; ++s) {
+                const int e = s * kConvThreads + tid;
+                const int pix = px0 + 2 * (e & 31);
+                const bool ok = chunk * g.CK + (e >> 5) * 8 < g.Cin && pix < P;
+                src[s] = ok ? item_src[s] : 0u;
+                second[s] = (ok && pix + 1 < P) ? ES : 0u;
+                bad |= ok ? 0u : (1u << s);
+            }
+        }
+        pre_bad = bad;
+        pre_whole = whole;
+#pragma unroll
+        for (int s = 0; s < SS; ++s) {
+            if (item_on[s]) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const char* __restrict__ row = base + j * row_bytes;
+                    if constexpr (LM == LOAD_PAIR32) {
+                        pre[s][j][0] = *reinterpret_cast<const uint32_t*>(row + src[s]);
+                    } else if constexpr (LM == LOAD_2X16) {
+                        pre[s][j][0] = *reinterpret_cast<const uint16_t*>(row + src[s]);
+                        pre[s][j][1] = *reinterpret_cast<const uint16_t*>(row + src[s] + second[s]);
+                    } else {
+                        pre[s][j][0] = *reinterpret_cast<const uint32_t*>(row + src[s]);
+                        pre[s][j][1] = *reinterpret_cast<const uint32_t*>(row + src[s] + second[s]);
+                    }
+                }
+            }
+        }
+    };
+
+    // Registers -> LDS, transposed to [pixel][channel]: 8 channels of a pixel are one 16-byte write.
+    auto write_lds = [&](int buf) __attribute__((always_inline)) {
+        unsigned char* __restrict__ xb = lds + buf * x_buf_bytes;
+#pragma unroll
+        for (int s = 0; s < SS; ++s) {
+            if (item_on[s]) {
+                cv_u32x4 lo, hi;
+                if constexpr (LM == LOAD_PAIR32) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        lo[k] = __builtin_amdgcn_perm(pre[s][2 * k + 1][0], pre[s][2 * k][0], 0x05040100u);
+                        hi[k] = __builtin_amdgcn_perm(pre[s][2 * k + 1][0], pre[s][2 * k][0], 0x07060302u);
+                    }
+                } else {
+                    uint32_t e0[8], e1[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if constexpr (LM == LOAD_2X16) {
+                            e0[j] = pre[s][j][0];
+                            e1[j] = pre[s][j][1];
+                        } else {
+                            e0[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][0]));
+                            e1[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][1]));
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        lo[k] = e0[2 * k] | (e0[2 * k + 1] << 16);
+                        hi[k] = e1[2 * k] | (e1[2 * k + 1] << 16);
+                    }
+                }
+                if (!pre_whole) {
+                    const bool zero = (pre_bad >> s) & 1u;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        lo[k] = zero ? 0u : lo[k];
+                        hi[k] = zero ? 0u : hi[k];
+                    }
+                }
+                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s]) = lo;
+                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s] + g.pitch) = hi;
+            }
+        }
+    };
+
+    // ---- tile walk: pixel tiles congruent to this workgroup's XCD, consecutive work items = output-channel tiles.
+    const int xcd = blockIdx.x & 7;
+    const int slots_per_xcd = gridDim.x >> 3;
+    const int n_px_tiles = g.tiles_x * g.tiles_y;
+    const int work_per_xcd = ((n_px_tiles + 7) >> 3) * g.oc_tiles;
+    int work = blockIdx.x >> 3;
+    int oc_tile = 0, img = 0, px0 = 0;
+    auto decode = [&](int w, int& oc_t, int& n, int& p0) __attribute__((always_inline)) -> bool {
+        if (w >= work_per_xcd) return false;
+        const int pt = fast_div(w, g.d_oc_tiles);
+        const int px_tile = pt * 8 + xcd;
+        if (px_tile >= n_px_tiles) return false;
+        oc_t = w - pt * g.oc_tiles;
+        n = fast_div(px_tile, g.d_tiles_x);
+        p0 = (px_tile - n * g.tiles_x) * kPwTile;
+        return true;
+    };
+    bool have_tile = decode(work, oc_tile, img, px0);
+    if (have_tile) issue_loads(0, 0, img, px0);
+
+    // ---- kernel constants of the matrix loop and the epilogue.
+    const uint32_t b_off0 = static_cast<uint32_t>((2 * l32) * g.pitch + half * 16);   // this lane's pixels 2 l32, 2 l32 + 1
+    const unsigned char* __restrict__ wl = wlds + (static_cast<size_t>(wave) * total_pairs * 64 + lane) * 16;
+    float* __restrict__ stage_wr = stage + (half * 4) * kPwStagePitch + 2 * l32;
+    const float* __restrict__ stage_rd = stage + rg * kPwStagePitch + pcx * 8;
+    const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
+    const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+
+    // Bias fragment: row l32 of the weight operand carries the fp32 bias as three 16-bit terms (exact to 24 bits) in its
+    // first k-slots; the activation fragments of ones differ in slots the bias fragment leaves zero, only so that the
+    // two start-of-timestep matrix instructions stay two instructions.
+    cv_u32x4 a_bias = {0u, 0u, 0u, 0u};
+    const uint32_t one16 = F16 ? 0x3C00u : 0x3F80u;
+    const cv_u32x4 b_ones0 = {one16 | (one16 << 16), one16, 0u, 0u};
+    const cv_u32x4 b_ones1 = {one16 | (one16 << 16), one16 | (one16 << 16), 0u, 0u};
+    const cv_f32x16 acc_zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    int bias_ocf = -1;
+    int loaded_oc_tile = -1;
+    int buf = 0;
+
+    while (have_tile) {
+        const int ocf = oc_tile * 4 + wave;
+        const bool wave_has_work = ocf < nocf;
+        const bool full = px0 + kPwTile <= P;
+        const bool fast = g.vec8 && full;
+        uint32_t okmask = 0xffu;
+        if (!full) {
+            okmask = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) okmask |= (px0 + pcx * 8 + k < P) ? (1u << k) : 0u;
+        }
+        const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * P + px0;   // uniform element offset into [N, Cout, P]
+
+        if (ocf != bias_ocf) {
+            bias_ocf = ocf;
+            const int oc = ocf * 32 + l32;
+            const float b = (wave_has_work && half == 0 && oc < g.Cout) ? bias[oc] : 0.0f;
+            const uint32_t t1 = F16 ? float_to_f16_bits(b) : float_to_bf16_bits(b);
+            const float r1 = b - (F16 ? f16_bits_to_float(t1) : bf16_bits_to_float(t1));
+            const uint32_t t2 = F16 ? float_to_f16_bits(r1) : float_to_bf16_bits(r1);
+            const float r2 = r1 - (F16 ? f16_bits_to_float(t2) : bf16_bits_to_float(t2));
+            const uint32_t t3 = F16 ? float_to_f16_bits(r2) : float_to_bf16_bits(r2);
+            a_bias[0] = t1 | (t2 << 16);
+            a_bias[1] = t3;
+        }
+        if (WL && oc_tile != loaded_oc_tile) {
+            // (Re)load the weight fragments of this output-channel tile: [wave][pair][lane] x 16 bytes.
+            __syncthreads();
+            const int vec_per_wave = total_pairs * 64;
+            for (int i = tid; i < 4 * vec_per_wave; i += kConvThreads) {
+                const int wv = i / vec_per_wave;
+                const int within = i - wv * vec_per_wave;
+                const int src_ocf = min(oc_tile * 4 + wv, nocf - 1);
+                const cv_u32x4 val = *reinterpret_cast<const cv_u32x4*>(wpacked + static_cast<int64_t>(src_ocf) * frag_stride_ocf + static_cast<int64_t>(within) * 8);
+                *reinterpret_cast<cv_u32x4*>(wlds + static_cast<size_t>(i) * 16) = val;
+            }
+            loaded_oc_tile = oc_tile;
+            __syncthreads();
+        }
+        const uint16_t* __restrict__ wg = wpacked + static_cast<int64_t>(min(ocf, nocf - 1)) * frag_stride_ocf + lane * 8;
+
+        // ---- membrane of this lane's 4 x 8 neurons (group gi: channel ocf * 32 + gi * 8 + rg, pixels 8 pcx ..), all T steps.
+        uint32_t lane_off[NG];   // bytes into a spike-typed [Cout, P] image
+        bool row_ok[NG];
+        float v[NG][8];
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            const int oc = ocf * 32 + gi * 8 + rg;
+            row_ok[gi] = wave_has_work && oc < g.Cout && okmask != 0;
+            lane_off[gi] = static_cast<uint32_t>(oc * P + pcx * 8) * ES;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[gi][k] = 0.0f;
+        }
+        if (v_init != nullptr) {
+            if (fast && g.v_is_f32) {
+                const char* vbase = reinterpret_cast<const char*>(static_cast<const float*>(v_init) + tile_off);
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) {
+                    if (row_ok[gi]) {
+                        const float* src = reinterpret_cast<const float*>(vbase + lane_off[gi] * (4u / ES));
+                        const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
+                        const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) { v[gi][k] = lo.v[k]; v[gi][4 + k] = hi.v[k]; }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) {
+                    if (row_ok[gi]) {
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            if (okmask & (1u << k)) {
+                                v[gi][k] = g.v_is_f32 ? static_cast<const float*>(v_init)[tile_off + lane_off[gi] / ES + k]
+                                                      : to_float(static_cast<const XT*>(v_init)[tile_off + lane_off[gi] / ES + k]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+
+        // Spikes of a timestep wait here until the next stage has left its load registers.
+        Pack<XT, 8> pend[NG];
+        int pend_step = -1;
+        auto flush_spikes = [&]() __attribute__((always_inline)) {
+            char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
+            if (fast) {
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi)
+                    if (row_ok[gi]) *reinterpret_cast<Pack<XT, 8>*>(out + lane_off[gi]) = pend[gi];
+            } else {
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) {
+                    if (row_ok[gi]) {
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
+                            if (okmask & (1u << k)) *reinterpret_cast<XT*>(out + lane_off[gi] + k * ES) = pend[gi].v[k];
+                    }
+                }
+            }
+            pend_step = -1;
+        };
+
+        cv_f32x16 acc[kNPF];
+        int next_work = work, next_oc_tile = oc_tile, next_img = img, next_px0 = px0;
+        bool next_tile = false;
+        for (int step = 0; step < g.T; ++step) {
+            if (step < steps_with_input) {
+                acc[0] = cv_mfma<F16>(a_bias, b_ones0, acc_zero);
+                acc[1] = cv_mfma<F16>(a_bias, b_ones1, acc_zero);
+                for (int chunk = 0; chunk < g.nchunks; ++chunk) {
+                    if (!dbl) __syncthreads();   // single buffer: every wave is done reading the previous stage
+                    write_lds(buf);              // waits for the stage's loads
+                    __syncthreads();
+                    if (pend_step >= 0) flush_spikes();
+                    // ---- the stage after this one: next chunk, next timestep, or the first stage of the next tile.
+                    int ns = step, nc = chunk + 1, nimg = img, npx = px0;
+                    bool more = true;
+                    if (nc == g.nchunks) {
+                        nc = 0;
+                        ns = step + 1;
+                        if (ns == steps_with_input) {
+                            ns = 0;
+                            next_work = work + slots_per_xcd;
+                            next_tile = decode(next_work, next_oc_tile, next_img, next_px0);
+                            more = next_tile;
+                            nimg = next_img;
+                            npx = next_px0;
+                        }
+                    }
+                    if (WL && more) issue_loads(ns, nc, nimg, npx);
+                    if (wave_has_work) {
+                        const unsigned char* __restrict__ bp0 = lds + buf * x_buf_bytes + b_off0;
+                        const unsigned char* __restrict__ bp1 = bp0 + g.pitch;
+                        int pair = 0;
+                        if constexpr (WL) {
+                            const unsigned char* __restrict__ ap = wl + static_cast<size_t>(chunk * g.npairs) * kFragBytes;
+                            for (; pair + 2 <= g.npairs; pair += 2) {
+                                const cv_u32x4 a0 = *reinterpret_cast<const cv_u32x4*>(ap + pair * kFragBytes);
+                                const cv_u32x4 a1 = *reinterpret_cast<const cv_u32x4*>(ap + (pair + 1) * kFragBytes);
+                                const cv_u32x4 b00 = *reinterpret_cast<const cv_u32x4*>(bp0 + pair * 32);
+                                const cv_u32x4 b01 = *reinterpret_cast<const cv_u32x4*>(bp1 + pair * 32);
+                                const cv_u32x4 b10 = *reinterpret_cast<const cv_u32x4*>(bp0 + pair * 32 + 32);
+                                const cv_u32x4 b11 = *reinterpret_cast<const cv_u32x4*>(bp1 + pair * 32 + 32);
+                                acc[0] = cv_mfma<F16>(a0, b00, acc[0]);
+                                acc[1] = cv_mfma<F16>(a0, b01, acc[1]);
+                                acc[0] = cv_mfma<F16>(a1, b10, acc[0]);
+                                acc[1] = cv_mfma<F16>(a1, b11, acc[1]);
+                            }
+                            if (pair < g.npairs) {
+                                const cv_u32x4 a0 = *reinterpret_cast<const cv_u32x4*>(ap + pair * kFragBytes);
+                                const cv_u32x4 b00 = *reinterpret_cast<const cv_u32x4*>(bp0 + pair * 32);
+                                const cv_u32x4 b01 = *reinterpret_cast<const cv_u32x4*>(bp1 + pair * 32);
+                                acc[0] = cv_mfma<F16>(a0, b00, acc[0]);
+                                acc[1] = cv_mfma<F16>(a0, b01, acc[1]);
+                            }
+                        } else {
+                            // Weights streamed from global memory (L2 resident), one fragment ahead.
+                            const uint16_t* __restrict__ ap = wg + static_cast<int64_t>(chunk * g.npairs) * (kFragBytes / 2);
+                            cv_u32x4 a_cur = *reinterpret_cast<const cv_u32x4*>(ap);
+                            for (; pair < g.npairs; ++pair) {
+                                const int pn = pair + 1 < g.npairs ? pair + 1 : pair;
+                                const cv_u32x4 a_nxt = *reinterpret_cast<const cv_u32x4*>(ap + pn * (kFragBytes / 2));
+                                const cv_u32x4 b0 = *reinterpret_cast<const cv_u32x4*>(bp0 + pair * 32);
+                                const cv_u32x4 b1 = *reinterpret_cast<const cv_u32x4*>(bp1 + pair * 32);
+                                acc[0] = cv_mfma<F16>(a_cur, b0, acc[0]);
+                                acc[1] = cv_mfma<F16>(a_cur, b1, acc[1]);
+                                a_cur = a_nxt;
+                            }
+                        }
+                    }
+                    // Streaming weights share the load counter: the next stage's loads go out behind them.
+                    if (!WL && more) issue_loads(ns, nc, nimg, npx);
+                    buf ^= dbl;
+                }
+            }
+
+            // ---- LIF step: 8 channel rows at a time through the wave's stage, so that a lane owns 8 consecutive pixels.
+            if (wave_has_work) {
+                if (pend_step >= 0) flush_spikes();   // only when a timestep had no stage of its own (shared frame)
+                const char* __restrict__ res_t =
+                    has_residual ? reinterpret_cast<const char*>(static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), step)) + tile_off) : nullptr;
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) {
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const cv_f32x2 two = {acc[0][gi * 4 + rr], acc[1][gi * 4 + rr]};
+                        *reinterpret_cast<cv_f32x2*>(stage_wr + rr * kPwStagePitch) = two;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    const Pack<float, 4> xlo = *reinterpret_cast<const Pack<float, 4>*>(stage_rd);
+                    const Pack<float, 4> xhi = *reinterpret_cast<const Pack<float, 4>*>(stage_rd + 4);
+                    float x[8];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) { x[k] = xlo.v[k]; x[4 + k] = xhi.v[k]; }
+                    if (res_t != nullptr && row_ok[gi]) {
+                        if (fast) {
+                            const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + lane_off[gi]);
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < 8; ++k)
+                                if (okmask & (1u << k)) x[k] += to_float(*reinterpret_cast<const XT*>(res_t + lane_off[gi] + k * ES));
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        bool fired;
+                        if constexpr (STD) {
+                            const float h = v[gi][k] + (x[k] - v[gi][k]) * lif.inv_tau;
+                            fired = h >= lif.v_threshold;
+                            v[gi][k] = fired ? lif.v_reset : h;
+                        } else {
+                            const float h = v[gi][k] + (x[k] - v[gi][k] * c0f) * c1f;
+                            fired = h >= lif.v_threshold;
+                            v[gi][k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                        }
+                        pend[gi].v[k] = spike_value<XT>(fired);
+                    }
+                }
+                pend_step = step;
+            }
+        }
+
+        // ---- last timestep's spikes and the final membrane.
+        if (pend_step >= 0) flush_spikes();
+        if (fast && g.v_is_f32) {
+            char* vbase = reinterpret_cast<char*>(static_cast<float*>(v_out) + tile_off);
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) {
+                if (row_ok[gi]) {
+                    float* dst = reinterpret_cast<float*>(vbase + lane_off[gi] * (4u / ES));
+                    Pack<float, 4> lo, hi;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) { lo.v[k] = v[gi][k]; hi.v[k] = v[gi][4 + k]; }
+                    *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
+                    *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) {
+                if (row_ok[gi]) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        if (okmask & (1u << k)) {
+                            if (g.v_is_f32) static_cast<float*>(v_out)[tile_off + lane_off[gi] / ES + k] = v[gi][k];
+                            else static_cast<XT*>(v_out)[tile_off + lane_off[gi] / ES + k] = from_float<XT>(v[gi][k]);
+                        }
+                    }
+                }
+            }
+        }
+        work = next_work;
+        oc_tile = next_oc_tile;
+        img = next_img;
+        px0 = next_px0;
+        have_tile = next_tile;
+    }
+}
+
+template <typename XT>
+int launch_conv_pw(const ConvLaunch& L, int load_mode) {
+    auto run = [&](auto kernel) -> int {
+        if (L.lds_bytes > 64 * 1024) {
+            static bool raised[64] = {};
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+            if (!raised[dev]) {
+                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                     static_cast<int>(kMaxLds));
+                if (err != hipSuccess)
+                    return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: cannot reserve %zu bytes of LDS: %s", L.lds_bytes, hipGetErrorString(err));
+                raised[dev] = true;
+            }
+        }
+        kernel<<<dim3(L.grid), kConvThreads, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
+                                                                      static_cast<XT*>(L.spikes), L.v_out, L.lif);
+        return check_launch("snnf_conv_lif");
+    };
+    const bool std_lif = L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset;
+    auto pick = [&](auto lm) -> int {
+        constexpr int LMV = decltype(lm)::value;
+        if (L.g.w_lds)
+            return std_lif ? run(conv_pw_lif_kernel<XT, LMV, true, true>) : run(conv_pw_lif_kernel<XT, LMV, false, true>);
+        return std_lif ? run(conv_pw_lif_kernel<XT, LMV, true, false>) : run(conv_pw_lif_kernel<XT, LMV, false, false>);
+    };
+    if constexpr (sizeof(XT) == 4) {
+        return pick(std::integral_constant<int, LOAD_2XF32>{});
+    } else {
+        if (load_mode == LOAD_PAIR32) return pick(std::integral_constant<int, LOAD_PAIR32>{});
+        return pick(std::integral_constant<int, LOAD_2X16>{});
+    }
+}
+
+}  // namespace snnf
