@@ -105,8 +105,9 @@ struct ConvGeom {
     int64_t spike_step_stride;
     int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
     int debug;
-    int w_lds;                // time-outer kernels: this workgroup's weight fragments are kept in LDS
+    int w_lds;                // time-outer kernels: weight fragments streamed from L2 (0), kept in LDS (1) or in registers (2)
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
+    int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts
     FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
 };
 
@@ -127,7 +128,7 @@ struct ConvLaunch {
 };
 
 // One launcher per activation dtype (each in its own translation unit so they compile in parallel).
-// tt: 1, 2, 4 = timesteps accumulated side by side; 0 = time-outer kernel; -1 = pointwise kernel.
+// tt: 1, 2, 4 = timesteps accumulated side by side; 0 = time-outer kernel; -1 / -2 = pointwise kernel, general / fast.
 int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode);

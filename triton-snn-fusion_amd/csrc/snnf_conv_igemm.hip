@@ -208,7 +208,25 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     Plan pl = {};
     bool planned = false;
     bool pw_kernel = false;
-    size_t pw_lds = 0;
+    // Pointwise kernel: where the weight fragments live (registers only in the fast variant) and the LDS that takes.
+    auto pw_config = [&](bool allow_regs, ConvGeom& gg) -> size_t {
+        const size_t xb = static_cast<size_t>(64) * gg.pitch;
+        const size_t wbytes = static_cast<size_t>(4) * gg.nchunks * gg.npairs * kFragBytes;
+        size_t bytes = xb + kPwStageBytes;
+        gg.x_bufs = 1;
+        gg.w_lds = 0;   // streamed from L2
+        if (allow_regs && gg.nchunks == 1 && gg.npairs == 8) {
+            gg.w_lds = 2;   // a wave's 8 fragments in registers
+        } else if ((bytes + wbytes) * 2 <= kMaxLds) {
+            gg.w_lds = 1;   // the workgroup's fragments in LDS, two workgroups per CU
+            bytes += wbytes;
+        }
+        if ((bytes + xb) * 2 <= kMaxLds) {
+            gg.x_bufs = 2;
+            bytes += xb;
+        }
+        return bytes;
+    };
     if (time_outer && pointwise && Cin % 8 == 0 && static_cast<int64_t>(Cout) * g.Wo < (1LL << 30) &&
         !(force != nullptr && force[0] == 't' && force[1] == 'o')) {
         // Pointwise kernel: flat tiles of 64 pixels x 128 output channels, no planning needed.
@@ -216,19 +234,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
         pl.TH = 1; pl.TW = 64; pl.tiles_x = (g.Wo + 63) / 64; pl.tiles_y = N; pl.NR = 1; pl.WT = 64;
         pl.wm_log2 = 0; pl.wn_log2 = 2; pl.oc_tiles = (Cout + 127) / 128;
-        const size_t xb = static_cast<size_t>(64) * g.pitch;
-        const size_t wbytes = static_cast<size_t>(4) * g.nchunks * g.npairs * kFragBytes;
-        pw_lds = xb + kPwStageBytes;
-        g.x_bufs = 1;
-        if ((pw_lds + wbytes) * 2 <= kMaxLds) {
-            g.w_lds = 1;
-            pw_lds += wbytes;
-        }
-        if ((pw_lds + xb) * 2 <= kMaxLds) {
-            g.x_bufs = 2;
-            pw_lds += xb;
-        }
-        pl.lds_bytes = pw_lds;
+        pl.lds_bytes = 0;
     } else if (time_outer) {
         planned = plan(g, 1, 0, load_mode, vec_ok, pl);
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
@@ -266,12 +272,43 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
             lds_bytes += wbytes;
         }
     }
-    const int n_px_tiles = g.tiles_x * g.tiles_y;
-    const int work_per_xcd = ((n_px_tiles + 7) / 8) * g.oc_tiles;
     const int cu_per_xcd = (compute_units() + 7) / 8;
+    auto grid_for = [&](const ConvGeom& gg, int per_cu) {
+        const int work_per_xcd = ((gg.tiles_x * gg.tiles_y + 7) / 8) * gg.oc_tiles;
+        int slots = cu_per_xcd * per_cu;
+        if (slots > work_per_xcd) slots = work_per_xcd;
+        return slots * 8;
+    };
     const int per_cu = time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1);
-    int slots = cu_per_xcd * per_cu;
-    if (slots > work_per_xcd) slots = work_per_xcd;
+
+    // Pointwise layers: the fast variant takes the tiles that lie inside their image when the layer qualifies (common
+    // neuron, aligned outputs, fp32 membrane, whole channel fragments); the general variant takes the ragged last tile of
+    // each image, or everything.
+    struct Part { ConvGeom g; size_t lds; int tt; };
+    Part parts[2];
+    int nparts = 0;
+    if (pw_kernel) {
+        const int P = g.Wo;
+        const bool fast_ok = lif.charge_mode == CHARGE_SCALE && !lif.soft_reset && vec_ok && Cout % 32 == 0 && v_dtype == SNNF_F32;
+        const int full_tiles = fast_ok ? P / 64 : 0;
+        if (full_tiles > 0) {
+            Part& f = parts[nparts++];
+            f.g = g; f.tt = -2;
+            f.g.tiles_x = full_tiles; f.g.px_base = 0;
+            f.g.d_tiles_x = make_fast_div(full_tiles);
+            f.lds = pw_config(true, f.g);
+        }
+        if (full_tiles * 64 < P) {
+            Part& r = parts[nparts++];
+            r.g = g; r.tt = -1;
+            r.g.tiles_x = (P - full_tiles * 64 + 63) / 64; r.g.px_base = full_tiles * 64;
+            r.g.d_tiles_x = make_fast_div(r.g.tiles_x);
+            r.lds = pw_config(false, r.g);
+        }
+    } else {
+        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = time_outer ? 0 : window;
+        nparts = 1;
+    }
 
     for (int t0 = 0; t0 < T; t0 += window) {
         const int tw = (T - t0) < window ? (T - t0) : window;
@@ -281,7 +318,8 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
             if (residuals != nullptr) L.residuals.p[t] = residuals[t0 + (t < tw ? t : 0)];
         }
         L.has_residual = residuals != nullptr ? 1 : 0;
-        L.g = g;
+      for (int part = 0; part < nparts; ++part) {
+        L.g = parts[part].g;
         L.g.T = tw;
         L.g.debug = getenv("SNNF_DEBUG_CONV") ? atoi(getenv("SNNF_DEBUG_CONV")) : 0;
         L.g.shared_x = (all_shared && (window > 1 || time_outer)) ? 1 : 0;
@@ -291,15 +329,16 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         L.spikes = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
         L.v_out = v_out;
         L.lif = lif;
-        L.grid = slots * 8;
-        L.lds_bytes = lds_bytes;
+        L.grid = grid_for(L.g, per_cu);
+        L.lds_bytes = parts[part].lds;
         L.stream = hs;
         int rc;
-        const int tt = pw_kernel ? -1 : (time_outer ? 0 : window);
+        const int tt = parts[part].tt;
         if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, load_mode);
         else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, load_mode);
         else rc = launch_conv_f16(L, tt, load_mode);
         if (rc != SNNF_OK) return rc;
+      }
     }
     return SNNF_OK;
 }

@@ -3,9 +3,9 @@
 #include "snnf_conv_tout_kernel.h"
 
 namespace snnf {
-// tt < 0 selects the pointwise kernel, tt == 0 the time-outer kernel, tt in {1, 2, 4} the kernel that accumulates tt timesteps side by side.
+// tt < 0 selects the pointwise kernel (-2: its fast variant), tt == 0 the time-outer kernel, tt in {1, 2, 4} the kernel that accumulates tt timesteps side by side.
 int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode) {
-    if (tt < 0) return launch_conv_pw<f16_t>(L, load_mode);
+    if (tt < 0) return launch_conv_pw<f16_t>(L, load_mode, tt == -2);
     if (tt == 0) return launch_conv_tout<f16_t>(L, load_mode);
     return launch_conv_tt<f16_t>(L, tt, load_mode);
 }

@@ -14,9 +14,14 @@
 //     issued from a single place in the loop (copies between two sets of load registers would force a wait right after
 //     the loads), and a timestep's spikes wait in registers until the next stage has been taken out of its load
 //     registers, so that the wait for those loads never finds fresh stores in front of it.
-//   * The activation tile is double buffered in LDS when it fits (one workgroup barrier per stage); WL: the weight
-//     fragments of the workgroup's 128 channels stay in LDS, otherwise they stream from L2 one fragment ahead.
-// Requires Cin % 8 == 0 (channel groups of 8 are whole). Operand mapping and the packed weight format are those of
+//   * The activation tile is double buffered in LDS when it fits (one workgroup barrier per stage). A wave's weight
+//     fragments stay in registers when there are exactly 8 of them (Cin of 113..128), else the workgroup's fragments stay in
+//     LDS when they fit, else they stream from L2 one fragment ahead. LDS bandwidth is the next limit after the vector
+//     unit, so LDS rows are laid out for conflict-free 16-byte reads.
+// FAST: every tile of the launch lies inside its image, outputs are 16-byte aligned, Cout % 32 == 0 and the membrane is
+// fp32, so the per-pixel and per-row masks and the element-wise load/store paths (and the scalar registers they pin)
+// drop out; the host sends the ragged last tile of each image, and any layer that fails these conditions, to the
+// general variant. Requires Cin % 8 == 0 (channel groups of 8 are whole). Operand mapping and the packed weight format are those of
 // snnf_conv_kernel.h.
 #pragma once
 
@@ -31,6 +36,9 @@ constexpr int kPwStageFloats = 8 * kPwStagePitch;          // 8 channel rows
 static_assert(4 * kPwStageFloats * sizeof(float) == kPwStageBytes, "host and kernel disagree on the stage size");
 constexpr int kPwTile = 64;                                // pixels per tile
 constexpr int kPwSlots = 2;                                // staging items per thread and chunk (128 channels x 64 pixels)
+constexpr int kPwRegPairs = 8;                             // weight fragments a wave can keep in registers
+
+enum PwWeights : int { PW_WEIGHTS_STREAM = 0, PW_WEIGHTS_LDS = 1, PW_WEIGHTS_REGS = 2 };
 
 // Entry i of a pointer table passed by value as a kernel argument, read from the kernel-argument segment (explicit
 // arguments start at offset 0 of that segment, in declaration order and naturally aligned).
@@ -43,8 +51,8 @@ __device__ __forceinline__ const void* kernarg_table_entry(int table_offset_byte
 }
 
 // The two pointer tables MUST be the first two kernel parameters (offsets 0 and sizeof(StepPtrs)).
-template <typename XT, int LM, bool STD, bool WL>
-__global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const StepPtrs xs, const StepPtrs residuals,
+template <typename XT, int LM, bool STD, int WM, bool FAST>
+__global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pw_lif_kernel(const StepPtrs xs, const StepPtrs residuals,
                                                                       const int has_residual, const ConvGeom g,
                                                                       const uint16_t* __restrict__ wpacked,
                                                                       const float* __restrict__ bias,
@@ -57,6 +65,8 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
     constexpr int SS = kPwSlots;
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
     constexpr int NG = 4;                          // epilogue row groups (8 channel rows each) of the wave's 32 channels
+    constexpr bool WL = WM == PW_WEIGHTS_LDS;      // weight fragments of the workgroup's 128 channels live in LDS
+    constexpr bool WR = WM == PW_WEIGHTS_REGS;     // the wave's weight fragments (exactly 8, one chunk) live in registers
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
@@ -86,7 +96,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
         const int cg = e >> 5, pp = e & 31;
         item_on[s] = cg < groups;
         item_src[s] = (static_cast<uint32_t>(cg) * 8u * static_cast<uint32_t>(P) + 2u * pp) * ES;
-        item_dst[s] = static_cast<uint32_t>(2 * pp * g.pitch + cg * 16);
+        item_dst[s] = static_cast<uint32_t>(pp * g.pitch + cg * 16);   // pixel 2 pp -> row pp, pixel 2 pp + 1 -> row pp + 32
     }
     // The 16 bytes of padding behind a pixel's channels are read as a second channel group when a chunk has only one:
     // keep them zero (staging never writes there).
@@ -104,8 +114,8 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
     // outside are redirected to the tile's first pixels (always valid) and zeroed on their way into LDS.
     auto issue_loads = [&](int step, int chunk, int n, int px0) __attribute__((always_inline)) {
         const char* __restrict__ base = static_cast<const char*>(kernarg_table_entry(0, step)) +
-                                        (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES;
-        const bool whole = px0 + kPwTile <= P && (chunk + 1) * g.CK <= g.Cin;
+                                        (static_cast<int64_t>(((g.debug & 1) ? 0 : n) * g.Cin + chunk * g.CK) * P + ((g.debug & 1) ? 0 : px0)) * ES;
+        const bool whole = (FAST || px0 + kPwTile <= P) && (chunk + 1) * g.CK <= g.Cin;
         uint32_t src[SS], second[SS];
         uint32_t bad = 0;
 #pragma unroll
@@ -118,9 +128,9 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
             for (int s = 0; s < SS; ++s) {
                 const int e = s * kConvThreads + tid;
                 const int pix = px0 + 2 * (e & 31);
-                const bool ok = chunk * g.CK + (e >> 5) * 8 < g.Cin && pix < P;
+                const bool ok = chunk * g.CK + (e >> 5) * 8 < g.Cin && (FAST || pix < P);
                 src[s] = ok ? item_src[s] : 0u;
-                second[s] = (ok && pix + 1 < P) ? ES : 0u;
+                second[s] = (ok && (FAST || pix + 1 < P)) ? ES : 0u;
                 bad |= ok ? 0u : (1u << s);
             }
         }
@@ -186,7 +196,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
                     }
                 }
                 *reinterpret_cast<cv_u32x4*>(xb + item_dst[s]) = lo;
-                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s] + g.pitch) = hi;
+                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s] + 32 * g.pitch) = hi;
             }
         }
     };
@@ -205,17 +215,21 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
         if (px_tile >= n_px_tiles) return false;
         oc_t = w - pt * g.oc_tiles;
         n = fast_div(px_tile, g.d_tiles_x);
-        p0 = (px_tile - n * g.tiles_x) * kPwTile;
+        p0 = g.px_base + (px_tile - n * g.tiles_x) * kPwTile;
         return true;
     };
     bool have_tile = decode(work, oc_tile, img, px0);
     if (have_tile) issue_loads(0, 0, img, px0);
 
     // ---- kernel constants of the matrix loop and the epilogue.
-    const uint32_t b_off0 = static_cast<uint32_t>((2 * l32) * g.pitch + half * 16);   // this lane's pixels 2 l32, 2 l32 + 1
+    // This lane's pixels 2 l32 and 2 l32 + 1 sit in rows l32 and l32 + 32 of the tile (consecutive lanes one pitch apart:
+    // 16-byte reads without bank conflicts).
+    const uint32_t b_off0 = static_cast<uint32_t>(l32 * g.pitch + half * 16);
     const unsigned char* __restrict__ wl = wlds + (static_cast<size_t>(wave) * total_pairs * 64 + lane) * 16;
-    float* __restrict__ stage_wr = stage + (half * 4) * kPwStagePitch + 2 * l32;
-    const float* __restrict__ stage_rd = stage + rg * kPwStagePitch + pcx * 8;
+    // Stage columns are permuted so that both 16-byte reads of a lane's 8 pixels are free of bank conflicts: pixel q sits
+    // in column (q & 3) + 4 ((q >> 3) & 7) + 32 ((q >> 2) & 1); a lane's pixel pair stays adjacent.
+    float* __restrict__ stage_wr = stage + (half * 4) * kPwStagePitch + 2 * (l32 & 1) + 4 * (l32 >> 2) + 32 * ((l32 >> 1) & 1);
+    const float* __restrict__ stage_rd = stage + rg * kPwStagePitch + pcx * 4;
     const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
     const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
 
@@ -227,6 +241,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
     const cv_u32x4 b_ones0 = {one16 | (one16 << 16), one16, 0u, 0u};
     const cv_u32x4 b_ones1 = {one16 | (one16 << 16), one16 | (one16 << 16), 0u, 0u};
     const cv_f32x16 acc_zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    cv_u32x4 a_reg[kPwRegPairs];
     int bias_ocf = -1;
     int loaded_oc_tile = -1;
     int buf = 0;
@@ -234,8 +249,9 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
     while (have_tile) {
         const int ocf = oc_tile * 4 + wave;
         const bool wave_has_work = ocf < nocf;
-        const bool full = px0 + kPwTile <= P;
-        const bool fast = g.vec8 && full;
+        const bool full = FAST || px0 + kPwTile <= P;
+        const bool fast = FAST || (g.vec8 && full);
+        const bool vf32 = FAST || g.v_is_f32;
         uint32_t okmask = 0xffu;
         if (!full) {
             okmask = 0;
@@ -255,6 +271,15 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
             const uint32_t t3 = F16 ? float_to_f16_bits(r2) : float_to_bf16_bits(r2);
             a_bias[0] = t1 | (t2 << 16);
             a_bias[1] = t3;
+        }
+        if (WR && ocf != loaded_oc_tile) {
+            loaded_oc_tile = ocf;
+            const uint16_t* __restrict__ src = wpacked + static_cast<int64_t>(min(ocf, nocf - 1)) * frag_stride_ocf + lane * 8;
+#pragma unroll
+            for (int q = 0; q < kPwRegPairs; ++q)
+                a_reg[q] = *reinterpret_cast<const cv_u32x4*>(src + q * (kFragBytes / 2));
+            // Wait here, once: otherwise every later use of a fragment waits for ALL outstanding loads, prefetch included.
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         }
         if (WL && oc_tile != loaded_oc_tile) {
             // (Re)load the weight fragments of this output-channel tile: [wave][pair][lane] x 16 bytes.
@@ -279,13 +304,13 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi) {
             const int oc = ocf * 32 + gi * 8 + rg;
-            row_ok[gi] = wave_has_work && oc < g.Cout && okmask != 0;
+            row_ok[gi] = FAST ? wave_has_work : (wave_has_work && oc < g.Cout && okmask != 0);
             lane_off[gi] = static_cast<uint32_t>(oc * P + pcx * 8) * ES;
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[gi][k] = 0.0f;
         }
         if (v_init != nullptr) {
-            if (fast && g.v_is_f32) {
+            if (fast && vf32) {
                 const char* vbase = reinterpret_cast<const char*>(static_cast<const float*>(v_init) + tile_off);
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi) {
@@ -304,7 +329,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
 #pragma unroll
                         for (int k = 0; k < 8; ++k) {
                             if (okmask & (1u << k)) {
-                                v[gi][k] = g.v_is_f32 ? static_cast<const float*>(v_init)[tile_off + lane_off[gi] / ES + k]
+                                v[gi][k] = vf32 ? static_cast<const float*>(v_init)[tile_off + lane_off[gi] / ES + k]
                                                       : to_float(static_cast<const XT*>(v_init)[tile_off + lane_off[gi] / ES + k]);
                             }
                         }
@@ -318,7 +343,8 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
         int pend_step = -1;
         auto flush_spikes = [&]() __attribute__((always_inline)) {
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
-            if (fast) {
+            if (g.debug & 2) {
+            } else if (fast) {
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi)
                     if (row_ok[gi]) *reinterpret_cast<Pack<XT, 8>*>(out + lane_off[gi]) = pend[gi];
@@ -345,7 +371,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
                 for (int chunk = 0; chunk < g.nchunks; ++chunk) {
                     if (!dbl) __syncthreads();   // single buffer: every wave is done reading the previous stage
                     write_lds(buf);              // waits for the stage's loads
-                    __syncthreads();
+                    if (!(g.debug & 4)) __syncthreads();
                     if (pend_step >= 0) flush_spikes();
                     // ---- the stage after this one: next chunk, next timestep, or the first stage of the next tile.
                     int ns = step, nc = chunk + 1, nimg = img, npx = px0;
@@ -362,13 +388,55 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
                             npx = next_px0;
                         }
                     }
-                    if (WL && more) issue_loads(ns, nc, nimg, npx);
+                    if (WM != PW_WEIGHTS_STREAM && more) issue_loads(ns, nc, nimg, npx);
                     if (wave_has_work) {
                         const unsigned char* __restrict__ bp0 = lds + buf * x_buf_bytes + b_off0;
-                        const unsigned char* __restrict__ bp1 = bp0 + g.pitch;
+                        const unsigned char* __restrict__ bp1 = bp0 + 32 * g.pitch;
                         int pair = 0;
-                        if constexpr (WL) {
+                        if constexpr (WR) {
+                            // Exactly kPwRegPairs pairs, straight-line: operand reads run two pairs ahead of the matrix unit.
+                            cv_u32x4 b0[kPwRegPairs], b1[kPwRegPairs];
+#pragma unroll
+                            for (int q = 0; q < kPwRegPairs; ++q) {
+                                b0[q] = *reinterpret_cast<const cv_u32x4*>(bp0 + q * 32);
+                                b1[q] = *reinterpret_cast<const cv_u32x4*>(bp1 + q * 32);
+                            }
+#pragma unroll
+                            for (int q = 0; q < kPwRegPairs; ++q) {
+                                acc[0] = cv_mfma<F16>(a_reg[q], b0[q], acc[0]);
+                                acc[1] = cv_mfma<F16>(a_reg[q], b1[q], acc[1]);
+                            }
+                            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                            for (int q = 0; q < kPwRegPairs - 2; ++q) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                            }
+                            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                        } else if constexpr (WL) {
                             const unsigned char* __restrict__ ap = wl + static_cast<size_t>(chunk * g.npairs) * kFragBytes;
+                            for (; pair + 4 <= g.npairs; pair += 4) {
+                                // All twelve operand reads go out before the first matrix instruction.
+                                cv_u32x4 a[4], b0[4], b1[4];
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    a[q] = *reinterpret_cast<const cv_u32x4*>(ap + (pair + q) * kFragBytes);
+                                    b0[q] = *reinterpret_cast<const cv_u32x4*>(bp0 + (pair + q) * 32);
+                                    b1[q] = *reinterpret_cast<const cv_u32x4*>(bp1 + (pair + q) * 32);
+                                }
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) {
+                                    acc[0] = cv_mfma<F16>(a[q], b0[q], acc[0]);
+                                    acc[1] = cv_mfma<F16>(a[q], b1[q], acc[1]);
+                                }
+                                // Instruction order for the scheduler: two pairs' operands in flight ahead of the matrix unit.
+                                __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            }
                             for (; pair + 2 <= g.npairs; pair += 2) {
                                 const cv_u32x4 a0 = *reinterpret_cast<const cv_u32x4*>(ap + pair * kFragBytes);
                                 const cv_u32x4 a1 = *reinterpret_cast<const cv_u32x4*>(ap + (pair + 1) * kFragBytes);
@@ -404,7 +472,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
                         }
                     }
                     // Streaming weights share the load counter: the next stage's loads go out behind them.
-                    if (!WL && more) issue_loads(ns, nc, nimg, npx);
+                    if (WM == PW_WEIGHTS_STREAM && more) issue_loads(ns, nc, nimg, npx);
                     buf ^= dbl;
                 }
             }
@@ -424,7 +492,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
                     }
                     __builtin_amdgcn_wave_barrier();
                     const Pack<float, 4> xlo = *reinterpret_cast<const Pack<float, 4>*>(stage_rd);
-                    const Pack<float, 4> xhi = *reinterpret_cast<const Pack<float, 4>*>(stage_rd + 4);
+                    const Pack<float, 4> xhi = *reinterpret_cast<const Pack<float, 4>*>(stage_rd + 32);
                     float x[8];
 #pragma unroll
                     for (int k = 0; k < 4; ++k) { x[k] = xlo.v[k]; x[4 + k] = xhi.v[k]; }
@@ -460,7 +528,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
 
         // ---- last timestep's spikes and the final membrane.
         if (pend_step >= 0) flush_spikes();
-        if (fast && g.v_is_f32) {
+        if (fast && vf32) {
             char* vbase = reinterpret_cast<char*>(static_cast<float*>(v_out) + tile_off);
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi) {
@@ -480,7 +548,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         if (okmask & (1u << k)) {
-                            if (g.v_is_f32) static_cast<float*>(v_out)[tile_off + lane_off[gi] / ES + k] = v[gi][k];
+                            if (vf32) static_cast<float*>(v_out)[tile_off + lane_off[gi] / ES + k] = v[gi][k];
                             else static_cast<XT*>(v_out)[tile_off + lane_off[gi] / ES + k] = from_float<XT>(v[gi][k]);
                         }
                     }
@@ -496,10 +564,10 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_pw_lif_kernel(const Step
 }
 
 template <typename XT>
-int launch_conv_pw(const ConvLaunch& L, int load_mode) {
+int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     auto run = [&](auto kernel) -> int {
         if (L.lds_bytes > 64 * 1024) {
-            static bool raised[64] = {};
+            static bool raised[64] = {};   // per kernel instantiation and device
             int dev = 0;
             if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
             if (!raised[dev]) {
@@ -514,12 +582,17 @@ int launch_conv_pw(const ConvLaunch& L, int load_mode) {
                                                                       static_cast<XT*>(L.spikes), L.v_out, L.lif);
         return check_launch("snnf_conv_lif");
     };
-    const bool std_lif = L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset;
+    // Fast variants exist for the common neuron only (power-of-two tau, hard reset); the general variants take any
+    // neuron through the generic update and keep their weights in LDS or stream them.
     auto pick = [&](auto lm) -> int {
         constexpr int LMV = decltype(lm)::value;
-        if (L.g.w_lds)
-            return std_lif ? run(conv_pw_lif_kernel<XT, LMV, true, true>) : run(conv_pw_lif_kernel<XT, LMV, false, true>);
-        return std_lif ? run(conv_pw_lif_kernel<XT, LMV, true, false>) : run(conv_pw_lif_kernel<XT, LMV, false, false>);
+        if (fast) {
+            if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true>);
+            if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_LDS, true>);
+            return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_STREAM, true>);
+        }
+        if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LMV, false, PW_WEIGHTS_LDS, false>);
+        return run(conv_pw_lif_kernel<XT, LMV, false, PW_WEIGHTS_STREAM, false>);
     };
     if constexpr (sizeof(XT) == 4) {
         return pick(std::integral_constant<int, LOAD_2XF32>{});
