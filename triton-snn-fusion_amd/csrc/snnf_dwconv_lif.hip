@@ -12,6 +12,12 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kItems = 2;     // output strips per thread
 constexpr int kColOffset = 4;  // LDS column of input column 0 (keeps 16-byte alignment; column 3 is the left halo)
+constexpr size_t kDwMaxLds = 64 * 1024;
+typedef float dw_f32x4 __attribute__((ext_vector_type(4)));   // one 16-byte LDS access
+
+// Input vectors a thread prefetches per timestep: a stride-2 band has about four input vectors per output strip.
+template <int STRIDE>
+__host__ __device__ constexpr int kLoadSlots() { return STRIDE == 1 ? 3 : 8; }
 
 struct DwGeom {
     int planes;      // N * C
@@ -32,7 +38,23 @@ __device__ __forceinline__ void load_strip_as_float(const XT* __restrict__ p, fl
     for (int i = 0; i < PX; ++i) out[i] = to_float(raw.v[i]);
 }
 
-template <typename XT, typename VT, int STRIDE, int PX>
+// Entry i of a pointer table passed by value as a kernel argument, read from the kernel-argument segment with a scalar
+// load (explicit arguments start at offset 0 of that segment, in declaration order).
+__device__ __forceinline__ const void* dw_table_entry(int table_offset_bytes, int i) {
+    typedef const void* cvp;
+    typedef const __attribute__((address_space(4))) unsigned char* ka_bytes;
+    typedef const __attribute__((address_space(4))) cvp* ka_entry;
+    ka_bytes ka = (ka_bytes)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(ka_entry)(ka + table_offset_bytes + i * 8);
+}
+
+// Pipeline of one timestep: the step's input vectors, prefetched into registers during the previous step, are widened
+// to fp32 and written into one of two LDS tiles; one workgroup barrier; the previous step's spikes leave (they waited
+// in registers so that the wait for the prefetched loads never finds fresh stores in front of it); the next step's
+// loads are issued; then the 3x3 taps and the LIF update run on the tile. The two pointer tables MUST be the first two
+// kernel parameters.
+// STD: the common neuron (power-of-two tau, hard reset) inlined without per-element mode branches.
+template <typename XT, typename VT, int STRIDE, int PX, bool STD>
 __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, StepPtrs residuals, int has_residual,
                                                                  int T, DwGeom g, const XT* __restrict__ weight,
                                                                  const XT* __restrict__ bias,
@@ -41,7 +63,10 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
                                                                  VT* __restrict__ v_out, LifParams lif) {
     extern __shared__ __align__(16) float tile[];
     constexpr int IN_COLS = (PX - 1) * STRIDE + 3;
+    constexpr int KL = kLoadSlots<STRIDE>();           // input vectors a thread prefetches per timestep
+    constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
 
+    const int tid = threadIdx.x;
     const int band = blockIdx.x % g.bands;
     const int plane0 = (blockIdx.x / g.bands) * g.PB;
     const int planes_here = min(g.PB, g.planes - plane0);
@@ -49,100 +74,169 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
     const int rows_here = min(g.TH, g.Ho - row0);
     const int in_row0 = row0 * STRIDE - 1;              // input row held in LDS row 0
     const int plane_floats = g.RIN * g.pitch;
+    const int buf_floats = g.PB * plane_floats;
 
-    // Zero the whole tile once: halo columns and out-of-image rows stay zero for every timestep.
-    for (int i = threadIdx.x; i < g.PB * plane_floats; i += kThreads) tile[i] = 0.0f;
+    // Zero both tiles once: halo columns and out-of-image rows stay zero for every timestep.
+    for (int i = tid; i < 2 * buf_floats; i += kThreads) tile[i] = 0.0f;
 
-    // Fixed ownership of output strips for the whole time loop.
+    // ---- fixed ownership of input vectors (PX elements of one input row) for the whole time loop.
+    const int load_vectors = planes_here * g.RIN * g.WV;
+    uint32_t ld_src[KL];     // byte offset from the first plane of this workgroup; 0 for an idle slot
+    int ld_dst[KL];          // float offset into a tile; -1 for an idle slot
+#pragma unroll
+    for (int k = 0; k < KL; ++k) {
+        const int i = tid + k * kThreads;
+        ld_src[k] = 0;
+        ld_dst[k] = -1;
+        if (i < load_vectors) {
+            const int p = i / (g.RIN * g.WV);
+            const int rem = i - p * (g.RIN * g.WV);
+            const int r = rem / g.WV;
+            const int cv = rem - r * g.WV;
+            const int ih = in_row0 + r;
+            if (ih >= 0 && ih < g.H) {
+                ld_src[k] = static_cast<uint32_t>((p * g.H + ih) * g.W + cv * PX) * ES;
+                ld_dst[k] = p * plane_floats + r * g.pitch + kColOffset + cv * PX;
+            }
+        }
+    }
+    const int64_t in_base = static_cast<int64_t>(plane0) * g.H * g.W;    // elements
+
+    // ---- fixed ownership of output strips.
     const int strips_per_plane = rows_here * g.SW;
     const int strips = planes_here * strips_per_plane;
-    int item_plane[kItems], item_row[kItems], item_col[kItems];
+    int item_src[kItems];          // float offset of the strip's top-left input (left halo) inside a tile
+    uint32_t item_out[kItems];     // element offset of the strip from the first output plane of this workgroup
     bool item_live[kItems];
     float v[kItems][PX];
     float w[kItems][9];
     float b[kItems];
+    const int64_t out_base = (static_cast<int64_t>(plane0) * g.Ho + row0) * g.Wo;   // elements
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
-        const int i = threadIdx.x + k * kThreads;
+        const int i = tid + k * kThreads;
         item_live[k] = i < strips;
         const int ii = item_live[k] ? i : 0;
-        item_plane[k] = ii / strips_per_plane;
-        const int rem = ii - item_plane[k] * strips_per_plane;
-        item_row[k] = rem / g.SW;
-        item_col[k] = (rem - item_row[k] * g.SW) * PX;
-        const int c = (plane0 + item_plane[k]) % g.C;
+        const int ip = ii / strips_per_plane;
+        const int rem = ii - ip * strips_per_plane;
+        const int ir = rem / g.SW;
+        const int ic = (rem - ir * g.SW) * PX;
+        item_src[k] = ip * plane_floats + (ir * STRIDE) * g.pitch + (kColOffset - 1) + ic * STRIDE;
+        item_out[k] = static_cast<uint32_t>((ip * g.Ho + ir) * g.Wo + ic);
+        const int c = (plane0 + ip) % g.C;
 #pragma unroll
         for (int j = 0; j < 9; ++j) w[k][j] = to_float(weight[c * 9 + j]);
         b[k] = to_float(bias[c]);
-        const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
         if (item_live[k] && v_init != nullptr) {
-            load_strip_as_float<VT, PX>(v_init + o, v[k]);
+            load_strip_as_float<VT, PX>(v_init + out_base + item_out[k], v[k]);
         } else {
 #pragma unroll
             for (int j = 0; j < PX; ++j) v[k][j] = 0.0f;
         }
     }
 
-    const int load_vectors = planes_here * g.RIN * g.WV;
-    for (int t = 0; t < T; ++t) {
-        __syncthreads();  // previous step's reads (or the zero fill) are complete
-        const XT* __restrict__ x = static_cast<const XT*>(xs.p[t]);
-        for (int i = threadIdx.x; i < load_vectors; i += kThreads) {
-            const int p = i / (g.RIN * g.WV);
-            const int rem = i - p * (g.RIN * g.WV);
-            const int r = rem / g.WV;
-            const int cv = rem - r * g.WV;
-            const int ih = in_row0 + r;
-            if (ih < 0 || ih >= g.H) continue;
-            float vals[PX];
-            load_strip_as_float<XT, PX>(x + (static_cast<int64_t>(plane0 + p) * g.H + ih) * g.W + cv * PX, vals);
-            float* dst = tile + p * plane_floats + r * g.pitch + kColOffset + cv * PX;
+    // ---- prefetch registers and the spikes waiting to be stored.
+    Pack<XT, PX> pre[KL];
+    auto issue_loads = [&](int t) __attribute__((always_inline)) {
+        const char* __restrict__ x = reinterpret_cast<const char*>(static_cast<const XT*>(dw_table_entry(0, t)) + in_base);
 #pragma unroll
-            for (int j = 0; j < PX; ++j) dst[j] = vals[j];
-        }
-        __syncthreads();
+        for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const Pack<XT, PX>*>(x + ld_src[k]);
+    };
+    Pack<XT, PX> pend[kItems];
+    int pend_t = -1;
+    auto flush = [&]() __attribute__((always_inline)) {
+        XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k)
+            if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+        pend_t = -1;
+    };
 
+    issue_loads(0);
+    __syncthreads();   // zero fill complete
+    int buf = 0;
+    for (int t = 0; t < T; ++t) {
+        float* __restrict__ cur = tile + buf * buf_floats;
+#pragma unroll
+        for (int k = 0; k < KL; ++k) {
+            if (ld_dst[k] >= 0) {
+                float* dst = cur + ld_dst[k];
+                if constexpr (PX % 4 == 0) {
+#pragma unroll
+                    for (int q = 0; q < PX / 4; ++q) {
+                        const dw_f32x4 four = {to_float(pre[k].v[4 * q]), to_float(pre[k].v[4 * q + 1]),
+                                               to_float(pre[k].v[4 * q + 2]), to_float(pre[k].v[4 * q + 3])};
+                        *reinterpret_cast<dw_f32x4*>(dst + 4 * q) = four;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < PX; ++j) dst[j] = to_float(pre[k].v[j]);
+                }
+            }
+        }
+        __syncthreads();   // tile of step t complete; every wave is past its reads of the other tile
+        if (pend_t >= 0) flush();
+        if (t + 1 < T) issue_loads(t + 1);
+
+        const XT* __restrict__ res = has_residual ? static_cast<const XT*>(dw_table_entry(sizeof(StepPtrs), t)) + out_base : nullptr;
 #pragma unroll
         for (int k = 0; k < kItems; ++k) {
-            if (!item_live[k]) continue;
-            const float* src = tile + item_plane[k] * plane_floats + (item_row[k] * STRIDE) * g.pitch +
-                               (kColOffset - 1) + item_col[k] * STRIDE;
+            const float* __restrict__ src = cur + item_src[k];
             float acc[PX];
 #pragma unroll
             for (int j = 0; j < PX; ++j) acc[j] = b[k];
 #pragma unroll
             for (int kh = 0; kh < 3; ++kh) {
                 float in[IN_COLS];
+                if constexpr (PX == 8 && STRIDE == 1) {
+                    // left halo, two aligned 16-byte reads, right halo
+                    const float* row = src + kh * g.pitch;
+                    in[0] = row[0];
+                    const dw_f32x4 lo = *reinterpret_cast<const dw_f32x4*>(row + 1);
+                    const dw_f32x4 hi = *reinterpret_cast<const dw_f32x4*>(row + 5);
+                    in[9] = row[9];
 #pragma unroll
-                for (int j = 0; j < IN_COLS; ++j) in[j] = src[kh * g.pitch + j];
+                    for (int j = 0; j < 4; ++j) { in[1 + j] = lo[j]; in[5 + j] = hi[j]; }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < IN_COLS; ++j) in[j] = src[kh * g.pitch + j];
+                }
 #pragma unroll
                 for (int j = 0; j < PX; ++j) {
 #pragma unroll
                     for (int kw = 0; kw < 3; ++kw) acc[j] = fmaf(in[j * STRIDE + kw], w[k][kh * 3 + kw], acc[j]);
                 }
             }
-            const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
-            if (has_residual) {
-                float res[PX];
-                load_strip_as_float<XT, PX>(static_cast<const XT*>(residuals.p[t]) + o, res);
+            if (res != nullptr && item_live[k]) {
+                float r8[PX];
+                load_strip_as_float<XT, PX>(res + item_out[k], r8);
 #pragma unroll
-                for (int j = 0; j < PX; ++j) acc[j] += res[j];
+                for (int j = 0; j < PX; ++j) acc[j] += r8[j];
             }
-            Pack<XT, PX> out;
 #pragma unroll
-            for (int j = 0; j < PX; ++j) out.v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
-            *reinterpret_cast<Pack<XT, PX>*>(spikes + t * spike_step_stride + o) = out;
+            for (int j = 0; j < PX; ++j) {
+                if constexpr (STD) {
+                    const float h = v[k][j] + (acc[j] - v[k][j]) * lif.inv_tau;
+                    const bool fired = h >= lif.v_threshold;
+                    v[k][j] = fired ? lif.v_reset : h;
+                    pend[k].v[j] = spike_value<XT>(fired);
+                } else {
+                    pend[k].v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
+                }
+            }
         }
+        pend_t = t;
+        buf ^= 1;
     }
+    if (pend_t >= 0) flush();
 
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (!item_live[k]) continue;
-        const int64_t o = (static_cast<int64_t>(plane0 + item_plane[k]) * g.Ho + row0 + item_row[k]) * g.Wo + item_col[k];
         Pack<VT, PX> vo;
 #pragma unroll
         for (int j = 0; j < PX; ++j) vo.v[j] = from_float<VT>(v[k][j]);
-        *reinterpret_cast<Pack<VT, PX>*>(v_out + o) = vo;
+        *reinterpret_cast<Pack<VT, PX>*>(v_out + out_base + item_out[k]) = vo;
     }
 }
 
@@ -163,26 +257,33 @@ int launch(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g
         g.PB = max_strips / per_plane;
         if (g.PB > g.planes) g.PB = g.planes;
     }
-    g.bands = (g.Ho + g.TH - 1) / g.TH;
-    g.RIN = (g.TH - 1) * STRIDE + 3;
+    // Row pitch: a multiple of 4 floats (16-byte vectors) but not of 8, so that the 16-byte reads of lanes that sit in
+    // consecutive rows fall into different banks.
     g.pitch = ((g.W + kColOffset + 1) + 3) / 4 * 4;
-    size_t lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
-    while (lds > 64 * 1024 && g.PB > 1) {
-        g.PB = (g.PB + 1) / 2;
-        lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
-    }
-    while (lds > 64 * 1024 && g.TH > 1) {
-        g.TH = (g.TH + 1) / 2;
+    if (g.pitch % 8 == 0) g.pitch += 4;
+    // Two LDS tiles (double buffering) must fit, and a thread prefetches at most kLoadSlots input vectors per timestep.
+    const int max_vectors = kThreads * kLoadSlots<STRIDE>();
+    auto fits = [&]() {
         g.bands = (g.Ho + g.TH - 1) / g.TH;
         g.RIN = (g.TH - 1) * STRIDE + 3;
-        lds = static_cast<size_t>(g.PB) * g.RIN * g.pitch * sizeof(float);
-    }
-    if (lds > 64 * 1024) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: input row of %d pixels does not fit LDS", g.W);
+        const size_t bytes = static_cast<size_t>(2) * g.PB * g.RIN * g.pitch * sizeof(float);
+        return bytes <= kDwMaxLds && g.PB * g.RIN * g.WV <= max_vectors;
+    };
+    while (!fits() && g.PB > 1) g.PB = (g.PB + 1) / 2;
+    while (!fits() && g.TH > 1) g.TH = (g.TH + 1) / 2;
+    if (!fits()) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: input row of %d pixels does not fit LDS", g.W);
+    const size_t lds = static_cast<size_t>(2) * g.PB * g.RIN * g.pitch * sizeof(float);
     const int64_t blocks = static_cast<int64_t>((g.planes + g.PB - 1) / g.PB) * g.bands;
     if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: too many planes");
-    dwconv3x3_lif_kernel<XT, VT, STRIDE, PX><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
-        xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
-        static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    if (lif.charge_mode == CHARGE_SCALE && !lif.soft_reset) {
+        dwconv3x3_lif_kernel<XT, VT, STRIDE, PX, true><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+            xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
+            static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    } else {
+        dwconv3x3_lif_kernel<XT, VT, STRIDE, PX, false><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+            xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
+            static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    }
     return check_launch("snnf_dwconv3x3_lif");
 }
 
