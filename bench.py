@@ -36,6 +36,9 @@ def _parse():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-operator timings of the other workloads")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only copy 256 MiB device to device three times: the known-size kernel that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     return ap.parse_args()
 
 
@@ -81,6 +84,51 @@ def _time_graph(fn, steps: int, warmup: int):
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
+
+
+def _time_kernel(fn, steps: int, warmup: int, reps: int = 10):
+    """Average milliseconds per launch of the operator `fn`: `reps` launches captured into one HIP graph and replayed,
+    HIP events on the replay stream, so that the figure is the kernel's own duration and not the Python call around it.
+    Falls back to timing eager launches when capture is not possible."""
+    import torch
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(reps):
+                fn()
+        replays = max(1, steps // reps)
+        for _ in range(max(1, warmup // reps)):
+            graph.replay()
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop) / (replays * reps)
+        del graph
+        return ms, "graph"
+    except Exception:
+        torch.cuda.synchronize()
+        return _time_gpu(fn, steps, warmup)[0], "eager"
+
+
+# HBM bytes per launch of the default workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE (KiB per dispatch),
+# each scaled by what the same counter reads for a plain 256 MiB device copy (FETCH_SIZE reads half the bytes copied,
+# factor 2.0; WRITE_SIZE reads them exactly, factor 1.0). Valid for mobilenet_block in bf16 only.
+MEASURED_TRAFFIC_BYTES = {
+    ("mobilenet_block", "bf16", "layer0_depthwise3x3"): (50262.5 * 2.0 + 150532.5) * 1024,
+    ("mobilenet_block", "bf16", "layer1_pointwise1x1"): (50522.2 * 2.0 + 301076.0) * 1024,
+}
 
 
 class Prepared:
@@ -220,6 +268,14 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
+    if args.copy_probe:
+        a = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device="cuda:0").normal_()
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes": a.numel() * 4, "copies": 3}))
+        return 0
     from triton_snn_fusion_amd import _lib, workloads as W
     if not _lib.library_available():
         import importlib
@@ -263,13 +319,16 @@ def main() -> int:
         inputs = prep.layer_inputs()
         torch.cuda.synchronize()
         for i, xs in enumerate(inputs):
-            ms, _ = _time_gpu(lambda i=i, xs=xs: prep.run_layer(i, xs), args.steps, max(3, args.warmup // 2))
+            ms, how = _time_kernel(lambda i=i, xs=xs: prep.run_layer(i, xs), args.steps, max(3, args.warmup // 2))
             nbytes, flops = prep.layer_work(i, xs)
             groups = prep.layers[i][5]
             kind = "depthwise3x3" if groups > 1 else ("pointwise1x1" if tuple(prep.layers[i][1].shape[2:]) == (1, 1) else "conv")
+            traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype, f"layer{i}_{kind}"))
+            traffic = None if traffic is None else int(traffic)
             kernels[f"layer{i}_{kind}"] = {
-                "ms": round(ms, 4), "algorithmic_bytes": nbytes, "flops": flops,
-                "hbm": _roofline("hbm", nbytes, ms), "mfma": None if groups > 1 else _roofline("mfma", flops, ms),
+                "ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "flops": flops,
+                "hbm": _roofline("hbm", nbytes, ms, traffic),
+                "mfma": None if groups > 1 else _roofline("mfma", flops, ms, traffic),
             }
         dominant = max(kernels.items(), key=lambda kv: kv[1]["ms"])
         ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
