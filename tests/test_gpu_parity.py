@@ -277,6 +277,43 @@ def test_conv_residual_chaining_packed_out_single_step_and_batched_tn(hip_ops):
     _no_fallback(hip_ops, 8)
 
 
+POINTWISE_CASES = [  # Cin, Cout, H, W, dtype, vdtype, lif, T, residual, tensor v_init
+    (128, 256, 16, 16, BF16, F32, (1.0, 0.0, 2.0), 4, False, False),   # weights in registers, every tile inside its image
+    (128, 256, 14, 14, BF16, F32, (1.0, 0.0, 2.0), 4, True, True),     # + ragged last tile (second launch), residual, v_init
+    (64, 96, 8, 8, BF16, F32, (1.0, 0.0, 4.0), 3, False, False),       # weights in LDS, one chunk of 64 channels
+    (64, 80, 8, 8, BF16, F32, (1.0, 0.0, 2.0), 2, False, True),        # Cout not a multiple of 32: row masks
+    (256, 128, 7, 7, BF16, F32, (1.0, 0.0, 2.0), 4, True, False),      # odd plane (unaligned loads), two chunks
+    (1024, 64, 8, 8, BF16, F32, (1.0, 0.0, 2.0), 2, False, False),     # weights streamed from L2
+    (1024, 64, 5, 5, BF16, F32, (1.0, 0.0, 2.0), 2, False, True),      # streamed + odd plane
+    (24, 32, 10, 10, BF16, F32, (1.0, 0.0, 2.0), 4, False, False),     # channel tail inside a chunk
+    (8, 32, 8, 8, BF16, F32, (1.0, 0.0, 2.0), 4, False, False),        # a single channel group
+    (128, 64, 16, 16, BF16, F32, (1.0, -1.0, 2.0), 4, False, False),   # soft reset: general variant
+    (128, 64, 16, 16, BF16, F32, (0.5, 0.0, 1.0), 5, False, True),     # IF neuron
+    (128, 64, 8, 8, F32, F32, (1.0, 0.0, 2.0), 4, True, False),        # fp32 activations (rounded to bf16 on the way in)
+    (128, 96, 8, 16, F16, F16, (1.0, 0.0, 2.0), 4, False, True),       # f16 with an f16 membrane
+    (192, 64, 16, 8, F16, F32, (1.0, 0.0, 2.0), 17, False, False),     # channel tail in the second chunk, two launch windows
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,dtype,vdtype,lif,T,residual,tensor_v", POINTWISE_CASES)
+def test_pointwise_conv_lif_variants(hip_ops, Cin, Cout, H, W, dtype, vdtype, lif, T, residual, tensor_v):
+    N = 3
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(900 + Cin + Cout + H, T, N, Cin, Cout, H, W, 1, dtype, p=0.25)
+    g = gen(901 + Cin)
+    rs = [q(torch.randn(N, Cout, H, W, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = q(torch.randn(N, Cout, H, W, generator=g) * 0.3, vdtype) if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (1, 1), (0, 0), (1, 1), 1, *lif, residuals=rs)
+    dx, dw, db = [dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype)
+    dv = dev(v0, vdtype) if tensor_v else zero_v(vdtype)
+    if residual:
+        sp, v = S.fused_temporal_conv_add_lif_state(dx, [dev(r, dtype) for r in rs], dw, db, dv, [1, 1], [0, 0], [1, 1], 1, *lif, False)
+    else:
+        sp, v = S.fused_temporal_pointwise_conv_lif_state(dx, dw, db, dv, [1, 1], [0, 0], [1, 1], 1, *lif, False)
+    assert sp.dtype == dtype and v.dtype == vdtype and tuple(sp.shape) == (T, N, Cout, H, W)
+    check(sp, v, ref, v_threshold=lif[0], v_dtype=vdtype, what=f"pointwise {Cin}->{Cout} {H}x{W}")
+    _no_fallback(hip_ops, 1)
+
+
 def test_conv_shared_analog_frame_is_convolved_once_and_matches(hip_ops):
     """Direct encoding: the same analog frame feeds every timestep (the T list entries alias one tensor)."""
     g = gen(41)

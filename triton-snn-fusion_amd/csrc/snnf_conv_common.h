@@ -104,7 +104,6 @@ struct ConvGeom {
     int vec8;                 // runs of 8 output pixels may be stored as one 16-byte-aligned vector
     int64_t spike_step_stride;
     int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
-    int debug;
     int w_lds;                // time-outer kernels: weight fragments streamed from L2 (0), kept in LDS (1) or in registers (2)
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
     int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts

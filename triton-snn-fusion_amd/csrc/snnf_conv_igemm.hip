@@ -200,10 +200,6 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
                                                        static_cast<double>(T) * N * Cout * Ho_real * Wo_real) +
                          4.0 * N * Cout * Ho_real * Wo_real;
     bool time_outer = all_shared || flops / bytes < 200.0;
-    const char* force = getenv("SNNF_CONV_KERNEL");   // "tout" / "tin": override for experiments
-    if (force != nullptr && force[0] == 't' && force[1] == 'o') time_outer = true;
-    if (force != nullptr && force[0] == 't' && force[1] == 'i') time_outer = false;
-
     int window = 0;
     Plan pl = {};
     bool planned = false;
@@ -227,8 +223,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         }
         return bytes;
     };
-    if (time_outer && pointwise && Cin % 8 == 0 && static_cast<int64_t>(Cout) * g.Wo < (1LL << 30) &&
-        !(force != nullptr && force[0] == 't' && force[1] == 'o')) {
+    if (time_outer && pointwise && Cin % 8 == 0 && static_cast<int64_t>(Cout) * g.Wo < (1LL << 30)) {
         // Pointwise kernel: flat tiles of 64 pixels x 128 output channels, no planning needed.
         pw_kernel = planned = true;
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
@@ -321,7 +316,6 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
       for (int part = 0; part < nparts; ++part) {
         L.g = parts[part].g;
         L.g.T = tw;
-        L.g.debug = getenv("SNNF_DEBUG_CONV") ? atoi(getenv("SNNF_DEBUG_CONV")) : 0;
         L.g.shared_x = (all_shared && (window > 1 || time_outer)) ? 1 : 0;
         L.wpacked = static_cast<const uint16_t*>(packed_weight);
         L.bias = reinterpret_cast<const float*>(L.wpacked + packed_weight_elems(pg));

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             const int t = u % TT;
             const int s = u / TT;
             const uint32_t flags = st_meta[s] >> 20;
-            if (!(g.debug & 1) && t < t_in && (flags & 4)) {
+            if (t < t_in && (flags & 4)) {
                 const char* __restrict__ base = static_cast<const char*>(xs.p[t]) + chunk_bytes;  // uniform
                 const int nval = g.Cin - (chunk * g.CK + static_cast<int>((st_meta[s] >> 24) & 31u) * 8);
                 const bool ok0 = flags & 1, ok1 = flags & 2;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
         for (int u = 0; u < MI; ++u) {
             const int t = u % TT;
             const int s = u / TT;
-            if (!(g.debug & 8) && t < t_in && ((st_meta[s] >> 20) & 4)) {
+            if (t < t_in && ((st_meta[s] >> 20) & 4)) {
                 uint32_t e0[8], e1[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             int cg = half & (groups - 1);
             int kh = 0, kw = 0;
             if (half >> g.groups_log2) { kw = 1; if (kw == g.KW) { kw = 0; kh = 1; } }
-            for (int pair = 0; pair < ((g.debug & 2) ? 0 : g.npairs); ++pair, ++gp) {
+            for (int pair = 0; pair < g.npairs; ++pair, ++gp) {
                 if (gp + 1 < total_pairs) {
 #pragma unroll
                     for (int f = 0; f < kNOF; ++f)
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
 #pragma unroll
                     for (int p = 0; p < kNPF; ++p) acc[t][f][p] = acc[0][f][p];
         }
-        if (wave_has_work && !(g.debug & 4)) {
+        if (wave_has_work) {
             float* __restrict__ stage = reinterpret_cast<float*>(lds) + wave * (TT * 8 * kEpiPitch);
             const int rg = lane >> 3;            // channel row of this lane inside a group of 8
             const int pcx = lane & 7;            // pixel chunk: pixels 8 * pcx .. 8 * pcx + 7 of the wave's 64

@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
     // outside are redirected to the tile's first pixels (always valid) and zeroed on their way into LDS.
     auto issue_loads = [&](int step, int chunk, int n, int px0) __attribute__((always_inline)) {
         const char* __restrict__ base = static_cast<const char*>(kernarg_table_entry(0, step)) +
-                                        (static_cast<int64_t>(((g.debug & 1) ? 0 : n) * g.Cin + chunk * g.CK) * P + ((g.debug & 1) ? 0 : px0)) * ES;
+                                        (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES;
         const bool whole = (FAST || px0 + kPwTile <= P) && (chunk + 1) * g.CK <= g.Cin;
         uint32_t src[SS], second[SS];
         uint32_t bad = 0;
@@ -343,8 +343,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         int pend_step = -1;
         auto flush_spikes = [&]() __attribute__((always_inline)) {
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
-            if (g.debug & 2) {
-            } else if (fast) {
+            if (fast) {
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi)
                     if (row_ok[gi]) *reinterpret_cast<Pack<XT, 8>*>(out + lane_off[gi]) = pend[gi];
@@ -371,7 +370,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                 for (int chunk = 0; chunk < g.nchunks; ++chunk) {
                     if (!dbl) __syncthreads();   // single buffer: every wave is done reading the previous stage
                     write_lds(buf);              // waits for the stage's loads
-                    if (!(g.debug & 4)) __syncthreads();
+                    __syncthreads();
                     if (pend_step >= 0) flush_spikes();
                     // ---- the stage after this one: next chunk, next timestep, or the first stage of the next tile.
                     int ns = step, nc = chunk + 1, nimg = img, npx = px0;

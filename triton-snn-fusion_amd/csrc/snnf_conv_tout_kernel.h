@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
 #pragma unroll
         for (int s = 0; s < SS; ++s) {
             const uint32_t flags = st_meta[s] >> 20;
-            if ((flags & 4) && !(g.debug & 1)) {
+            if (flags & 4) {
                 const int nval = g.Cin - (chunk * g.CK + static_cast<int>((st_meta[s] >> 24) & 31u) * 8);
                 const bool ok0 = flags & 1, ok1 = flags & 2;
 #pragma unroll
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
     auto write_lds = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < SS; ++s) {
-            if (((st_meta[s] >> 20) & 4) && !(g.debug & 8)) {
+            if ((st_meta[s] >> 20) & 4) {
                 cv_u32x4 lo, hi;
                 if constexpr (LM == LOAD_PAIR32) {
                     // dword j = (pixel 0, pixel 1) of channel j -> per pixel, channel pairs: one byte permute each.
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
                             issue_loads(0, 0);
                         }
                     }
-                    if (!wave_has_work || (g.debug & 2)) continue;
+                    if (!wave_has_work) continue;
                     int cg = half & (groups - 1);
                     int kh = 0, kw = 0;
                     if (half >> g.groups_log2) { kw = 1; if (kw == g.KW) { kw = 0; kh = 1; } }
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
             }
 
             // ---- LIF step on this wave's 64 x 64 outputs: transpose 8 channel rows at a time through the wave's stage.
-            if (wave_has_work && !(g.debug & 4)) {
+            if (wave_has_work) {
                 XT* __restrict__ out_t = spikes + step * g.spike_step_stride;
                 const XT* __restrict__ res_t = has_residual ? static_cast<const XT*>(step_pointer(residuals, step)) : nullptr;
 #pragma unroll
@@ -466,8 +466,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
                             }
                             sp.v[k] = spike_value<XT>(fired);
                         }
-                        if ((g.debug & 16) && v[gi][0] != 12345.0f) {
-                        } else if (fast) {
+                        if (fast) {
                             *reinterpret_cast<Pack<XT, 8>*>(out_t + row_off + pxoff[0]) = sp;
                         } else {
 #pragma unroll
@@ -480,7 +479,7 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
         }
 
         // ---- final membrane.
-        if (wave_has_work && okmask != 0 && !(g.debug & 32)) {
+        if (wave_has_work && okmask != 0) {
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi) {
                 const int oc = (ocf0 + (gi >> 2)) * 32 + (gi & 3) * 8 + rg;
