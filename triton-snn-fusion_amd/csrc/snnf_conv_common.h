@@ -14,6 +14,7 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kEpiPitch = 68;       // floats per channel row of the epilogue stage (64 pixels + padding)
 constexpr size_t kToutStageBytes = 4 * 64 * 12 * sizeof(float);   // time-outer kernel: four waves x 64 pixels x (8 rows + padding)
 constexpr size_t kPwStageBytes = 4 * 8 * 68 * sizeof(float);      // pointwise kernel: four waves x 8 channel rows x (64 pixels + padding)
+constexpr size_t kMmStageBytes = 8 * 16 * 40 * sizeof(float);     // matrix kernel: eight waves x 16 channel rows x (32 pixels + padding)
 constexpr size_t kEpiBytes = 4 * 4 * 8 * kEpiPitch * sizeof(float);  // four waves x (up to 4 steps x 8 channel rows)
 
 // Channels per chunk staged in LDS; fixed by (Cin, taps, activation width) alone so that packing and the kernel agree.
@@ -107,7 +108,10 @@ struct ConvGeom {
     int w_lds;                // time-outer kernels: weight fragments streamed from L2 (0), kept in LDS (1) or in registers (2)
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
     int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts
+    int tiles_img;            // matrix kernel: tiles per image (tiles_x * tiles_y, tiles never straddle images)
+    int run8;                 // matrix kernel: runs of 8 tile pixels are contiguous and 16-byte aligned in memory
     FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
+    FastDiv d_tiles_img, d_KW;
 };
 
 struct ConvLaunch {
@@ -127,7 +131,8 @@ struct ConvLaunch {
 };
 
 // One launcher per activation dtype (each in its own translation unit so they compile in parallel).
-// tt: 1, 2, 4 = timesteps accumulated side by side; 0 = time-outer kernel; -1 / -2 = pointwise kernel, general / fast.
+// tt: 1, 2, 4 = timesteps accumulated side by side (4-wave kernel); 10 + tt / 20 + tt = 8-wave matrix kernel, general /
+// fast; 0 = time-outer kernel; -1 / -2 = pointwise kernel, general / fast.
 int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode);

@@ -99,6 +99,78 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
     return best > 0.0;
 }
 
+// Tile plan of the 8-wave matrix kernel: wave arrangement WM x WN (WM * WN == 8; a wave owns 32 pixels x 64 channels)
+// and an output tile of TH x TW pixels inside one image (TH * TW <= WM * 32). `fast`: every tile is full and runs of 8
+// tile pixels are contiguous, 16-byte aligned runs in memory.
+struct MmPlan {
+    int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, oc_tiles, run8, all_full;
+    size_t lds_bytes;
+};
+
+bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, bool want_vec8, MmPlan& best_plan) {
+    const bool pair_shift = load_mode == LOAD_PAIR32;
+    const int groups = 1 << g0.groups_log2;
+    const int max_items = 512 * (load_mode == LOAD_PAIR32 ? 2 : 1);
+    const int cus = compute_units();
+    double best = -1.0;
+    for (int wn_log2 = 0; wn_log2 <= 3; ++wn_log2) {
+        const int wm_log2 = 3 - wn_log2;
+        const int PT = (1 << wm_log2) * 32;
+        const int OT = (1 << wn_log2) * 64;
+        const int oc_tiles = (g0.Cout + OT - 1) / OT;
+        const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
+        for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
+            int th = PT / tw;
+            if (th > g0.Ho) th = g0.Ho;
+            const int tiles_x = (g0.Wo + tw - 1) / tw;
+            const int tiles_y = (g0.Ho + th - 1) / th;
+            const int NR = (th - 1) * g0.sh + g0.KH;
+            int WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
+            WT = (WT + 1) & ~1;
+            const size_t bytes = static_cast<size_t>(tt) * NR * WT * g0.pitch + kMmStageBytes;
+            if (bytes > kMaxLds) continue;
+            if (groups * NR * (WT / 2) > max_items) continue;
+            const bool full_width = tw == g0.Wo;
+            const bool run8 = want_vec8 && (full_width ? ((th * g0.Wo) % 8 == 0) : (tw % 8 == 0 && g0.Wo % 8 == 0));
+            const bool all_full = g0.Ho % th == 0 && g0.Wo % tw == 0;
+            const double work = static_cast<double>(g0.N) * tiles_x * tiles_y * oc_tiles;
+            const double lane_eff = static_cast<double>(g0.Ho) * g0.Wo / (static_cast<double>(tiles_x) * tiles_y * PT);
+            const double waves = work < cus ? 1.0 : static_cast<double>(static_cast<long long>((work + cus - 1) / cus));
+            const double fill = work / (waves * cus);
+            const double halo = static_cast<double>(NR) * WT / (static_cast<double>(th) * tw);
+            double score = lane_eff * oc_eff * fill / (1.0 + 0.1 * (halo - 1.0)) / (1.0 + 0.05 * (oc_tiles - 1));
+            if (!run8) score *= 0.4;           // element-wise 2-byte stores are very slow
+            else if (!all_full) score *= 0.8;  // the masked variant
+            if (score > best) {
+                best = score;
+                best_plan = MmPlan{th, tw, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, oc_tiles, run8 ? 1 : 0, all_full ? 1 : 0, bytes};
+            }
+        }
+    }
+    return best > 0.0;
+}
+
+bool plan_mm(const ConvGeom& g, int tt, int load_mode, bool want_vec8, MmPlan& out) {
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
+    static std::mutex mu;
+    static std::map<Key, std::pair<bool, MmPlan>> plans;
+    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, tt, load_mode, want_vec8 ? 1 : 0);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = plans.find(key);
+        if (it != plans.end()) {
+            out = it->second.second;
+            return it->second.first;
+        }
+    }
+    MmPlan p = {};
+    const bool ok = plan_mm_uncached(g, tt, load_mode, want_vec8, p);
+    std::lock_guard<std::mutex> lock(mu);
+    plans[key] = std::make_pair(ok, p);
+    out = p;
+    return ok;
+}
+
 bool plan(const ConvGeom& g, int t_in, int tt, int load_mode, bool want_vec8, Plan& out) {
     using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
     static std::mutex mu;
@@ -235,7 +307,24 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
         if (!planned) time_outer = false;
     }
-    if (!time_outer) {
+    bool mm_kernel = false;
+    MmPlan mp = {};
+    if (!time_outer && !all_shared && pg.CK >= 16 && Cin % 8 == 0) {
+        // 8-wave matrix kernel: the largest window of 4, 2 or 1 timesteps whose halo tiles fit LDS.
+        int w2 = 1;
+        while (w2 < T && w2 < kMaxTT) w2 *= 2;
+        for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
+            if (plan_mm(g, w2, load_mode, vec_ok, mp)) {
+                mm_kernel = planned = true;
+                window = w2;
+            }
+        }
+        if (mm_kernel) {
+            pl.TH = mp.TH; pl.TW = mp.TW; pl.tiles_x = mp.tiles_x; pl.tiles_y = mp.tiles_y; pl.NR = mp.NR; pl.WT = mp.WT;
+            pl.wm_log2 = mp.wm_log2; pl.wn_log2 = mp.wn_log2; pl.oc_tiles = mp.oc_tiles; pl.lds_bytes = mp.lds_bytes;
+        }
+    }
+    if (!time_outer && !mm_kernel) {
         // Timesteps per launch: as many (<= 4) as fit LDS side by side; a shared analog frame needs one tile for any window.
         window = T < kMaxTT ? T : kMaxTT;
         int w2 = 1;
@@ -256,6 +345,8 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.d_TW = make_fast_div(g.TW); g.d_Ho = make_fast_div(g.Ho); g.d_H = make_fast_div(g.H);
     g.d_WTP = make_fast_div(g.WT / 2); g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
     g.d_tiles_x = make_fast_div(g.tiles_x); g.d_oc_tiles = make_fast_div(g.oc_tiles);
+    g.tiles_img = g.tiles_x * g.tiles_y; g.d_tiles_img = make_fast_div(g.tiles_img); g.d_KW = make_fast_div(g.KW);
+    g.run8 = mm_kernel ? mp.run8 : 0;
 
     size_t lds_bytes = pl.lds_bytes;
     if (time_outer && !pw_kernel) {
@@ -269,12 +360,13 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     }
     const int cu_per_xcd = (compute_units() + 7) / 8;
     auto grid_for = [&](const ConvGeom& gg, int per_cu) {
-        const int work_per_xcd = ((gg.tiles_x * gg.tiles_y + 7) / 8) * gg.oc_tiles;
+        const int px_tiles = mm_kernel ? gg.N * gg.tiles_img : gg.tiles_x * gg.tiles_y;
+        const int work_per_xcd = ((px_tiles + 7) / 8) * gg.oc_tiles;
         int slots = cu_per_xcd * per_cu;
         if (slots > work_per_xcd) slots = work_per_xcd;
         return slots * 8;
     };
-    const int per_cu = time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1);
+    const int per_cu = mm_kernel ? 1 : (time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1));
 
     // Pointwise layers: the fast variant takes the tiles that lie inside their image when the layer qualifies (common
     // neuron, aligned outputs, fp32 membrane, whole channel fragments); the general variant takes the ragged last tile of
@@ -300,6 +392,10 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
             r.g.d_tiles_x = make_fast_div(r.g.tiles_x);
             r.lds = pw_config(false, r.g);
         }
+    } else if (mm_kernel) {
+        const bool fast_ok = mp.all_full && mp.run8 && vec_ok && Cout % 64 == 0 && v_dtype == SNNF_F32;
+        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + window;
+        nparts = 1;
     } else {
         parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = time_outer ? 0 : window;
         nparts = 1;

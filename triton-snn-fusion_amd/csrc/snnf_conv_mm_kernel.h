@@ -1,0 +1,464 @@
+// Dense convolution + bias (+ residual) + LIF over up to 4 timesteps side by side, for layers bound by the matrix
+// cores (3x3 and larger kernels with tens to hundreds of channels).
+//
+// Same implicit GEMM as snnf_conv_kernel.h (M = output channels, N = pixels, K = taps x channels, packed weights), built
+// around what limits such a kernel on this machine:
+//   * 8 waves per workgroup, one workgroup per CU: two waves per SIMD, so that one wave's operand reads, LIF epilogue and
+//     stores overlap the other's matrix instructions. A wave owns 64 channels x 32 pixels x TT timesteps (8 accumulator
+//     tiles, 128 registers): a weight fragment feeds TT matrix instructions, an activation fragment two.
+//   * A tile is TH x TW output pixels of ONE image, so a lane's pixel, its LDS address and its output offset are kernel
+//     constants; a tile contributes uniform bases only. The halo tile in LDS holds explicit zeros for padding, so the
+//     matrix loop has no bounds logic: per pair of k-slots the (tap, channel group) offsets are walked on the scalar unit.
+//   * Staging loads are unconditional (out-of-image items read a valid address and are zeroed on their way into LDS)
+//     and issued from a single place one stage ahead; the LIF epilogue runs on a wave-private LDS stage, 16 channel rows
+//     x 32 pixels at a time, so that a lane owns 8 consecutive pixels: 16-byte spike stores, membrane in registers
+//     across the TT steps.
+// FAST: every tile is full, runs of 8 pixels are contiguous and 16-byte aligned, Cout % 64 == 0, fp32 membrane; the
+// general variant masks pixels and rows. Requires Cin > 8 (chunks of at least 16 channels: every pair of k-slots real).
+#pragma once
+
+#include "snnf_conv_pw_kernel.h"
+
+namespace snnf {
+
+constexpr int kMmThreads = 512;
+constexpr int kMmWaves = 8;
+constexpr int kMmStagePitch = 40;                          // floats per channel row of a wave's stage (32 pixels + padding)
+constexpr int kMmStageFloats = 16 * kMmStagePitch;         // 16 channel rows
+static_assert(kMmWaves * kMmStageFloats * sizeof(float) == kMmStageBytes, "host and kernel disagree on the stage size");
+// Spatial staging items per thread, chunk and timestep: 64 prefetch registers in every load mode.
+__host__ __device__ constexpr int mm_staging_slots(int load_mode) { return load_mode == LOAD_PAIR32 ? 2 : 1; }
+typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename XT, int TT, int LM, bool FAST>
+__global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_mm_lif_kernel(
+    const StepPtrs xs, const StepPtrs residuals, const int has_residual, const ConvGeom g,
+    const uint16_t* __restrict__ wpacked, const float* __restrict__ bias, const void* __restrict__ v_init,
+    XT* __restrict__ spikes, void* __restrict__ v_out, const LifParams lif) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
+    constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
+    constexpr int SS = mm_staging_slots(LM);
+    constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int wm = wave & ((1 << g.wm_log2) - 1);
+    const int wn = wave >> g.wm_log2;
+
+    const int groups = 1 << g.groups_log2;
+    const int WTP = g.WT >> 1;
+    const int tile_bytes = g.NR * g.WT * g.pitch;            // one timestep's halo tile
+    float* __restrict__ stage = reinterpret_cast<float*>(lds + TT * tile_bytes) + wave * kMmStageFloats;
+    const int nocf = (g.Cout + 31) >> 5;
+    const int total_pairs = g.nchunks * g.npairs;
+    const int64_t frag_stride_ocf = static_cast<int64_t>(total_pairs) * (kFragBytes / 2);
+    const int64_t plane = static_cast<int64_t>(g.H) * g.W;
+    const int po = g.Ho * g.Wo;
+    const bool pair_shift = LM == LOAD_PAIR32;               // tile columns start at an even input column
+
+    // ---- kernel constants of the staging: item e = (channel group, tile row, column pair).
+    int item_cg[SS], item_r[SS], item_c[SS];                 // item_cg < 0: idle slot
+    uint32_t item_dst[SS];
+    int item_src[SS];                                        // element offset of (cg * 8, row r, column 2 cp) from the tile origin
+#pragma unroll
+    for (int s = 0; s < SS; ++s) {
+        const int e = s * kMmThreads + tid;
+        const int cg = fast_div(e, g.d_stage_rows);
+        const int rem = e - cg * (g.NR * WTP);
+        const int r = fast_div(rem, g.d_WTP);
+        const int cp = rem - r * WTP;
+        item_cg[s] = cg < groups ? cg : -1;
+        item_r[s] = r;
+        item_c[s] = 2 * cp;
+        item_dst[s] = static_cast<uint32_t>((r * g.WT + 2 * cp) * g.pitch + cg * 16);
+        item_src[s] = (cg * 8 * g.H + r) * g.W + 2 * cp;
+    }
+
+    // ---- the stage in flight.
+    uint32_t pre[SS][TT][8][RPE];
+    uint32_t pre_zero0 = 0, pre_zero1 = 0;                   // bit s: first / second column of item s is padding or beyond Cin
+
+    // Loads of channel chunk `chunk` of the tile whose halo starts at input (row ih_lo, column iw_lo) of image n.
+    auto issue_loads = [&](int chunk, int n, int ih_lo, int iw_lo) __attribute__((always_inline)) {
+        const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
+        const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
+        uint32_t off0[SS], off1[SS];
+        uint32_t z0 = 0, z1 = 0;
+#pragma unroll
+        for (int s = 0; s < SS; ++s) {
+            const int ih = ih_lo + item_r[s];
+            const int iw = iw_lo + item_c[s];
+            const bool cok = item_cg[s] >= 0 && chunk * g.CK + item_cg[s] * 8 < g.Cin && ih >= 0 && ih < g.H;
+            const bool ok0 = cok && iw >= 0 && iw < g.W;
+            const bool ok1 = cok && iw + 1 >= 0 && iw + 1 < g.W;
+            const uint32_t src = static_cast<uint32_t>(item_src[s] + tile_rel) * ES;
+            off0[s] = ok0 ? src : 0u;
+            off1[s] = ok1 ? src + ES : 0u;
+            z0 |= ok0 ? 0u : (1u << s);
+            z1 |= ok1 ? 0u : (1u << s);
+        }
+        pre_zero0 = z0;
+        pre_zero1 = z1;
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+            const char* __restrict__ base = reinterpret_cast<const char*>(static_cast<const XT*>(kernarg_table_entry(0, t)) + origin);
+#pragma unroll
+            for (int s = 0; s < SS; ++s) {
+                if (item_cg[s] >= 0) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const char* __restrict__ row = base + j * plane * ES;
+                        if constexpr (LM == LOAD_PAIR32) {
+                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(row + off0[s]);
+                        } else if constexpr (LM == LOAD_2X16) {
+                            pre[s][t][j][0] = *reinterpret_cast<const uint16_t*>(row + off0[s]);
+                            pre[s][t][j][1] = *reinterpret_cast<const uint16_t*>(row + off1[s]);
+                        } else {
+                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(row + off0[s]);
+                            pre[s][t][j][1] = *reinterpret_cast<const uint32_t*>(row + off1[s]);
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    // Registers -> LDS, transposed to [pixel][channel]; padding and absent channels become zeros.
+    auto write_lds = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < SS; ++s) {
+            if (item_cg[s] >= 0) {
+                const bool zero0 = (pre_zero0 >> s) & 1u, zero1 = (pre_zero1 >> s) & 1u;
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    cv_u32x4 lo, hi;
+                    if constexpr (LM == LOAD_PAIR32) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            lo[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], 0x05040100u);
+                            hi[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], 0x07060302u);
+                        }
+                    } else {
+                        uint32_t e0[8], e1[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            if constexpr (LM == LOAD_2X16) {
+                                e0[j] = pre[s][t][j][0];
+                                e1[j] = pre[s][t][j][1];
+                            } else {
+                                e0[j] = float_to_bf16_bits(__uint_as_float(pre[s][t][j][0]));
+                                e1[j] = float_to_bf16_bits(__uint_as_float(pre[s][t][j][1]));
+                            }
+                        }
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            lo[k] = e0[2 * k] | (e0[2 * k + 1] << 16);
+                            hi[k] = e1[2 * k] | (e1[2 * k + 1] << 16);
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        lo[k] = zero0 ? 0u : lo[k];
+                        hi[k] = zero1 ? 0u : hi[k];
+                    }
+                    unsigned char* dst = lds + t * tile_bytes + item_dst[s];
+                    *reinterpret_cast<cv_u32x4*>(dst) = lo;
+                    *reinterpret_cast<cv_u32x4*>(dst + g.pitch) = hi;
+                }
+            }
+        }
+    };
+
+    // ---- tile walk: pixel tiles congruent to this workgroup's XCD; consecutive work items = output-channel tiles.
+    const int xcd = blockIdx.x & 7;
+    const int slots_per_xcd = gridDim.x >> 3;
+    const int n_px_tiles = g.N * g.tiles_img;
+    const int work_per_xcd = ((n_px_tiles + 7) >> 3) * g.oc_tiles;
+    int work = blockIdx.x >> 3;
+    int oc_tile = 0, img = 0, oh0 = 0, ow0 = 0;
+    auto decode = [&](int w, int& oc_t, int& n, int& r0, int& c0) __attribute__((always_inline)) -> bool {
+        if (w >= work_per_xcd) return false;
+        const int pt = fast_div(w, g.d_oc_tiles);
+        const int px_tile = pt * 8 + xcd;
+        if (px_tile >= n_px_tiles) return false;
+        oc_t = w - pt * g.oc_tiles;
+        n = fast_div(px_tile, g.d_tiles_img);
+        const int in_img = px_tile - n * g.tiles_img;
+        const int ty = fast_div(in_img, g.d_tiles_x);
+        r0 = ty * g.TH;
+        c0 = (in_img - ty * g.tiles_x) * g.TW;
+        return true;
+    };
+    auto halo_origin = [&](int r0, int c0, int& ih_lo, int& iw_lo) __attribute__((always_inline)) {
+        ih_lo = r0 * g.sh - g.ph;
+        iw_lo = c0 * g.sw - g.pw;
+        if (pair_shift && (iw_lo & 1)) iw_lo -= 1;
+    };
+    bool have_tile = decode(work, oc_tile, img, oh0, ow0);
+    if (have_tile) {
+        int ih_lo, iw_lo;
+        halo_origin(oh0, ow0, ih_lo, iw_lo);
+        issue_loads(0, img, ih_lo, iw_lo);
+    }
+
+    // ---- kernel constants of the matrix loop: this lane's pixel (block pixel wm * 32 + l32) inside the halo tile.
+    const int mpix = wm * 32 + l32;
+    const int mpr = fast_div(mpix, g.d_TW);
+    const int mpc = mpix - mpr * g.TW;
+    const bool m_inside = mpr < g.TH;                        // lanes beyond the tile read pixel (0, 0): finite, never stored
+    const uint32_t b_base = static_cast<uint32_t>(m_inside ? ((mpr * g.sh) * g.WT + mpc * g.sw) * g.pitch : 0);
+
+    // ---- kernel constants of the epilogue: lane = (channel row lane >> 2 of 16, pixels 8 (lane & 3) .. + 7 of the wave's 32).
+    const int row16 = lane >> 2;
+    const int pcx = lane & 3;
+    const int epix = wm * 32 + pcx * 8;
+    const int epr = fast_div(epix, g.d_TW);
+    const int epc = epix - epr * g.TW;
+    const bool run_inside = epix + 8 <= g.TH * g.TW;         // FAST: runs are whole, so inside or outside as a whole
+    const uint32_t lane_px = static_cast<uint32_t>(epr * g.Wo + epc);
+    float* __restrict__ stage_wr = stage + (half * 4) * kMmStagePitch + l32;
+    const float* __restrict__ stage_rd = stage + row16 * kMmStagePitch + pcx * 8;
+    const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
+    const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+
+    while (have_tile) {
+        int ih_lo, iw_lo;
+        halo_origin(oh0, ow0, ih_lo, iw_lo);
+        // Column of the tile's first output pixel inside the halo tile (0, or 1 when the halo start was aligned down).
+        const int col0 = (ow0 * g.sw - g.pw) - iw_lo;
+        const int ocf0 = ((oc_tile << g.wn_log2) + wn) * 2;
+        const bool wave_has_work = ocf0 < nocf;
+        const uint16_t* __restrict__ wlane = wpacked + lane * 8;
+        const int64_t w_off0 = static_cast<int64_t>(min(ocf0, nocf - 1)) * frag_stride_ocf;
+        const int64_t w_off1 = static_cast<int64_t>(min(ocf0 + 1, nocf - 1)) * frag_stride_ocf;
+
+        cv_f32x16 acc[TT][2];
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[t][f][r] = 0.0f;
+
+        int next_work = work, next_oc_tile = oc_tile, next_img = img, next_oh0 = oh0, next_ow0 = ow0;
+        bool next_tile = false;
+        int gp = 0;                                          // chunk * npairs + pair
+        cv_u32x4 a_cur0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0);
+        cv_u32x4 a_cur1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1);
+        for (int chunk = 0; chunk < g.nchunks; ++chunk) {
+            __syncthreads();   // every wave is done reading the previous stage
+            write_lds();       // waits for the stage's loads
+            __syncthreads();
+            // ---- the stage after this one: next chunk, or the first chunk of the next tile.
+            {
+                int nc = chunk + 1, nimg = img, nih = ih_lo, niw = iw_lo;
+                bool more = true;
+                if (nc == g.nchunks) {
+                    nc = 0;
+                    next_work = work + slots_per_xcd;
+                    next_tile = decode(next_work, next_oc_tile, next_img, next_oh0, next_ow0);
+                    more = next_tile;
+                    nimg = next_img;
+                    halo_origin(next_oh0, next_ow0, nih, niw);
+                }
+                if (more) issue_loads(nc, nimg, nih, niw);
+            }
+            if (wave_has_work) {
+                // k-slot 2 * pair + half -> (tap, channel group); both halves' offsets walked on the scalar unit.
+                const unsigned char* __restrict__ bp = lds + b_base + static_cast<uint32_t>(col0 * g.pitch);
+                for (int pair = 0; pair < g.npairs; ++pair, ++gp) {
+                    const int gn = gp + 1 < total_pairs ? gp + 1 : gp;
+                    const cv_u32x4 a_nxt0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + static_cast<int64_t>(gn) * (kFragBytes / 2));
+                    const cv_u32x4 a_nxt1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + static_cast<int64_t>(gn) * (kFragBytes / 2));
+                    const int s0 = 2 * pair, s1 = 2 * pair + 1;
+                    const int tap0 = s0 >> g.groups_log2, tap1 = s1 >> g.groups_log2;
+                    const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
+                    const int off_even = ((kh0 * g.WT) + (tap0 - kh0 * g.KW)) * g.pitch + (s0 & (groups - 1)) * 16;
+                    const int off_odd = ((kh1 * g.WT) + (tap1 - kh1 * g.KW)) * g.pitch + (s1 & (groups - 1)) * 16;
+                    const unsigned char* __restrict__ bq = bp + (half ? off_odd : off_even);
+                    cv_u32x4 b[TT];
+#pragma unroll
+                    for (int t = 0; t < TT; ++t) b[t] = *reinterpret_cast<const cv_u32x4*>(bq + t * tile_bytes);
+#pragma unroll
+                    for (int t = 0; t < TT; ++t) {
+                        acc[t][0] = cv_mfma<F16>(a_cur0, b[t], acc[t][0]);
+                        acc[t][1] = cv_mfma<F16>(a_cur1, b[t], acc[t][1]);
+                    }
+                    a_cur0 = a_nxt0;
+                    a_cur1 = a_nxt1;
+                }
+            } else {
+                gp += g.npairs;
+            }
+        }
+
+        // ---- epilogue: 16 channel rows x 32 pixels at a time through the wave's stage; the membrane of a lane's 8 pixels
+        // lives in registers across the TT steps. h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
+        if (wave_has_work) {
+            const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo);
+            const bool fast = FAST || (g.vec8 && full && g.run8);
+            const bool vf32 = FAST || g.v_is_f32;
+            uint32_t okmask = 0xffu;
+            uint32_t pxoff[8];
+            if (!fast) {
+                okmask = 0;
+                int pr = epr, pc = epc;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const bool ok = pr < g.TH && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
+                    okmask |= ok ? (1u << k) : 0u;
+                    pxoff[k] = ok ? static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
+                    if (++pc == g.TW) { pc = 0; ++pr; }
+                }
+            } else {
+                okmask = run_inside ? 0xffu : 0u;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pxoff[k] = lane_px + k;
+            }
+            const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * po + oh0 * g.Wo + ow0;   // uniform, elements
+#pragma unroll
+            for (int f = 0; f < 2; ++f) {
+#pragma unroll
+                for (int ps = 0; ps < 2; ++ps) {
+                    // rows of this pass: channels (ocf0 + f) * 32 + 16 * ps + [0, 16); accumulator rows r = 8 ps .. 8 ps + 7.
+                    const int oc = (ocf0 + f) * 32 + ps * 16 + row16;
+                    const bool row_ok = (FAST || oc < g.Cout) && okmask != 0;
+                    const uint32_t row_off = static_cast<uint32_t>(oc) * static_cast<uint32_t>(po);
+                    const float bvv = (FAST || oc < g.Cout) ? bias[oc] : 0.0f;
+                    float v[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) v[k] = 0.0f;
+                    if (v_init != nullptr && row_ok) {
+                        if (fast && vf32) {
+                            const float* src = static_cast<const float*>(v_init) + tile_off + row_off + pxoff[0];
+                            const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
+                            const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { v[k] = lo.v[k]; v[4 + k] = hi.v[k]; }
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) {
+                                if (okmask & (1u << k)) {
+                                    v[k] = vf32 ? static_cast<const float*>(v_init)[tile_off + row_off + pxoff[k]]
+                                                : to_float(static_cast<const XT*>(v_init)[tile_off + row_off + pxoff[k]]);
+                                }
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < TT; ++t) {
+                        if (t < g.T) {
+                            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                            for (int rr = 0; rr < 8; ++rr)
+                                stage_wr[((rr >> 2) * 8 + (rr & 3)) * kMmStagePitch] = acc[t][f][ps * 8 + rr];
+                            __builtin_amdgcn_wave_barrier();
+                            const cv_f32x4 xlo = *reinterpret_cast<const cv_f32x4*>(stage_rd);
+                            const cv_f32x4 xhi = *reinterpret_cast<const cv_f32x4*>(stage_rd + 4);
+                            float x[8];
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { x[k] = xlo[k] + bvv; x[4 + k] = xhi[k] + bvv; }
+                            XT* __restrict__ out_t = spikes + t * g.spike_step_stride + tile_off + row_off;
+                            if (has_residual && row_ok) {
+                                const XT* __restrict__ res_t = static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), t)) + tile_off + row_off;
+                                if (fast) {
+                                    const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + pxoff[0]);
+#pragma unroll
+                                    for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
+                                } else {
+#pragma unroll
+                                    for (int k = 0; k < 8; ++k)
+                                        if (okmask & (1u << k)) x[k] += to_float(res_t[pxoff[k]]);
+                                }
+                            }
+                            Pack<XT, 8> sp;
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) {
+                                const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
+                                const bool fired = h >= lif.v_threshold;
+                                v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                                sp.v[k] = spike_value<XT>(fired);
+                            }
+                            if (row_ok) {
+                                if (fast) {
+                                    *reinterpret_cast<Pack<XT, 8>*>(out_t + pxoff[0]) = sp;
+                                } else {
+#pragma unroll
+                                    for (int k = 0; k < 8; ++k)
+                                        if (okmask & (1u << k)) out_t[pxoff[k]] = sp.v[k];
+                                }
+                            }
+                        }
+                    }
+                    if (row_ok) {
+                        if (fast && vf32) {
+                            float* dst = static_cast<float*>(v_out) + tile_off + row_off + pxoff[0];
+                            Pack<float, 4> lo, hi;
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
+                            *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
+                            *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) {
+                                if (okmask & (1u << k)) {
+                                    if (vf32) static_cast<float*>(v_out)[tile_off + row_off + pxoff[k]] = v[k];
+                                    else static_cast<XT*>(v_out)[tile_off + row_off + pxoff[k]] = from_float<XT>(v[k]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        work = next_work;
+        oc_tile = next_oc_tile;
+        img = next_img;
+        oh0 = next_oh0;
+        ow0 = next_ow0;
+        have_tile = next_tile;
+    }
+}
+
+template <typename XT, int TT>
+int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
+    auto run = [&](auto kernel) -> int {
+        if (L.lds_bytes > 64 * 1024) {
+            static bool raised[64] = {};   // per kernel instantiation and device
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+            if (!raised[dev]) {
+                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                     static_cast<int>(kMaxLds));
+                if (err != hipSuccess)
+                    return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: cannot reserve %zu bytes of LDS: %s", L.lds_bytes, hipGetErrorString(err));
+                raised[dev] = true;
+            }
+        }
+        kernel<<<dim3(L.grid), kMmThreads, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
+                                                                    static_cast<XT*>(L.spikes), L.v_out, L.lif);
+        return check_launch("snnf_conv_lif");
+    };
+    auto pick = [&](auto lm) -> int {
+        constexpr int LMV = decltype(lm)::value;
+        return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true>) : run(conv_mm_lif_kernel<XT, TT, LMV, false>);
+    };
+    if constexpr (sizeof(XT) == 4) {
+        return pick(std::integral_constant<int, LOAD_2XF32>{});
+    } else {
+        if (load_mode == LOAD_PAIR32) return pick(std::integral_constant<int, LOAD_PAIR32>{});
+        return pick(std::integral_constant<int, LOAD_2X16>{});
+    }
+}
+
+template <typename XT>
+int launch_conv_mm(const ConvLaunch& L, int tt, int load_mode, bool fast) {
+    if (tt == 4) return launch_conv_mm_tt<XT, 4>(L, load_mode, fast);
+    if (tt == 2) return launch_conv_mm_tt<XT, 2>(L, load_mode, fast);
+    return launch_conv_mm_tt<XT, 1>(L, load_mode, fast);
+}
+
+}  // namespace snnf
