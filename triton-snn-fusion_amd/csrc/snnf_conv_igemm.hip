@@ -271,7 +271,10 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     const double bytes = static_cast<double>(xsize) * ((all_shared ? 1 : T) * static_cast<double>(N) * Cin * H * W +
                                                        static_cast<double>(T) * N * Cout * Ho_real * Wo_real) +
                          4.0 * N * Cout * Ho_real * Wo_real;
-    bool time_outer = all_shared || flops / bytes < 200.0;
+    // Dense layers with at least 16 input channels go to the 8-wave matrix kernel whatever their intensity (its per-tile
+    // cost is the lower one); pointwise, few-channel and shared-frame layers stay with the time-outer kernels.
+    const bool matrix_candidate = !pointwise && !all_shared && pg.CK >= 16 && Cin % 8 == 0;
+    bool time_outer = all_shared || (flops / bytes < 200.0 && !matrix_candidate);
     int window = 0;
     Plan pl = {};
     bool planned = false;

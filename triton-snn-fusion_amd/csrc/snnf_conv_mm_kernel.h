@@ -245,10 +245,33 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
 
         int next_work = work, next_oc_tile = oc_tile, next_img = img, next_oh0 = oh0, next_ow0 = ow0;
         bool next_tile = false;
-        int gp = 0;                                          // chunk * npairs + pair
-        cv_u32x4 a_cur0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0);
-        cv_u32x4 a_cur1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1);
+        // One pair of k-slots: slot 2 * pair + half -> (tap, channel group); both halves' LDS offsets are computed on the
+        // scalar unit, a lane picks its half's.
+        auto mma_pair = [&](int pair, const unsigned char* __restrict__ bp, const cv_u32x4& a0, const cv_u32x4& a1) __attribute__((always_inline)) {
+            const int s0 = 2 * pair, s1 = 2 * pair + 1;
+            const int tap0 = s0 >> g.groups_log2, tap1 = s1 >> g.groups_log2;
+            const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
+            const int off_even = ((kh0 * g.WT) + (tap0 - kh0 * g.KW)) * g.pitch + (s0 & (groups - 1)) * 16;
+            const int off_odd = ((kh1 * g.WT) + (tap1 - kh1 * g.KW)) * g.pitch + (s1 & (groups - 1)) * 16;
+            const unsigned char* __restrict__ bq = bp + (half ? off_odd : off_even);
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                const cv_u32x4 b = *reinterpret_cast<const cv_u32x4*>(bq + t * tile_bytes);
+                acc[t][0] = cv_mfma<F16>(a0, b, acc[t][0]);
+                acc[t][1] = cv_mfma<F16>(a1, b, acc[t][1]);
+            }
+        };
+        // Weight fragments stream from L2 two pairs ahead of their use, through three register sets.
+        auto load_frags = [&](int gpair, cv_u32x4& a0, cv_u32x4& a1) __attribute__((always_inline)) {
+            const int64_t o = static_cast<int64_t>(min(gpair, total_pairs - 1)) * (kFragBytes / 2);
+            a0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + o);
+            a1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + o);
+        };
+        cv_u32x4 wa[3][2];
         for (int chunk = 0; chunk < g.nchunks; ++chunk) {
+            const int gp0 = chunk * g.npairs;
+            load_frags(gp0, wa[0][0], wa[0][1]);       // in flight across the barriers and the LDS writes below
+            load_frags(gp0 + 1, wa[1][0], wa[1][1]);
             __syncthreads();   // every wave is done reading the previous stage
             write_lds();       // waits for the stage's loads
             __syncthreads();
@@ -267,31 +290,19 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                 if (more) issue_loads(nc, nimg, nih, niw);
             }
             if (wave_has_work) {
-                // k-slot 2 * pair + half -> (tap, channel group); both halves' offsets walked on the scalar unit.
                 const unsigned char* __restrict__ bp = lds + b_base + static_cast<uint32_t>(col0 * g.pitch);
-                for (int pair = 0; pair < g.npairs; ++pair, ++gp) {
-                    const int gn = gp + 1 < total_pairs ? gp + 1 : gp;
-                    const cv_u32x4 a_nxt0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + static_cast<int64_t>(gn) * (kFragBytes / 2));
-                    const cv_u32x4 a_nxt1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + static_cast<int64_t>(gn) * (kFragBytes / 2));
-                    const int s0 = 2 * pair, s1 = 2 * pair + 1;
-                    const int tap0 = s0 >> g.groups_log2, tap1 = s1 >> g.groups_log2;
-                    const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
-                    const int off_even = ((kh0 * g.WT) + (tap0 - kh0 * g.KW)) * g.pitch + (s0 & (groups - 1)) * 16;
-                    const int off_odd = ((kh1 * g.WT) + (tap1 - kh1 * g.KW)) * g.pitch + (s1 & (groups - 1)) * 16;
-                    const unsigned char* __restrict__ bq = bp + (half ? off_odd : off_even);
-                    cv_u32x4 b[TT];
-#pragma unroll
-                    for (int t = 0; t < TT; ++t) b[t] = *reinterpret_cast<const cv_u32x4*>(bq + t * tile_bytes);
-#pragma unroll
-                    for (int t = 0; t < TT; ++t) {
-                        acc[t][0] = cv_mfma<F16>(a_cur0, b[t], acc[t][0]);
-                        acc[t][1] = cv_mfma<F16>(a_cur1, b[t], acc[t][1]);
+                for (int pair = 0; pair < g.npairs; pair += 3) {
+                    load_frags(gp0 + pair + 2, wa[2][0], wa[2][1]);
+                    mma_pair(pair, bp, wa[0][0], wa[0][1]);
+                    if (pair + 1 < g.npairs) {
+                        load_frags(gp0 + pair + 3, wa[0][0], wa[0][1]);
+                        mma_pair(pair + 1, bp, wa[1][0], wa[1][1]);
                     }
-                    a_cur0 = a_nxt0;
-                    a_cur1 = a_nxt1;
+                    if (pair + 2 < g.npairs) {
+                        load_frags(gp0 + pair + 4, wa[1][0], wa[1][1]);
+                        mma_pair(pair + 2, bp, wa[2][0], wa[2][1]);
+                    }
                 }
-            } else {
-                gp += g.npairs;
             }
         }
 
