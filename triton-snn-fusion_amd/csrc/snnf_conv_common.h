@@ -109,7 +109,10 @@ struct ConvGeom {
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
     int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts
     int tiles_img;            // matrix kernel: tiles per image (tiles_x * tiles_y, tiles never straddle images)
-    int run8;                 // matrix kernel: runs of 8 tile pixels are contiguous and 16-byte aligned in memory
+    int run8;                 // matrix kernel: runs of 8 tile pixels are contiguous in memory and aligned for 16-byte
+                              // (8) or 8-byte (4) spike accesses; 0: neither
+    int wk_log2;              // matrix kernel: waves that split K of one output tile
+    int mm_stage_off;         // matrix kernel: LDS offset of the waves' epilogue stages
     FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
     FastDiv d_tiles_img, d_KW;
 };

@@ -103,58 +103,74 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
 // and an output tile of TH x TW pixels inside one image (TH * TW <= WM * 32). `fast`: every tile is full and runs of 8
 // tile pixels are contiguous, 16-byte aligned runs in memory.
 struct MmPlan {
-    int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, oc_tiles, run8, all_full;
+    int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full, stage_off;
     size_t lds_bytes;
 };
 
-bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, bool want_vec8, MmPlan& best_plan) {
+// `vec`: widest aligned spike access the operands allow (8 or 4 elements, 0 = none). The WK waves that split K of one
+// tile cost an LDS reduction, so K is only split when the unsplit tiling leaves most of the machine idle.
+bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan& best_plan) {
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int groups = 1 << g0.groups_log2;
     const int max_items = 512 * (load_mode == LOAD_PAIR32 ? 2 : 1);
     const int cus = compute_units();
     double best = -1.0;
-    for (int wn_log2 = 0; wn_log2 <= 3; ++wn_log2) {
-        const int wm_log2 = 3 - wn_log2;
-        const int PT = (1 << wm_log2) * 32;
-        const int OT = (1 << wn_log2) * 64;
-        const int oc_tiles = (g0.Cout + OT - 1) / OT;
-        const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
-        for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
-            int th = PT / tw;
-            if (th > g0.Ho) th = g0.Ho;
-            const int tiles_x = (g0.Wo + tw - 1) / tw;
-            const int tiles_y = (g0.Ho + th - 1) / th;
-            const int NR = (th - 1) * g0.sh + g0.KH;
-            int WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
-            WT = (WT + 1) & ~1;
-            const size_t bytes = static_cast<size_t>(tt) * NR * WT * g0.pitch + kMmStageBytes;
-            if (bytes > kMaxLds) continue;
-            if (groups * NR * (WT / 2) > max_items) continue;
-            const bool full_width = tw == g0.Wo;
-            const bool run8 = want_vec8 && (full_width ? ((th * g0.Wo) % 8 == 0) : (tw % 8 == 0 && g0.Wo % 8 == 0));
-            const bool all_full = g0.Ho % th == 0 && g0.Wo % tw == 0;
-            const double work = static_cast<double>(g0.N) * tiles_x * tiles_y * oc_tiles;
-            const double lane_eff = static_cast<double>(g0.Ho) * g0.Wo / (static_cast<double>(tiles_x) * tiles_y * PT);
-            const double waves = work < cus ? 1.0 : static_cast<double>(static_cast<long long>((work + cus - 1) / cus));
-            const double fill = work / (waves * cus);
-            const double halo = static_cast<double>(NR) * WT / (static_cast<double>(th) * tw);
-            double score = lane_eff * oc_eff * fill / (1.0 + 0.1 * (halo - 1.0)) / (1.0 + 0.05 * (oc_tiles - 1));
-            if (!run8) score *= 0.4;           // element-wise 2-byte stores are very slow
-            else if (!all_full) score *= 0.8;  // the masked variant
-            if (score > best) {
-                best = score;
-                best_plan = MmPlan{th, tw, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, oc_tiles, run8 ? 1 : 0, all_full ? 1 : 0, bytes};
+    for (int wk_log2 = 0; wk_log2 <= 3; ++wk_log2) {
+        if ((1 << wk_log2) > g0.npairs) break;
+        if (wk_log2 > 0 && g0.nchunks * g0.npairs < 72) break;   // measured: splitting pays from K of about 1152 on
+        for (int wn_log2 = 0; wn_log2 + wk_log2 <= 3; ++wn_log2) {
+            const int wm_log2 = 3 - wn_log2 - wk_log2;
+            const int PT = (1 << wm_log2) * 32;
+            const int OT = (1 << wn_log2) * 64;
+            const int oc_tiles = (g0.Cout + OT - 1) / OT;
+            const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
+            for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
+                int th = PT / tw;
+                if (th > g0.Ho) th = g0.Ho;
+                const int tiles_x = (g0.Wo + tw - 1) / tw;
+                const int tiles_y = (g0.Ho + th - 1) / th;
+                const int NR = (th - 1) * g0.sh + g0.KH;
+                int WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
+                WT = (WT + 1) & ~1;
+                size_t tiles_bytes = static_cast<size_t>(tt) * NR * WT * g0.pitch;
+                if (wk_log2 > 0 && tiles_bytes < 64 * 1024) tiles_bytes = 64 * 1024;    // the split-K partial sums of one timestep
+                const size_t bytes = tiles_bytes + kMmStageBytes;
+                if (bytes > kMaxLds) continue;
+                if (groups * NR * (WT / 2) > max_items) continue;
+                const bool full_width = tw == g0.Wo;
+                int run = 0;
+                for (int cand : {8, 4}) {
+                    if (cand > vec || run != 0) continue;
+                    if (full_width ? ((th * g0.Wo) % cand == 0) : (tw % cand == 0 && g0.Wo % cand == 0)) run = cand;
+                }
+                // `all_full`: every tile is whole and made of whole runs.
+                const bool all_full = g0.Ho % th == 0 && g0.Wo % tw == 0 && run != 0 && (th * tw) % run == 0;
+                const double work = static_cast<double>(g0.N) * tiles_x * tiles_y * oc_tiles;
+                const double lane_eff = static_cast<double>(g0.Ho) * g0.Wo / (static_cast<double>(tiles_x) * tiles_y * PT);
+                const double waves = work < cus ? 1.0 : static_cast<double>(static_cast<long long>((work + cus - 1) / cus));
+                const double fill = work / (waves * cus);
+                const double halo = static_cast<double>(NR) * WT / (static_cast<double>(th) * tw);
+                double score = lane_eff * oc_eff * fill / (1.0 + 0.1 * (halo - 1.0)) / (1.0 + 0.05 * (oc_tiles - 1));
+                score /= 1.0 + 0.08 * ((1 << wk_log2) - 1);
+                if (run == 0) score *= 0.4;        // element-wise 2-byte stores are very slow
+                else if (!all_full) score *= 0.8;  // the masked variant
+                else if (run == 4) score *= 0.95;
+                if (score > best) {
+                    best = score;
+                    best_plan = MmPlan{th, tw, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full ? 1 : 0,
+                                       static_cast<int>(tiles_bytes), bytes};
+                }
             }
         }
     }
     return best > 0.0;
 }
 
-bool plan_mm(const ConvGeom& g, int tt, int load_mode, bool want_vec8, MmPlan& out) {
-    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
+bool plan_mm(const ConvGeom& g, int tt, int load_mode, int vec, MmPlan& out) {
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
     static std::mutex mu;
     static std::map<Key, std::pair<bool, MmPlan>> plans;
-    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, tt, load_mode, want_vec8 ? 1 : 0);
+    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, g.npairs, tt, load_mode, vec);
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = plans.find(key);
@@ -164,7 +180,7 @@ bool plan_mm(const ConvGeom& g, int tt, int load_mode, bool want_vec8, MmPlan& o
         }
     }
     MmPlan p = {};
-    const bool ok = plan_mm_uncached(g, tt, load_mode, want_vec8, p);
+    const bool ok = plan_mm_uncached(g, tt, load_mode, vec, p);
     std::lock_guard<std::mutex> lock(mu);
     plans[key] = std::make_pair(ok, p);
     out = p;
@@ -257,10 +273,14 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     // 8 consecutive output pixels start 16-byte aligned whenever their first pixel offset is a multiple of 8.
     bool vec_ok = ((static_cast<int64_t>(g.Ho) * g.Wo) % 8 == 0) && (spike_step_stride % 8 == 0) && aligned_to(spikes, 16) &&
                   aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16));
+    // The same for runs of 4 pixels (8-byte spike accesses, 16-byte membrane accesses).
+    bool vec4_ok = ((static_cast<int64_t>(g.Ho) * g.Wo) % 4 == 0) && (spike_step_stride % 4 == 0) && aligned_to(spikes, 8) &&
+                   aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16)) && xsize == 2;
     for (int t = 0; t < T; ++t) {
         all_shared = all_shared && xs[t] == xs[0];
         pair_aligned = pair_aligned && aligned_to(xs[t], 4);
         if (residuals != nullptr) vec_ok = vec_ok && aligned_to(residuals[t], 16);
+        if (residuals != nullptr) vec4_ok = vec4_ok && aligned_to(residuals[t], 8);
     }
     const int load_mode = xsize == 4 ? LOAD_2XF32 : (pair_aligned ? LOAD_PAIR32 : LOAD_2X16);
 
@@ -317,7 +337,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         int w2 = 1;
         while (w2 < T && w2 < kMaxTT) w2 *= 2;
         for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
-            if (plan_mm(g, w2, load_mode, vec_ok, mp)) {
+            if (plan_mm(g, w2, load_mode, vec_ok ? 8 : (vec4_ok ? 4 : 0), mp)) {
                 mm_kernel = planned = true;
                 window = w2;
             }
@@ -349,7 +369,9 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.d_WTP = make_fast_div(g.WT / 2); g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
     g.d_tiles_x = make_fast_div(g.tiles_x); g.d_oc_tiles = make_fast_div(g.oc_tiles);
     g.tiles_img = g.tiles_x * g.tiles_y; g.d_tiles_img = make_fast_div(g.tiles_img); g.d_KW = make_fast_div(g.KW);
-    g.run8 = mm_kernel ? mp.run8 : 0;
+    g.run8 = mm_kernel ? mp.run : 0;
+    g.wk_log2 = mm_kernel ? mp.wk_log2 : 0;
+    g.mm_stage_off = mm_kernel ? mp.stage_off : 0;
 
     size_t lds_bytes = pl.lds_bytes;
     if (time_outer && !pw_kernel) {
@@ -396,7 +418,8 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
             r.lds = pw_config(false, r.g);
         }
     } else if (mm_kernel) {
-        const bool fast_ok = mp.all_full && mp.run8 && vec_ok && Cout % 64 == 0 && v_dtype == SNNF_F32;
+        const bool fast_ok = mp.all_full && mp.run >= 4 && Cout % 64 == 0 && v_dtype == SNNF_F32 &&
+                             lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
         parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + window;
         nparts = 1;
     } else {

@@ -13,8 +13,10 @@
 //     and issued from a single place one stage ahead; the LIF epilogue runs on a wave-private LDS stage, 16 channel rows
 //     x 32 pixels at a time, so that a lane owns 8 consecutive pixels: 16-byte spike stores, membrane in registers
 //     across the TT steps.
-// FAST: every tile is full, runs of 8 pixels are contiguous and 16-byte aligned, Cout % 64 == 0, fp32 membrane; the
-// general variant masks pixels and rows. Requires Cin > 8 (chunks of at least 16 channels: every pair of k-slots real).
+//   * SK: layers with few pixels and many channels (deep stages) do not fill the machine with 64 x 32 wave tiles, so
+//     WK waves share an output tile, each taking every WK-th pair of k-slots, and add their sums through LDS.
+// FAST: every tile is full, runs of 8 pixels are contiguous and 16-byte aligned, Cout % 64 == 0, fp32 membrane, the
+// common neuron (power-of-two tau, hard reset); the general variant masks pixels and rows and takes any neuron. Requires Cin > 8 (chunks of at least 16 channels: every pair of k-slots real).
 #pragma once
 
 #include "snnf_conv_pw_kernel.h"
@@ -30,7 +32,7 @@ static_assert(kMmWaves * kMmStageFloats * sizeof(float) == kMmStageBytes, "host 
 __host__ __device__ constexpr int mm_staging_slots(int load_mode) { return load_mode == LOAD_PAIR32 ? 2 : 1; }
 typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
 
-template <typename XT, int TT, int LM, bool FAST>
+template <typename XT, int TT, int LM, bool FAST, bool SK>
 __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_mm_lif_kernel(
     const StepPtrs xs, const StepPtrs residuals, const int has_residual, const ConvGeom g,
     const uint16_t* __restrict__ wpacked, const float* __restrict__ bias, const void* __restrict__ v_init,
@@ -46,12 +48,14 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     const int half = lane >> 5;
     const int l32 = lane & 31;
     const int wm = wave & ((1 << g.wm_log2) - 1);
-    const int wn = wave >> g.wm_log2;
+    const int wn = (wave >> g.wm_log2) & ((1 << g.wn_log2) - 1);
+    const int wk = SK ? (wave >> (g.wm_log2 + g.wn_log2)) : 0;     // K slice of this wave (split-K variant)
+    const int WK = SK ? (1 << g.wk_log2) : 1;
 
     const int groups = 1 << g.groups_log2;
     const int WTP = g.WT >> 1;
     const int tile_bytes = g.NR * g.WT * g.pitch;            // one timestep's halo tile
-    float* __restrict__ stage = reinterpret_cast<float*>(lds + TT * tile_bytes) + wave * kMmStageFloats;
+    float* __restrict__ stage = reinterpret_cast<float*>(lds + g.mm_stage_off) + wave * kMmStageFloats;
     const int nocf = (g.Cout + 31) >> 5;
     const int total_pairs = g.nchunks * g.npairs;
     const int64_t frag_stride_ocf = static_cast<int64_t>(total_pairs) * (kFragBytes / 2);
@@ -217,7 +221,8 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     const int epix = wm * 32 + pcx * 8;
     const int epr = fast_div(epix, g.d_TW);
     const int epc = epix - epr * g.TW;
-    const bool run_inside = epix + 8 <= g.TH * g.TW;         // FAST: runs are whole, so inside or outside as a whole
+    const bool lo_inside = epix + 4 <= g.TH * g.TW;          // FAST: tile sizes are multiples of 4 (8 with 16-byte runs), so
+    const bool hi_inside = epix + 8 <= g.TH * g.TW;          // each half of a lane's run of 8 pixels is inside or outside as a whole
     const uint32_t lane_px = static_cast<uint32_t>(epr * g.Wo + epc);
     float* __restrict__ stage_wr = stage + (half * 4) * kMmStagePitch + l32;
     const float* __restrict__ stage_rd = stage + row16 * kMmStagePitch + pcx * 8;
@@ -270,8 +275,8 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         cv_u32x4 wa[3][2];
         for (int chunk = 0; chunk < g.nchunks; ++chunk) {
             const int gp0 = chunk * g.npairs;
-            load_frags(gp0, wa[0][0], wa[0][1]);       // in flight across the barriers and the LDS writes below
-            load_frags(gp0 + 1, wa[1][0], wa[1][1]);
+            load_frags(gp0 + wk, wa[0][0], wa[0][1]);  // in flight across the barriers and the LDS writes below
+            load_frags(gp0 + wk + WK, wa[1][0], wa[1][1]);
             __syncthreads();   // every wave is done reading the previous stage
             write_lds();       // waits for the stage's loads
             __syncthreads();
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                     nc = 0;
                     next_work = work + slots_per_xcd;
                     next_tile = decode(next_work, next_oc_tile, next_img, next_oh0, next_ow0);
-                    more = next_tile;
+                    more = next_tile && !SK;   // split K: the next tile's loads go out after the epilogue (registers)
                     nimg = next_img;
                     halo_origin(next_oh0, next_ow0, nih, niw);
                 }
@@ -291,139 +296,247 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             }
             if (wave_has_work) {
                 const unsigned char* __restrict__ bp = lds + b_base + static_cast<uint32_t>(col0 * g.pitch);
-                for (int pair = 0; pair < g.npairs; pair += 3) {
-                    load_frags(gp0 + pair + 2, wa[2][0], wa[2][1]);
+                // This wave's pairs of the chunk: wk, wk + WK, ... (every pair when K is not split).
+                for (int pair = wk; pair < g.npairs; pair += 3 * WK) {
+                    load_frags(gp0 + pair + 2 * WK, wa[2][0], wa[2][1]);
                     mma_pair(pair, bp, wa[0][0], wa[0][1]);
-                    if (pair + 1 < g.npairs) {
-                        load_frags(gp0 + pair + 3, wa[0][0], wa[0][1]);
-                        mma_pair(pair + 1, bp, wa[1][0], wa[1][1]);
+                    if (pair + WK < g.npairs) {
+                        load_frags(gp0 + pair + 3 * WK, wa[0][0], wa[0][1]);
+                        mma_pair(pair + WK, bp, wa[1][0], wa[1][1]);
                     }
-                    if (pair + 2 < g.npairs) {
-                        load_frags(gp0 + pair + 4, wa[1][0], wa[1][1]);
-                        mma_pair(pair + 2, bp, wa[2][0], wa[2][1]);
+                    if (pair + 2 * WK < g.npairs) {
+                        load_frags(gp0 + pair + 4 * WK, wa[1][0], wa[1][1]);
+                        mma_pair(pair + 2 * WK, bp, wa[2][0], wa[2][1]);
                     }
                 }
             }
         }
 
-        // ---- epilogue: 16 channel rows x 32 pixels at a time through the wave's stage; the membrane of a lane's 8 pixels
-        // lives in registers across the TT steps. h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
-        if (wave_has_work) {
-            const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo);
-            const bool fast = FAST || (g.vec8 && full && g.run8);
-            const bool vf32 = FAST || g.v_is_f32;
-            uint32_t okmask = 0xffu;
-            uint32_t pxoff[8];
-            if (!fast) {
-                okmask = 0;
-                int pr = epr, pc = epc;
+        // ---- epilogue: 16 channel rows x 32 pixels at a time through the wave's stage, so that a lane owns 8 consecutive
+        // pixels of one channel row; the membrane of those 8 neurons lives in registers across the TT steps.
+        // h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
+        const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo);
+        const bool fast = FAST || (g.vec8 && full && g.run8 == 8);
+        const bool vf32 = FAST || g.v_is_f32;
+        const bool wide = !FAST || g.run8 == 8;          // FAST: 16-byte spike accesses, or 8-byte ones when runs are only 8-byte aligned
+        uint32_t okmask = 0xffu;
+        uint32_t pxoff[8];
+        if (!fast) {
+            okmask = 0;
+            int pr = epr, pc = epc;
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const bool ok = pr < g.TH && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
-                    okmask |= ok ? (1u << k) : 0u;
-                    pxoff[k] = ok ? static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
-                    if (++pc == g.TW) { pc = 0; ++pr; }
-                }
-            } else {
-                okmask = run_inside ? 0xffu : 0u;
-#pragma unroll
-                for (int k = 0; k < 8; ++k) pxoff[k] = lane_px + k;
+            for (int k = 0; k < 8; ++k) {
+                const bool ok = pr < g.TH && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
+                okmask |= ok ? (1u << k) : 0u;
+                pxoff[k] = ok ? static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
+                if (++pc == g.TW) { pc = 0; ++pr; }
             }
-            const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * po + oh0 * g.Wo + ow0;   // uniform, elements
+        } else {
+            okmask = (lo_inside ? 0x0fu : 0u) | (hi_inside ? 0xf0u : 0u);
 #pragma unroll
-            for (int f = 0; f < 2; ++f) {
+            for (int k = 0; k < 8; ++k) pxoff[k] = lane_px + k;
+        }
+        const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * po + oh0 * g.Wo + ow0;   // uniform, elements
+
+        // One group = 16 channel rows (fragment f, half ps) x the wave's 32 pixels; `rows_ok`: this lane's row exists.
+        auto group_row = [&](int gidx, bool& row_ok, uint32_t& row_off, float& bvv) __attribute__((always_inline)) {
+            const int oc = (ocf0 + (gidx >> 1)) * 32 + (gidx & 1) * 16 + row16;
+            row_ok = wave_has_work && (FAST || oc < g.Cout) && okmask != 0;
+            row_off = static_cast<uint32_t>(min(oc, g.Cout - 1)) * static_cast<uint32_t>(po);
+            bvv = (wave_has_work && (FAST || oc < g.Cout)) ? bias[oc] : 0.0f;
+        };
+        auto load_membrane = [&](bool row_ok, uint32_t row_off, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll
-                for (int ps = 0; ps < 2; ++ps) {
-                    // rows of this pass: channels (ocf0 + f) * 32 + 16 * ps + [0, 16); accumulator rows r = 8 ps .. 8 ps + 7.
-                    const int oc = (ocf0 + f) * 32 + ps * 16 + row16;
-                    const bool row_ok = (FAST || oc < g.Cout) && okmask != 0;
-                    const uint32_t row_off = static_cast<uint32_t>(oc) * static_cast<uint32_t>(po);
-                    const float bvv = (FAST || oc < g.Cout) ? bias[oc] : 0.0f;
-                    float v[8];
+            for (int k = 0; k < 8; ++k) v[k] = 0.0f;
+            if (v_init != nullptr && row_ok) {
+                if (fast && vf32) {
+                    const float* src = static_cast<const float*>(v_init) + tile_off + row_off + pxoff[0];
+                    if (okmask & 0x0fu) {
+                        const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) v[k] = 0.0f;
-                    if (v_init != nullptr && row_ok) {
-                        if (fast && vf32) {
-                            const float* src = static_cast<const float*>(v_init) + tile_off + row_off + pxoff[0];
-                            const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
-                            const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+                        for (int k = 0; k < 4; ++k) v[k] = lo.v[k];
+                    }
+                    if (okmask & 0xf0u) {
+                        const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
 #pragma unroll
-                            for (int k = 0; k < 4; ++k) { v[k] = lo.v[k]; v[4 + k] = hi.v[k]; }
-                        } else {
+                        for (int k = 0; k < 4; ++k) v[4 + k] = hi.v[k];
+                    }
+                } else {
 #pragma unroll
-                            for (int k = 0; k < 8; ++k) {
-                                if (okmask & (1u << k)) {
-                                    v[k] = vf32 ? static_cast<const float*>(v_init)[tile_off + row_off + pxoff[k]]
-                                                : to_float(static_cast<const XT*>(v_init)[tile_off + row_off + pxoff[k]]);
-                                }
-                            }
+                    for (int k = 0; k < 8; ++k) {
+                        if (okmask & (1u << k)) {
+                            v[k] = vf32 ? static_cast<const float*>(v_init)[tile_off + row_off + pxoff[k]]
+                                        : to_float(static_cast<const XT*>(v_init)[tile_off + row_off + pxoff[k]]);
                         }
                     }
+                }
+            }
+        };
+        auto store_membrane = [&](bool row_ok, uint32_t row_off, const float (&v)[8]) __attribute__((always_inline)) {
+            if (!row_ok) return;
+            if (fast && vf32) {
+                float* dst = static_cast<float*>(v_out) + tile_off + row_off + pxoff[0];
+                Pack<float, 4> lo, hi;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
+                if (okmask & 0x0fu) *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
+                if (okmask & 0xf0u) *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (okmask & (1u << k)) {
+                        if (vf32) static_cast<float*>(v_out)[tile_off + row_off + pxoff[k]] = v[k];
+                        else static_cast<XT*>(v_out)[tile_off + row_off + pxoff[k]] = from_float<XT>(v[k]);
+                    }
+                }
+            }
+        };
+        // One LIF step of a group: the lane's 8 sums arrive in MFMA layout (xin = accumulator rows 8 ps .. 8 ps + 7 of its
+        // pixel), are transposed through the wave's stage, then bias (+ residual), LIF, spike store.
+        auto lif_step_group = [&](int t, bool row_ok, uint32_t row_off, float bvv, const float (&xin)[8], float (&v)[8]) __attribute__((always_inline)) {
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int rr = 0; rr < 8; ++rr) stage_wr[((rr >> 2) * 8 + (rr & 3)) * kMmStagePitch] = xin[rr];
+            __builtin_amdgcn_wave_barrier();
+            const cv_f32x4 xlo = *reinterpret_cast<const cv_f32x4*>(stage_rd);
+            const cv_f32x4 xhi = *reinterpret_cast<const cv_f32x4*>(stage_rd + 4);
+            float x[8];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { x[k] = xlo[k] + bvv; x[4 + k] = xhi[k] + bvv; }
+            XT* __restrict__ out_t = spikes + t * g.spike_step_stride + tile_off + row_off;
+            if (has_residual && row_ok) {
+                const XT* __restrict__ res_t = static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), t)) + tile_off + row_off;
+                if (fast && wide) {
+                    const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + pxoff[0]);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
+                } else if (fast) {
+                    if (okmask & 0x0fu) {
+                        const Pack<XT, 4> ra = *reinterpret_cast<const Pack<XT, 4>*>(res_t + pxoff[0]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) x[k] += to_float(ra.v[k]);
+                    }
+                    if (okmask & 0xf0u) {
+                        const Pack<XT, 4> rb = *reinterpret_cast<const Pack<XT, 4>*>(res_t + pxoff[0] + 4);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) x[4 + k] += to_float(rb.v[k]);
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (okmask & (1u << k)) x[k] += to_float(res_t[pxoff[k]]);
+                }
+            }
+            Pack<XT, 8> sp;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                bool fired;
+                if constexpr (FAST) {   // the common neuron: power-of-two tau, hard reset
+                    const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
+                    fired = h >= lif.v_threshold;
+                    v[k] = fired ? lif.v_reset : h;
+                } else {
+                    const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
+                    fired = h >= lif.v_threshold;
+                    v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                }
+                sp.v[k] = spike_value<XT>(fired);
+            }
+            if (row_ok) {
+                if (fast && wide) {
+                    *reinterpret_cast<Pack<XT, 8>*>(out_t + pxoff[0]) = sp;
+                } else if (fast) {
+                    Pack<XT, 4> sa, sb;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) { sa.v[k] = sp.v[k]; sb.v[k] = sp.v[4 + k]; }
+                    if (okmask & 0x0fu) *reinterpret_cast<Pack<XT, 4>*>(out_t + pxoff[0]) = sa;
+                    if (okmask & 0xf0u) *reinterpret_cast<Pack<XT, 4>*>(out_t + pxoff[0] + 4) = sb;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (okmask & (1u << k)) out_t[pxoff[k]] = sp.v[k];
+                }
+            }
+        };
+
+        if constexpr (!SK) {
+            if (wave_has_work) {
+#pragma unroll
+                for (int gidx = 0; gidx < 4; ++gidx) {
+                    bool row_ok;
+                    uint32_t row_off;
+                    float bvv, v[8];
+                    group_row(gidx, row_ok, row_off, bvv);
+                    load_membrane(row_ok, row_off, v);
 #pragma unroll
                     for (int t = 0; t < TT; ++t) {
                         if (t < g.T) {
-                            __builtin_amdgcn_wave_barrier();
+                            float xin[8];
 #pragma unroll
-                            for (int rr = 0; rr < 8; ++rr)
-                                stage_wr[((rr >> 2) * 8 + (rr & 3)) * kMmStagePitch] = acc[t][f][ps * 8 + rr];
-                            __builtin_amdgcn_wave_barrier();
-                            const cv_f32x4 xlo = *reinterpret_cast<const cv_f32x4*>(stage_rd);
-                            const cv_f32x4 xhi = *reinterpret_cast<const cv_f32x4*>(stage_rd + 4);
-                            float x[8];
-#pragma unroll
-                            for (int k = 0; k < 4; ++k) { x[k] = xlo[k] + bvv; x[4 + k] = xhi[k] + bvv; }
-                            XT* __restrict__ out_t = spikes + t * g.spike_step_stride + tile_off + row_off;
-                            if (has_residual && row_ok) {
-                                const XT* __restrict__ res_t = static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), t)) + tile_off + row_off;
-                                if (fast) {
-                                    const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + pxoff[0]);
-#pragma unroll
-                                    for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
-                                } else {
-#pragma unroll
-                                    for (int k = 0; k < 8; ++k)
-                                        if (okmask & (1u << k)) x[k] += to_float(res_t[pxoff[k]]);
-                                }
-                            }
-                            Pack<XT, 8> sp;
-#pragma unroll
-                            for (int k = 0; k < 8; ++k) {
-                                const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
-                                const bool fired = h >= lif.v_threshold;
-                                v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
-                                sp.v[k] = spike_value<XT>(fired);
-                            }
-                            if (row_ok) {
-                                if (fast) {
-                                    *reinterpret_cast<Pack<XT, 8>*>(out_t + pxoff[0]) = sp;
-                                } else {
-#pragma unroll
-                                    for (int k = 0; k < 8; ++k)
-                                        if (okmask & (1u << k)) out_t[pxoff[k]] = sp.v[k];
-                                }
-                            }
+                            for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[t][gidx >> 1][(gidx & 1) * 8 + rr];
+                            lif_step_group(t, row_ok, row_off, bvv, xin, v);
                         }
                     }
-                    if (row_ok) {
-                        if (fast && vf32) {
-                            float* dst = static_cast<float*>(v_out) + tile_off + row_off + pxoff[0];
-                            Pack<float, 4> lo, hi;
+                    store_membrane(row_ok, row_off, v);
+                }
+            }
+        } else {
+            // Split K: the WK waves that share an output tile add their partial sums through LDS, one timestep per round (the
+            // halo tiles are dead by then). A group has one owner wave, which adds the WK partial sums in a fixed order and
+            // runs that step's LIF right away, so only the membranes stay in registers between rounds.
+            float* __restrict__ part = reinterpret_cast<float*>(lds);      // [tile wave][wk][quad 0..7][lane][4]
+            const int wt = wave & ((1 << (g.wm_log2 + g.wn_log2)) - 1);
+            bool row_ok[2];
+            uint32_t row_off[2];
+            float bvv[2], v[2][8];
 #pragma unroll
-                            for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
-                            *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
-                            *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
-                        } else {
+            for (int gidx = 0; gidx < 4; ++gidx) {
+                const int owner = g.wk_log2 == 1 ? (gidx >> 1) : (gidx << (g.wk_log2 - 2));
+                if (owner == wk) {
+                    group_row(gidx, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1]);
+                    load_membrane(row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
+                }
+            }
 #pragma unroll
-                            for (int k = 0; k < 8; ++k) {
-                                if (okmask & (1u << k)) {
-                                    if (vf32) static_cast<float*>(v_out)[tile_off + row_off + pxoff[k]] = v[k];
-                                    else static_cast<XT*>(v_out)[tile_off + row_off + pxoff[k]] = from_float<XT>(v[k]);
-                                }
+            for (int t = 0; t < TT; ++t) {
+                if (t < g.T) {   // uniform: every wave takes the same rounds
+                    __syncthreads();   // previous round read; first round: every wave is done with the halo tiles
+#pragma unroll
+                    for (int f = 0; f < 2; ++f)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const cv_f32x4 four = {acc[t][f][4 * q], acc[t][f][4 * q + 1], acc[t][f][4 * q + 2], acc[t][f][4 * q + 3]};
+                            *reinterpret_cast<cv_f32x4*>(part + (((wt * WK + wk) * 8 + f * 4 + q) * 64 + lane) * 4) = four;
+                        }
+                    __syncthreads();
+#pragma unroll
+                    for (int gidx = 0; gidx < 4; ++gidx) {
+                        const int owner = g.wk_log2 == 1 ? (gidx >> 1) : (gidx << (g.wk_log2 - 2));
+                        if (owner == wk) {
+                            cv_f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+                            for (int k = 0; k < WK; ++k) {
+                                const float* __restrict__ src = part + (((wt * WK + k) * 8 + gidx * 2) * 64 + lane) * 4;
+                                lo += *reinterpret_cast<const cv_f32x4*>(src);
+                                hi += *reinterpret_cast<const cv_f32x4*>(src + 256);
                             }
+                            float xin[8];
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { xin[k] = lo[k]; xin[4 + k] = hi[k]; }
+                            lif_step_group(t, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
                         }
                     }
                 }
             }
+#pragma unroll
+            for (int gidx = 0; gidx < 4; ++gidx) {
+                const int owner = g.wk_log2 == 1 ? (gidx >> 1) : (gidx << (g.wk_log2 - 2));
+                if (owner == wk) store_membrane(row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
+            }
+        }
+        if (SK && next_tile) {
+            int nih, niw;
+            halo_origin(next_oh0, next_ow0, nih, niw);
+            issue_loads(0, next_img, nih, niw);
         }
         work = next_work;
         oc_tile = next_oc_tile;
@@ -436,6 +549,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
 
 template <typename XT, int TT>
 int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
+    const bool split_k = L.g.wk_log2 > 0;
     auto run = [&](auto kernel) -> int {
         if (L.lds_bytes > 64 * 1024) {
             static bool raised[64] = {};   // per kernel instantiation and device
@@ -455,7 +569,9 @@ int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
     };
     auto pick = [&](auto lm) -> int {
         constexpr int LMV = decltype(lm)::value;
-        return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true>) : run(conv_mm_lif_kernel<XT, TT, LMV, false>);
+        if (split_k)
+            return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, true>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, true>);
+        return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, false>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, false>);
     };
     if constexpr (sizeof(XT) == 4) {
         return pick(std::integral_constant<int, LOAD_2XF32>{});
