@@ -314,6 +314,42 @@ def test_pointwise_conv_lif_variants(hip_ops, Cin, Cout, H, W, dtype, vdtype, li
     _no_fallback(hip_ops, 1)
 
 
+DENSE_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, residual, tensor v_init
+    (64, 64, 16, 16, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False),    # whole tiles, 16-byte runs
+    (128, 128, 14, 14, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True),    # K split across waves, 8-byte runs
+    (256, 64, 7, 7, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 3, False, True),      # odd plane: masked variant, K split
+    (32, 96, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 3, 2, True, False),     # Cout % 64 != 0, window of 4 with 3 live steps
+    (64, 64, 10, 10, 3, 1, 1, BF16, F32, (1.0, -1.0, 2.0), 2, 2, False, False),   # two steps side by side, soft reset
+    (64, 128, 9, 9, 3, 1, 1, BF16, F32, (0.5, 0.0, 1.0), 1, 2, True, True),       # single step, IF neuron
+    (48, 64, 16, 16, 5, 1, 2, F16, F16, (1.0, 0.0, 2.0), 4, 2, False, True),      # 5x5, f16 with an f16 membrane
+    (64, 64, 16, 16, 3, 2, 1, F32, F32, (1.0, 0.0, 2.0), 4, 2, False, False),     # stride 2, fp32 activations
+    (64, 64, 15, 15, 3, 1, 1, BF16, F32, (1.0, 0.0, 4.0), 4, 2, False, False),    # odd width: unaligned loads
+    (512, 128, 4, 4, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 4, False, False),    # deep and tiny: K split eight ways
+    (64, 64, 16, 16, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 6, 2, True, True),      # two launch windows (4 + 2)
+    (64, 192, 8, 24, 1, 2, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False),    # strided 1x1 (downsample shortcut)
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,stride,pad,dtype,vdtype,lif,T,N,residual,tensor_v", DENSE_CASES)
+def test_dense_conv_lif_matrix_kernel_variants(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, residual, tensor_v):
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(1200 + Cin + Cout + H + k, T, N, Cin, Cout, H, W, k, dtype, p=0.25)
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    g = gen(1201 + Cin)
+    rs = [q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, vdtype) if tensor_v else torch.tensor(0.0)
+    geo = ([stride, stride], [pad, pad], [1, 1], 1)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (stride, stride), (pad, pad), (1, 1), 1, *lif, residuals=rs)
+    dx, dw, db = [dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype)
+    dv = dev(v0, vdtype) if tensor_v else zero_v(vdtype)
+    if residual:
+        sp, v = S.fused_temporal_conv_add_lif_state(dx, [dev(r, dtype) for r in rs], dw, db, dv, *geo, *lif, False)
+    else:
+        sp, v = S.fused_temporal_conv_lif_state(dx, dw, db, dv, *geo, *lif, False)
+    assert sp.dtype == dtype and v.dtype == vdtype and tuple(sp.shape) == (T, N, Cout, Ho, Wo)
+    check(sp, v, ref, v_threshold=lif[0], v_dtype=vdtype, what=f"dense {Cin}->{Cout} k{k} s{stride} {H}x{W}")
+    _no_fallback(hip_ops, 1)
+
+
 def test_conv_shared_analog_frame_is_convolved_once_and_matches(hip_ops):
     """Direct encoding: the same analog frame feeds every timestep (the T list entries alias one tensor)."""
     g = gen(41)
