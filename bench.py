@@ -36,6 +36,9 @@ def _parse():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-operator timings of the other workloads")
+    ap.add_argument("--layers", default=None, choices=["resnet18", "vgg11"],
+                    help="instead of a workload: time every fused conv layer shape of the spiking ResNet-18 (T=4, B=16, "
+                         "224x224) or VGG-11 (T=4, B=64, 32x32) configuration on its own, synthetic spike inputs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only copy 256 MiB device to device three times: the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -210,6 +213,66 @@ def _roofline(bound: str, work: float, ms: float, traffic=None):
             "frac": round(achieved / peak, 4), "traffic": traffic}
 
 
+# (name, Cin, Cout, input size, kernel, stride, padding, residual added before the LIF, one analog frame for all T, count)
+RESNET18_LAYERS = [
+    ("stem 7x7/2 3->64", 3, 64, 224, 7, 2, 3, False, True, 1),
+    ("3x3 64->64 @56", 64, 64, 56, 3, 1, 1, False, False, 2), ("3x3 64->64 @56 +res", 64, 64, 56, 3, 1, 1, True, False, 2),
+    ("3x3/2 64->128 @56", 64, 128, 56, 3, 2, 1, False, False, 1), ("1x1/2 64->128 @56", 64, 128, 56, 1, 2, 0, False, False, 1),
+    ("3x3 128->128 @28", 128, 128, 28, 3, 1, 1, False, False, 1), ("3x3 128->128 @28 +res", 128, 128, 28, 3, 1, 1, True, False, 2),
+    ("3x3/2 128->256 @28", 128, 256, 28, 3, 2, 1, False, False, 1), ("1x1/2 128->256 @28", 128, 256, 28, 1, 2, 0, False, False, 1),
+    ("3x3 256->256 @14", 256, 256, 14, 3, 1, 1, False, False, 1), ("3x3 256->256 @14 +res", 256, 256, 14, 3, 1, 1, True, False, 2),
+    ("3x3/2 256->512 @14", 256, 512, 14, 3, 2, 1, False, False, 1), ("1x1/2 256->512 @14", 256, 512, 14, 1, 2, 0, False, False, 1),
+    ("3x3 512->512 @7", 512, 512, 7, 3, 1, 1, False, False, 1), ("3x3 512->512 @7 +res", 512, 512, 7, 3, 1, 1, True, False, 2),
+]
+VGG11_LAYERS = [
+    ("3x3 3->64 @32", 3, 64, 32, 3, 1, 1, False, True, 1), ("3x3 64->128 @16", 64, 128, 16, 3, 1, 1, False, False, 1),
+    ("3x3 128->256 @8", 128, 256, 8, 3, 1, 1, False, False, 1), ("3x3 256->256 @8", 256, 256, 8, 3, 1, 1, False, False, 1),
+    ("3x3 256->512 @4", 256, 512, 4, 3, 1, 1, False, False, 1), ("3x3 512->512 @4", 512, 512, 4, 3, 1, 1, False, False, 1),
+    ("3x3 512->512 @2", 512, 512, 2, 3, 1, 1, False, False, 2),
+]
+
+
+def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
+    """Times every fused conv(+residual)+LIF layer shape of a network configuration on its own (graph replay, HIP events)."""
+    import torch
+    from triton_snn_fusion_amd import workloads as W
+    ops = torch.ops.snn_custom
+    layers, batch = (RESNET18_LAYERS, 16) if which == "resnet18" else (VGG11_LAYERS, 64)
+    T, dev = 4, torch.device("cuda:0")
+    esize = torch.empty((), dtype=dtype).element_size()
+    g = torch.Generator(device="cpu")
+    g.manual_seed(0)
+    v0 = torch.zeros((), dtype=torch.float32, device=dev)
+    rows, total_ms, total_flops = [], 0.0, 0
+    for name, cin, cout, size, k, stride, pad, residual, analog, count in layers:
+        if analog:
+            frame = torch.randn(batch, cin, size, size, generator=g).to(dev, dtype)
+            xs = [frame] * T
+        else:
+            xs = [(torch.rand(batch, cin, size, size, generator=g) < 0.15).to(dev, dtype) for _ in range(T)]
+        w = (torch.randn(cout, cin, k, k, generator=g) * (2.0 / (cin * k * k)) ** 0.5).to(dev, dtype)
+        b = (torch.randn(cout, generator=g) * 0.1).to(dev, dtype)
+        out = (size + 2 * pad - k) // stride + 1
+        rs = [(torch.rand(batch, cout, out, out, generator=g) < 0.15).to(dev, dtype) for _ in range(T)] if residual else None
+        if residual:
+            fn = lambda: ops.fused_temporal_conv_add_lif_state(xs, rs, w, b, v0, [stride, stride], [pad, pad], [1, 1], 1, 1.0, 0.0, 2.0, False)
+        else:
+            fn = lambda: ops.fused_temporal_conv_lif_state(xs, w, b, v0, [stride, stride], [pad, pad], [1, 1], 1, 1.0, 0.0, 2.0, False)
+        ms, how = _time_kernel(fn, steps, warmup)
+        flops = W.conv_flops(T, batch, cin, cout, out, out, k, k, 1)
+        nbytes = W.algorithmic_conv_bytes(T, batch, cin, size, size, cout, out, out, k, k, 1, esize, 4, shared_input=analog)
+        if residual:
+            nbytes += T * batch * cout * out * out * esize
+        rows.append({"layer": name, "count": count, "ms": round(ms, 4), "timed": how,
+                     "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+        total_ms += ms * count
+        total_flops += flops * count
+    return {"metric": METRIC, "workload": f"{which}_layers", "dtype": dtype_name, "T": T, "batch": batch,
+            "conv_ms_per_forward": round(total_ms, 4), "images_T_per_s_conv_only": round(batch * T / (total_ms * 1e-3), 1),
+            "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
+
+
 def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
     """Eager fp32 PyTorch-CPU path (the oracle's restatement of the reference's eager ops) on a bounded sample."""
     import torch
@@ -284,6 +347,13 @@ def main() -> int:
     ops.configure_fused_op("hip", strict_triton=True)
     device = torch.device("cuda:0")
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+
+    if args.layers is not None:
+        sweep = _layer_sweep(args.layers, dtype, args.dtype, args.steps, args.warmup)
+        stats = ops.get_fused_op_call_stats()
+        sweep["native_calls"], sweep["fallback_calls"] = stats["triton"], stats["fallback"]
+        print(json.dumps(sweep))
+        return 0 if stats["fallback"] == 0 else 1
 
     wl = getattr(W, args.workload)()
     prep = Prepared(wl, dtype, device)
