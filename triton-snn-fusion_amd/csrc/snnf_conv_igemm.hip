@@ -336,8 +336,13 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         // 8-wave matrix kernel: the largest window of 4, 2 or 1 timesteps whose halo tiles fit LDS.
         int w2 = 1;
         while (w2 < T && w2 < kMaxTT) w2 *= 2;
+        const bool fast_layer = Cout % 64 == 0 && v_dtype == SNNF_F32 && lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
         for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
             if (plan_mm(g, w2, load_mode, vec_ok ? 8 : (vec4_ok ? 4 : 0), mp)) {
+                // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
+                // the activation prefetch): it runs windows of 2.
+                const bool fast_plan = fast_layer && mp.all_full && mp.run >= 4;
+                if (w2 == 4 && !fast_plan) continue;
                 mm_kernel = planned = true;
                 window = w2;
             }
@@ -419,7 +424,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         }
     } else if (mm_kernel) {
         const bool fast_ok = mp.all_full && mp.run >= 4 && Cout % 64 == 0 && v_dtype == SNNF_F32 &&
-                             lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+                             lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;   // = fast_plan above
         parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + window;
         nparts = 1;
     } else {
