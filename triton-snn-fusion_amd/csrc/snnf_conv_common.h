@@ -113,8 +113,9 @@ struct ConvGeom {
                               // (8) or 8-byte (4) spike accesses; 0: neither
     int wk_log2;              // matrix kernel: waves that split K of one output tile
     int mm_stage_off;         // matrix kernel: LDS offset of the waves' epilogue stages
+    int stage_chunks;         // matrix kernel: packed channel chunks held by one LDS stage (pitch = stage_chunks * CK * 2 + 16)
     FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
-    FastDiv d_tiles_img, d_KW;
+    FastDiv d_tiles_img, d_KW, d_npairs;
 };
 
 struct ConvLaunch {

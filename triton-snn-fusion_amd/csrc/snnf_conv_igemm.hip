@@ -103,7 +103,7 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
 // and an output tile of TH x TW pixels inside one image (TH * TW <= WM * 32). `fast`: every tile is full and runs of 8
 // tile pixels are contiguous, 16-byte aligned runs in memory.
 struct MmPlan {
-    int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full, stage_off;
+    int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full, stage_off, stage_chunks, pitch;
     size_t lds_bytes;
 };
 
@@ -132,11 +132,18 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan
                 const int NR = (th - 1) * g0.sh + g0.KH;
                 int WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
                 WT = (WT + 1) & ~1;
-                size_t tiles_bytes = static_cast<size_t>(tt) * NR * WT * g0.pitch;
+                // An LDS stage holds as many packed channel chunks as fit (fewer barriers and exposed load latencies per tile).
+                int sc = 1;
+                while (sc * 2 <= g0.nchunks && sc * 2 * g0.CK <= 256 &&
+                       static_cast<size_t>(tt) * NR * WT * (sc * 2 * g0.CK * 2 + 16) + kMmStageBytes <= kMaxLds &&
+                       sc * 2 * groups * NR * (WT / 2) <= max_items)
+                    sc *= 2;
+                const int pitch = sc * g0.CK * 2 + 16;
+                size_t tiles_bytes = static_cast<size_t>(tt) * NR * WT * pitch;
                 if (wk_log2 > 0 && tiles_bytes < 64 * 1024) tiles_bytes = 64 * 1024;    // the split-K partial sums of one timestep
                 const size_t bytes = tiles_bytes + kMmStageBytes;
                 if (bytes > kMaxLds) continue;
-                if (groups * NR * (WT / 2) > max_items) continue;
+                if (sc * groups * NR * (WT / 2) > max_items) continue;
                 const bool full_width = tw == g0.Wo;
                 int run = 0;
                 for (int cand : {8, 4}) {
@@ -158,7 +165,7 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan
                 if (score > best) {
                     best = score;
                     best_plan = MmPlan{th, tw, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full ? 1 : 0,
-                                       static_cast<int>(tiles_bytes), bytes};
+                                       static_cast<int>(tiles_bytes), sc, pitch, bytes};
                 }
             }
         }
@@ -167,10 +174,10 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan
 }
 
 bool plan_mm(const ConvGeom& g, int tt, int load_mode, int vec, MmPlan& out) {
-    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
     static std::mutex mu;
     static std::map<Key, std::pair<bool, MmPlan>> plans;
-    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, g.npairs, tt, load_mode, vec);
+    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, g.npairs, g.nchunks, tt, load_mode, vec);
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = plans.find(key);
@@ -377,6 +384,10 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.run8 = mm_kernel ? mp.run : 0;
     g.wk_log2 = mm_kernel ? mp.wk_log2 : 0;
     g.mm_stage_off = mm_kernel ? mp.stage_off : 0;
+    g.stage_chunks = mm_kernel ? mp.stage_chunks : 1;
+    if (mm_kernel) g.pitch = mp.pitch;
+    g.d_npairs = make_fast_div(g.npairs);
+    if (mm_kernel) g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
 
     size_t lds_bytes = pl.lds_bytes;
     if (time_outer && !pw_kernel) {

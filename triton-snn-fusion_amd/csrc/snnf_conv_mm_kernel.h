@@ -52,7 +52,9 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     const int wk = SK ? (wave >> (g.wm_log2 + g.wn_log2)) : 0;     // K slice of this wave (split-K variant)
     const int WK = SK ? (1 << g.wk_log2) : 1;
 
-    const int groups = 1 << g.groups_log2;
+    const int groups = 1 << g.groups_log2;                   // channel groups of 8 per packed chunk
+    const int stage_groups = groups * g.stage_chunks;        // ... per LDS stage (a stage holds stage_chunks chunks)
+    const int nstages = (g.nchunks + g.stage_chunks - 1) / g.stage_chunks;
     const int WTP = g.WT >> 1;
     const int tile_bytes = g.NR * g.WT * g.pitch;            // one timestep's halo tile
     float* __restrict__ stage = reinterpret_cast<float*>(lds + g.mm_stage_off) + wave * kMmStageFloats;
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         const int rem = e - cg * (g.NR * WTP);
         const int r = fast_div(rem, g.d_WTP);
         const int cp = rem - r * WTP;
-        item_cg[s] = cg < groups ? cg : -1;
+        item_cg[s] = cg < stage_groups ? cg : -1;
         item_r[s] = r;
         item_c[s] = 2 * cp;
         item_dst[s] = static_cast<uint32_t>((r * g.WT + 2 * cp) * g.pitch + cg * 16);
@@ -85,8 +87,10 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     uint32_t pre[SS][TT][8][RPE];
     uint32_t pre_zero0 = 0, pre_zero1 = 0;                   // bit s: first / second column of item s is padding or beyond Cin
 
-    // Loads of channel chunk `chunk` of the tile whose halo starts at input (row ih_lo, column iw_lo) of image n.
-    auto issue_loads = [&](int chunk, int n, int ih_lo, int iw_lo) __attribute__((always_inline)) {
+    // Loads of stage `stg` (stage_chunks channel chunks) of the tile whose halo starts at input (row ih_lo, column iw_lo)
+    // of image n.
+    auto issue_loads = [&](int stg, int n, int ih_lo, int iw_lo) __attribute__((always_inline)) {
+        const int chunk = stg * g.stage_chunks;                                                  // first chunk of the stage
         const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
         const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
         uint32_t off0[SS], off1[SS];
@@ -252,7 +256,10 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         bool next_tile = false;
         // One pair of k-slots: slot 2 * pair + half -> (tap, channel group); both halves' LDS offsets are computed on the
         // scalar unit, a lane picks its half's.
-        auto mma_pair = [&](int pair, const unsigned char* __restrict__ bp, const cv_u32x4& a0, const cv_u32x4& a1) __attribute__((always_inline)) {
+        auto mma_pair = [&](int q, const unsigned char* __restrict__ bp0, const cv_u32x4& a0, const cv_u32x4& a1) __attribute__((always_inline)) {
+            const int sub = fast_div(q, g.d_npairs);                 // chunk inside the stage
+            const int pair = q - sub * g.npairs;
+            const unsigned char* __restrict__ bp = bp0 + sub * (groups * 16);
             const int s0 = 2 * pair, s1 = 2 * pair + 1;
             const int tap0 = s0 >> g.groups_log2, tap1 = s1 >> g.groups_log2;
             const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
@@ -273,8 +280,9 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             a1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + o);
         };
         cv_u32x4 wa[3][2];
-        for (int chunk = 0; chunk < g.nchunks; ++chunk) {
-            const int gp0 = chunk * g.npairs;
+        for (int chunk = 0; chunk < nstages; ++chunk) {        // `chunk` counts LDS stages from here on
+            const int gp0 = chunk * g.stage_chunks * g.npairs;
+            const int spairs = min(g.stage_chunks, g.nchunks - chunk * g.stage_chunks) * g.npairs;   // pairs of this stage
             load_frags(gp0 + wk, wa[0][0], wa[0][1]);  // in flight across the barriers and the LDS writes below
             load_frags(gp0 + wk + WK, wa[1][0], wa[1][1]);
             __syncthreads();   // every wave is done reading the previous stage
@@ -284,7 +292,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             {
                 int nc = chunk + 1, nimg = img, nih = ih_lo, niw = iw_lo;
                 bool more = true;
-                if (nc == g.nchunks) {
+                if (nc == nstages) {
                     nc = 0;
                     next_work = work + slots_per_xcd;
                     next_tile = decode(next_work, next_oc_tile, next_img, next_oh0, next_ow0);
@@ -297,14 +305,14 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             if (wave_has_work) {
                 const unsigned char* __restrict__ bp = lds + b_base + static_cast<uint32_t>(col0 * g.pitch);
                 // This wave's pairs of the chunk: wk, wk + WK, ... (every pair when K is not split).
-                for (int pair = wk; pair < g.npairs; pair += 3 * WK) {
+                for (int pair = wk; pair < spairs; pair += 3 * WK) {
                     load_frags(gp0 + pair + 2 * WK, wa[2][0], wa[2][1]);
                     mma_pair(pair, bp, wa[0][0], wa[0][1]);
-                    if (pair + WK < g.npairs) {
+                    if (pair + WK < spairs) {
                         load_frags(gp0 + pair + 3 * WK, wa[0][0], wa[0][1]);
                         mma_pair(pair + WK, bp, wa[1][0], wa[1][1]);
                     }
-                    if (pair + 2 * WK < g.npairs) {
+                    if (pair + 2 * WK < spairs) {
                         load_frags(gp0 + pair + 4 * WK, wa[1][0], wa[1][1]);
                         mma_pair(pair + 2 * WK, bp, wa[2][0], wa[2][1]);
                     }
