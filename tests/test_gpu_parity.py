@@ -364,6 +364,40 @@ def test_conv_shared_analog_frame_is_convolved_once_and_matches(hip_ops):
     assert torch.equal(s, s2) and torch.equal(v, v2)
 
 
+SHARED_FRAME_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, lif, T, N, residual, tensor v_init
+    (3, 64, 64, 64, 7, 2, 3, BF16, (1.0, 0.0, 2.0), 4, 2, False, False),     # ResNet stem
+    (3, 64, 31, 31, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 2, False, True),      # odd plane: masked variant
+    (1, 32, 28, 28, 5, 1, 2, BF16, (1.0, 0.0, 2.0), 6, 3, False, False),     # one input channel, Cout % 64 != 0
+    (2, 64, 32, 32, 3, 1, 1, F32, (1.0, -1.0, 2.0), 4, 2, True, False),      # fp32 frame, soft reset, residual per step
+    (64, 64, 16, 16, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 5, 2, False, True),     # analog frame with whole channel groups
+    (128, 64, 8, 8, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 2, True, True),       # K split across waves, T steps per round
+    (3, 64, 32, 32, 3, 1, 1, F16, (0.5, 0.0, 1.0), 20, 1, False, False),     # two launch windows (16 + 4), IF neuron
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,stride,pad,dtype,lif,T,N,residual,tensor_v", SHARED_FRAME_CASES)
+def test_conv_shared_analog_frame_variants(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, lif, T, N, residual, tensor_v):
+    """One analog frame for all T timesteps: convolved once, T LIF steps on the same accumulators."""
+    g = gen(1300 + Cin + Cout + H + k)
+    op_dtype = BF16 if dtype == F32 else dtype     # fp32 frames and weights enter the matrix cores as bf16
+    x = q(torch.randn(N, Cin, H, W, generator=g), op_dtype)
+    w = q(torch.randn(Cout, Cin, k, k, generator=g) * (1.5 / (Cin * k * k) ** 0.5), op_dtype)
+    b = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    rs = [q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, F32) if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif([x] * T, w, b, v0, (stride, stride), (pad, pad), (1, 1), 1, *lif, residuals=rs)
+    geo = ([stride, stride], [pad, pad], [1, 1], 1)
+    dx, dv = dev(x, dtype), (dev(v0, F32) if tensor_v else zero_v())
+    if residual:
+        sp, v = S.fused_temporal_conv_add_lif_state([dx] * T, [dev(r, dtype) for r in rs], dev(w, dtype), dev(b, dtype), dv, *geo, *lif, False)
+    else:
+        sp, v = S.fused_temporal_conv_lif_state([dx] * T, dev(w, dtype), dev(b, dtype), dv, *geo, *lif, False)
+    assert tuple(sp.shape) == (T, N, Cout, Ho, Wo)
+    check(sp, v, ref, v_threshold=lif[0], what=f"shared frame {Cin}->{Cout} k{k} s{stride} {H}x{W} T={T}")
+    _no_fallback(hip_ops, 1)
+
+
 def test_conv_and_linear_known_answers_exact(hip_ops):
     """tests/golden/conv_kat.json: exact sums (multiples of 1/8), so bf16 matrix operands must reproduce them bit for
     bit. An integrate-and-fire neuron (tau <= 1) with an unreachable threshold makes v_out the convolution output."""

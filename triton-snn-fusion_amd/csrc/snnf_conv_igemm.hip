@@ -112,7 +112,7 @@ struct MmPlan {
 bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan& best_plan) {
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int groups = 1 << g0.groups_log2;
-    const int max_items = 512 * (load_mode == LOAD_PAIR32 ? 2 : 1);
+    const int max_items = 512 * ((load_mode == LOAD_PAIR32 ? 8 : 4) / tt);
     const int cus = compute_units();
     double best = -1.0;
     for (int wk_log2 = 0; wk_log2 <= 3; ++wk_log2) {
@@ -298,14 +298,39 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     const double bytes = static_cast<double>(xsize) * ((all_shared ? 1 : T) * static_cast<double>(N) * Cin * H * W +
                                                        static_cast<double>(T) * N * Cout * Ho_real * Wo_real) +
                          4.0 * N * Cout * Ho_real * Wo_real;
-    // Dense layers with at least 16 input channels go to the 8-wave matrix kernel whatever their intensity (its per-tile
-    // cost is the lower one); pointwise, few-channel and shared-frame layers stay with the time-outer kernels.
-    const bool matrix_candidate = !pointwise && !all_shared && pg.CK >= 16 && Cin % 8 == 0;
-    bool time_outer = all_shared || (flops / bytes < 200.0 && !matrix_candidate);
+    // Dense layers whose input channels fill whole groups of 8 (or fit a single group) go to the 8-wave matrix kernel
+    // whatever their intensity (its per-tile cost is the lower one); pointwise layers stay with the pointwise kernel.
+    const bool matrix_candidate = !pointwise && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
     Plan pl = {};
     bool planned = false;
     bool pw_kernel = false;
+    bool mm_kernel = false;
+    MmPlan mp = {};
+    if (matrix_candidate) {
+        // 8-wave matrix kernel: the largest window of 4, 2 or 1 timesteps whose halo tiles fit LDS.
+        // One analog frame for all T: a single stage of input (TT = 1), up to 16 LIF steps per launch.
+        int w2 = 1;
+        while (!all_shared && w2 < T && w2 < kMaxTT) w2 *= 2;
+        const bool fast_layer = Cout % 64 == 0 && v_dtype == SNNF_F32 && lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+        for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
+            if (plan_mm(g, w2, load_mode, vec_ok ? 8 : (vec4_ok ? 4 : 0), mp)) {
+                // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
+                // the activation prefetch): it runs windows of 2.
+                const bool fast_plan = fast_layer && mp.all_full && mp.run >= 4;
+                if (w2 == 4 && !fast_plan) continue;
+                mm_kernel = planned = true;
+                window = w2;
+            }
+        }
+        if (mm_kernel && all_shared) window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
+        if (mm_kernel) {
+            pl.TH = mp.TH; pl.TW = mp.TW; pl.tiles_x = mp.tiles_x; pl.tiles_y = mp.tiles_y; pl.NR = mp.NR; pl.WT = mp.WT;
+            pl.wm_log2 = mp.wm_log2; pl.wn_log2 = mp.wn_log2; pl.oc_tiles = mp.oc_tiles; pl.lds_bytes = mp.lds_bytes;
+        }
+    }
+    // Everything else: the time-outer kernels for a shared frame or a low intensity, the 4-wave T-in-M kernel otherwise.
+    bool time_outer = !mm_kernel && (all_shared || flops / bytes < 200.0);
     // Pointwise kernel: where the weight fragments live (registers only in the fast variant) and the LDS that takes.
     auto pw_config = [&](bool allow_regs, ConvGeom& gg) -> size_t {
         const size_t xb = static_cast<size_t>(64) * gg.pitch;
@@ -336,28 +361,6 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         planned = plan(g, 1, 0, load_mode, vec_ok, pl);
         window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
         if (!planned) time_outer = false;
-    }
-    bool mm_kernel = false;
-    MmPlan mp = {};
-    if (!time_outer && !all_shared && pg.CK >= 16 && Cin % 8 == 0) {
-        // 8-wave matrix kernel: the largest window of 4, 2 or 1 timesteps whose halo tiles fit LDS.
-        int w2 = 1;
-        while (w2 < T && w2 < kMaxTT) w2 *= 2;
-        const bool fast_layer = Cout % 64 == 0 && v_dtype == SNNF_F32 && lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
-        for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
-            if (plan_mm(g, w2, load_mode, vec_ok ? 8 : (vec4_ok ? 4 : 0), mp)) {
-                // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
-                // the activation prefetch): it runs windows of 2.
-                const bool fast_plan = fast_layer && mp.all_full && mp.run >= 4;
-                if (w2 == 4 && !fast_plan) continue;
-                mm_kernel = planned = true;
-                window = w2;
-            }
-        }
-        if (mm_kernel) {
-            pl.TH = mp.TH; pl.TW = mp.TW; pl.tiles_x = mp.tiles_x; pl.tiles_y = mp.tiles_y; pl.NR = mp.NR; pl.WT = mp.WT;
-            pl.wm_log2 = mp.wm_log2; pl.wn_log2 = mp.wn_log2; pl.oc_tiles = mp.oc_tiles; pl.lds_bytes = mp.lds_bytes;
-        }
     }
     if (!time_outer && !mm_kernel) {
         // Timesteps per launch: as many (<= 4) as fit LDS side by side; a shared analog frame needs one tile for any window.
@@ -436,7 +439,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     } else if (mm_kernel) {
         const bool fast_ok = mp.all_full && mp.run >= 4 && Cout % 64 == 0 && v_dtype == SNNF_F32 &&
                              lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;   // = fast_plan above
-        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + window;
+        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + (all_shared ? 1 : window);
         nparts = 1;
     } else {
         parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = time_outer ? 0 : window;

@@ -16,7 +16,9 @@
 //   * SK: layers with few pixels and many channels (deep stages) do not fill the machine with 64 x 32 wave tiles, so
 //     WK waves share an output tile, each taking every WK-th pair of k-slots, and add their sums through LDS.
 // FAST: every tile is full, runs of 8 pixels are contiguous and 16-byte aligned, Cout % 64 == 0, fp32 membrane, the
-// common neuron (power-of-two tau, hard reset); the general variant masks pixels and rows and takes any neuron. Requires Cin > 8 (chunks of at least 16 channels: every pair of k-slots real).
+// common neuron (power-of-two tau, hard reset); the general variant masks pixels and rows and takes any neuron. Requires whole
+// channel groups (Cin % 8 == 0) or Cin < 8. With TT == 1 the single stage may be one analog frame shared by all g.T
+// timesteps: it is convolved once.
 #pragma once
 
 #include "snnf_conv_pw_kernel.h"
@@ -28,8 +30,8 @@ constexpr int kMmWaves = 8;
 constexpr int kMmStagePitch = 40;                          // floats per channel row of a wave's stage (32 pixels + padding)
 constexpr int kMmStageFloats = 16 * kMmStagePitch;         // 16 channel rows
 static_assert(kMmWaves * kMmStageFloats * sizeof(float) == kMmStageBytes, "host and kernel disagree on the stage size");
-// Spatial staging items per thread, chunk and timestep: 64 prefetch registers in every load mode.
-__host__ __device__ constexpr int mm_staging_slots(int load_mode) { return load_mode == LOAD_PAIR32 ? 2 : 1; }
+// Spatial staging items per thread and stage: 64 prefetch registers whatever the load mode and the timesteps per stage.
+__host__ __device__ constexpr int mm_staging_slots(int load_mode, int tt) { return (load_mode == LOAD_PAIR32 ? 8 : 4) / tt; }
 typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
 
 template <typename XT, int TT, int LM, bool FAST, bool SK>
@@ -40,7 +42,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
-    constexpr int SS = mm_staging_slots(LM);
+    constexpr int SS = mm_staging_slots(LM, TT);
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,6 +85,8 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         item_src[s] = (cg * 8 * g.H + r) * g.W + 2 * cp;
     }
 
+    const int last_channel = g.Cin < 8 ? g.Cin - 1 : 7;
+    const int taps = g.KH * g.KW;
     // ---- the stage in flight.
     uint32_t pre[SS][TT][8][RPE];
     uint32_t pre_zero0 = 0, pre_zero1 = 0;                   // bit s: first / second column of item s is padding or beyond Cin
@@ -118,7 +122,8 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                 if (item_cg[s] >= 0) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        const char* __restrict__ row = base + j * plane * ES;
+                        // Fewer than 8 input channels in all: the absent ones re-read the last real one (their weights are 0).
+                        const char* __restrict__ row = base + min(j, last_channel) * plane * ES;
                         if constexpr (LM == LOAD_PAIR32) {
                             pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(row + off0[s]);
                         } else if constexpr (LM == LOAD_2X16) {
@@ -261,7 +266,8 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             const int pair = q - sub * g.npairs;
             const unsigned char* __restrict__ bp = bp0 + sub * (groups * 16);
             const int s0 = 2 * pair, s1 = 2 * pair + 1;
-            const int tap0 = s0 >> g.groups_log2, tap1 = s1 >> g.groups_log2;
+            // With a single channel group an odd tap count leaves the last k-slot empty (zero weights): it re-reads the last tap.
+            const int tap0 = s0 >> g.groups_log2, tap1 = min(s1 >> g.groups_log2, taps - 1);
             const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
             const int off_even = ((kh0 * g.WT) + (tap0 - kh0 * g.KW)) * g.pitch + (s0 & (groups - 1)) * 16;
             const int off_odd = ((kh1 * g.WT) + (tap1 - kh1 * g.KW)) * g.pitch + (s1 & (groups - 1)) * 16;
@@ -476,13 +482,21 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                     float bvv, v[8];
                     group_row(gidx, row_ok, row_off, bvv);
                     load_membrane(row_ok, row_off, v);
+                    if constexpr (TT == 1) {
+                        // One stage of input: a single timestep, or one analog frame that feeds all g.T timesteps.
+                        float xin[8];
 #pragma unroll
-                    for (int t = 0; t < TT; ++t) {
-                        if (t < g.T) {
-                            float xin[8];
+                        for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[0][gidx >> 1][(gidx & 1) * 8 + rr];
+                        for (int t = 0; t < g.T; ++t) lif_step_group(t, row_ok, row_off, bvv, xin, v);
+                    } else {
 #pragma unroll
-                            for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[t][gidx >> 1][(gidx & 1) * 8 + rr];
-                            lif_step_group(t, row_ok, row_off, bvv, xin, v);
+                        for (int t = 0; t < TT; ++t) {
+                            if (t < g.T) {
+                                float xin[8];
+#pragma unroll
+                                for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[t][gidx >> 1][(gidx & 1) * 8 + rr];
+                                lif_step_group(t, row_ok, row_off, bvv, xin, v);
+                            }
                         }
                     }
                     store_membrane(row_ok, row_off, v);
@@ -530,7 +544,12 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                             float xin[8];
 #pragma unroll
                             for (int k = 0; k < 4; ++k) { xin[k] = lo[k]; xin[4 + k] = hi[k]; }
-                            lif_step_group(t, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
+                            if constexpr (TT == 1) {   // one stage of input feeds all g.T timesteps
+                                for (int ts = 0; ts < g.T; ++ts)
+                                    lif_step_group(ts, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
+                            } else {
+                                lif_step_group(t, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
+                            }
                         }
                     }
                 }
