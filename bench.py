@@ -39,6 +39,9 @@ def _parse():
     ap.add_argument("--layers", default=None, choices=["resnet18", "vgg11"],
                     help="instead of a workload: time every fused conv layer shape of the spiking ResNet-18 (T=4, B=16, "
                          "224x224) or VGG-11 (T=4, B=64, 32x32) configuration on its own, synthetic spike inputs")
+    ap.add_argument("--model", default=None, choices=["resnet18", "vgg11"],
+                    help="end-to-end forward of the spiking ResNet-18 (T=4, B=16, 224x224) or VGG-11 (T=4, B=64, 32x32) "
+                         "network through the fused operators, replayed as one HIP graph")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only copy 256 MiB device to device three times: the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -273,6 +276,44 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
             "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
 
 
+MODEL_CONFIGS = {"resnet18": dict(batch=16, size=224, T=4), "vgg11": dict(batch=64, size=32, T=4)}
+
+
+def _model_forward(name: str, dtype, steps: int, warmup: int):
+    """End-to-end forward of a whole spiking network (direct encoding: one N(0, 1) frame repeated over T) through the
+    fused temporal operators: eager launches and one HIP graph replay per forward; images*T/s = B*T / forward time."""
+    import torch
+    from triton_snn_fusion_amd import models as M
+    cfg = MODEL_CONFIGS[name]
+    g = torch.Generator(device="cpu")
+    g.manual_seed(0)
+    frame = torch.randn(cfg["batch"], 3, cfg["size"], cfg["size"], generator=g)
+    net = M.fuse_network(M.build_network(name, seed=0), cfg["T"], dtype, "cuda:0")
+    net.record = []
+    net(frame)
+    torch.cuda.synchronize()
+    fused_calls = sum(1 for e in net.record if e["kind"] in ("conv_lif", "tail"))
+    library_calls = sum(1 for e in net.record if e["kind"] in ("plain_conv", "pool", "add"))
+    net.record = None
+    x = net._prepare(frame)
+    ms_eager, wall = _time_gpu(lambda: net(x), max(5, steps // 2), max(2, warmup // 2))
+    out = {"workload": f"{name}_end_to_end", "T": cfg["T"], "batch": cfg["batch"], "input": [cfg["batch"], 3, cfg["size"], cfg["size"]],
+           "fused_operator_calls": fused_calls, "pytorch_operator_calls": library_calls,
+           "eager_launch_ms_per_forward": round(ms_eager, 4), "host_ms_per_forward": round(wall, 4)}
+    try:
+        replay, _, _ = net.capture(frame)
+        ms_graph, _ = _time_gpu(replay, steps, warmup)
+        out["graph_ms_per_forward"] = round(ms_graph, 4)
+    except Exception as exc:  # pragma: no cover - reported, the eager number stands
+        ms_graph = None
+        out["graph_error"] = str(exc)[:200]
+    best = ms_graph if ms_graph is not None else ms_eager
+    out["ms_per_forward"] = round(best, 4)
+    out["images_T_per_s"] = round(cfg["batch"] * cfg["T"] / (best * 1e-3), 1)
+    out["images_per_s"] = round(cfg["batch"] / (best * 1e-3), 1)
+    return out
+
+
 def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
     """Eager fp32 PyTorch-CPU path (the oracle's restatement of the reference's eager ops) on a bounded sample."""
     import torch
@@ -355,6 +396,14 @@ def main() -> int:
         print(json.dumps(sweep))
         return 0 if stats["fallback"] == 0 else 1
 
+    if args.model is not None:
+        res = _model_forward(args.model, dtype, args.steps, args.warmup)
+        res.update({"metric": METRIC, "dtype": args.dtype, "data": "synthetic (seed 0, N(0,1) frame, Kaiming-normal weights, random eval-mode BN folded)"})
+        stats = ops.get_fused_op_call_stats()
+        res["native_calls"], res["fallback_calls"] = stats["triton"], stats["fallback"]
+        print(json.dumps(res))
+        return 0 if stats["fallback"] == 0 else 1
+
     wl = getattr(W, args.workload)()
     prep = Prepared(wl, dtype, device)
     prep.step()
@@ -434,6 +483,11 @@ def main() -> int:
             except Exception as exc:
                 entry["graph_error"] = str(exc)[:200]
             extra[name] = entry
+        for name in MODEL_CONFIGS:
+            try:
+                extra[f"{name}_end_to_end"] = _model_forward(name, dtype, max(10, args.steps // 2), max(3, args.warmup // 2))
+            except Exception as exc:  # the headline workload stands on its own
+                extra[f"{name}_end_to_end"] = {"error": str(exc)[:300]}
         result["extra"] = extra
 
     stats = ops.get_fused_op_call_stats()

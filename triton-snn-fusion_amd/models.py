@@ -1,0 +1,415 @@
+"""Spiking VGG-11-style and ResNet-18-style networks, as single-step eager modules and as fused temporal executors.
+
+Counterpart of the reference's model harness (benchmarks/validate_chronos_baselines.py:234-244 `SingleStepModeLoopWrapper`,
+:286-293 the (v_th 1, v_reset 0, tau 2) neuron, :304-309 state reset, :748-790 the VGG / ResNet constructors; the neuron
+contract `CustomStatefulIFNode` as used in benchmarks/benchmark_tensorrt_runtime.py:42-79). The reference builds these
+networks from spikingjelly's model zoo and lets its FX compiler group the T unrolled single-step iterations into
+temporal operators; here the two networks are defined directly and each has
+
+  * an eager form (`SpikingVGG11`, `SpikingResNet18`): one timestep per call, Conv2d -> BatchNorm2d -> neuron, state kept
+    in the neuron modules, driven by `SingleStepModeLoopWrapper` (same analog frame every step, readout = sum / T);
+  * a fused form (`FusedSpikingVGG11`, `FusedSpikingResNet18`): layer-major execution of the same network through
+    `torch.ops.snn_custom.fused_temporal_*` (BatchNorm folded into the convolution, all T steps of a layer in one
+    call, the last neuron + global average pool + classifier in `fused_temporal_lif_avgpool_linear`). This is the
+    operator sequence the reference's temporal rewrite produces for such a graph.
+
+What stays on stock PyTorch in the fused form is what the reference leaves as ordinary graph nodes too: the pooling
+between stages, the LIF-free 1x1 downsample shortcuts and the last convolution whose neuron belongs to the tail.
+"""
+from __future__ import annotations
+
+import copy
+import math
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .workloads import BN_EPS, LIF_DEFAULT, fold_bn_into_conv_params
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Neuron and wrappers
+# ---------------------------------------------------------------------------------------------------------------
+class CustomStatefulIFNode(nn.Module):
+    """Single-step LIF neuron that keeps its membrane in `self.v` between calls (forward only).
+
+    forward(x) = `torch.ops.snn_custom.lif_forward_state(x, self.v, v_threshold, v_reset, tau, detach_reset)`; a 0-dim
+    (or otherwise mismatching) `self.v` means "start from zeros" (reference runtime/snn_custom_ops.py:378-381)."""
+
+    def __init__(self, v_threshold: float = 1.0, v_reset: float = 0.0, tau: float = 2.0, detach_reset: bool = False,
+                 surrogate_function: Optional[Callable] = None, step_mode: str = "s"):
+        super().__init__()
+        self.v_threshold = float(v_threshold)
+        self.v_reset = float(v_reset)
+        self.tau = float(tau)
+        self.detach_reset = bool(detach_reset)
+        self.surrogate_function = surrogate_function     # forward-only: kept for interface compatibility
+        self.step_mode = step_mode
+        self.v: torch.Tensor = torch.tensor(0.0)
+
+    def reset(self) -> None:
+        self.v = torch.tensor(0.0)
+
+    def reset_state_if_needed(self, x: torch.Tensor) -> None:
+        v = self.v
+        if not isinstance(v, torch.Tensor) or v.shape != x.shape or v.dtype != x.dtype or v.device != x.device:
+            self.v = torch.zeros((), dtype=x.dtype, device=x.device)
+
+    @property
+    def lif_params(self) -> Tuple[float, float, float]:
+        return (self.v_threshold, self.v_reset, self.tau)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        from .runtime import snn_custom_ops  # noqa: F401  (registers torch.ops.snn_custom)
+        self.reset_state_if_needed(x)
+        spike, self.v = torch.ops.snn_custom.lif_forward_state(x, self.v, self.v_threshold, self.v_reset, self.tau,
+                                                               self.detach_reset)
+        return spike
+
+
+def reset_custom_stateful_lif_modules(model: nn.Module) -> None:
+    for m in model.modules():
+        if isinstance(m, CustomStatefulIFNode):
+            m.reset()
+
+
+reset_lif_modules = reset_custom_stateful_lif_modules
+
+
+class SingleStepModeLoopWrapper(nn.Module):
+    """Feeds the same frame to a single-step network T times and averages its outputs."""
+
+    def __init__(self, layer: nn.Module, T: int):
+        super().__init__()
+        self.layer = layer
+        self.T = int(T)
+
+    def forward(self, x):
+        out_spikes_counter = 0
+        for _ in range(self.T):
+            out_spikes_counter = out_spikes_counter + self.layer(x)
+        return out_spikes_counter / self.T
+
+
+def _neuron() -> CustomStatefulIFNode:
+    v_th, v_reset, tau = LIF_DEFAULT
+    return CustomStatefulIFNode(v_threshold=v_th, v_reset=v_reset, tau=tau)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Eager single-step networks
+# ---------------------------------------------------------------------------------------------------------------
+class ConvBNNeuron(nn.Module):
+    """Conv2d (no bias) -> BatchNorm2d -> neuron; `sn` is None for a LIF-free convolution (shortcut, pre-tail)."""
+
+    def __init__(self, cin: int, cout: int, kernel: int, stride: int, padding: int, neuron: bool = True):
+        super().__init__()
+        self.conv = nn.Conv2d(cin, cout, kernel, stride, padding, bias=False)
+        self.bn = nn.BatchNorm2d(cout, eps=BN_EPS)
+        self.sn = _neuron() if neuron else None
+
+    def forward(self, x):
+        y = self.bn(self.conv(x))
+        return self.sn(y) if self.sn is not None else y
+
+
+VGG11_STAGES = ((64,), (128,), (256, 256), (512, 512), (512, 512))
+
+
+class SpikingVGG11(nn.Module):
+    """Conv3x3+BN+LIF stages 64 | 128 | 256-256 | 512-512 | 512-512 with a 2x2 average pool between stages; the last
+    convolution's neuron opens the tail LIF -> global average pool -> Linear. `width` scales every channel count."""
+
+    def __init__(self, num_classes: int = 10, in_channels: int = 3, width: int = 64):
+        super().__init__()
+        layers: List[nn.Module] = []
+        cin = in_channels
+        convs = [(max(1, c * width // 64), si) for si, stage in enumerate(VGG11_STAGES) for c in stage]
+        for i, (cout, si) in enumerate(convs):
+            if i > 0 and si != convs[i - 1][1]:
+                layers.append(nn.AvgPool2d(2))
+            layers.append(ConvBNNeuron(cin, cout, 3, 1, 1, neuron=i + 1 < len(convs)))
+            cin = cout
+        self.features = nn.Sequential(*layers)
+        self.tail_sn = _neuron()
+        self.avgpool = nn.AdaptiveAvgPool2d((1, 1))
+        self.fc = nn.Linear(cin, num_classes)
+
+    def forward(self, x):
+        y = self.tail_sn(self.features(x))
+        return self.fc(torch.flatten(self.avgpool(y), 1))
+
+
+class SpikingBasicBlock(nn.Module):
+    """conv3x3-BN-LIF, conv3x3-BN, + identity (1x1/stride conv + BN when the shape changes), LIF."""
+
+    def __init__(self, cin: int, cout: int, stride: int):
+        super().__init__()
+        self.conv1 = ConvBNNeuron(cin, cout, 3, stride, 1)
+        self.conv2 = ConvBNNeuron(cout, cout, 3, 1, 1, neuron=False)
+        self.downsample = ConvBNNeuron(cin, cout, 1, stride, 0, neuron=False) if (stride != 1 or cin != cout) else None
+        self.sn2: Optional[CustomStatefulIFNode] = _neuron()
+
+    def pre_activation(self, x):
+        identity = x if self.downsample is None else self.downsample(x)
+        return self.conv2(self.conv1(x)) + identity
+
+    def forward(self, x):
+        y = self.pre_activation(x)
+        return self.sn2(y) if self.sn2 is not None else y
+
+
+class SpikingResNet18(nn.Module):
+    """Stem 7x7/2 + BN + LIF + 3x3/2 max pool, four stages of two BasicBlocks (64/128/256/512, stride 2 from the
+    second stage on, 1x1 downsample shortcuts), tail LIF -> global average pool -> Linear. The last block's output
+    neuron is the tail's neuron."""
+
+    def __init__(self, num_classes: int = 1000, in_channels: int = 3, width: int = 64, blocks: Sequence[int] = (2, 2, 2, 2)):
+        super().__init__()
+        self.stem = ConvBNNeuron(in_channels, width, 7, 2, 3)
+        self.maxpool = nn.MaxPool2d(3, 2, 1)
+        layers: List[nn.Module] = []
+        cin = width
+        for si, n in enumerate(blocks):
+            cout = width << si
+            for bi in range(n):
+                layers.append(SpikingBasicBlock(cin, cout, 2 if (si > 0 and bi == 0) else 1))
+                cin = cout
+        self.blocks = nn.Sequential(*layers)
+        self.tail_sn = self.blocks[-1].sn2
+        self.blocks[-1].sn2 = None                  # applied as the tail's neuron
+        self.avgpool = nn.AdaptiveAvgPool2d((1, 1))
+        self.fc = nn.Linear(cin, num_classes)
+
+    def forward(self, x):
+        y = self.tail_sn(self.blocks(self.maxpool(self.stem(x))))
+        return self.fc(torch.flatten(self.avgpool(y), 1))
+
+
+def init_synthetic_(model: nn.Module, seed: int = 0, gain: float = 1.0) -> nn.Module:
+    """Kaiming-normal convolution and classifier weights (scaled by `gain`), classifier bias N(0, 0.01^2), BatchNorm
+    gamma U(0.8, 1.2), beta N(0, 0.1^2), running mean N(0, 0.1^2), running variance U(0.5, 1.5); CPU generator `seed`."""
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, (nn.Conv2d, nn.Linear)):
+                fan_in = m.weight[0].numel()
+                m.weight.copy_(torch.randn(m.weight.shape, generator=g) * math.sqrt(2.0 / fan_in) * gain)
+                if m.bias is not None:
+                    m.bias.copy_(torch.randn(m.bias.shape, generator=g) * 0.01)
+            elif isinstance(m, nn.BatchNorm2d):
+                c = m.num_features
+                m.weight.copy_(torch.rand(c, generator=g) * 0.4 + 0.8)
+                m.bias.copy_(torch.randn(c, generator=g) * 0.1)
+                m.running_mean.copy_(torch.randn(c, generator=g) * 0.1)
+                m.running_var.copy_(torch.rand(c, generator=g) + 0.5)
+    return model.eval()
+
+
+def fold_batchnorm(model: nn.Module, round_to: Optional[torch.dtype] = None) -> nn.Module:
+    """Copy of `model` with every eval-mode BatchNorm folded into its convolution (which gains a bias) and, when
+    `round_to` is given, all convolution / classifier parameters rounded to that dtype (values kept in fp32). The eager
+    form of the copy computes with exactly the operands the fused form feeds to the kernels."""
+    model = copy.deepcopy(model).eval()
+
+    def rounded(t: torch.Tensor) -> torch.Tensor:
+        return t if round_to is None else t.to(round_to).to(torch.float32)
+
+    with torch.no_grad():
+        for m in list(model.modules()):
+            if isinstance(m, ConvBNNeuron) and isinstance(m.bn, nn.BatchNorm2d):
+                w, b = fold_bn_into_conv_params(m.conv.weight.float(), m.conv.bias, m.bn.running_mean.float(),
+                                                m.bn.running_var.float(), m.bn.weight.float(), m.bn.bias.float(), m.bn.eps)
+                conv = nn.Conv2d(m.conv.in_channels, m.conv.out_channels, m.conv.kernel_size, m.conv.stride, m.conv.padding, bias=True)
+                conv.weight.copy_(rounded(w))
+                conv.bias.copy_(rounded(b))
+                m.conv, m.bn = conv.to(w.device), nn.Identity()
+            elif isinstance(m, nn.Linear):
+                m.weight.copy_(rounded(m.weight.float()))
+                if m.bias is not None:
+                    m.bias.copy_(rounded(m.bias.float()))
+    return model
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Fused temporal executors
+# ---------------------------------------------------------------------------------------------------------------
+class _FusedLayer:
+    """Folded parameters of one ConvBNNeuron in the activation dtype on the target device."""
+
+    def __init__(self, m: ConvBNNeuron, dtype: torch.dtype, device: torch.device):
+        with torch.no_grad():
+            if isinstance(m.bn, nn.BatchNorm2d):
+                w, b = fold_bn_into_conv_params(m.conv.weight.float(), m.conv.bias, m.bn.running_mean.float(),
+                                                m.bn.running_var.float(), m.bn.weight.float(), m.bn.bias.float(), m.bn.eps)
+            else:
+                w = m.conv.weight.float()
+                b = m.conv.bias.float() if m.conv.bias is not None else torch.zeros(w.shape[0])
+            self.weight = w.to(device=device, dtype=dtype).contiguous()
+            self.bias = b.to(device=device, dtype=dtype).contiguous()
+        self.stride = [int(s) for s in m.conv.stride]
+        self.padding = [int(p) for p in m.conv.padding]
+        self.lif = m.sn.lif_params if m.sn is not None else None
+
+    @property
+    def geometry(self):
+        return (self.stride, self.padding, [1, 1], 1)
+
+
+class _FusedNetwork(nn.Module):
+    """Shared plumbing: parameter folding, operator calls, optional recording of every operator call (inputs and
+    outputs, for layer-by-layer verification), and whole-forward HIP graph capture."""
+
+    def __init__(self, T: int, dtype: torch.dtype, device, v_dtype: torch.dtype = torch.float32):
+        super().__init__()
+        from .runtime import snn_custom_ops
+        if torch.device(device).type == "cuda":
+            # Native kernels only: an operator call they cannot serve raises instead of running the eager ops.
+            snn_custom_ops.configure_fused_op("hip", strict_triton=True)
+        self.T = int(T)
+        self.dtype = dtype
+        self.device_ = torch.device(device)
+        self.zero_v = torch.zeros((), dtype=v_dtype, device=self.device_)
+        self.record: Optional[List[Dict]] = None
+        self._graph = None
+
+    # -- operator calls ------------------------------------------------------------------------------------------
+    def _log(self, **entry):
+        if self.record is not None:
+            self.record.append(entry)
+
+    def conv_lif(self, name: str, xs: List[torch.Tensor], layer: _FusedLayer, residuals: Optional[List[torch.Tensor]] = None):
+        S = torch.ops.snn_custom
+        if residuals is None:
+            spikes, v = S.fused_temporal_conv_lif_state(xs, layer.weight, layer.bias, self.zero_v, *layer.geometry, *layer.lif, False)
+        else:
+            spikes, v = S.fused_temporal_conv_add_lif_state(xs, residuals, layer.weight, layer.bias, self.zero_v,
+                                                            *layer.geometry, *layer.lif, False)
+        self._log(kind="conv_lif", name=name, xs=xs, residuals=residuals, layer=layer, spikes=spikes, v=v)
+        return spikes
+
+    def plain_conv(self, name: str, x_seq: torch.Tensor, layer: _FusedLayer) -> torch.Tensor:
+        """LIF-free convolution of all T*N frames at once (stock PyTorch, bias = folded BatchNorm shift)."""
+        y = F.conv2d(x_seq.flatten(0, 1), layer.weight, layer.bias, layer.stride, layer.padding)
+        y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
+        self._log(kind="plain_conv", name=name, x=x_seq, layer=layer, y=y)
+        return y
+
+    def pooled(self, name: str, x_seq: torch.Tensor, pool: nn.Module) -> torch.Tensor:
+        y = pool(x_seq.flatten(0, 1))
+        y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
+        self._log(kind="pool", name=name, x=x_seq, pool=pool, y=y)
+        return y
+
+    def tail(self, x_seq: torch.Tensor, lif, fc_weight, fc_bias) -> torch.Tensor:
+        out_sum, v = torch.ops.snn_custom.fused_temporal_lif_avgpool_linear(x_seq, self.zero_v, fc_weight, fc_bias, *lif, False)
+        self._log(kind="tail", name="tail", x=x_seq, lif=lif, fc_weight=fc_weight, fc_bias=fc_bias, out_sum=out_sum, v=v)
+        return out_sum / self.T
+
+    # -- driver --------------------------------------------------------------------------------------------------
+    def _prepare(self, x: torch.Tensor) -> torch.Tensor:
+        return x.to(device=self.device_, dtype=self.dtype).contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        with torch.no_grad():
+            return self.run(self._prepare(x))
+
+    def run(self, x: torch.Tensor) -> torch.Tensor:     # pragma: no cover - implemented by the subclasses
+        raise NotImplementedError
+
+    def capture(self, example: torch.Tensor, warmup: int = 3):
+        """Captures the whole forward into one HIP graph; returns (replay, static_input, static_output).
+
+        The warm-up forwards run on a side stream first (weight packing, library handles and the caching allocator
+        settle outside the capture). Kernels are enqueued by every operator on the current stream without allocating
+        or synchronising, so the capture holds kernel nodes only."""
+        static_in = self._prepare(example).clone()
+        side = torch.cuda.Stream(device=self.device_)
+        side.wait_stream(torch.cuda.current_stream(self.device_))
+        with torch.cuda.stream(side):
+            for _ in range(max(1, warmup)):
+                self.forward(static_in)
+        torch.cuda.current_stream(self.device_).wait_stream(side)
+        torch.cuda.synchronize(self.device_)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = self.forward(static_in)
+        self._graph = graph
+        return graph.replay, static_in, static_out
+
+
+class FusedSpikingVGG11(_FusedNetwork):
+    def __init__(self, model: SpikingVGG11, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0"):
+        super().__init__(T, dtype, device)
+        self.steps: List[Tuple[str, object]] = []
+        for i, m in enumerate(model.features):
+            if isinstance(m, ConvBNNeuron):
+                self.steps.append(("conv" if m.sn is not None else "plain", _FusedLayer(m, dtype, self.device_)))
+            else:
+                self.steps.append(("pool", copy.deepcopy(m)))
+        self.tail_lif = model.tail_sn.lif_params
+        self.fc_weight = model.fc.weight.detach().to(device=self.device_, dtype=dtype).contiguous()
+        self.fc_bias = model.fc.bias.detach().to(device=self.device_, dtype=dtype).contiguous()
+
+    def run(self, x):
+        seq: Optional[torch.Tensor] = None          # [T, N, C, H, W] spikes; None while the input is the analog frame
+        for i, (kind, item) in enumerate(self.steps):
+            if kind == "conv":
+                xs = [x] * self.T if seq is None else list(seq.unbind(0))
+                seq = self.conv_lif(f"features.{i}", xs, item)
+            elif kind == "pool":
+                seq = self.pooled(f"features.{i}", seq, item)
+            else:
+                seq = self.plain_conv(f"features.{i}", seq, item)
+        return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
+
+
+class FusedSpikingResNet18(_FusedNetwork):
+    def __init__(self, model: SpikingResNet18, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0"):
+        super().__init__(T, dtype, device)
+        self.stem = _FusedLayer(model.stem, dtype, self.device_)
+        self.maxpool = copy.deepcopy(model.maxpool)
+        self.block_layers = []
+        for b in model.blocks:
+            conv2 = _FusedLayer(b.conv2, dtype, self.device_)
+            conv2.lif = b.sn2.lif_params if b.sn2 is not None else None
+            down = _FusedLayer(b.downsample, dtype, self.device_) if b.downsample is not None else None
+            self.block_layers.append((_FusedLayer(b.conv1, dtype, self.device_), conv2, down))
+        self.tail_lif = model.tail_sn.lif_params
+        self.fc_weight = model.fc.weight.detach().to(device=self.device_, dtype=dtype).contiguous()
+        self.fc_bias = model.fc.bias.detach().to(device=self.device_, dtype=dtype).contiguous()
+
+    def run(self, x):
+        seq = self.conv_lif("stem", [x] * self.T, self.stem)
+        seq = self.pooled("maxpool", seq, self.maxpool)
+        for i, (conv1, conv2, down) in enumerate(self.block_layers):
+            identity = seq if down is None else self.plain_conv(f"blocks.{i}.downsample", seq, down)
+            hidden = self.conv_lif(f"blocks.{i}.conv1", list(seq.unbind(0)), conv1)
+            if conv2.lif is not None:
+                seq = self.conv_lif(f"blocks.{i}.conv2", list(hidden.unbind(0)), conv2, residuals=list(identity.unbind(0)))
+            else:   # last block: its neuron is the tail's
+                seq = self.plain_conv(f"blocks.{i}.conv2", hidden, conv2) + identity
+                self._log(kind="add", name=f"blocks.{i}.add", y=seq)
+        return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
+
+
+def build_network(name: str, width: int = 64, num_classes: Optional[int] = None, seed: int = 0, gain: float = 1.0) -> nn.Module:
+    """`vgg11` (10 classes) or `resnet18` (1000 classes) with the synthetic initialisation."""
+    if name == "vgg11":
+        model = SpikingVGG11(num_classes=10 if num_classes is None else num_classes, width=width)
+    elif name == "resnet18":
+        model = SpikingResNet18(num_classes=1000 if num_classes is None else num_classes, width=width)
+    else:
+        raise ValueError(f"unsupported model: {name}")
+    return init_synthetic_(model, seed=seed, gain=gain)
+
+
+def fuse_network(model: nn.Module, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0") -> _FusedNetwork:
+    if isinstance(model, SpikingVGG11):
+        return FusedSpikingVGG11(model, T, dtype, device)
+    if isinstance(model, SpikingResNet18):
+        return FusedSpikingResNet18(model, T, dtype, device)
+    raise TypeError(f"no fused executor for {type(model).__name__}")
