@@ -293,7 +293,8 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
     net(frame)
     torch.cuda.synchronize()
     fused_calls = sum(1 for e in net.record if e["kind"] in ("conv_lif", "tail"))
-    library_calls = sum(1 for e in net.record if e["kind"] in ("plain_conv", "pool", "add"))
+    library_calls = sum(1 for e in net.record if e["kind"] == "pool" or (e["kind"] == "plain_conv" and not e["native"]))
+    fused_calls += sum(1 for e in net.record if e["kind"] == "plain_conv" and e["native"])
     net.record = None
     x = net._prepare(frame)
     ms_eager, wall = _time_gpu(lambda: net(x), max(5, steps // 2), max(2, warmup // 2))

@@ -141,6 +141,26 @@ int snnf_conv_lif(const void* const* xs, const void* const* residuals, int T,
                   void* spikes, int64_t spike_step_stride, void* v_out,
                   float v_threshold, float v_reset, float tau, void* stream);
 
+/* Convolution + bias (+ residual) WITHOUT a neuron: out[t] = conv2d(xs[t]) + b (+ residuals[t]) in the activation dtype,
+ * for T independent frames, with the same packed weight and matrix kernel as snnf_conv_lif. No fused operator of the
+ * reference corresponds to it: its rewrite leaves LIF-free Conv+BN nodes (the 1x1 downsample shortcuts of a ResNet,
+ * whose output is the `residuals` operand of fused_temporal_conv_add_lif_state, runtime/snn_custom_ops.py:491-518) to
+ * the framework's convolution; this entry point keeps such a layer on the NCHW tensors the fused operators exchange.
+ * Supported: Cin % 8 == 0 or Cin < 8, anything but a plain 1x1 stride-1 convolution; SNNF_ERR_UNSUPPORTED otherwise.
+ *   out : [T, N, Cout, Ho, Wo] x_dtype (frame stride `out_step_stride` elements) */
+int snnf_conv_bias(const void* const* xs, const void* const* residuals /* nullable */, int T,
+                   int N, int Cin, int H, int W, int x_dtype,
+                   const void* packed_weight, int Cout, int KH, int KW,
+                   int stride_h, int stride_w, int pad_h, int pad_w,
+                   void* out, int64_t out_step_stride, void* stream);
+
+/* Describes what the most recent snnf_conv_lif / snnf_conv_bias call on this thread selected: kernel family, timesteps per launch, tile
+ * and wave decomposition, LDS bytes, grid ("key=value" pairs, empty before the first call). Plays the role of the
+ * reference's get_autotune_best_config (kernels/benchmark_conv_lif_temporal_general.py:1332-1369), whose result the
+ * operator layer publishes as kernel_temporal_config (runtime/snn_custom_ops.py:341-353): selection here is a
+ * deterministic planner, and this is how a host reads its decision. The pointer stays valid for the thread's lifetime. */
+const char* snnf_conv_last_plan(void);
+
 #ifdef __cplusplus
 }
 #endif

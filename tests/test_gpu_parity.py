@@ -327,6 +327,11 @@ DENSE_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, re
     (512, 128, 4, 4, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 4, False, False),    # deep and tiny: K split eight ways
     (64, 64, 16, 16, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 6, 2, True, True),      # two launch windows (4 + 2)
     (64, 192, 8, 24, 1, 2, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False),    # strided 1x1 (downsample shortcut)
+    (128, 128, 2, 2, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 16, True, True),     # 2x2 planes: 8 images per tile
+    (64, 64, 4, 4, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 6, False, True),       # 4x4 planes, batch not a multiple of the images per tile
+    (256, 128, 4, 4, 3, 1, 1, BF16, F32, (1.0, -1.0, 2.0), 3, 5, True, False),    # several images per tile, K split, masked variant, soft reset
+    (64, 64, 8, 8, 3, 2, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 8, False, False),      # stride 2 onto 4x4 planes, several images per tile
+    (32, 64, 6, 6, 5, 1, 2, F16, F32, (1.0, 0.0, 2.0), 2, 7, True, True),         # 6x6 planes (no aligned runs), 5x5 kernel, f16
 ]
 
 
@@ -396,6 +401,62 @@ def test_conv_shared_analog_frame_variants(hip_ops, Cin, Cout, H, W, k, stride, 
     assert tuple(sp.shape) == (T, N, Cout, Ho, Wo)
     check(sp, v, ref, v_threshold=lif[0], what=f"shared frame {Cin}->{Cout} k{k} s{stride} {H}x{W} T={T}")
     _no_fallback(hip_ops, 1)
+
+
+CONV_BIAS_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, T, N, residual, analog input
+    (64, 128, 16, 16, 1, 2, 0, BF16, 4, 2, False, False),     # ResNet downsample shortcut
+    (64, 64, 12, 12, 3, 1, 1, BF16, 4, 2, True, False),       # conv + bias + residual (pre-tail sum)
+    (128, 96, 7, 7, 3, 1, 1, BF16, 3, 3, True, False),        # odd plane, Cout % 64 != 0, 3 frames
+    (3, 32, 20, 20, 5, 1, 2, BF16, 2, 2, False, True),        # few input channels, analog frames
+    (32, 64, 16, 16, 3, 2, 1, F16, 4, 2, False, True),        # fp16
+    (64, 64, 8, 8, 3, 1, 1, F32, 1, 4, False, False),         # fp32 in and out (bf16 matrix operands)
+    (256, 64, 6, 6, 3, 1, 1, BF16, 4, 2, True, False),        # deep: K split across waves
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,stride,pad,dtype,T,N,residual,analog", CONV_BIAS_CASES)
+def test_conv_bias_without_neuron(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, T, N, residual, analog):
+    """snnf_conv_bias: the matrix kernel's neuron-free output against F.conv2d in fp32 on the same (rounded) operands;
+    the only rounding on the kernel's side is the store in the activation dtype."""
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan, run_hip_temporal_conv_bias
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(1400 + Cin + Cout + H + k, T, N, Cin, Cout, H, W, k, dtype, analog=analog, p=0.3)
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    g = gen(1401 + Cin)
+    rs = [q(torch.randn(N, Cout, Ho, Wo, generator=g), dtype) for _ in range(T)] if residual else None
+    want = torch.stack([torch.nn.functional.conv2d(x, w_ref, b_ref, stride, pad) for x in xs])
+    if residual:
+        want = want + torch.stack(rs)
+    got = run_hip_temporal_conv_bias([dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype), [stride, stride], [pad, pad],
+                                     None if rs is None else [dev(r, dtype) for r in rs])
+    assert got.dtype == dtype and tuple(got.shape) == (T, N, Cout, Ho, Wo)
+    assert last_conv_plan()["kernel"] == "matrix"
+    rtol = {F32: 1e-4, BF16: 2 ** -8, F16: 2 ** -10}[dtype]
+    assert torch.allclose(got.float().cpu(), want, rtol=rtol, atol=1e-4 if dtype == F32 else 1e-3), (got.float().cpu() - want).abs().max()
+
+
+def test_conv_bias_rejects_what_the_matrix_kernel_does_not_take(hip_ops):
+    x = [torch.zeros(2, 64, 8, 8, device=DEV, dtype=BF16)]
+    w = torch.zeros(64, 64, 1, 1, device=DEV, dtype=BF16)
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import run_hip_temporal_conv_bias
+    with pytest.raises(RuntimeError, match="unsupported_shape"):
+        run_hip_temporal_conv_bias(x, w, None, [1, 1], [0, 0])      # plain 1x1 / stride 1
+    w12 = torch.zeros(64, 12, 3, 3, device=DEV, dtype=BF16)
+    with pytest.raises(RuntimeError, match="unsupported_shape"):
+        run_hip_temporal_conv_bias([torch.zeros(2, 12, 8, 8, device=DEV, dtype=BF16)], w12, None, [1, 1], [1, 1])   # Cin % 8 != 0
+
+
+def test_conv_plan_is_reported(hip_ops):
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    xs = [torch.zeros(2, 64, 16, 16, device=DEV, dtype=BF16) for _ in range(4)]
+    w, b = torch.zeros(64, 64, 3, 3, device=DEV, dtype=BF16), torch.zeros(64, device=DEV, dtype=BF16)
+    S.fused_temporal_conv_lif_state(xs, w, b, zero_v(), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+    plan = last_conv_plan()
+    assert plan["kernel"] == "matrix" and plan["variant"] == 24 and plan["window"] == 4 and plan["launches"] == 1
+    w1 = torch.zeros(128, 64, 1, 1, device=DEV, dtype=BF16)
+    S.fused_temporal_pointwise_conv_lif_state(xs, w1, torch.zeros(128, device=DEV, dtype=BF16), zero_v(), [1, 1], [0, 0], [1, 1], 1, *LIF, False)
+    assert last_conv_plan()["kernel"] == "pointwise"
+    configs = hip_ops.get_kernel_temporal_configs()
+    assert any("BTILE_T=4" in key for key in configs), configs
 
 
 def test_conv_and_linear_known_answers_exact(hip_ops):

@@ -31,6 +31,7 @@ SIGNATURES = {
     "snnf_abi_version": (_i, []),
     "snnf_status_string": (ctypes.c_char_p, [_i]),
     "snnf_last_error": (ctypes.c_char_p, []),
+    "snnf_conv_last_plan": (ctypes.c_char_p, []),
     "snnf_lif_scan": (_i, [_pp, _i, _i64, _i, _vp, _i, _vp, _i64, _vp, _f, _f, _f, _vp]),
     "snnf_dwconv3x3_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _i64, _vp,
                                 _f, _f, _f, _vp]),
@@ -42,6 +43,7 @@ SIGNATURES = {
     "snnf_conv_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "snnf_conv_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i64,
                            _vp, _f, _f, _f, _vp]),
+    "snnf_conv_bias": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
 }
 
 _LIB: Optional[ctypes.CDLL] = None

@@ -14,7 +14,7 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kEpiPitch = 68;       // floats per channel row of the epilogue stage (64 pixels + padding)
 constexpr size_t kToutStageBytes = 4 * 64 * 12 * sizeof(float);   // time-outer kernel: four waves x 64 pixels x (8 rows + padding)
 constexpr size_t kPwStageBytes = 4 * 8 * 68 * sizeof(float);      // pointwise kernel: four waves x 8 channel rows x (64 pixels + padding)
-constexpr size_t kMmStageBytes = 8 * 16 * 40 * sizeof(float);     // matrix kernel: eight waves x 16 channel rows x (32 pixels + padding)
+constexpr size_t kMmStageBytesPerWave = 16 * 40 * sizeof(float);  // matrix kernel, per wave: 16 channel rows x (32 pixels + padding)
 constexpr size_t kEpiBytes = 4 * 4 * 8 * kEpiPitch * sizeof(float);  // four waves x (up to 4 steps x 8 channel rows)
 
 // Channels per chunk staged in LDS; fixed by (Cin, taps, activation width) alone so that packing and the kernel agree.
@@ -105,6 +105,8 @@ struct ConvGeom {
     int vec8;                 // runs of 8 output pixels may be stored as one 16-byte-aligned vector
     int64_t spike_step_stride;
     int v_is_f32;             // membrane dtype in memory: fp32 (1) or the activation dtype (0)
+    int analog_out;         // matrix kernel: write conv + bias (+ residual) instead of spikes, no membrane
+    int TI, img_groups;      // matrix kernel: images per tile (> 1 only when a tile is a whole output plane), ceil(N / TI)
     int w_lds;                // time-outer kernels: weight fragments streamed from L2 (0), kept in LDS (1) or in registers (2)
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
     int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts
@@ -116,6 +118,7 @@ struct ConvGeom {
     int stage_chunks;         // matrix kernel: packed channel chunks held by one LDS stage (pitch = stage_chunks * CK * 2 + 16)
     FastDiv d_TW, d_Ho, d_H, d_WTP, d_stage_rows, d_tiles_x, d_oc_tiles;   // d_stage_rows: NR * (WT / 2)
     FastDiv d_tiles_img, d_KW, d_npairs;
+    FastDiv d_NR, d_tile_px;                                               // matrix kernel: halo rows per image, TH * TW
 };
 
 struct ConvLaunch {
@@ -140,5 +143,9 @@ struct ConvLaunch {
 int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode);
 int launch_conv_f16(const ConvLaunch& L, int tt, int load_mode);
+// Matrix kernel with 4-wave workgroups (fast variant, shared input frame: tt == 1): separate translation units.
+int launch_conv_mm_w4_f32(const ConvLaunch& L, int tt, int load_mode);
+int launch_conv_mm_w4_bf16(const ConvLaunch& L, int tt, int load_mode);
+int launch_conv_mm_w4_f16(const ConvLaunch& L, int tt, int load_mode);
 
 }  // namespace snnf

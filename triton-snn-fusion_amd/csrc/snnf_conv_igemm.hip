@@ -1,4 +1,6 @@
 // Host side of the implicit-GEMM conv+LIF operator: argument validation, tile planning and launch.
+#include <algorithm>
+#include <cstdio>
 #include "snnf_conv_common.h"
 
 #include <cstdlib>
@@ -105,21 +107,27 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
 struct MmPlan {
     int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full, stage_off, stage_chunks, pitch;
     size_t lds_bytes;
+    int nw;          // waves per workgroup: 8 (one workgroup per CU) or 4 (two)
+    double score;
+    int TI;          // images per tile: > 1 only for tiles that are whole output planes (small planes, deep stages)
 };
 
 // `vec`: widest aligned spike access the operands allow (8 or 4 elements, 0 = none). The WK waves that split K of one
 // tile cost an LDS reduction, so K is only split when the unsplit tiling leaves most of the machine idle.
-bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan& best_plan) {
+bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw, MmPlan& best_plan) {
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int groups = 1 << g0.groups_log2;
-    const int max_items = 512 * ((load_mode == LOAD_PAIR32 ? 8 : 4) / tt);
-    const int cus = compute_units();
+    const int max_items = nw * 64 * ((load_mode == LOAD_PAIR32 ? 8 : 4) / tt);
+    const int nw_log2 = nw == 8 ? 3 : 2;
+    const int cus = compute_units() * (8 / nw);                  // workgroup slots of the machine
+    const size_t lds_cap = kMaxLds * nw / 8;                      // per workgroup
+    const size_t stage_bytes = nw * kMmStageBytesPerWave;
     double best = -1.0;
-    for (int wk_log2 = 0; wk_log2 <= 3; ++wk_log2) {
+    for (int wk_log2 = 0; wk_log2 <= nw_log2; ++wk_log2) {
         if ((1 << wk_log2) > g0.npairs) break;
         if (wk_log2 > 0 && g0.nchunks * g0.npairs < 72) break;   // measured: splitting pays from K of about 1152 on
-        for (int wn_log2 = 0; wn_log2 + wk_log2 <= 3; ++wn_log2) {
-            const int wm_log2 = 3 - wn_log2 - wk_log2;
+        for (int wn_log2 = 0; wn_log2 + wk_log2 <= nw_log2; ++wn_log2) {
+            const int wm_log2 = nw_log2 - wn_log2 - wk_log2;
             const int PT = (1 << wm_log2) * 32;
             const int OT = (1 << wn_log2) * 64;
             const int oc_tiles = (g0.Cout + OT - 1) / OT;
@@ -132,31 +140,38 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan
                 const int NR = (th - 1) * g0.sh + g0.KH;
                 int WT = (tw - 1) * g0.sw + g0.KW + (pair_shift ? 1 : 0);
                 WT = (WT + 1) & ~1;
+                // A tile that is a whole output plane may take several images (stacked halo tiles): small planes then
+                // still fill the 32-pixel waves.
+                const int ti_max = (th == g0.Ho && tw == g0.Wo) ? std::max(1, std::min(g0.N, PT / (th * tw))) : 1;
+              for (int ti = 1; ti <= ti_max; ++ti) {
+                const int NRT = ti * NR;                           // stacked halo rows
+                const int img_groups = (g0.N + ti - 1) / ti;
                 // An LDS stage holds as many packed channel chunks as fit (fewer barriers and exposed load latencies per tile).
                 int sc = 1;
                 while (sc * 2 <= g0.nchunks && sc * 2 * g0.CK <= 256 &&
-                       static_cast<size_t>(tt) * NR * WT * (sc * 2 * g0.CK * 2 + 16) + kMmStageBytes <= kMaxLds &&
-                       sc * 2 * groups * NR * (WT / 2) <= max_items)
+                       static_cast<size_t>(tt) * NRT * WT * (sc * 2 * g0.CK * 2 + 16) + stage_bytes <= lds_cap &&
+                       sc * 2 * groups * NRT * (WT / 2) <= max_items)
                     sc *= 2;
                 const int pitch = sc * g0.CK * 2 + 16;
-                size_t tiles_bytes = static_cast<size_t>(tt) * NR * WT * pitch;
-                if (wk_log2 > 0 && tiles_bytes < 64 * 1024) tiles_bytes = 64 * 1024;    // the split-K partial sums of one timestep
-                const size_t bytes = tiles_bytes + kMmStageBytes;
-                if (bytes > kMaxLds) continue;
-                if (sc * groups * NR * (WT / 2) > max_items) continue;
+                size_t tiles_bytes = static_cast<size_t>(tt) * NRT * WT * pitch;
+                const size_t partial_bytes = static_cast<size_t>(nw) * 8 * 1024;        // the split-K partial sums of one timestep
+                if (wk_log2 > 0 && tiles_bytes < partial_bytes) tiles_bytes = partial_bytes;
+                const size_t bytes = tiles_bytes + stage_bytes;
+                if (bytes > lds_cap) continue;
+                if (sc * groups * NRT * (WT / 2) > max_items) continue;
                 const bool full_width = tw == g0.Wo;
                 int run = 0;
                 for (int cand : {8, 4}) {
                     if (cand > vec || run != 0) continue;
                     if (full_width ? ((th * g0.Wo) % cand == 0) : (tw % cand == 0 && g0.Wo % cand == 0)) run = cand;
                 }
-                // `all_full`: every tile is whole and made of whole runs.
-                const bool all_full = g0.Ho % th == 0 && g0.Wo % tw == 0 && run != 0 && (th * tw) % run == 0;
-                const double work = static_cast<double>(g0.N) * tiles_x * tiles_y * oc_tiles;
-                const double lane_eff = static_cast<double>(g0.Ho) * g0.Wo / (static_cast<double>(tiles_x) * tiles_y * PT);
+                // `all_full`: every tile is whole and made of whole runs (runs never straddle two images of a tile).
+                const bool all_full = g0.Ho % th == 0 && g0.Wo % tw == 0 && run != 0 && (th * tw) % run == 0 && g0.N % ti == 0;
+                const double work = static_cast<double>(img_groups) * tiles_x * tiles_y * oc_tiles;
+                const double lane_eff = static_cast<double>(g0.N) * g0.Ho * g0.Wo / (static_cast<double>(img_groups) * tiles_x * tiles_y * PT);
                 const double waves = work < cus ? 1.0 : static_cast<double>(static_cast<long long>((work + cus - 1) / cus));
                 const double fill = work / (waves * cus);
-                const double halo = static_cast<double>(NR) * WT / (static_cast<double>(th) * tw);
+                const double halo = static_cast<double>(NR) * WT / (static_cast<double>(th) * tw);   // per image
                 double score = lane_eff * oc_eff * fill / (1.0 + 0.1 * (halo - 1.0)) / (1.0 + 0.05 * (oc_tiles - 1));
                 score /= 1.0 + 0.08 * ((1 << wk_log2) - 1);
                 if (run == 0) score *= 0.4;        // element-wise 2-byte stores are very slow
@@ -165,19 +180,20 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, MmPlan
                 if (score > best) {
                     best = score;
                     best_plan = MmPlan{th, tw, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, wk_log2, oc_tiles, run, all_full ? 1 : 0,
-                                       static_cast<int>(tiles_bytes), sc, pitch, bytes};
+                                       static_cast<int>(tiles_bytes), sc, pitch, bytes, nw, score, ti};
                 }
+              }
             }
         }
     }
     return best > 0.0;
 }
 
-bool plan_mm(const ConvGeom& g, int tt, int load_mode, int vec, MmPlan& out) {
-    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
+bool plan_mm(const ConvGeom& g, int tt, int load_mode, int vec, int nw, MmPlan& out) {
+    using Key = std::tuple<int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int, int>;
     static std::mutex mu;
     static std::map<Key, std::pair<bool, MmPlan>> plans;
-    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, g.npairs, g.nchunks, tt, load_mode, vec);
+    const Key key(g.N, g.H, g.W, g.KH, g.KW, g.sh, g.sw, g.ph, g.pw, g.pitch, g.Cout, g.npairs, g.nchunks, tt, load_mode, vec, nw);
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = plans.find(key);
@@ -187,7 +203,7 @@ bool plan_mm(const ConvGeom& g, int tt, int load_mode, int vec, MmPlan& out) {
         }
     }
     MmPlan p = {};
-    const bool ok = plan_mm_uncached(g, tt, load_mode, vec, p);
+    const bool ok = plan_mm_uncached(g, tt, load_mode, vec, nw, p);
     std::lock_guard<std::mutex> lock(mu);
     plans[key] = std::make_pair(ok, p);
     out = p;
@@ -219,12 +235,24 @@ bool plan(const ConvGeom& g, int t_in, int tt, int load_mode, bool want_vec8, Pl
 }  // namespace
 }  // namespace snnf
 
-extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,
-                             int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
-                             int pad_h, int pad_w, const void* v_init, int v_dtype, void* spikes,
-                             int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
-                             void* stream) {
-    using namespace snnf;
+namespace snnf {
+char* conv_plan_buffer() {
+    static thread_local char buffer[256] = {0};
+    return buffer;
+}
+}  // namespace snnf
+
+extern "C" const char* snnf_conv_last_plan(void) { return snnf::conv_plan_buffer(); }
+
+namespace snnf {
+namespace {
+// Shared body of snnf_conv_lif and snnf_conv_bias. `analog_out`: no neuron - the convolution output (+ bias, + residual)
+// is written in the activation dtype where the spikes would go, and no membrane is read or written.
+int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,
+                  int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
+                  int pad_h, int pad_w, const void* v_init, int v_dtype, void* spikes,
+                  int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
+                  void* stream, bool analog_out) {
     if (xs == nullptr || packed_weight == nullptr || spikes == nullptr || v_out == nullptr)
         return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_conv_lif: xs, packed_weight, spikes and v_out must be non-null");
     if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 ||
@@ -270,6 +298,7 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.pitch = pg.CK * 2 + 16;
     g.spike_step_stride = spike_step_stride;
     g.v_is_f32 = v_dtype == SNNF_F32 ? 1 : 0;
+    g.analog_out = analog_out ? 1 : 0;
     const int xsize = dtype_size(x_dtype);
     const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
     hipStream_t hs = as_stream(stream);
@@ -313,15 +342,22 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
         int w2 = 1;
         while (!all_shared && w2 < T && w2 < kMaxTT) w2 *= 2;
         const bool fast_layer = Cout % 64 == 0 && v_dtype == SNNF_F32 && lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+        const int vec = vec_ok ? 8 : (vec4_ok ? 4 : 0);
         for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
-            if (plan_mm(g, w2, load_mode, vec_ok ? 8 : (vec4_ok ? 4 : 0), mp)) {
-                // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
-                // the activation prefetch): it runs windows of 2.
-                const bool fast_plan = fast_layer && mp.all_full && mp.run >= 4;
-                if (w2 == 4 && !fast_plan) continue;
-                mm_kernel = planned = true;
-                window = w2;
-            }
+            MmPlan p8 = {}, p4 = {};
+            const bool ok8 = plan_mm(g, w2, load_mode, vec, 8, p8);
+            // One shared frame: a single short matrix stage, then T steps of epilogue per tile. Two 4-wave workgroups per
+            // CU (fast variant only) overlap one's epilogue with the other's loads and matrix work; measured 15 % faster on
+            // a 7x7/2 stem, slower on every layer with a deep matrix loop.
+            const bool ok4 = all_shared && fast_layer && plan_mm(g, w2, load_mode, vec, 4, p4) && p4.all_full && p4.run >= 4;
+            if (!ok8 && !ok4) continue;
+            mp = ok4 ? p4 : p8;
+            // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
+            // the activation prefetch): it runs windows of 2.
+            const bool fast_plan = fast_layer && mp.all_full && mp.run >= 4;
+            if (w2 == 4 && !fast_plan) continue;
+            mm_kernel = planned = true;
+            window = w2;
         }
         if (mm_kernel && all_shared) window = T < SNNF_MAX_T_PER_LAUNCH ? T : SNNF_MAX_T_PER_LAUNCH;
         if (mm_kernel) {
@@ -329,6 +365,9 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
             pl.wm_log2 = mp.wm_log2; pl.wn_log2 = mp.wn_log2; pl.oc_tiles = mp.oc_tiles; pl.lds_bytes = mp.lds_bytes;
         }
     }
+    if (analog_out && !mm_kernel)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_bias: unsupported_shape: only layers the 8-wave matrix kernel takes "
+                    "(Cin %% 8 == 0 or Cin < 8, not a plain 1x1/1 convolution, tiles that fit LDS)");
     // Everything else: the time-outer kernels for a shared frame or a low intensity, the 4-wave T-in-M kernel otherwise.
     bool time_outer = !mm_kernel && (all_shared || flops / bytes < 200.0);
     // Pointwise kernel: where the weight fragments live (registers only in the fast variant) and the LDS that takes.
@@ -390,7 +429,11 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     g.stage_chunks = mm_kernel ? mp.stage_chunks : 1;
     if (mm_kernel) g.pitch = mp.pitch;
     g.d_npairs = make_fast_div(g.npairs);
-    if (mm_kernel) g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
+    g.TI = mm_kernel ? mp.TI : 1;
+    g.img_groups = (g.N + g.TI - 1) / g.TI;
+    g.d_NR = make_fast_div(g.NR);
+    g.d_tile_px = make_fast_div(g.TH * g.TW);
+    if (mm_kernel) g.d_stage_rows = make_fast_div(g.TI * g.NR * (g.WT / 2));
 
     size_t lds_bytes = pl.lds_bytes;
     if (time_outer && !pw_kernel) {
@@ -404,13 +447,13 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     }
     const int cu_per_xcd = (compute_units() + 7) / 8;
     auto grid_for = [&](const ConvGeom& gg, int per_cu) {
-        const int px_tiles = mm_kernel ? gg.N * gg.tiles_img : gg.tiles_x * gg.tiles_y;
+        const int px_tiles = mm_kernel ? gg.img_groups * gg.tiles_img : gg.tiles_x * gg.tiles_y;
         const int work_per_xcd = ((px_tiles + 7) / 8) * gg.oc_tiles;
         int slots = cu_per_xcd * per_cu;
         if (slots > work_per_xcd) slots = work_per_xcd;
         return slots * 8;
     };
-    const int per_cu = mm_kernel ? 1 : (time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1));
+    const int per_cu = mm_kernel ? 8 / mp.nw : (time_outer ? 2 : ((pl.lds_bytes * 2 <= kMaxLds && window < 4) ? 2 : 1));
 
     // Pointwise layers: the fast variant takes the tiles that lie inside their image when the layer qualifies (common
     // neuron, aligned outputs, fp32 membrane, whole channel fragments); the general variant takes the ragged last tile of
@@ -439,13 +482,20 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
     } else if (mm_kernel) {
         const bool fast_ok = mp.all_full && mp.run >= 4 && Cout % 64 == 0 && v_dtype == SNNF_F32 &&
                              lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;   // = fast_plan above
-        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (fast_ok ? 20 : 10) + (all_shared ? 1 : window);
+        parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = (mp.nw == 4 ? 30 : (fast_ok ? 20 : 10)) + (all_shared ? 1 : window);
         nparts = 1;
     } else {
         parts[0].g = g; parts[0].lds = lds_bytes; parts[0].tt = time_outer ? 0 : window;
         nparts = 1;
     }
 
+    snprintf(snnf::conv_plan_buffer(), 256,
+             "kernel=%s variant=%d window=%d launches=%d tile=%dx%dx%d halo=%dx%d waves=%dx%dx%d oc_tiles=%d px_tiles=%d "
+             "stage_chunks=%d run=%d lds=%zu grid=%d",
+             pw_kernel ? "pointwise" : (mm_kernel ? "matrix" : (time_outer ? "time_outer" : "t_in_m")), parts[0].tt, window,
+             nparts * ((T + window - 1) / window), g.TI, g.TH, g.TW, g.NR, g.WT, 1 << g.wm_log2, 1 << g.wn_log2, 1 << g.wk_log2,
+             g.oc_tiles, mm_kernel ? g.img_groups * g.tiles_img : g.tiles_x * g.tiles_y, g.stage_chunks, g.run8, parts[0].lds,
+             grid_for(parts[0].g, per_cu));
     for (int t0 = 0; t0 < T; t0 += window) {
         const int tw = (T - t0) < window ? (T - t0) : window;
         ConvLaunch L = {};
@@ -476,4 +526,23 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
       }
     }
     return SNNF_OK;
+}
+}  // namespace
+}  // namespace snnf
+
+extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,
+                             int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
+                             int pad_h, int pad_w, const void* v_init, int v_dtype, void* spikes,
+                             int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
+                             void* stream) {
+    return snnf::conv_lif_impl(xs, residuals, T, N, Cin, H, W, x_dtype, packed_weight, Cout, KH, KW, stride_h, stride_w, pad_h,
+                               pad_w, v_init, v_dtype, spikes, spike_step_stride, v_out, v_threshold, v_reset, tau, stream, false);
+}
+
+extern "C" int snnf_conv_bias(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,
+                              int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
+                              int pad_h, int pad_w, void* out, int64_t out_step_stride, void* stream) {
+    // The neuron parameters only steer the variant selection (the common neuron qualifies for the fast variant).
+    return snnf::conv_lif_impl(xs, residuals, T, N, Cin, H, W, x_dtype, packed_weight, Cout, KH, KW, stride_h, stride_w, pad_h,
+                               pad_w, nullptr, SNNF_F32, out, out_step_stride, out, 1.0f, 0.0f, 2.0f, stream, true);
 }

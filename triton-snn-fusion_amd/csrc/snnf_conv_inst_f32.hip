@@ -7,6 +7,7 @@ namespace snnf {
 // tt < 0 selects the pointwise kernel (-2: its fast variant), tt == 0 the time-outer kernel, tt in {1, 2, 4} the kernel that accumulates tt timesteps side by side.
 int launch_conv_f32(const ConvLaunch& L, int tt, int load_mode) {
     if (tt < 0) return launch_conv_pw<float>(L, load_mode, tt == -2);
+    if (tt >= 30) return launch_conv_mm_w4_f32(L, tt - 30, load_mode);
     if (tt >= 20) return launch_conv_mm<float>(L, tt - 20, load_mode, true);
     if (tt >= 10) return launch_conv_mm<float>(L, tt - 10, load_mode, false);
     if (tt == 0) return launch_conv_tout<float>(L, load_mode);

@@ -25,17 +25,30 @@
 
 namespace snnf {
 
-constexpr int kMmThreads = 512;
-constexpr int kMmWaves = 8;
 constexpr int kMmStagePitch = 40;                          // floats per channel row of a wave's stage (32 pixels + padding)
 constexpr int kMmStageFloats = 16 * kMmStagePitch;         // 16 channel rows
-static_assert(kMmWaves * kMmStageFloats * sizeof(float) == kMmStageBytes, "host and kernel disagree on the stage size");
+static_assert(kMmStageFloats * sizeof(float) == kMmStageBytesPerWave, "host and kernel disagree on the stage size");
 // Spatial staging items per thread and stage: 64 prefetch registers whatever the load mode and the timesteps per stage.
 __host__ __device__ constexpr int mm_staging_slots(int load_mode, int tt) { return (load_mode == LOAD_PAIR32 ? 8 : 4) / tt; }
 typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
 
-template <typename XT, int TT, int LM, bool FAST, bool SK>
-__global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_mm_lif_kernel(
+// Phase timestamps of the first tile of the first 64 workgroups (development builds with -DSNNF_MM_TRACE only): slot 0
+// kernel start, 1 first loads issued, 2 + 2 s / 3 + 2 s stage s in LDS / stage s multiplied (s < 4), 10 / 11 epilogue
+// start / end. Read back with snnf_debug_mm_trace() of the translation unit that launched the kernel.
+#ifdef SNNF_MM_TRACE
+__device__ unsigned long long mm_trace[64 * 16];
+#define SNNF_MM_STAMP(slot)                                                                                  \
+    do {                                                                                                     \
+        if (threadIdx.x == 0 && blockIdx.x < 64 && trace_on) mm_trace[blockIdx.x * 16 + (slot)] = __builtin_amdgcn_s_memtime(); \
+    } while (0)
+#else
+#define SNNF_MM_STAMP(slot) do {} while (0)
+#endif
+
+// NW waves per workgroup: 8 (one workgroup per CU) or 4 (two independent workgroups per CU, whose load, matrix and
+// epilogue phases overlap each other instead of running in lockstep across the whole CU).
+template <typename XT, int TT, int LM, bool FAST, bool SK, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_mm_lif_kernel(
     const StepPtrs xs, const StepPtrs residuals, const int has_residual, const ConvGeom g,
     const uint16_t* __restrict__ wpacked, const float* __restrict__ bias, const void* __restrict__ v_init,
     XT* __restrict__ spikes, void* __restrict__ v_out, const LifParams lif) {
@@ -44,7 +57,12 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
     constexpr int SS = mm_staging_slots(LM, TT);
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
+    constexpr int NT = NW * 64;                               // threads per workgroup
     const int tid = threadIdx.x;
+#ifdef SNNF_MM_TRACE
+    bool trace_on = true;
+#endif
+    SNNF_MM_STAMP(0);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int half = lane >> 5;
@@ -54,11 +72,14 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     const int wk = SK ? (wave >> (g.wm_log2 + g.wn_log2)) : 0;     // K slice of this wave (split-K variant)
     const int WK = SK ? (1 << g.wk_log2) : 1;
 
+    if (g.wm_log2 >= 0) SNNF_MM_STAMP(12);
     const int groups = 1 << g.groups_log2;                   // channel groups of 8 per packed chunk
     const int stage_groups = groups * g.stage_chunks;        // ... per LDS stage (a stage holds stage_chunks chunks)
     const int nstages = (g.nchunks + g.stage_chunks - 1) / g.stage_chunks;
     const int WTP = g.WT >> 1;
-    const int tile_bytes = g.NR * g.WT * g.pitch;            // one timestep's halo tile
+    const int rows_all = g.TI * g.NR;                        // halo rows of the TI images of a tile, stacked
+    const int tile_px = g.TH * g.TW;                         // output pixels per image and tile
+    const int tile_bytes = rows_all * g.WT * g.pitch;        // one timestep's halo tile(s)
     float* __restrict__ stage = reinterpret_cast<float*>(lds + g.mm_stage_off) + wave * kMmStageFloats;
     const int nocf = (g.Cout + 31) >> 5;
     const int total_pairs = g.nchunks * g.npairs;
@@ -68,23 +89,28 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     const bool pair_shift = LM == LOAD_PAIR32;               // tile columns start at an even input column
 
     // ---- kernel constants of the staging: item e = (channel group, tile row, column pair).
-    int item_cg[SS], item_r[SS], item_c[SS];                 // item_cg < 0: idle slot
+    int item_cg[SS], item_r[SS], item_c[SS], item_i[SS];     // item_cg < 0: idle slot; item_i: image of the tile
     uint32_t item_dst[SS];
-    int item_src[SS];                                        // element offset of (cg * 8, row r, column 2 cp) from the tile origin
+    int item_src[SS];                                        // element offset of (image i, channel cg * 8, row r, column 2 cp) from the tile origin
+    const int image_elems = g.Cin * g.H * g.W;
 #pragma unroll
     for (int s = 0; s < SS; ++s) {
-        const int e = s * kMmThreads + tid;
+        const int e = s * NT + tid;
         const int cg = fast_div(e, g.d_stage_rows);
-        const int rem = e - cg * (g.NR * WTP);
-        const int r = fast_div(rem, g.d_WTP);
-        const int cp = rem - r * WTP;
+        const int rem = e - cg * (rows_all * WTP);
+        const int rr = fast_div(rem, g.d_WTP);               // stacked row
+        const int cp = rem - rr * WTP;
+        const int ii = fast_div(rr, g.d_NR);
+        const int r = rr - ii * g.NR;
         item_cg[s] = cg < stage_groups ? cg : -1;
         item_r[s] = r;
+        item_i[s] = ii;
         item_c[s] = 2 * cp;
-        item_dst[s] = static_cast<uint32_t>((r * g.WT + 2 * cp) * g.pitch + cg * 16);
-        item_src[s] = (cg * 8 * g.H + r) * g.W + 2 * cp;
+        item_dst[s] = static_cast<uint32_t>((rr * g.WT + 2 * cp) * g.pitch + cg * 16);
+        item_src[s] = ii * image_elems + (cg * 8 * g.H + r) * g.W + 2 * cp;
     }
 
+    if (item_src[0] != -12345) SNNF_MM_STAMP(13);
     const int last_channel = g.Cin < 8 ? g.Cin - 1 : 7;
     const int taps = g.KH * g.KW;
     // ---- the stage in flight.
@@ -103,7 +129,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         for (int s = 0; s < SS; ++s) {
             const int ih = ih_lo + item_r[s];
             const int iw = iw_lo + item_c[s];
-            const bool cok = item_cg[s] >= 0 && chunk * g.CK + item_cg[s] * 8 < g.Cin && ih >= 0 && ih < g.H;
+            const bool cok = item_cg[s] >= 0 && chunk * g.CK + item_cg[s] * 8 < g.Cin && ih >= 0 && ih < g.H && n + item_i[s] < g.N;
             const bool ok0 = cok && iw >= 0 && iw < g.W;
             const bool ok1 = cok && iw + 1 >= 0 && iw + 1 < g.W;
             const uint32_t src = static_cast<uint32_t>(item_src[s] + tile_rel) * ES;
@@ -188,7 +214,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     // ---- tile walk: pixel tiles congruent to this workgroup's XCD; consecutive work items = output-channel tiles.
     const int xcd = blockIdx.x & 7;
     const int slots_per_xcd = gridDim.x >> 3;
-    const int n_px_tiles = g.N * g.tiles_img;
+    const int n_px_tiles = g.img_groups * g.tiles_img;       // a tile spans TI images (TI > 1: whole output planes)
     const int work_per_xcd = ((n_px_tiles + 7) >> 3) * g.oc_tiles;
     int work = blockIdx.x >> 3;
     int oc_tile = 0, img = 0, oh0 = 0, ow0 = 0;
@@ -198,8 +224,9 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         const int px_tile = pt * 8 + xcd;
         if (px_tile >= n_px_tiles) return false;
         oc_t = w - pt * g.oc_tiles;
-        n = fast_div(px_tile, g.d_tiles_img);
-        const int in_img = px_tile - n * g.tiles_img;
+        const int group = fast_div(px_tile, g.d_tiles_img);
+        const int in_img = px_tile - group * g.tiles_img;
+        n = group * g.TI;
         const int ty = fast_div(in_img, g.d_tiles_x);
         r0 = ty * g.TH;
         c0 = (in_img - ty * g.tiles_x) * g.TW;
@@ -211,28 +238,35 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         if (pair_shift && (iw_lo & 1)) iw_lo -= 1;
     };
     bool have_tile = decode(work, oc_tile, img, oh0, ow0);
+    if (oh0 != -12345) SNNF_MM_STAMP(14);
     if (have_tile) {
         int ih_lo, iw_lo;
         halo_origin(oh0, ow0, ih_lo, iw_lo);
         issue_loads(0, img, ih_lo, iw_lo);
     }
+    SNNF_MM_STAMP(1);
 
     // ---- kernel constants of the matrix loop: this lane's pixel (block pixel wm * 32 + l32) inside the halo tile.
     const int mpix = wm * 32 + l32;
-    const int mpr = fast_div(mpix, g.d_TW);
-    const int mpc = mpix - mpr * g.TW;
-    const bool m_inside = mpr < g.TH;                        // lanes beyond the tile read pixel (0, 0): finite, never stored
-    const uint32_t b_base = static_cast<uint32_t>(m_inside ? ((mpr * g.sh) * g.WT + mpc * g.sw) * g.pitch : 0);
+    const int mpi = fast_div(mpix, g.d_tile_px);             // image of the tile
+    const int mrem = mpix - mpi * tile_px;
+    const int mpr = fast_div(mrem, g.d_TW);
+    const int mpc = mrem - mpr * g.TW;
+    const bool m_inside = mpi < g.TI;                        // lanes beyond the tile read pixel (0, 0): finite, never stored
+    const uint32_t b_base = static_cast<uint32_t>(m_inside ? ((mpi * g.NR + mpr * g.sh) * g.WT + mpc * g.sw) * g.pitch : 0);
 
     // ---- kernel constants of the epilogue: lane = (channel row lane >> 2 of 16, pixels 8 (lane & 3) .. + 7 of the wave's 32).
     const int row16 = lane >> 2;
     const int pcx = lane & 3;
     const int epix = wm * 32 + pcx * 8;
-    const int epr = fast_div(epix, g.d_TW);
-    const int epc = epix - epr * g.TW;
-    const bool lo_inside = epix + 4 <= g.TH * g.TW;          // FAST: tile sizes are multiples of 4 (8 with 16-byte runs), so
-    const bool hi_inside = epix + 8 <= g.TH * g.TW;          // each half of a lane's run of 8 pixels is inside or outside as a whole
-    const uint32_t lane_px = static_cast<uint32_t>(epr * g.Wo + epc);
+    const int epi = fast_div(epix, g.d_tile_px);
+    const int erem = epix - epi * tile_px;
+    const int epr = fast_div(erem, g.d_TW);
+    const int epc = erem - epr * g.TW;
+    const bool lo_inside = epix + 4 <= g.TI * tile_px;       // FAST: planes and tiles are multiples of 4 (8 with 16-byte runs), so
+    const bool hi_inside = epix + 8 <= g.TI * tile_px;       // each half of a lane's run of 8 pixels is inside or outside as a whole
+    const uint32_t image_out = static_cast<uint32_t>(g.Cout) * static_cast<uint32_t>(g.Ho * g.Wo);
+    const uint32_t lane_px = static_cast<uint32_t>(epi) * image_out + static_cast<uint32_t>(epr * g.Wo + epc);
     float* __restrict__ stage_wr = stage + (half * 4) * kMmStagePitch + l32;
     const float* __restrict__ stage_rd = stage + row16 * kMmStagePitch + pcx * 8;
     const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
@@ -281,6 +315,9 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         };
         // Weight fragments stream from L2 two pairs ahead of their use, through three register sets.
         auto load_frags = [&](int gpair, cv_u32x4& a0, cv_u32x4& a1) __attribute__((always_inline)) {
+#ifdef SNNF_MM_EXPERIMENT_NO_WEIGHT_STREAM
+            if (gpair >= 2 * WK) return;   // timing experiment (wrong results): only the first fragments of a tile are loaded
+#endif
             const int64_t o = static_cast<int64_t>(min(gpair, total_pairs - 1)) * (kFragBytes / 2);
             a0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + o);
             a1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + o);
@@ -294,6 +331,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             __syncthreads();   // every wave is done reading the previous stage
             write_lds();       // waits for the stage's loads
             __syncthreads();
+            if (chunk < 4) SNNF_MM_STAMP(2 + 2 * chunk);
             // ---- the stage after this one: next chunk, or the first chunk of the next tile.
             {
                 int nc = chunk + 1, nimg = img, nih = ih_lo, niw = iw_lo;
@@ -324,12 +362,14 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                     }
                 }
             }
+            if (chunk < 4) SNNF_MM_STAMP(3 + 2 * chunk);
         }
+        SNNF_MM_STAMP(10);
 
         // ---- epilogue: 16 channel rows x 32 pixels at a time through the wave's stage, so that a lane owns 8 consecutive
         // pixels of one channel row; the membrane of those 8 neurons lives in registers across the TT steps.
         // h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
-        const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo);
+        const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo && img + g.TI <= g.N);
         const bool fast = FAST || (g.vec8 && full && g.run8 == 8);
         const bool vf32 = FAST || g.v_is_f32;
         const bool wide = !FAST || g.run8 == 8;          // FAST: 16-byte spike accesses, or 8-byte ones when runs are only 8-byte aligned
@@ -337,13 +377,16 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
         uint32_t pxoff[8];
         if (!fast) {
             okmask = 0;
-            int pr = epr, pc = epc;
+            int pi = epi, pr = epr, pc = epc;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                const bool ok = pr < g.TH && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
+                const bool ok = pi < g.TI && img + pi < g.N && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
                 okmask |= ok ? (1u << k) : 0u;
-                pxoff[k] = ok ? static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
-                if (++pc == g.TW) { pc = 0; ++pr; }
+                pxoff[k] = ok ? static_cast<uint32_t>(pi) * image_out + static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
+                if (++pc == g.TW) {
+                    pc = 0;
+                    if (++pr == g.TH) { pr = 0; ++pi; }
+                }
             }
         } else {
             okmask = (lo_inside ? 0x0fu : 0u) | (hi_inside ? 0xf0u : 0u);
@@ -359,6 +402,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             row_off = static_cast<uint32_t>(min(oc, g.Cout - 1)) * static_cast<uint32_t>(po);
             bvv = (wave_has_work && (FAST || oc < g.Cout)) ? bias[oc] : 0.0f;
         };
+        const bool analog = g.analog_out != 0;   // neuron-free output: conv + bias (+ residual) where the spikes would go
         auto load_membrane = [&](bool row_ok, uint32_t row_off, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[k] = 0.0f;
@@ -387,7 +431,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
             }
         };
         auto store_membrane = [&](bool row_ok, uint32_t row_off, const float (&v)[8]) __attribute__((always_inline)) {
-            if (!row_ok) return;
+            if (!row_ok || analog) return;
             if (fast && vf32) {
                 float* dst = static_cast<float*>(v_out) + tile_off + row_off + pxoff[0];
                 Pack<float, 4> lo, hi;
@@ -442,19 +486,24 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                 }
             }
             Pack<XT, 8> sp;
+            if (analog) {   // uniform: no neuron, the sums themselves go out
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                bool fired;
-                if constexpr (FAST) {   // the common neuron: power-of-two tau, hard reset
-                    const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
-                    fired = h >= lif.v_threshold;
-                    v[k] = fired ? lif.v_reset : h;
-                } else {
-                    const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
-                    fired = h >= lif.v_threshold;
-                    v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                for (int k = 0; k < 8; ++k) sp.v[k] = from_float<XT>(x[k]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    bool fired;
+                    if constexpr (FAST) {   // the common neuron: power-of-two tau, hard reset
+                        const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
+                        fired = h >= lif.v_threshold;
+                        v[k] = fired ? lif.v_reset : h;
+                    } else {
+                        const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
+                        fired = h >= lif.v_threshold;
+                        v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
+                    }
+                    sp.v[k] = spike_value<XT>(fired);
                 }
-                sp.v[k] = spike_value<XT>(fired);
             }
             if (row_ok) {
                 if (fast && wide) {
@@ -560,6 +609,10 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
                 if (owner == wk) store_membrane(row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
             }
         }
+        SNNF_MM_STAMP(11);
+#ifdef SNNF_MM_TRACE
+        trace_on = false;
+#endif
         if (SK && next_tile) {
             int nih, niw;
             halo_origin(next_oh0, next_ow0, nih, niw);
@@ -574,7 +627,7 @@ __global__ __launch_bounds__(kMmThreads, 1) __attribute__((amdgpu_waves_per_eu(2
     }
 }
 
-template <typename XT, int TT>
+template <typename XT, int TT, int NW>
 int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
     const bool split_k = L.g.wk_log2 > 0;
     auto run = [&](auto kernel) -> int {
@@ -590,15 +643,20 @@ int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
                 raised[dev] = true;
             }
         }
-        kernel<<<dim3(L.grid), kMmThreads, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
+        kernel<<<dim3(L.grid), NW * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
                                                                     static_cast<XT*>(L.spikes), L.v_out, L.lif);
         return check_launch("snnf_conv_lif");
     };
     auto pick = [&](auto lm) -> int {
         constexpr int LMV = decltype(lm)::value;
-        if (split_k)
-            return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, true>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, true>);
-        return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, false>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, false>);
+        if constexpr (NW == 8) {
+            if (split_k)
+                return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, true, 8>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, true, 8>);
+            return fast ? run(conv_mm_lif_kernel<XT, TT, LMV, true, false, 8>) : run(conv_mm_lif_kernel<XT, TT, LMV, false, false, 8>);
+        } else {   // half-size workgroups exist in the fast variant only
+            if (!fast) return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: no general variant with %d waves", NW);
+            return split_k ? run(conv_mm_lif_kernel<XT, TT, LMV, true, true, NW>) : run(conv_mm_lif_kernel<XT, TT, LMV, true, false, NW>);
+        }
     };
     if constexpr (sizeof(XT) == 4) {
         return pick(std::integral_constant<int, LOAD_2XF32>{});
@@ -608,11 +666,11 @@ int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
     }
 }
 
-template <typename XT>
+template <typename XT, int NW = 8>
 int launch_conv_mm(const ConvLaunch& L, int tt, int load_mode, bool fast) {
-    if (tt == 4) return launch_conv_mm_tt<XT, 4>(L, load_mode, fast);
-    if (tt == 2) return launch_conv_mm_tt<XT, 2>(L, load_mode, fast);
-    return launch_conv_mm_tt<XT, 1>(L, load_mode, fast);
+    if (tt == 4) return launch_conv_mm_tt<XT, 4, NW>(L, load_mode, fast);
+    if (tt == 2) return launch_conv_mm_tt<XT, 2, NW>(L, load_mode, fast);
+    return launch_conv_mm_tt<XT, 1, NW>(L, load_mode, fast);
 }
 
 }  // namespace snnf

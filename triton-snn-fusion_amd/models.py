@@ -274,6 +274,7 @@ class _FusedNetwork(nn.Module):
         self.device_ = torch.device(device)
         self.zero_v = torch.zeros((), dtype=v_dtype, device=self.device_)
         self.record: Optional[List[Dict]] = None
+        self.native_plain_conv = True        # False: LIF-free convolutions always go to the framework's convolution
         self._graph = None
 
     # -- operator calls ------------------------------------------------------------------------------------------
@@ -291,11 +292,26 @@ class _FusedNetwork(nn.Module):
         self._log(kind="conv_lif", name=name, xs=xs, residuals=residuals, layer=layer, spikes=spikes, v=v)
         return spikes
 
-    def plain_conv(self, name: str, x_seq: torch.Tensor, layer: _FusedLayer) -> torch.Tensor:
-        """LIF-free convolution of all T*N frames at once (stock PyTorch, bias = folded BatchNorm shift)."""
-        y = F.conv2d(x_seq.flatten(0, 1), layer.weight, layer.bias, layer.stride, layer.padding)
-        y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
-        self._log(kind="plain_conv", name=name, x=x_seq, layer=layer, y=y)
+    def plain_conv(self, name: str, x_seq: torch.Tensor, layer: _FusedLayer, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """LIF-free convolution (+ residual) of T frames, bias = folded BatchNorm shift: the matrix kernel's neuron-free
+        mode where it takes the layer, the framework's convolution otherwise (and on CPU tensors)."""
+        y = None
+        if x_seq.is_cuda and self.native_plain_conv:
+            from .runtime.hip_convlif_backend import run_hip_temporal_conv_bias
+            try:
+                y = run_hip_temporal_conv_bias(list(x_seq.unbind(0)), layer.weight, layer.bias, layer.stride, layer.padding,
+                                               None if residual is None else list(residual.unbind(0)))
+                native = True
+            except RuntimeError as exc:
+                if "unsupported" not in str(exc):
+                    raise
+        if y is None:
+            native = False
+            y = F.conv2d(x_seq.flatten(0, 1), layer.weight, layer.bias, layer.stride, layer.padding)
+            y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
+            if residual is not None:
+                y = y + residual
+        self._log(kind="plain_conv", name=name, x=x_seq, layer=layer, residual=residual, y=y, native=native)
         return y
 
     def pooled(self, name: str, x_seq: torch.Tensor, pool: nn.Module) -> torch.Tensor:
@@ -391,8 +407,7 @@ class FusedSpikingResNet18(_FusedNetwork):
             if conv2.lif is not None:
                 seq = self.conv_lif(f"blocks.{i}.conv2", list(hidden.unbind(0)), conv2, residuals=list(identity.unbind(0)))
             else:   # last block: its neuron is the tail's
-                seq = self.plain_conv(f"blocks.{i}.conv2", hidden, conv2) + identity
-                self._log(kind="add", name=f"blocks.{i}.add", y=seq)
+                seq = self.plain_conv(f"blocks.{i}.conv2", hidden, conv2, residual=identity)
         return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
 
 

@@ -237,6 +237,33 @@ def get_autotune_best_config(kernel_key: str, residual_add: bool = False, T: int
     return {"BTILE_T": window, "REUSE_GROUPS": 1, "kernel_temporal_window": window, "residual_add": bool(residual_add)}
 
 
+def last_conv_plan() -> Dict:
+    """What the planner selected for this thread's most recent matrix-core convolution launch (snnf_conv_last_plan):
+    kernel family, timesteps per launch, tile and wave decomposition, LDS bytes and grid, as a dict."""
+    text = _lib.lib().snnf_conv_last_plan().decode("ascii", "replace")
+    plan: Dict = {}
+    for item in text.split():
+        key, _, value = item.partition("=")
+        plan[key] = int(value) if value.lstrip("-").isdigit() else value
+    return plan
+
+
+def _planned_temporal_config(kernel_key: str, residual_add: bool, T: int) -> Dict:
+    config = get_autotune_best_config(kernel_key, residual_add=residual_add, T=T)
+    if kernel_key.startswith("depthwise_"):
+        return config
+    plan = last_conv_plan()
+    if plan:
+        variant = int(plan.get("variant", 0))
+        # Timesteps accumulated side by side against one weight fragment load: the matrix kernels encode it in the
+        # variant number (10 + n general, 20 + n fast, 30 + n fast with 4-wave workgroups), the 4-wave T-in-M kernel uses the variant itself, the time-outer and
+        # pointwise kernels take one step at a time with the weights resident.
+        side_by_side = variant % 10 if variant >= 10 else max(1, variant)
+        config.update({"BTILE_T": side_by_side, "kernel_temporal_window": int(plan.get("window", config["kernel_temporal_window"])),
+                       "plan": plan})
+    return config
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # Packed-weight cache: the implicit-GEMM kernel reads weights in matrix-core fragment order; the repack runs once per
 # (weight tensor object, version) and is reused by every later call with the same tensors.
@@ -326,6 +353,42 @@ def _launch(kernel_key: str, steps: Sequence[torch.Tensor], residuals: Optional[
             float(v_threshold), float(v_reset), float(tau), stream))
 
 
+def run_hip_temporal_conv_bias(xs: Sequence[torch.Tensor], weight, bias, stride, padding,
+                               residuals: Optional[Sequence[torch.Tensor]] = None) -> torch.Tensor:
+    """Neuron-free convolution + bias (+ residual) of T independent frames on the matrix kernel (snnf_conv_bias):
+    returns [T, N, Cout, Ho, Wo] in the activation dtype. For the LIF-free Conv+BN layers between fused operators
+    (ResNet shortcuts, whose output feeds `fused_temporal_conv_add_lif_state` as `residuals`); the reference leaves
+    those to the framework's convolution. Raises RuntimeError("unsupported_...") for layers the kernel does not take."""
+    steps = _contiguous_steps(xs)
+    first = steps[0]
+    if not first.is_cuda or first.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise RuntimeError("unsupported_device: snnf_conv_bias needs fp32 / bf16 / fp16 tensors on the GPU")
+    if any(s.shape != first.shape or s.dtype != first.dtype for s in steps):
+        raise RuntimeError("unsupported_shape: frames must share shape and dtype")
+    T = len(steps)
+    n, cin, h, w = (int(d) for d in first.shape)
+    cout, wcin, kh, kw = (int(d) for d in weight.shape)
+    if wcin != cin:
+        raise RuntimeError(f"unsupported_groups: weight has {wcin} input channels, frames have {cin}")
+    sh, sw = _as_pair(stride)
+    ph, pw = _as_pair(padding)
+    ho, wo = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
+    res = None
+    if residuals is not None:
+        res = _contiguous_steps(residuals)
+        if len(res) != T or any(tuple(r.shape) != (n, cout, ho, wo) or r.dtype != first.dtype for r in res):
+            raise RuntimeError("unsupported_residual_shape: residuals must be T tensors of the output shape and dtype")
+    if bias is None:
+        bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    out = torch.empty((T, n, cout, ho, wo), dtype=first.dtype, device=first.device)
+    packed = _packed_weight(weight, bias, first.dtype)
+    _lib.check("snnf_conv_bias", _lib.lib().snnf_conv_bias(
+        _lib.step_pointers(steps), _lib.step_pointers(res) if res is not None else None, T, n, cin, h, w,
+        _lib.dtype_code(first.dtype), packed.data_ptr(), cout, kh, kw, sh, sw, ph, pw,
+        out.data_ptr(), int(out.stride(0)), _lib.current_stream(first.device)))
+    return out
+
+
 def _contiguous_steps(xs: Sequence[torch.Tensor]) -> List[torch.Tensor]:
     return [x if x.is_contiguous() else x.contiguous() for x in xs]
 
@@ -385,7 +448,7 @@ def _run_temporal(kind: str, xs, residuals, weight, bias, v_init, stride, paddin
         diagnostics["kernel_kind"] = "temporal_residual"
     return TritonConvLIFResult(
         spikes, v_next, True, kernel_key=kernel_key,
-        kernel_temporal_config=get_autotune_best_config(kernel_key, residual_add=residuals is not None, T=T),
+        kernel_temporal_config=_planned_temporal_config(kernel_key, residuals is not None, T),
         kernel_diagnostics=diagnostics,
     )
 
