@@ -61,6 +61,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     const int tid = threadIdx.x;
 #ifdef SNNF_MM_TRACE
     bool trace_on = true;
+    int trace_tile = 0;
 #endif
     SNNF_MM_STAMP(0);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -110,7 +111,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         item_src[s] = ii * image_elems + (cg * 8 * g.H + r) * g.W + 2 * cp;
     }
 
-    if (item_src[0] != -12345) SNNF_MM_STAMP(13);
     const int last_channel = g.Cin < 8 ? g.Cin - 1 : 7;
     const int taps = g.KH * g.KW;
     // ---- the stage in flight.
@@ -365,159 +365,170 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             if (chunk < 4) SNNF_MM_STAMP(3 + 2 * chunk);
         }
         SNNF_MM_STAMP(10);
+#ifdef SNNF_MM_TRACE
+        if (trace_tile == 1 && threadIdx.x == 0 && blockIdx.x < 64) mm_trace[blockIdx.x * 16 + 13] = __builtin_amdgcn_s_memtime();
+#endif
 
-        // ---- epilogue: 16 channel rows x 32 pixels at a time through the wave's stage, so that a lane owns 8 consecutive
-        // pixels of one channel row; the membrane of those 8 neurons lives in registers across the TT steps.
-        // h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
-        const bool full = FAST || (oh0 + g.TH <= g.Ho && ow0 + g.TW <= g.Wo && img + g.TI <= g.N);
-        const bool fast = FAST || (g.vec8 && full && g.run8 == 8);
+        // ---- epilogue. h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
+        // FAST: 16 channel rows x 32 pixels at a time go through the wave's LDS stage, so that a lane owns 8 consecutive pixels
+        // of one channel row (16- or 8-byte accesses); the membrane of those 8 neurons lives in registers across the TT steps.
+        // General variant: straight from the accumulator layout - a lane owns ONE pixel and 8 channel rows per group, the 32
+        // lanes of a half-wave store 32 consecutive pixels of a row (coalesced 2-byte spike stores whatever the alignment of
+        // the planes), one validity bit per lane instead of one per element.
         const bool vf32 = FAST || g.v_is_f32;
         const bool wide = !FAST || g.run8 == 8;          // FAST: 16-byte spike accesses, or 8-byte ones when runs are only 8-byte aligned
-        uint32_t okmask = 0xffu;
-        uint32_t pxoff[8];
-        if (!fast) {
-            okmask = 0;
-            int pi = epi, pr = epr, pc = epc;
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const bool ok = pi < g.TI && img + pi < g.N && oh0 + pr < g.Ho && ow0 + pc < g.Wo;
-                okmask |= ok ? (1u << k) : 0u;
-                pxoff[k] = ok ? static_cast<uint32_t>(pi) * image_out + static_cast<uint32_t>(pr * g.Wo + pc) : 0u;
-                if (++pc == g.TW) {
-                    pc = 0;
-                    if (++pr == g.TH) { pr = 0; ++pi; }
-                }
-            }
-        } else {
-            okmask = (lo_inside ? 0x0fu : 0u) | (hi_inside ? 0xf0u : 0u);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) pxoff[k] = lane_px + k;
-        }
+        const uint32_t okmask = FAST ? ((lo_inside ? 0x0fu : 0u) | (hi_inside ? 0xf0u : 0u))
+                                     : ((m_inside && img + mpi < g.N && oh0 + mpr < g.Ho && ow0 + mpc < g.Wo) ? 0xffu : 0u);
+        // Element offset of the lane's first pixel (FAST: of its run of 8) from the tile origin of its channel row.
+        const uint32_t px0 = FAST ? lane_px : static_cast<uint32_t>(mpi) * image_out + static_cast<uint32_t>(mpr * g.Wo + mpc);
         const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * po + oh0 * g.Wo + ow0;   // uniform, elements
+        const bool analog = g.analog_out != 0;   // neuron-free output: conv + bias (+ residual) where the spikes would go
 
-        // One group = 16 channel rows (fragment f, half ps) x the wave's 32 pixels; `rows_ok`: this lane's row exists.
-        auto group_row = [&](int gidx, bool& row_ok, uint32_t& row_off, float& bvv) __attribute__((always_inline)) {
-            const int oc = (ocf0 + (gidx >> 1)) * 32 + (gidx & 1) * 16 + row16;
+        // One group = 8 accumulator registers of a 32-row fragment: FAST, after the transposition, this lane's channel row
+        // row16 of the group's 16 rows; general variant, the lane's 8 rows first + {0..3, 8..11} with
+        // first = 32 fragment + 16 (gidx & 1) + 4 half. `row_ok`: the lane has anything to load or store in the group.
+        auto first_row = [&](int gidx) __attribute__((always_inline)) -> int {
+            return (ocf0 + (gidx >> 1)) * 32 + (gidx & 1) * 16 + (FAST ? row16 : 4 * half);
+        };
+        auto row_delta = [&](int rr) __attribute__((always_inline)) -> int { return 8 * (rr >> 2) + (rr & 3); };
+        auto group_row = [&](int gidx, bool& row_ok, uint32_t& row_off, float (&bvv)[8]) __attribute__((always_inline)) {
+            const int oc = first_row(gidx);
             row_ok = wave_has_work && (FAST || oc < g.Cout) && okmask != 0;
             row_off = static_cast<uint32_t>(min(oc, g.Cout - 1)) * static_cast<uint32_t>(po);
-            bvv = (wave_has_work && (FAST || oc < g.Cout)) ? bias[oc] : 0.0f;
+            if constexpr (FAST) {
+                bvv[0] = wave_has_work ? bias[oc] : 0.0f;
+            } else {
+#pragma unroll
+                for (int rr = 0; rr < 8; ++rr) bvv[rr] = (wave_has_work && oc + row_delta(rr) < g.Cout) ? bias[oc + row_delta(rr)] : 0.0f;
+            }
         };
-        const bool analog = g.analog_out != 0;   // neuron-free output: conv + bias (+ residual) where the spikes would go
-        auto load_membrane = [&](bool row_ok, uint32_t row_off, float (&v)[8]) __attribute__((always_inline)) {
+        auto load_membrane = [&](int gidx, bool row_ok, uint32_t row_off, float (&v)[8]) __attribute__((always_inline)) {
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[k] = 0.0f;
-            if (v_init != nullptr && row_ok) {
-                if (fast && vf32) {
-                    const float* src = static_cast<const float*>(v_init) + tile_off + row_off + pxoff[0];
-                    if (okmask & 0x0fu) {
-                        const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
+            if (v_init == nullptr || !row_ok) return;
+            if constexpr (FAST) {
+                const float* src = static_cast<const float*>(v_init) + tile_off + row_off + px0;
+                if (okmask & 0x0fu) {
+                    const Pack<float, 4> lo = *reinterpret_cast<const Pack<float, 4>*>(src);
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) v[k] = lo.v[k];
-                    }
-                    if (okmask & 0xf0u) {
-                        const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+                    for (int k = 0; k < 4; ++k) v[k] = lo.v[k];
+                }
+                if (okmask & 0xf0u) {
+                    const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) v[4 + k] = hi.v[k];
-                    }
-                } else {
+                    for (int k = 0; k < 4; ++k) v[4 + k] = hi.v[k];
+                }
+            } else {
+                const int oc = first_row(gidx);
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        if (okmask & (1u << k)) {
-                            v[k] = vf32 ? static_cast<const float*>(v_init)[tile_off + row_off + pxoff[k]]
-                                        : to_float(static_cast<const XT*>(v_init)[tile_off + row_off + pxoff[k]]);
-                        }
+                for (int rr = 0; rr < 8; ++rr) {
+                    if (oc + row_delta(rr) < g.Cout) {
+                        const int64_t at = tile_off + row_off + static_cast<uint32_t>(row_delta(rr) * po) + px0;
+                        v[rr] = vf32 ? static_cast<const float*>(v_init)[at] : to_float(static_cast<const XT*>(v_init)[at]);
                     }
                 }
             }
         };
-        auto store_membrane = [&](bool row_ok, uint32_t row_off, const float (&v)[8]) __attribute__((always_inline)) {
+        auto store_membrane = [&](int gidx, bool row_ok, uint32_t row_off, const float (&v)[8]) __attribute__((always_inline)) {
             if (!row_ok || analog) return;
-            if (fast && vf32) {
-                float* dst = static_cast<float*>(v_out) + tile_off + row_off + pxoff[0];
+            if constexpr (FAST) {
+                float* dst = static_cast<float*>(v_out) + tile_off + row_off + px0;
                 Pack<float, 4> lo, hi;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
                 if (okmask & 0x0fu) *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
                 if (okmask & 0xf0u) *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
             } else {
+                const int oc = first_row(gidx);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    if (okmask & (1u << k)) {
-                        if (vf32) static_cast<float*>(v_out)[tile_off + row_off + pxoff[k]] = v[k];
-                        else static_cast<XT*>(v_out)[tile_off + row_off + pxoff[k]] = from_float<XT>(v[k]);
+                for (int rr = 0; rr < 8; ++rr) {
+                    if (oc + row_delta(rr) < g.Cout) {
+                        const int64_t at = tile_off + row_off + static_cast<uint32_t>(row_delta(rr) * po) + px0;
+                        if (vf32) static_cast<float*>(v_out)[at] = v[rr];
+                        else static_cast<XT*>(v_out)[at] = from_float<XT>(v[rr]);
                     }
                 }
             }
         };
-        // One LIF step of a group: the lane's 8 sums arrive in MFMA layout (xin = accumulator rows 8 ps .. 8 ps + 7 of its
-        // pixel), are transposed through the wave's stage, then bias (+ residual), LIF, spike store.
-        auto lif_step_group = [&](int t, bool row_ok, uint32_t row_off, float bvv, const float (&xin)[8], float (&v)[8]) __attribute__((always_inline)) {
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int rr = 0; rr < 8; ++rr) stage_wr[((rr >> 2) * 8 + (rr & 3)) * kMmStagePitch] = xin[rr];
-            __builtin_amdgcn_wave_barrier();
-            const cv_f32x4 xlo = *reinterpret_cast<const cv_f32x4*>(stage_rd);
-            const cv_f32x4 xhi = *reinterpret_cast<const cv_f32x4*>(stage_rd + 4);
-            float x[8];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) { x[k] = xlo[k] + bvv; x[4 + k] = xhi[k] + bvv; }
-            XT* __restrict__ out_t = spikes + t * g.spike_step_stride + tile_off + row_off;
-            if (has_residual && row_ok) {
-                const XT* __restrict__ res_t = static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), t)) + tile_off + row_off;
-                if (fast && wide) {
-                    const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + pxoff[0]);
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
-                } else if (fast) {
-                    if (okmask & 0x0fu) {
-                        const Pack<XT, 4> ra = *reinterpret_cast<const Pack<XT, 4>*>(res_t + pxoff[0]);
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) x[k] += to_float(ra.v[k]);
-                    }
-                    if (okmask & 0xf0u) {
-                        const Pack<XT, 4> rb = *reinterpret_cast<const Pack<XT, 4>*>(res_t + pxoff[0] + 4);
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) x[4 + k] += to_float(rb.v[k]);
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-                        if (okmask & (1u << k)) x[k] += to_float(res_t[pxoff[k]]);
-                }
-            }
-            Pack<XT, 8> sp;
-            if (analog) {   // uniform: no neuron, the sums themselves go out
-#pragma unroll
-                for (int k = 0; k < 8; ++k) sp.v[k] = from_float<XT>(x[k]);
+        // The neuron (or, in the neuron-free mode, the conversion of the sum) of one element.
+        auto neuron = [&](float x, float& v) __attribute__((always_inline)) -> XT {
+            bool fired;
+            if constexpr (FAST) {   // the common neuron: power-of-two tau, hard reset
+                const float h = v + (x - v) * lif.inv_tau;
+                fired = h >= lif.v_threshold;
+                v = fired ? lif.v_reset : h;
             } else {
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    bool fired;
-                    if constexpr (FAST) {   // the common neuron: power-of-two tau, hard reset
-                        const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
-                        fired = h >= lif.v_threshold;
-                        v[k] = fired ? lif.v_reset : h;
-                    } else {
-                        const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
-                        fired = h >= lif.v_threshold;
-                        v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
-                    }
-                    sp.v[k] = spike_value<XT>(fired);
-                }
+                const float h = v + (x - v * c0f) * c1f;
+                fired = h >= lif.v_threshold;
+                v = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
             }
-            if (row_ok) {
-                if (fast && wide) {
-                    *reinterpret_cast<Pack<XT, 8>*>(out_t + pxoff[0]) = sp;
-                } else if (fast) {
-                    Pack<XT, 4> sa, sb;
+            return spike_value<XT>(fired);
+        };
+        // One LIF step of a group: the lane's 8 sums arrive in accumulator layout (xin = rows 8 (gidx & 1) .. + 7 of its
+        // 32-row fragment, for its pixel). FAST: transposed through the wave's stage, then bias (+ residual), LIF, one wide
+        // spike store. General variant: bias (+ residual), LIF and a 2-byte store per row, in place.
+        auto lif_step_group = [&](int t, int gidx, bool row_ok, uint32_t row_off, const float (&bvv)[8], const float (&xin)[8], float (&v)[8]) __attribute__((always_inline)) {
+            XT* __restrict__ out_t = spikes + t * g.spike_step_stride + tile_off + row_off;
+            const XT* __restrict__ res_t = nullptr;
+            if (has_residual) res_t = static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), t)) + tile_off + row_off;
+            if constexpr (FAST) {
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) { sa.v[k] = sp.v[k]; sb.v[k] = sp.v[4 + k]; }
-                    if (okmask & 0x0fu) *reinterpret_cast<Pack<XT, 4>*>(out_t + pxoff[0]) = sa;
-                    if (okmask & 0xf0u) *reinterpret_cast<Pack<XT, 4>*>(out_t + pxoff[0] + 4) = sb;
+                for (int rr = 0; rr < 8; ++rr) stage_wr[((rr >> 2) * 8 + (rr & 3)) * kMmStagePitch] = xin[rr];
+                __builtin_amdgcn_wave_barrier();
+                const cv_f32x4 xlo = *reinterpret_cast<const cv_f32x4*>(stage_rd);
+                const cv_f32x4 xhi = *reinterpret_cast<const cv_f32x4*>(stage_rd + 4);
+                float x[8];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) { x[k] = xlo[k] + bvv[0]; x[4 + k] = xhi[k] + bvv[0]; }
+                if (has_residual && row_ok) {
+                    if (wide) {
+                        const Pack<XT, 8> rr8 = *reinterpret_cast<const Pack<XT, 8>*>(res_t + px0);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) x[k] += to_float(rr8.v[k]);
+                    } else {
+                        if (okmask & 0x0fu) {
+                            const Pack<XT, 4> ra = *reinterpret_cast<const Pack<XT, 4>*>(res_t + px0);
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) x[k] += to_float(ra.v[k]);
+                        }
+                        if (okmask & 0xf0u) {
+                            const Pack<XT, 4> rb = *reinterpret_cast<const Pack<XT, 4>*>(res_t + px0 + 4);
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) x[4 + k] += to_float(rb.v[k]);
+                        }
+                    }
+                }
+                Pack<XT, 8> sp;
+                if (analog) {   // uniform: no neuron, the sums themselves go out
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) sp.v[k] = from_float<XT>(x[k]);
                 } else {
 #pragma unroll
-                    for (int k = 0; k < 8; ++k)
-                        if (okmask & (1u << k)) out_t[pxoff[k]] = sp.v[k];
+                    for (int k = 0; k < 8; ++k) sp.v[k] = neuron(x[k], v[k]);
+                }
+                if (row_ok) {
+                    if (wide) {
+                        *reinterpret_cast<Pack<XT, 8>*>(out_t + px0) = sp;
+                    } else {
+                        Pack<XT, 4> sa, sb;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) { sa.v[k] = sp.v[k]; sb.v[k] = sp.v[4 + k]; }
+                        if (okmask & 0x0fu) *reinterpret_cast<Pack<XT, 4>*>(out_t + px0) = sa;
+                        if (okmask & 0xf0u) *reinterpret_cast<Pack<XT, 4>*>(out_t + px0 + 4) = sb;
+                    }
+                }
+            } else {
+                if (!row_ok) return;
+                const int oc = first_row(gidx);
+#pragma unroll
+                for (int rr = 0; rr < 8; ++rr) {
+                    if (oc + row_delta(rr) < g.Cout) {
+                        const uint32_t at = static_cast<uint32_t>(row_delta(rr) * po) + px0;
+                        float x = xin[rr] + bvv[rr];
+                        if (has_residual) x += to_float(res_t[at]);
+                        out_t[at] = analog ? from_float<XT>(x) : neuron(x, v[rr]);
+                    }
                 }
             }
         };
@@ -528,15 +539,15 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 for (int gidx = 0; gidx < 4; ++gidx) {
                     bool row_ok;
                     uint32_t row_off;
-                    float bvv, v[8];
+                    float bvv[8], v[8];
                     group_row(gidx, row_ok, row_off, bvv);
-                    load_membrane(row_ok, row_off, v);
+                    load_membrane(gidx, row_ok, row_off, v);
                     if constexpr (TT == 1) {
                         // One stage of input: a single timestep, or one analog frame that feeds all g.T timesteps.
                         float xin[8];
 #pragma unroll
                         for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[0][gidx >> 1][(gidx & 1) * 8 + rr];
-                        for (int t = 0; t < g.T; ++t) lif_step_group(t, row_ok, row_off, bvv, xin, v);
+                        for (int t = 0; t < g.T; ++t) lif_step_group(t, gidx, row_ok, row_off, bvv, xin, v);
                     } else {
 #pragma unroll
                         for (int t = 0; t < TT; ++t) {
@@ -544,11 +555,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                                 float xin[8];
 #pragma unroll
                                 for (int rr = 0; rr < 8; ++rr) xin[rr] = acc[t][gidx >> 1][(gidx & 1) * 8 + rr];
-                                lif_step_group(t, row_ok, row_off, bvv, xin, v);
+                                lif_step_group(t, gidx, row_ok, row_off, bvv, xin, v);
                             }
                         }
                     }
-                    store_membrane(row_ok, row_off, v);
+                    store_membrane(gidx, row_ok, row_off, v);
                 }
             }
         } else {
@@ -559,13 +570,13 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             const int wt = wave & ((1 << (g.wm_log2 + g.wn_log2)) - 1);
             bool row_ok[2];
             uint32_t row_off[2];
-            float bvv[2], v[2][8];
+            float bvv[2][8], v[2][8];
 #pragma unroll
             for (int gidx = 0; gidx < 4; ++gidx) {
                 const int owner = g.wk_log2 == 1 ? (gidx >> 1) : (gidx << (g.wk_log2 - 2));
                 if (owner == wk) {
                     group_row(gidx, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1]);
-                    load_membrane(row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
+                    load_membrane(gidx, row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
                 }
             }
 #pragma unroll
@@ -595,9 +606,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                             for (int k = 0; k < 4; ++k) { xin[k] = lo[k]; xin[4 + k] = hi[k]; }
                             if constexpr (TT == 1) {   // one stage of input feeds all g.T timesteps
                                 for (int ts = 0; ts < g.T; ++ts)
-                                    lif_step_group(ts, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
+                                    lif_step_group(ts, gidx, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
                             } else {
-                                lif_step_group(t, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
+                                lif_step_group(t, gidx, row_ok[gidx & 1], row_off[gidx & 1], bvv[gidx & 1], xin, v[gidx & 1]);
                             }
                         }
                     }
@@ -606,12 +617,14 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int gidx = 0; gidx < 4; ++gidx) {
                 const int owner = g.wk_log2 == 1 ? (gidx >> 1) : (gidx << (g.wk_log2 - 2));
-                if (owner == wk) store_membrane(row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
+                if (owner == wk) store_membrane(gidx, row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
             }
         }
         SNNF_MM_STAMP(11);
 #ifdef SNNF_MM_TRACE
+        if (trace_tile == 1 && threadIdx.x == 0 && blockIdx.x < 64) mm_trace[blockIdx.x * 16 + 15] = __builtin_amdgcn_s_memtime();
         trace_on = false;
+        ++trace_tile;
 #endif
         if (SK && next_tile) {
             int nih, niw;
