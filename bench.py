@@ -276,6 +276,19 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
             "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
 
 
+def _bandwidth_probe():
+    """What plain streaming kernels reach on this device, next to the published 8 TB/s: a 1 GiB device-to-device copy
+    (read + write) and a 1 GiB fill (write only), both far beyond the 256 MB last-level cache."""
+    import torch
+    n = 256 * 1024 * 1024
+    a = torch.empty(n, dtype=torch.float32, device="cuda:0").normal_()
+    b = torch.empty_like(a)
+    copy_ms, _ = _time_gpu(lambda: b.copy_(a), 10, 3)
+    fill_ms, _ = _time_gpu(lambda: b.fill_(1.0), 10, 3)
+    del a, b
+    return {"copy_1GiB_GBs": round(2 * n * 4 / (copy_ms * 1e-3) / 1e9, 1), "fill_1GiB_GBs": round(n * 4 / (fill_ms * 1e-3) / 1e9, 1)}
+
+
 MODEL_CONFIGS = {"resnet18": dict(batch=16, size=224, T=4), "vgg11": dict(batch=64, size=32, T=4)}
 
 
@@ -308,6 +321,21 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
     except Exception as exc:  # pragma: no cover - reported, the eager number stands
         ms_graph = None
         out["graph_error"] = str(exc)[:200]
+    # The same network through the FX temporal rewrite (trace of the T-step loop -> fused operator graph).
+    try:
+        from triton_snn_fusion_amd import fx_temporal_rewrite as R
+        wrapper = M.SingleStepModeLoopWrapper(M.build_network(name, seed=0), cfg["T"])
+        gm, stats = R.compile_temporal(wrapper, tail_first=True, device="cuda:0", dtype=dtype)
+        with torch.no_grad():
+            gm(x)
+            torch.cuda.synchronize()
+            ms_fx, _ = _time_gpu(lambda: gm(x), max(5, steps // 2), max(2, warmup // 2))
+            out["fx_rewrite"] = {"fused_groups": stats.temporal_conv_bn_lif_groups + stats.temporal_conv_bn_add_lif_groups
+                                 + stats.temporal_lif_avgpool_linear_groups, "skipped": len(stats.skipped),
+                                 "eager_launch_ms_per_forward": round(ms_fx, 4)}
+            out["fx_rewrite"]["graph_ms_per_forward"] = round(_time_graph(lambda: gm(x), steps, warmup), 4)
+    except Exception as exc:  # pragma: no cover - reported, the executor numbers stand
+        out.setdefault("fx_rewrite", {})["error"] = str(exc)[:200]
     best = ms_graph if ms_graph is not None else ms_eager
     out["ms_per_forward"] = round(best, 4)
     out["images_T_per_s"] = round(cfg["batch"] * cfg["T"] / (best * 1e-3), 1)
@@ -462,6 +490,13 @@ def main() -> int:
                                  "hbm": _roofline("hbm", nbytes, ms_step), "mfma": _roofline("mfma", flops, ms_step)}
         result["roofline"] = dict(kernels["linear_lif"]["hbm"], kernel="linear_lif")
     result["kernels"] = kernels
+    try:
+        probe = _bandwidth_probe()
+        result["hbm_probe"] = probe
+        if result["roofline"]["bound"] == "hbm":
+            result["roofline"]["frac_of_copy_probe"] = round(result["roofline"]["achieved"] / probe["copy_1GiB_GBs"], 4)
+    except Exception as exc:  # the probe is context, not part of the measurement
+        result["hbm_probe"] = {"error": str(exc)[:200]}
     try:
         result["graph_ms_per_step"] = round(_time_graph(prep.step, args.steps, args.warmup), 4)
     except Exception as exc:  # graph capture is a convenience measurement only

@@ -11,6 +11,7 @@ import torch.nn.functional as F
 
 from helpers import DEV, check, gen, q
 from oracle import snn_oracle as O
+from triton_snn_fusion_amd import fx_temporal_rewrite as R
 from triton_snn_fusion_amd import models as M
 
 BF16, F32 = torch.bfloat16, torch.float32
@@ -110,6 +111,82 @@ def test_network_shapes_follow_the_benchmark_configurations():
 
 
 # ---------------------------------------------------------------------------------------------------------------
+# FX temporal rewrite (CPU: the snn_custom operators evaluate the eager formulas there)
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("tail_first", [False, True])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_rewrite_graph_invariants_and_numerical_equality(name, tail_first):
+    T = 4
+    model = M.build_network(name, width=16, gain=5.0)
+    wrapper = M.SingleStepModeLoopWrapper(model, T)
+    x = torch.randn(2, 3, 64 if name == "resnet18" else 32, 64 if name == "resnet18" else 32, generator=gen(4))
+    with torch.no_grad():
+        want = wrapper(x)
+    traced = R.trace_single_step_loop(wrapper)
+    lifs = [n for n in traced.graph.nodes if R.is_custom_lif_state_node(n)]
+    assert len(lifs) == T * (8 if name == "vgg11" else 17)
+    assert all(n.v.dim() == 0 for n in model.modules() if isinstance(n, M.CustomStatefulIFNode))     # tracing left no proxies behind
+    gm, stats = R.compile_temporal(wrapper, tail_first=tail_first, batch_time=False)
+    S = torch.ops.snn_custom
+    targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+    n_conv = sum(t in (S.fused_temporal_conv_lif_state, S.fused_temporal_pointwise_conv_lif_state) for t in targets)
+    n_res = targets.count(S.fused_temporal_conv_add_lif_state)
+    n_tail = targets.count(S.fused_temporal_lif_avgpool_linear)
+    assert not any(R.is_custom_lif_state_node(n) for n in gm.graph.nodes), "every neuron call is inside a fused operator"
+    if name == "vgg11":
+        assert (n_conv, n_res, n_tail) == ((7, 0, 1) if tail_first else (8, 0, 0))
+    else:
+        assert (n_conv, n_res, n_tail) == ((9, 7, 1) if tail_first else (9, 8, 0))
+    assert stats.replaced_patterns == T * (8 if name == "vgg11" else 17) and not stats.skipped
+    # fused layers have no per-timestep Conv2d / BatchNorm2d calls left; LIF-free ones are called once per timestep
+    convs = [n for n in gm.graph.nodes if n.op == "call_module" and isinstance(gm.get_submodule(n.target), torch.nn.Conv2d)]
+    assert len(convs) == T * ({"vgg11": 0, "resnet18": 3}[name] + (1 if tail_first else 0))
+    # every fused operator takes its T inputs as a list of T nodes and starts from the scalar-zero membrane
+    for n in gm.graph.nodes:
+        if n.op == "call_function" and n.target in (S.fused_temporal_conv_lif_state, S.fused_temporal_conv_add_lif_state):
+            assert isinstance(n.args[0], (list, tuple)) and len(n.args[0]) == T
+            v0 = n.args[4] if n.target is S.fused_temporal_conv_add_lif_state else n.args[3]
+            assert v0.op == "get_attr" and getattr(gm, v0.target).dim() == 0
+    with torch.no_grad():
+        got = gm(x)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5), float((got - want).abs().max())
+    # Stateless layers batched over time: one call each instead of T, same result.
+    removed = R.batch_timestep_calls(gm)
+    modules = [n for n in gm.graph.nodes if n.op == "call_module"]
+    assert len(modules) == len({n.target for n in modules}), "every remaining layer is called once"
+    extra = (0 if tail_first else 1) + (1 if (tail_first and name == "resnet18") else 0)   # flatten before the classifier / pre-tail residual add
+    assert removed == T * (len(modules) + extra)
+    assert not any(n.op == "call_function" and n.target is torch.stack for n in gm.graph.nodes)
+    with torch.no_grad():
+        again = gm(x)
+    assert torch.allclose(again, want, rtol=1e-4, atol=1e-5), float((again - want).abs().max())
+
+
+def test_fx_rewrite_leaves_a_layer_alone_when_its_state_chain_is_broken():
+    """A neuron whose membrane is read between the steps (here: exported by the module) must not be fused."""
+    class Leaky(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.block = M.init_synthetic_(M.ConvBNNeuron(4, 8, 3, 1, 1), gain=5.0)
+
+        def forward(self, x):
+            a = self.block(x)
+            peek = self.block.sn.v          # the intermediate membrane escapes
+            b = self.block(x)
+            return a + b + peek.mean()
+
+    module = Leaky()
+    gm, stats = R.compile_temporal(module)
+    assert stats.replaced_patterns == 0 and len(stats.skipped) == 1 and "other users" in stats.skipped[0]
+    x = torch.randn(1, 4, 6, 6, generator=gen(8))
+    M.reset_lif_modules(module)
+    with torch.no_grad():
+        want = module(x)
+        M.reset_lif_modules(module)
+        assert torch.allclose(gm(x), want)
+
+
+# ---------------------------------------------------------------------------------------------------------------
 # Fused form (GPU)
 # ---------------------------------------------------------------------------------------------------------------
 def _fused(name, T=4, gain=5.0):
@@ -200,3 +277,24 @@ def test_fused_network_graph_replay_matches_eager_launches(hip_ops, name):
         torch.cuda.synchronize()
         assert torch.equal(static_out, want)
     assert hip_ops.get_fused_op_call_stats()["fallback"] == 0
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_rewritten_graph_runs_on_the_hip_kernels(hip_ops, name):
+    """compile on the CPU in fp32, move to the GPU in bf16: the rewritten graph calls the same fused operators with the
+    same operands as the hand-lowered executor (tail_first = the executor's lowering), so the logits agree closely (the
+    LIF-free convolutions differ: per-timestep framework calls here, one batched matrix-kernel call there)."""
+    T = 4
+    model, fused = _fused(name, T)
+    x = _frame(name)
+    gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16)
+    assert not stats.skipped
+    hip_ops.reset_fused_op_call_stats()
+    with torch.no_grad():
+        got = gm(x.to(DEV, BF16)).float().cpu()
+    stats_ops = hip_ops.get_fused_op_call_stats()
+    assert stats_ops["fallback"] == 0 and stats_ops["triton"] == (8 if name == "vgg11" else 17), stats_ops
+    want = fused(x).float().cpu()
+    cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
+    print(f"{name}: FX graph vs executor, cosine similarity of the logits {cos:.5f}")
+    assert cos > 0.8, cos

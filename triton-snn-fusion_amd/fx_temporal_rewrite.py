@@ -1,0 +1,537 @@
+"""Minimal temporal FX rewriter: T unrolled single-step iterations -> fused temporal operators.
+
+Counterpart of the reference's rewrite pipeline for the patterns the fused operators serve
+(compiler/fx_lif_temporal_rewrite.py: `collect_conv_bn_lif_state_patterns` :337, `collect_conv_bn_add_lif_state_patterns`
+:423, `collect_temporal_lif_avgpool_linear_patterns` :791, `group_temporal_patterns` :884, `check_temporal_state_chain`
+:929, `rewrite_temporal_conv_bn_lif_state_to_fused` :2037, residual :2214, tail :2745; BatchNorm folding
+compiler/fx_lif_rewrite.py:340-353). The reference obtains its graph from torch.compile and works on function-level
+nodes; this one traces a `SingleStepModeLoopWrapper`-style module with `torch.fx.symbolic_trace`, so convolutions,
+BatchNorms, pools and the classifier are `call_module` nodes and each neuron call is a
+`torch.ops.snn_custom.lif_forward_state` node whose membrane operand is the previous call's second output.
+
+Pipeline (`compile_temporal`):
+  1. `trace_single_step_loop`  - unrolls the T iterations; a neuron's first membrane is the scalar-zero constant.
+  2. collect                   - Conv2d -> BatchNorm2d -> LIF, Conv2d -> BatchNorm2d -> add(residual) -> LIF, and the tail
+                                 LIF -> AdaptiveAvgPool2d(1) -> flatten -> Linear -> running sum; one pattern per timestep.
+  3. group + check             - patterns of one layer (same conv and BN module) ordered by timestep; the state chain must be
+                                 v_getitem[t-1] -> v_prev[t] with a scalar-zero start, otherwise the layer is left alone.
+  4. rewrite                   - one fused operator node per layer over the list of its T inputs (operator chosen by
+                                 convolution kind: regular / pointwise / depthwise, as compiler/fx_lif_temporal_rewrite.py
+                                 :1625-1662), folded weights as graph attributes, per-timestep spikes as `spike_stack[t]`.
+The graph is then re-emitted in dependency order, which turns the time-major trace into layer-major execution.
+"""
+from __future__ import annotations
+
+import operator
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import torch
+import torch.fx as fx
+import torch.nn as nn
+
+from .workloads import fold_bn_into_conv_params
+
+
+def _lif_targets():
+    from .runtime import snn_custom_ops  # noqa: F401  (registers torch.ops.snn_custom)
+    return (torch.ops.snn_custom.lif_forward_state, torch.ops.snn_custom.lif_forward_state.default)
+
+
+def is_custom_lif_state_node(node: fx.Node) -> bool:
+    return node.op == "call_function" and node.target in _lif_targets()
+
+
+def _is_add_node(node: fx.Node) -> bool:
+    return node.op == "call_function" and node.target in (operator.add, operator.iadd, torch.add)
+
+
+def _module_of(gm: fx.GraphModule, node: fx.Node, kind) -> Optional[nn.Module]:
+    if node.op != "call_module":
+        return None
+    mod = gm.get_submodule(node.target)
+    return mod if isinstance(mod, kind) else None
+
+
+def find_tuple_getitems(node: fx.Node) -> Dict[int, fx.Node]:
+    out: Dict[int, fx.Node] = {}
+    for user in node.users:
+        if user.op == "call_function" and user.target is operator.getitem and isinstance(user.args[1], int):
+            out[user.args[1]] = user
+    return out
+
+
+def _is_scalar_zero(gm: fx.GraphModule, arg) -> bool:
+    """The membrane a neuron starts from: a 0-dim zero tensor held by the traced module."""
+    if isinstance(arg, fx.Node) and arg.op == "get_attr":
+        value = gm
+        for part in arg.target.split("."):
+            value = getattr(value, part)
+        return isinstance(value, torch.Tensor) and value.dim() == 0 and float(value) == 0.0
+    return False
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Tracing
+# ---------------------------------------------------------------------------------------------------------------
+def trace_single_step_loop(wrapper: nn.Module) -> fx.GraphModule:
+    """symbolic_trace of a module that calls a single-step network T times (the loop unrolls). Neuron modules are traced
+    through a forward that skips the shape check of the state (a 0-dim membrane means zeros to the operator anyway): the
+    first call of a neuron takes one shared scalar-zero constant, later calls the previous call's second output. The
+    modules are reset afterwards."""
+    from .models import CustomStatefulIFNode, reset_custom_stateful_lif_modules
+    from .runtime import snn_custom_ops  # noqa: F401  (registers torch.ops.snn_custom)
+
+    zero = torch.zeros(())
+
+    def traced_forward(self, x):
+        v_prev = self.v if isinstance(self.v, fx.Proxy) else zero
+        spike, self.v = torch.ops.snn_custom.lif_forward_state(x, v_prev, self.v_threshold, self.v_reset, self.tau, self.detach_reset)
+        return spike
+
+    reset_custom_stateful_lif_modules(wrapper)
+    original = CustomStatefulIFNode.forward
+    CustomStatefulIFNode.forward = traced_forward
+    try:
+        gm = fx.symbolic_trace(wrapper)
+    finally:
+        CustomStatefulIFNode.forward = original
+        reset_custom_stateful_lif_modules(wrapper)
+    return gm
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Patterns
+# ---------------------------------------------------------------------------------------------------------------
+@dataclass
+class TemporalPattern:
+    layer_id: str
+    timestep_index: int
+    conv_node: fx.Node
+    bn_node: fx.Node
+    lif_node: fx.Node
+    spike_getitem: Optional[fx.Node]
+    v_getitem: Optional[fx.Node]
+    conv_input: fx.Node
+    v_prev_node: object
+    lif_params: Tuple
+    add_node: Optional[fx.Node] = None          # residual form: lif(add(bn(conv(x)), residual))
+    residual_node: Optional[fx.Node] = None
+
+
+@dataclass
+class TemporalLifAvgPoolLinearPattern:
+    layer_id: str
+    timestep_index: int
+    lif_node: fx.Node
+    input_node: fx.Node
+    v_prev_node: object
+    spike_getitem: fx.Node
+    v_getitem: Optional[fx.Node]
+    pool_node: fx.Node
+    flatten_node: fx.Node
+    linear_node: fx.Node
+    acc_node: fx.Node
+    acc_prev: object
+    lif_params: Tuple
+
+
+@dataclass
+class TemporalGroup:
+    layer_id: str
+    patterns: List = field(default_factory=list)
+
+
+def _conv_bn_of(gm: fx.GraphModule, node) -> Optional[Tuple[fx.Node, fx.Node]]:
+    """(conv_node, bn_node) when `node` is BatchNorm2d(Conv2d(x)) with the convolution feeding only the BatchNorm."""
+    if not isinstance(node, fx.Node) or _module_of(gm, node, nn.BatchNorm2d) is None:
+        return None
+    conv = node.args[0]
+    if not isinstance(conv, fx.Node) or _module_of(gm, conv, nn.Conv2d) is None or len(conv.users) != 1:
+        return None
+    if gm.get_submodule(node.target).training:
+        return None
+    return conv, node
+
+
+def _lif_state_is_usable(node: fx.Node) -> Tuple[bool, str]:
+    if len(node.args) < 6 or node.kwargs:
+        return False, "unsupported lif args"
+    if not all(isinstance(a, (int, float, bool)) for a in node.args[2:6]):
+        return False, "lif parameters are not constants"
+    extra = [u for u in node.users if not (u.op == "call_function" and u.target is operator.getitem)]
+    return (not extra), ("lif output used as a tuple" if extra else "")
+
+
+def _collect(gm: fx.GraphModule, residual: bool) -> List[TemporalPattern]:
+    counts: Dict[str, int] = {}
+    patterns: List[TemporalPattern] = []
+    for node in gm.graph.nodes:
+        if not is_custom_lif_state_node(node) or not _lif_state_is_usable(node)[0]:
+            continue
+        source = node.args[0]
+        add_node = residual_node = None
+        if residual:
+            if not isinstance(source, fx.Node) or not _is_add_node(source) or len(source.users) != 1:
+                continue
+            a, b = source.args[0], source.args[1]
+            pair = _conv_bn_of(gm, a)
+            other = b
+            if pair is None:
+                pair, other = _conv_bn_of(gm, b), a
+            if pair is None or not isinstance(other, fx.Node) or len(pair[1].users) != 1:
+                continue
+            add_node, residual_node = source, other
+        else:
+            pair = _conv_bn_of(gm, source)
+            if pair is None or len(pair[1].users) != 1:
+                continue
+        conv_node, bn_node = pair
+        layer_id = f"conv={conv_node.target}|bn={bn_node.target}|params={tuple(node.args[2:6])!r}"
+        getitems = find_tuple_getitems(node)
+        t = counts.get(layer_id, 0)
+        counts[layer_id] = t + 1
+        patterns.append(TemporalPattern(layer_id, t, conv_node, bn_node, node, getitems.get(0), getitems.get(1),
+                                        conv_node.args[0], node.args[1], tuple(node.args[2:6]), add_node, residual_node))
+    return patterns
+
+
+def collect_conv_bn_lif_state_patterns(gm: fx.GraphModule) -> List[TemporalPattern]:
+    return _collect(gm, residual=False)
+
+
+def collect_conv_bn_add_lif_state_patterns(gm: fx.GraphModule) -> List[TemporalPattern]:
+    return _collect(gm, residual=True)
+
+
+def _single_user(node: Optional[fx.Node]) -> Optional[fx.Node]:
+    if node is None or len(node.users) != 1:
+        return None
+    return next(iter(node.users))
+
+
+def collect_temporal_lif_avgpool_linear_patterns(gm: fx.GraphModule, excluded_lif_nodes=None) -> List[TemporalLifAvgPoolLinearPattern]:
+    excluded = set(excluded_lif_nodes or [])
+    counts: Dict[str, int] = {}
+    patterns: List[TemporalLifAvgPoolLinearPattern] = []
+    for node in gm.graph.nodes:
+        if node in excluded or not is_custom_lif_state_node(node) or not _lif_state_is_usable(node)[0]:
+            continue
+        getitems = find_tuple_getitems(node)
+        pool = _single_user(getitems.get(0))
+        pool_mod = _module_of(gm, pool, nn.AdaptiveAvgPool2d) if pool is not None else None
+        if pool_mod is None or tuple(pool_mod.output_size if isinstance(pool_mod.output_size, (tuple, list)) else (pool_mod.output_size,) * 2) != (1, 1):
+            continue
+        flatten = _single_user(pool)
+        if flatten is None or not (flatten.op == "call_function" and flatten.target is torch.flatten and tuple(flatten.args[1:]) in ((1,), (1, -1))):
+            continue
+        linear = _single_user(flatten)
+        if linear is None or _module_of(gm, linear, nn.Linear) is None:
+            continue
+        acc = _single_user(linear)
+        if acc is None or not _is_add_node(acc):
+            continue
+        acc_prev = acc.args[1] if acc.args[0] is linear else acc.args[0]
+        layer_id = f"lif_avgpool_linear|fc={linear.target}|params={tuple(node.args[2:6])!r}"
+        t = counts.get(layer_id, 0)
+        counts[layer_id] = t + 1
+        patterns.append(TemporalLifAvgPoolLinearPattern(layer_id, t, node, node.args[0], node.args[1], getitems[0], getitems.get(1),
+                                                        pool, flatten, linear, acc, acc_prev, tuple(node.args[2:6])))
+    return patterns
+
+
+def group_temporal_patterns(patterns) -> List[TemporalGroup]:
+    grouped: Dict[str, List] = {}
+    for p in patterns:
+        grouped.setdefault(p.layer_id, []).append(p)
+    return [TemporalGroup(k, sorted(v, key=lambda p: p.timestep_index)) for k, v in grouped.items()]
+
+
+def check_temporal_state_chain(gm: fx.GraphModule, patterns) -> Tuple[bool, str]:
+    """The membrane of step t must be exactly the second output of step t-1, the first one the scalar zero, and nothing
+    else may read the intermediate membranes."""
+    if not _is_scalar_zero(gm, patterns[0].v_prev_node):
+        return False, f"{patterns[0].lif_node.name} does not start from the scalar-zero membrane"
+    for prev, nxt in zip(patterns, patterns[1:]):
+        if prev.v_getitem is None or nxt.v_prev_node is not prev.v_getitem:
+            return False, f"{prev.lif_node.name} membrane does not feed {nxt.lif_node.name} v_prev"
+        if len(prev.v_getitem.users) != 1:
+            return False, f"{prev.v_getitem.name} has other users"
+    last = patterns[-1].v_getitem
+    if last is not None and len(last.users) != 0:
+        return False, f"{last.name} (final membrane) is read by the graph"
+    return True, ""
+
+
+def check_temporal_lif_avgpool_linear_state_and_acc_chain(gm: fx.GraphModule, patterns) -> Tuple[bool, str]:
+    ok, reason = check_temporal_state_chain(gm, patterns)
+    if not ok:
+        return ok, reason
+    if not (isinstance(patterns[0].acc_prev, (int, float)) and patterns[0].acc_prev == 0):
+        return False, "the running sum does not start from 0"
+    for prev, nxt in zip(patterns, patterns[1:]):
+        if nxt.acc_prev is not prev.acc_node:
+            return False, f"{prev.acc_node.name} does not feed {nxt.acc_node.name}"
+        if len(prev.acc_node.users) != 1:
+            return False, f"{prev.acc_node.name} has other users"
+    return True, ""
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Rewrite
+# ---------------------------------------------------------------------------------------------------------------
+@dataclass
+class RewriteStats:
+    temporal_conv_bn_lif_groups: int = 0
+    temporal_conv_bn_add_lif_groups: int = 0
+    temporal_lif_avgpool_linear_groups: int = 0
+    replaced_patterns: int = 0
+    batched_timestep_calls: int = 0
+    skipped: List[str] = field(default_factory=list)
+
+
+def classify_conv_kind(conv: nn.Conv2d) -> str:
+    if conv.groups == conv.in_channels == conv.out_channels and conv.groups > 1:
+        return "depthwise"
+    if conv.groups == 1 and tuple(conv.kernel_size) == (1, 1) and tuple(conv.stride) == (1, 1) and tuple(conv.padding) == (0, 0):
+        return "pointwise"
+    return "regular"
+
+
+def _register(gm: fx.GraphModule, name: str, value: torch.Tensor) -> str:
+    base, i = name, 0
+    while hasattr(gm, name):
+        i += 1
+        name = f"{base}_{i}"
+    gm.register_buffer(name, value, persistent=False)
+    return name
+
+
+def _folded_params(gm: fx.GraphModule, group: TemporalGroup, index: int) -> Tuple[str, str, nn.Conv2d]:
+    conv = gm.get_submodule(group.patterns[0].conv_node.target)
+    bn = gm.get_submodule(group.patterns[0].bn_node.target)
+    with torch.no_grad():
+        w, b = fold_bn_into_conv_params(conv.weight.float(), conv.bias, bn.running_mean.float(), bn.running_var.float(),
+                                        None if bn.weight is None else bn.weight.float(), None if bn.bias is None else bn.bias.float(), bn.eps)
+        w = w.to(conv.weight.dtype).contiguous()
+        b = b.to(conv.weight.dtype).contiguous()
+    return _register(gm, f"fused_weight_{index}", w), _register(gm, f"fused_bias_{index}", b), conv
+
+
+def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] = None, tail_first: bool = False) -> RewriteStats:
+    """Replaces every layer whose T patterns pass the state-chain check by one fused temporal operator node."""
+    stats = stats or RewriteStats()
+    S = torch.ops.snn_custom
+    graph = gm.graph
+    output_node = next(n for n in graph.nodes if n.op == "output")
+    device = next((p.device for p in gm.parameters()), torch.device("cpu"))
+    zero_name = _register(gm, "chronos_zero_membrane", torch.zeros((), dtype=torch.float32, device=device))
+    index = 0
+    claimed = set()
+    tail_groups = []
+    if tail_first:
+        # The neuron in front of the classifier belongs to the tail operator; its convolution stays a plain layer.
+        tail_groups = group_temporal_patterns(collect_temporal_lif_avgpool_linear_patterns(gm))
+        for group in tail_groups:
+            if check_temporal_lif_avgpool_linear_state_and_acc_chain(gm, group.patterns)[0]:
+                claimed.update(p.lif_node for p in group.patterns)
+
+    conv_groups = [(g, False) for g in group_temporal_patterns(collect_conv_bn_lif_state_patterns(gm))]
+    conv_groups += [(g, True) for g in group_temporal_patterns(collect_conv_bn_add_lif_state_patterns(gm))]
+    for group, residual in conv_groups:
+        if any(p.lif_node in claimed for p in group.patterns):
+            continue
+        ok, reason = check_temporal_state_chain(gm, group.patterns)
+        if not ok:
+            stats.skipped.append(f"{group.layer_id}: {reason}")
+            continue
+        w_name, b_name, conv = _folded_params(gm, group, index)
+        index += 1
+        kind = classify_conv_kind(conv)
+        # Operands are read from the nodes now: an earlier rewrite may have redirected them to its spike_stack[t].
+        xs = [p.conv_node.args[0] for p in group.patterns]
+        residuals = [next(a for a in p.add_node.args if a is not p.bn_node) for p in group.patterns] if residual else None
+        # New nodes go in front of the output; the graph is re-emitted in dependency order at the end.
+        with graph.inserting_before(output_node):
+            w_node = graph.get_attr(w_name)
+            b_node = graph.get_attr(b_name)
+            v0 = graph.get_attr(zero_name)
+        geometry = (list(conv.stride), list(conv.padding), list(conv.dilation), int(conv.groups))
+        lif = tuple(group.patterns[0].lif_params)
+        if residual:
+            op = S.fused_temporal_conv_add_lif_state_depthwise if kind == "depthwise" else S.fused_temporal_conv_add_lif_state
+            args = (xs, residuals, w_node, b_node, v0, *geometry, *lif)
+        else:
+            op = {"regular": S.fused_temporal_conv_lif_state, "pointwise": S.fused_temporal_pointwise_conv_lif_state,
+                  "depthwise": S.fused_temporal_depthwise_conv_lif_state}[kind]
+            args = (xs, w_node, b_node, v0, *geometry, *lif)
+        with graph.inserting_before(output_node):
+            fused = graph.call_function(op, args)
+            spike_stack = graph.call_function(operator.getitem, (fused, 0))
+            for p in group.patterns:
+                if p.spike_getitem is not None:
+                    spike_t = graph.call_function(operator.getitem, (spike_stack, p.timestep_index))
+                    p.spike_getitem.replace_all_uses_with(spike_t)
+                claimed.add(p.lif_node)
+        if residual:
+            stats.temporal_conv_bn_add_lif_groups += 1
+        else:
+            stats.temporal_conv_bn_lif_groups += 1
+        stats.replaced_patterns += len(group.patterns)
+
+    if not tail_first:
+        tail_groups = group_temporal_patterns(collect_temporal_lif_avgpool_linear_patterns(gm, excluded_lif_nodes=claimed))
+    for group in tail_groups:
+        ok, reason = check_temporal_lif_avgpool_linear_state_and_acc_chain(gm, group.patterns)
+        if not ok:
+            stats.skipped.append(f"{group.layer_id}: {reason}")
+            continue
+        fc = gm.get_submodule(group.patterns[0].linear_node.target)
+        w_name = _register(gm, "fused_fc_weight", fc.weight.detach().contiguous())
+        b_name = _register(gm, "fused_fc_bias", fc.bias.detach().contiguous() if fc.bias is not None else torch.empty(0, dtype=fc.weight.dtype, device=fc.weight.device))
+        xs = [p.lif_node.args[0] for p in group.patterns]
+        with graph.inserting_before(output_node):
+            x_seq = graph.call_function(torch.stack, (xs,))
+            w_node = graph.get_attr(w_name)
+            b_node = graph.get_attr(b_name)
+            v0 = graph.get_attr(zero_name)
+            fused = graph.call_function(S.fused_temporal_lif_avgpool_linear, (x_seq, v0, w_node, b_node, *group.patterns[0].lif_params))
+            out_sum = graph.call_function(operator.getitem, (fused, 0))
+        group.patterns[-1].acc_node.replace_all_uses_with(out_sum)
+        stats.temporal_lif_avgpool_linear_groups += 1
+        stats.replaced_patterns += len(group.patterns)
+
+    _emit_in_dependency_order(gm)
+    gm.graph.lint()
+    gm.recompile()
+    return stats
+
+
+_TIME_BATCHABLE = (nn.Conv2d, nn.BatchNorm2d, nn.MaxPool2d, nn.AvgPool2d, nn.AdaptiveAvgPool2d, nn.Identity, nn.Linear)
+
+
+def batch_timestep_calls(gm: fx.GraphModule) -> int:
+    """Stateless layers that the trace applies once per timestep to `stack[t]`, t = 0..T-1, of one [T, N, ...] tensor
+    (pools, LIF-free convolutions and their BatchNorm, residual adds, flatten, the classifier) are applied once to the T*N frames
+    instead (the role of the reference's `_batched_tn` operator variants). Repeats until nothing changes, so chains such
+    as Conv2d -> BatchNorm2d batch link by link. Returns the number of per-timestep calls removed."""
+    removed = 0
+    changed = True
+    while changed:
+        changed = False
+        graph = gm.graph            # re-emission below replaces the graph object
+        groups: Dict[Tuple, Dict[int, fx.Node]] = {}
+        for node in graph.nodes:
+            key = None
+            if node.op == "call_module" and len(node.args) == 1 and not node.kwargs:
+                mod = gm.get_submodule(node.target)
+                if isinstance(mod, _TIME_BATCHABLE) and not (isinstance(mod, nn.BatchNorm2d) and mod.training):
+                    key = ("module", node.target)
+            elif node.op == "call_function" and node.target is torch.flatten and tuple(node.args[1:]) == (1,) and not node.kwargs:
+                key = ("flatten",)
+            elif _is_add_node(node) and len(node.args) == 2 and not node.kwargs:
+                key = ("add",)
+            if key is None:
+                continue
+            sources = node.args[:2] if key[0] == "add" else node.args[:1]
+            if not all(isinstance(src, fx.Node) and src.op == "call_function" and src.target is operator.getitem
+                       and isinstance(src.args[1], int) and isinstance(src.args[0], fx.Node) for src in sources):
+                continue
+            if len({src.args[1] for src in sources}) != 1:
+                continue    # operands of different timesteps
+            groups.setdefault(key + tuple(src.args[0] for src in sources), {})[sources[0].args[1]] = node
+        for key, members in groups.items():
+            stacks = key[2:] if key[0] == "module" else key[1:]
+            stack = stacks[0]
+            T = len(members)
+            complete = T >= 2 and sorted(members) == list(range(T))
+            for st in stacks:
+                steps = {u.args[1] for u in st.users if u.op == "call_function" and u.target is operator.getitem}
+                complete = complete and steps == set(range(T))
+            if not complete:
+                continue    # not every timestep of the stack goes through this layer
+            first = min(members.values(), key=lambda n: list(graph.nodes).index(n)) if key[0] == "add" else members[0]
+            with graph.inserting_before(first):
+                if key[0] == "module":
+                    flat = graph.call_method("flatten", (stack, 0, 1))
+                    y = graph.call_module(key[1], (flat,))
+                    y_seq = graph.call_method("unflatten", (y, 0, (T, -1)))
+                elif key[0] == "add":
+                    y_seq = graph.call_function(operator.add, (stacks[0], stacks[1]))
+                else:
+                    y_seq = graph.call_function(torch.flatten, (stack, 2))
+            for t, node in members.items():
+                with graph.inserting_after(y_seq):
+                    step = graph.call_function(operator.getitem, (y_seq, t))
+                node.replace_all_uses_with(step)
+            removed += T
+            changed = True
+        if changed:
+            _emit_in_dependency_order(gm)
+    # stack([y[0], ..., y[T-1]]) of one [T, ...] tensor is that tensor
+    for node in list(gm.graph.nodes):
+        if node.op == "call_function" and node.target is torch.stack and len(node.args) == 1 and not node.kwargs:
+            parts = node.args[0]
+            if (isinstance(parts, (list, tuple)) and parts and all(isinstance(p, fx.Node) and p.op == "call_function" and p.target is operator.getitem for p in parts)
+                    and len({p.args[0] for p in parts}) == 1 and [p.args[1] for p in parts] == list(range(len(parts)))):
+                whole = parts[0].args[0]
+                steps = {u.args[1] for u in whole.users if u.op == "call_function" and u.target is operator.getitem}
+                if steps == set(range(len(parts))):
+                    node.replace_all_uses_with(whole)
+    _emit_in_dependency_order(gm)
+    gm.graph.lint()
+    gm.recompile()
+    return removed
+
+
+def _emit_in_dependency_order(gm: fx.GraphModule) -> None:
+    """Rebuilds the graph from its output backwards: dead nodes (the replaced per-timestep chains) disappear and every
+    node lands after its operands, whatever position it was inserted at."""
+    old = gm.graph
+    new = fx.Graph()
+    env: Dict[fx.Node, fx.Node] = {}
+    for node in old.nodes:
+        if node.op == "placeholder":
+            env[node] = new.node_copy(node, lambda n: env[n])
+
+    def emit(node: fx.Node) -> fx.Node:
+        stack = [node]
+        while stack:
+            top = stack[-1]
+            if top in env:
+                stack.pop()
+                continue
+            pending = [a for a in top.all_input_nodes if a not in env]
+            if pending:
+                stack.extend(pending)
+                continue
+            env[top] = new.node_copy(top, lambda n: env[n])
+            stack.pop()
+        return env[node]
+
+    output = next(n for n in old.nodes if n.op == "output")
+    for dep in output.all_input_nodes:
+        emit(dep)
+    new.output(fx.node.map_arg(output.args[0], lambda n: env[n]))
+    gm.graph = new
+
+
+def compile_temporal(wrapper: nn.Module, tail_first: bool = False, device=None, dtype: Optional[torch.dtype] = None,
+                     batch_time: bool = True) -> Tuple[fx.GraphModule, RewriteStats]:
+    """Traces `wrapper` (a module that runs a single-step spiking network T times on the same input and averages) and
+    rewrites it to fused temporal operators. BatchNorm is folded with the parameters as they are at call time (fold in
+    fp32, before any cast); `device` / `dtype` then move and cast the rewritten module (weights and activations in
+    `dtype`, the membranes stay fp32). `tail_first`: give the neuron in front of the classifier to the
+    LIF -> AvgPool -> Linear operator (its convolution then stays a plain layer); by default the convolution patterns
+    claim it, as in the reference, whose tail rewrite only sees the neurons the convolution rewrites left over.
+    `batch_time`: also merge the per-timestep calls of stateless layers into one call over T*N frames."""
+    gm = trace_single_step_loop(wrapper)
+    stats = rewrite_temporal_to_fused(gm, tail_first=tail_first)
+    if batch_time:
+        stats.batched_timestep_calls = batch_timestep_calls(gm)
+    if device is not None or dtype is not None:
+        gm.to(device=device, dtype=dtype)
+        for name, buf in list(gm.named_buffers()):
+            if name.startswith("chronos_zero_membrane") or (buf.dim() == 0 and name.startswith("_tensor_constant")):
+                setattr(gm, name, torch.zeros((), dtype=torch.float32, device=buf.device))
+    return gm, stats
