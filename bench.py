@@ -306,13 +306,13 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
     net(frame)
     torch.cuda.synchronize()
     fused_calls = sum(1 for e in net.record if e["kind"] in ("conv_lif", "tail"))
-    library_calls = sum(1 for e in net.record if e["kind"] == "pool" or (e["kind"] == "plain_conv" and not e["native"]))
-    fused_calls += sum(1 for e in net.record if e["kind"] == "plain_conv" and e["native"])
+    library_calls = sum(1 for e in net.record if e["kind"] in ("pool", "plain_conv") and not e["native"])
+    fused_calls += sum(1 for e in net.record if e["kind"] in ("pool", "plain_conv") and e["native"])
     net.record = None
     x = net._prepare(frame)
     ms_eager, wall = _time_gpu(lambda: net(x), max(5, steps // 2), max(2, warmup // 2))
     out = {"workload": f"{name}_end_to_end", "T": cfg["T"], "batch": cfg["batch"], "input": [cfg["batch"], 3, cfg["size"], cfg["size"]],
-           "fused_operator_calls": fused_calls, "pytorch_operator_calls": library_calls,
+           "libsnnf_calls": fused_calls, "pytorch_operator_calls": library_calls,
            "eager_launch_ms_per_forward": round(ms_eager, 4), "host_ms_per_forward": round(wall, 4)}
     try:
         replay, _, _ = net.capture(frame)

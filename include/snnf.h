@@ -154,6 +154,15 @@ int snnf_conv_bias(const void* const* xs, const void* const* residuals /* nullab
                    int stride_h, int stride_w, int pad_h, int pad_w,
                    void* out, int64_t out_step_stride, void* stream);
 
+/* 2-D pooling of `planes` independent H x W planes (NCHW with planes = N * C, or T * N * C for a spike sequence):
+ * max 3x3 stride 2, max 2x2 stride 2 (padding <= kernel / 2, padded positions never win) and average 2x2 stride 2
+ * (no padding), floor output size. No fused operator of the reference corresponds to it: pooling layers stay ordinary
+ * framework calls between its fused operators (e.g. the stem's max pool and the 2x2 pools of the VGG / ResNet models in
+ * benchmarks/validate_chronos_baselines.py:748-790); this is the same layer for hosts that drive libsnnf directly.
+ *   x : [planes, H, W] x_dtype;  y : [planes, Ho, Wo] x_dtype */
+int snnf_pool2d(const void* x, void* y, int64_t planes, int H, int W, int kernel, int stride, int pad, int is_max,
+                int x_dtype, void* stream);
+
 /* Describes what the most recent snnf_conv_lif / snnf_conv_bias call on this thread selected: kernel family, timesteps per launch, tile
  * and wave decomposition, LDS bytes, grid ("key=value" pairs, empty before the first call). Plays the role of the
  * reference's get_autotune_best_config (kernels/benchmark_conv_lif_temporal_general.py:1332-1369), whose result the

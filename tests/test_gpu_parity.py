@@ -459,6 +459,34 @@ def test_conv_plan_is_reported(hip_ops):
     assert any("BTILE_T=4" in key for key in configs), configs
 
 
+@pytest.mark.parametrize("dtype", [BF16, F16, F32])
+@pytest.mark.parametrize("kind,k,s,p,shape", [("max", 3, 2, 1, (4, 2, 8, 112, 112)), ("max", 3, 2, 1, (3, 5, 9, 11)), ("max", 2, 2, 0, (2, 3, 7, 10)),
+                                              ("avg", 2, 2, 0, (4, 2, 16, 32, 32)), ("avg", 2, 2, 0, (3, 5, 7, 9)), ("max", 3, 2, 0, (2, 2, 3, 3)), ("max", 2, 2, 0, (2, 3, 8, 16)), ("max", 3, 2, 1, (5, 3, 14, 24))])
+def test_pool2d_matches_the_framework_pooling_exactly(snnf_lib, dtype, kind, k, s, p, shape):
+    """snnf_pool2d on spikes and on analog values: max pooling selects, 2x2 averaging of spikes is exact in every dtype."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd.runtime.hip_pool_backend import pool_config, run_hip_pool2d
+    g = gen(1500 + k + shape[-1])
+    x = spikes(shape, 0.3, g) if kind == "avg" else q(torch.randn(shape, generator=g), dtype)
+    module = torch.nn.MaxPool2d(k, s, p) if kind == "max" else torch.nn.AvgPool2d(k)
+    assert pool_config(module) == (kind == "max", k, s, p)
+    want = module(x.reshape(-1, 1, shape[-2], shape[-1])).reshape(*shape[:-2], -1, (shape[-1] + 2 * p - k) // s + 1)
+    got = run_hip_pool2d(dev(x, dtype), kind == "max", k, s, p)
+    assert got.dtype == dtype and tuple(got.shape) == tuple(want.shape)
+    assert torch.equal(got.float().cpu(), want)
+
+
+def test_pool2d_rejects_other_windows(snnf_lib):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd.runtime.hip_pool_backend import pool_config, run_hip_pool2d
+    assert pool_config(torch.nn.AvgPool2d(3)) is None and pool_config(torch.nn.MaxPool2d(3, 1, 1)) is None
+    assert pool_config(torch.nn.MaxPool2d(3, 2, 1, ceil_mode=True)) is None
+    with pytest.raises(RuntimeError, match="unsupported_kernel"):
+        run_hip_pool2d(torch.zeros(2, 8, 8, device=DEV, dtype=BF16), False, 3, 3, 0)
+
+
 def test_conv_and_linear_known_answers_exact(hip_ops):
     """tests/golden/conv_kat.json: exact sums (multiples of 1/8), so bf16 matrix operands must reproduce them bit for
     bit. An integrate-and-fire neuron (tau <= 1) with an unreachable threshold makes v_out the convolution output."""

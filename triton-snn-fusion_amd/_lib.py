@@ -43,6 +43,7 @@ SIGNATURES = {
     "snnf_conv_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "snnf_conv_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i64,
                            _vp, _f, _f, _f, _vp]),
+    "snnf_pool2d": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "snnf_conv_bias": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
 }
 

@@ -275,6 +275,7 @@ class _FusedNetwork(nn.Module):
         self.zero_v = torch.zeros((), dtype=v_dtype, device=self.device_)
         self.record: Optional[List[Dict]] = None
         self.native_plain_conv = True        # False: LIF-free convolutions always go to the framework's convolution
+        self.native_pool = True              # False: pooling layers always go to the framework's modules
         self._graph = None
 
     # -- operator calls ------------------------------------------------------------------------------------------
@@ -315,9 +316,16 @@ class _FusedNetwork(nn.Module):
         return y
 
     def pooled(self, name: str, x_seq: torch.Tensor, pool: nn.Module) -> torch.Tensor:
-        y = pool(x_seq.flatten(0, 1))
-        y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
-        self._log(kind="pool", name=name, x=x_seq, pool=pool, y=y)
+        """Pooling of all T*N frames at once: the HIP pooling kernel for the window shapes it has, the module itself
+        otherwise (and on CPU tensors)."""
+        from .runtime.hip_pool_backend import pool_config, run_hip_pool2d
+        config = pool_config(pool) if (x_seq.is_cuda and self.native_pool) else None
+        if config is not None:
+            y = run_hip_pool2d(x_seq, *config)
+        else:
+            y = pool(x_seq.flatten(0, 1))
+            y = y.view(x_seq.shape[0], x_seq.shape[1], *y.shape[1:])
+        self._log(kind="pool", name=name, x=x_seq, pool=pool, y=y, native=config is not None)
         return y
 
     def tail(self, x_seq: torch.Tensor, lif, fc_weight, fc_bias) -> torch.Tensor:
