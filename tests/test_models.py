@@ -154,8 +154,11 @@ def test_fx_rewrite_graph_invariants_and_numerical_equality(name, tail_first):
     removed = R.batch_timestep_calls(gm)
     modules = [n for n in gm.graph.nodes if n.op == "call_module"]
     assert len(modules) == len({n.target for n in modules}), "every remaining layer is called once"
-    extra = (0 if tail_first else 1) + (1 if (tail_first and name == "resnet18") else 0)   # flatten before the classifier / pre-tail residual add
-    assert removed == T * (len(modules) + extra)
+    assert removed > 0 and removed % T == 0
+    functions = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+    assert functions.count(R.pooled_frames) == (4 if name == "vgg11" else 1)                       # one call per pooling layer
+    assert functions.count(R.conv_bias_frames) == (3 if name == "resnet18" else 0) + (1 if tail_first else 0)   # LIF-free Conv+BN, folded
+    assert not any(isinstance(gm.get_submodule(n.target), (torch.nn.Conv2d, torch.nn.BatchNorm2d)) for n in modules)
     assert not any(n.op == "call_function" and n.target is torch.stack for n in gm.graph.nodes)
     with torch.no_grad():
         again = gm(x)

@@ -29,7 +29,9 @@ from typing import Dict, List, Optional, Tuple
 import torch
 import torch.fx as fx
 import torch.nn as nn
+import torch.nn.functional as F
 
+from .runtime.hip_pool_backend import pool_config
 from .workloads import fold_bn_into_conv_params
 
 
@@ -407,7 +409,45 @@ def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] 
     return stats
 
 
+def pooled_frames(x_seq: torch.Tensor, is_max: bool, kernel: int, stride: int, padding: int) -> torch.Tensor:
+    """Pooling of a [T, N, C, H, W] sequence: the HIP pooling kernel on the GPU, the framework's pooling on CPU tensors."""
+    if x_seq.is_cuda:
+        from .runtime.hip_pool_backend import run_hip_pool2d
+        return run_hip_pool2d(x_seq, is_max, kernel, stride, padding)
+    flat = x_seq.flatten(0, 1)
+    y = F.max_pool2d(flat, kernel, stride, padding) if is_max else F.avg_pool2d(flat, kernel, stride, padding)
+    return y.unflatten(0, (x_seq.shape[0], -1))
+
+
+def conv_bias_frames(x_seq: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, stride, padding) -> torch.Tensor:
+    """LIF-free convolution + folded BatchNorm of a [T, N, C, H, W] sequence: the matrix kernel's neuron-free mode where
+    it takes the layer, the framework's convolution otherwise."""
+    if x_seq.is_cuda:
+        from .runtime.hip_convlif_backend import run_hip_temporal_conv_bias
+        try:
+            return run_hip_temporal_conv_bias(list(x_seq.unbind(0)), weight, bias, stride, padding)
+        except RuntimeError as exc:
+            if "unsupported" not in str(exc):
+                raise
+    y = F.conv2d(x_seq.flatten(0, 1), weight, bias, stride, padding)
+    return y.unflatten(0, (x_seq.shape[0], -1))
+
+
 _TIME_BATCHABLE = (nn.Conv2d, nn.BatchNorm2d, nn.MaxPool2d, nn.AvgPool2d, nn.AdaptiveAvgPool2d, nn.Identity, nn.Linear)
+
+
+def _following_batchnorm(gm: fx.GraphModule, conv_members: Dict[int, fx.Node]) -> Optional[Dict[int, fx.Node]]:
+    """The eval-mode BatchNorm2d nodes (one module) that are the only users of the T convolution nodes, else None."""
+    out: Dict[int, fx.Node] = {}
+    target = None
+    for t, conv in conv_members.items():
+        user = _single_user(conv)
+        mod = _module_of(gm, user, nn.BatchNorm2d) if user is not None else None
+        if mod is None or mod.training or (target is not None and user.target != target):
+            return None
+        target = user.target
+        out[t] = user
+    return out
 
 
 def batch_timestep_calls(gm: fx.GraphModule) -> int:
@@ -451,16 +491,37 @@ def batch_timestep_calls(gm: fx.GraphModule) -> int:
             if not complete:
                 continue    # not every timestep of the stack goes through this layer
             first = min(members.values(), key=lambda n: list(graph.nodes).index(n)) if key[0] == "add" else members[0]
+            targets = members
             with graph.inserting_before(first):
                 if key[0] == "module":
-                    flat = graph.call_method("flatten", (stack, 0, 1))
-                    y = graph.call_module(key[1], (flat,))
-                    y_seq = graph.call_method("unflatten", (y, 0, (T, -1)))
+                    mod = gm.get_submodule(key[1])
+                    pool = pool_config(mod)
+                    bn_members = _following_batchnorm(gm, members) if isinstance(mod, nn.Conv2d) else None
+                    if pool is not None:
+                        y_seq = graph.call_function(pooled_frames, (stack, *pool))
+                    elif bn_members is not None and mod.groups == 1 and tuple(mod.dilation) == (1, 1):
+                        # Conv2d -> BatchNorm2d(eval) with no neuron behind it: one folded convolution over all frames.
+                        bn = gm.get_submodule(bn_members[0].target)
+                        with torch.no_grad():
+                            w, b = fold_bn_into_conv_params(mod.weight.float(), mod.bias, bn.running_mean.float(), bn.running_var.float(),
+                                                            None if bn.weight is None else bn.weight.float(),
+                                                            None if bn.bias is None else bn.bias.float(), bn.eps)
+                        index = sum(1 for name, _ in gm.named_buffers() if name.startswith("folded_weight_"))
+                        w_name = _register(gm, f"folded_weight_{index}", w.to(mod.weight.dtype).contiguous())
+                        b_name = _register(gm, f"folded_bias_{index}", b.to(mod.weight.dtype).contiguous())
+                        y_seq = graph.call_function(conv_bias_frames, (stack, graph.get_attr(w_name), graph.get_attr(b_name),
+                                                                       list(mod.stride), list(mod.padding)))
+                        targets = bn_members
+                        removed += T
+                    else:
+                        flat = graph.call_method("flatten", (stack, 0, 1))
+                        y = graph.call_module(key[1], (flat,))
+                        y_seq = graph.call_method("unflatten", (y, 0, (T, -1)))
                 elif key[0] == "add":
                     y_seq = graph.call_function(operator.add, (stacks[0], stacks[1]))
                 else:
                     y_seq = graph.call_function(torch.flatten, (stack, 2))
-            for t, node in members.items():
+            for t, node in targets.items():
                 with graph.inserting_after(y_seq):
                     step = graph.call_function(operator.getitem, (y_seq, t))
                 node.replace_all_uses_with(step)
