@@ -395,7 +395,7 @@ def main() -> int:
     args = _parse()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the operators shard over the batch axis with no "
-              "communication; see DESIGN.md) - run with --gpus 1", file=sys.stderr)
+              "communication) - run with --gpus 1", file=sys.stderr)
         return 2
     import torch
     if not torch.cuda.is_available():
