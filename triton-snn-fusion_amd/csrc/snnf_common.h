@@ -31,6 +31,20 @@ inline int check_launch(const char* what) {
 
 inline bool valid_dtype(int dt) { return dt == SNNF_F32 || dt == SNNF_BF16 || dt == SNNF_F16; }
 inline int dtype_size(int dt) { return dt == SNNF_F32 ? 4 : 2; }
+// Compute units of the current device (256 when it cannot be queried).
+inline int compute_units() {
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cached = n;
+        else
+            cached = 256;
+    }
+    return cached;
+}
+
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // ---------------------------------------------------------------------------------------------------------------

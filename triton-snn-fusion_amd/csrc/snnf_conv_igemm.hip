@@ -27,19 +27,6 @@ int max_tile_rows(const ConvGeom& g) {
     return worst;
 }
 
-int compute_units() {
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cached = n;
-        else
-            cached = 256;
-    }
-    return cached;
-}
-
 struct Plan {
     int TH, TW, tiles_x, tiles_y, NR, WT, wm_log2, wn_log2, oc_tiles;
     size_t lds_bytes;
@@ -121,7 +108,7 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw
     const int nw_log2 = nw == 8 ? 3 : 2;
     const int cus = compute_units() * (8 / nw);                  // workgroup slots of the machine
     const size_t lds_cap = kMaxLds * nw / 8;                      // per workgroup
-    const size_t stage_bytes = nw * kMmStageBytesPerWave;
+    const size_t stage_bytes = nw * kMmStageBytesPerWave + kMmBiasBytes;   // epilogue stages + the workgroup's bias values
     double best = -1.0;
     for (int wk_log2 = 0; wk_log2 <= nw_log2; ++wk_log2) {
         if ((1 << wk_log2) > g0.npairs) break;

@@ -82,6 +82,14 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     const int tile_px = g.TH * g.TW;                         // output pixels per image and tile
     const int tile_bytes = rows_all * g.WT * g.pitch;        // one timestep's halo tile(s)
     float* __restrict__ stage = reinterpret_cast<float*>(lds + g.mm_stage_off) + wave * kMmStageFloats;
+    // The workgroup's bias values (its 64 x WN output channels) are fetched with the first loads of a tile and parked in LDS
+    // until the epilogue, which would otherwise wait for them from memory group by group.
+    float* __restrict__ bias_lds = reinterpret_cast<float*>(lds + g.mm_stage_off) + NW * kMmStageFloats;
+    float bias_pre = 0.0f;
+    auto fetch_bias = [&](int oc_t) __attribute__((always_inline)) {
+        const int oc = (oc_t << g.wn_log2) * 64 + tid;
+        bias_pre = (tid < (64 << g.wn_log2) && oc < g.Cout) ? bias[oc] : 0.0f;
+    };
     const int nocf = (g.Cout + 31) >> 5;
     const int total_pairs = g.nchunks * g.npairs;
     const int64_t frag_stride_ocf = static_cast<int64_t>(total_pairs) * (kFragBytes / 2);
@@ -243,6 +251,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         int ih_lo, iw_lo;
         halo_origin(oh0, ow0, ih_lo, iw_lo);
         issue_loads(0, img, ih_lo, iw_lo);
+        fetch_bias(oc_tile);
     }
     SNNF_MM_STAMP(1);
 
@@ -328,8 +337,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             const int spairs = min(g.stage_chunks, g.nchunks - chunk * g.stage_chunks) * g.npairs;   // pairs of this stage
             load_frags(gp0 + wk, wa[0][0], wa[0][1]);  // in flight across the barriers and the LDS writes below
             load_frags(gp0 + wk + WK, wa[1][0], wa[1][1]);
-            __syncthreads();   // every wave is done reading the previous stage
+            __syncthreads();   // every wave is done reading the previous stage (and with the previous tile's epilogue)
             write_lds();       // waits for the stage's loads
+            if (chunk == 0 && tid < (64 << g.wn_log2)) bias_lds[tid] = bias_pre;
             __syncthreads();
             if (chunk < 4) SNNF_MM_STAMP(2 + 2 * chunk);
             // ---- the stage after this one: next chunk, or the first chunk of the next tile.
@@ -344,7 +354,10 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                     nimg = next_img;
                     halo_origin(next_oh0, next_ow0, nih, niw);
                 }
-                if (more) issue_loads(nc, nimg, nih, niw);
+                if (more) {
+                    issue_loads(nc, nimg, nih, niw);
+                    if (nc == 0) fetch_bias(next_oc_tile);
+                }
             }
             if (wave_has_work) {
                 const unsigned char* __restrict__ bp = lds + b_base + static_cast<uint32_t>(col0 * g.pitch);
@@ -391,15 +404,20 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             return (ocf0 + (gidx >> 1)) * 32 + (gidx & 1) * 16 + (FAST ? row16 : 4 * half);
         };
         auto row_delta = [&](int rr) __attribute__((always_inline)) -> int { return 8 * (rr >> 2) + (rr & 3); };
+        // General variant: all 16 channel rows of the group exist (uniform; true for every group when Cout % 16 == 0), so
+        // the per-row checks and their branches drop out.
+        auto group_full = [&](int gidx) __attribute__((always_inline)) -> bool {
+            return (ocf0 + (gidx >> 1)) * 32 + (gidx & 1) * 16 + 16 <= g.Cout;
+        };
         auto group_row = [&](int gidx, bool& row_ok, uint32_t& row_off, float (&bvv)[8]) __attribute__((always_inline)) {
             const int oc = first_row(gidx);
             row_ok = wave_has_work && (FAST || oc < g.Cout) && okmask != 0;
             row_off = static_cast<uint32_t>(min(oc, g.Cout - 1)) * static_cast<uint32_t>(po);
             if constexpr (FAST) {
-                bvv[0] = wave_has_work ? bias[oc] : 0.0f;
-            } else {
+                bvv[0] = bias_lds[oc - (oc_tile << g.wn_log2) * 64];
+            } else {   // rows beyond Cout hold zeros
 #pragma unroll
-                for (int rr = 0; rr < 8; ++rr) bvv[rr] = (wave_has_work && oc + row_delta(rr) < g.Cout) ? bias[oc + row_delta(rr)] : 0.0f;
+                for (int rr = 0; rr < 8; ++rr) bvv[rr] = bias_lds[oc - (oc_tile << g.wn_log2) * 64 + row_delta(rr)];
             }
         };
         auto load_membrane = [&](int gidx, bool row_ok, uint32_t row_off, float (&v)[8]) __attribute__((always_inline)) {
@@ -420,9 +438,10 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 }
             } else {
                 const int oc = first_row(gidx);
+                const bool all_rows = group_full(gidx);
 #pragma unroll
                 for (int rr = 0; rr < 8; ++rr) {
-                    if (oc + row_delta(rr) < g.Cout) {
+                    if (all_rows || oc + row_delta(rr) < g.Cout) {
                         const int64_t at = tile_off + row_off + static_cast<uint32_t>(row_delta(rr) * po) + px0;
                         v[rr] = vf32 ? static_cast<const float*>(v_init)[at] : to_float(static_cast<const XT*>(v_init)[at]);
                     }
@@ -440,6 +459,18 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 if (okmask & 0xf0u) *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
             } else {
                 const int oc = first_row(gidx);
+                if (group_full(gidx)) {
+                    if (vf32) {
+                        float* __restrict__ dst = static_cast<float*>(v_out) + tile_off + row_off;
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) dst[static_cast<uint32_t>(row_delta(rr) * po) + px0] = v[rr];
+                    } else {
+                        XT* __restrict__ dst = static_cast<XT*>(v_out) + tile_off + row_off;
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) dst[static_cast<uint32_t>(row_delta(rr) * po) + px0] = from_float<XT>(v[rr]);
+                    }
+                    return;
+                }
 #pragma unroll
                 for (int rr = 0; rr < 8; ++rr) {
                     if (oc + row_delta(rr) < g.Cout) {
@@ -521,6 +552,26 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             } else {
                 if (!row_ok) return;
                 const int oc = first_row(gidx);
+                if (group_full(gidx)) {
+                    float x[8];
+#pragma unroll
+                    for (int rr = 0; rr < 8; ++rr) x[rr] = xin[rr] + bvv[rr];
+                    if (has_residual) {
+                        XT res[8];
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) res[rr] = res_t[static_cast<uint32_t>(row_delta(rr) * po) + px0];
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) x[rr] += to_float(res[rr]);
+                    }
+                    if (analog) {
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) out_t[static_cast<uint32_t>(row_delta(rr) * po) + px0] = from_float<XT>(x[rr]);
+                    } else {
+#pragma unroll
+                        for (int rr = 0; rr < 8; ++rr) out_t[static_cast<uint32_t>(row_delta(rr) * po) + px0] = neuron(x[rr], v[rr]);
+                    }
+                    return;
+                }
 #pragma unroll
                 for (int rr = 0; rr < 8; ++rr) {
                     if (oc + row_delta(rr) < g.Cout) {
@@ -630,6 +681,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             int nih, niw;
             halo_origin(next_oh0, next_ow0, nih, niw);
             issue_loads(0, next_img, nih, niw);
+            fetch_bias(next_oc_tile);
         }
         work = next_work;
         oc_tile = next_oc_tile;
