@@ -148,25 +148,31 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         }
         pre_zero0 = z0;
         pre_zero1 = z1;
+        // A load address is a uniform base (timestep, image, chunk) plus a 32-bit lane offset that walks the 8 channels of
+        // the group: one vector add per load. Fewer than 8 input channels in all: the absent ones re-read the last real
+        // one (their weights are 0).
+        const uint32_t chan_stride = static_cast<uint32_t>(plane) * ES;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
             const char* __restrict__ base = reinterpret_cast<const char*>(static_cast<const XT*>(kernarg_table_entry(0, t)) + origin);
 #pragma unroll
             for (int s = 0; s < SS; ++s) {
                 if (item_cg[s] >= 0) {
+                    uint32_t v0 = off0[s], v1 = off1[s];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        // Fewer than 8 input channels in all: the absent ones re-read the last real one (their weights are 0).
-                        const char* __restrict__ row = base + min(j, last_channel) * plane * ES;
                         if constexpr (LM == LOAD_PAIR32) {
-                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(row + off0[s]);
+                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(base + v0);
                         } else if constexpr (LM == LOAD_2X16) {
-                            pre[s][t][j][0] = *reinterpret_cast<const uint16_t*>(row + off0[s]);
-                            pre[s][t][j][1] = *reinterpret_cast<const uint16_t*>(row + off1[s]);
+                            pre[s][t][j][0] = *reinterpret_cast<const uint16_t*>(base + v0);
+                            pre[s][t][j][1] = *reinterpret_cast<const uint16_t*>(base + v1);
                         } else {
-                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(row + off0[s]);
-                            pre[s][t][j][1] = *reinterpret_cast<const uint32_t*>(row + off1[s]);
+                            pre[s][t][j][0] = *reinterpret_cast<const uint32_t*>(base + v0);
+                            pre[s][t][j][1] = *reinterpret_cast<const uint32_t*>(base + v1);
                         }
+                        const uint32_t step = j < last_channel ? chan_stride : 0u;   // uniform
+                        v0 += step;
+                        v1 += step;
                     }
                 }
             }
