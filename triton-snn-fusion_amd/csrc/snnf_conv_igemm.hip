@@ -104,7 +104,7 @@ struct MmPlan {
 bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw, MmPlan& best_plan) {
     const bool pair_shift = load_mode == LOAD_PAIR32;
     const int groups = 1 << g0.groups_log2;
-    const int max_items = nw * 64 * ((load_mode == LOAD_PAIR32 ? 8 : 4) / tt);
+    const int slots = (load_mode == LOAD_PAIR32 ? 8 : 4) / tt;           // staging items per thread (mm_staging_slots)
     const int nw_log2 = nw == 8 ? 3 : 2;
     const int cus = compute_units() * (8 / nw);                  // workgroup slots of the machine
     const size_t lds_cap = kMaxLds * nw / 8;                      // per workgroup
@@ -113,6 +113,7 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw
     for (int wk_log2 = 0; wk_log2 <= nw_log2; ++wk_log2) {
         if ((1 << wk_log2) > g0.npairs) break;
         if (wk_log2 > 0 && g0.nchunks * g0.npairs < 72) break;   // measured: splitting pays from K of about 1152 on
+        const int max_items = nw * 64 * ((wk_log2 > 0 && load_mode == LOAD_PAIR32 && tt >= 2) ? slots / 2 : slots);
         for (int wn_log2 = 0; wn_log2 + wk_log2 <= nw_log2; ++wn_log2) {
             const int wm_log2 = nw_log2 - wn_log2 - wk_log2;
             const int PT = (1 << wm_log2) * 32;

@@ -29,7 +29,13 @@ constexpr int kMmStagePitch = 40;                          // floats per channel
 constexpr int kMmStageFloats = 16 * kMmStagePitch;         // 16 channel rows
 static_assert(kMmStageFloats * sizeof(float) == kMmStageBytesPerWave, "host and kernel disagree on the stage size");
 // Spatial staging items per thread and stage: 64 prefetch registers whatever the load mode and the timesteps per stage.
-__host__ __device__ constexpr int mm_staging_slots(int load_mode, int tt) { return (load_mode == LOAD_PAIR32 ? 8 : 4) / tt; }
+// The split-K variants stage deep layers with small tiles and are short of registers (with the full 64 prefetch registers
+// they spilled 30-140): with paired loads and 2 or 4 timesteps per stage they take half the slots, i.e. smaller LDS
+// stages (the unpaired load mode has half the slots to begin with and is better off with the larger stages).
+__host__ __device__ constexpr int mm_staging_slots(int load_mode, int tt, bool split_k = false) {
+    const int slots = (load_mode == LOAD_PAIR32 ? 8 : 4) / tt;
+    return (split_k && load_mode == LOAD_PAIR32 && tt >= 2) ? slots / 2 : slots;
+}
 typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
 
 // Phase timestamps of the first tile of the first 64 workgroups (development builds with -DSNNF_MM_TRACE only): slot 0
@@ -55,7 +61,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
-    constexpr int SS = mm_staging_slots(LM, TT);
+    constexpr int SS = mm_staging_slots(LM, TT, SK);
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
     constexpr int NT = NW * 64;                               // threads per workgroup
     const int tid = threadIdx.x;
