@@ -276,6 +276,40 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
             "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
 
 
+def _streaming_operators(dtype, steps: int, warmup: int):
+    """The two HBM-bound operators that no headline workload contains, each alone at a streaming size and at the size it
+    has in the spiking ResNet-18 of the configurations: temporal LIF scan (x once, spikes once, final membrane once) and
+    the LIF -> average pool -> linear tail (x once, final membrane once, classifier weight once)."""
+    import torch
+    S = torch.ops.snn_custom
+    dev = torch.device("cuda:0")
+    es = torch.empty((), dtype=dtype).element_size()
+    lif = (1.0, 0.0, 2.0, False)
+    v0 = torch.zeros((), device=dev, dtype=torch.float32)
+    out = {}
+    g = torch.Generator(device="cpu")
+    g.manual_seed(0)
+    for tag, shape in (("lif_scan_4x32x128x56x56", (4, 32, 128, 56, 56)), ("lif_scan_4x16x64x56x56", (4, 16, 64, 56, 56))):
+        x = (torch.randn(shape, generator=g) * 0.75 + 0.15).to(dev, dtype)
+        ms, how = _time_kernel(lambda: S.fused_temporal_lif_state(x, v0, *lif), steps, max(3, warmup // 2))
+        n = x[0].numel()
+        nbytes = (2 * shape[0] * es + 4) * n
+        out[tag] = {"ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "hbm": _roofline("hbm", nbytes, ms)}
+        del x
+    for tag, shape, classes in (("lif_tail_4x64x512x28x28_k1000", (4, 64, 512, 28, 28), 1000),
+                                ("lif_tail_4x16x512x7x7_k1000", (4, 16, 512, 7, 7), 1000),
+                                ("lif_tail_4x64x512x1x1_k10", (4, 64, 512, 1, 1), 10)):
+        x = (torch.randn(shape, generator=g) * 0.75 + 0.15).to(dev, dtype)
+        w = (torch.randn(classes, shape[2], generator=g) * 0.05).to(dev, dtype)
+        b = (torch.randn(classes, generator=g) * 0.05).to(dev, dtype)
+        ms, how = _time_kernel(lambda: S.fused_temporal_lif_avgpool_linear(x, v0, w, b, *lif), steps, max(3, warmup // 2))
+        n = x[0].numel()
+        nbytes = (shape[0] * es + 4) * n + (w.numel() + b.numel() + shape[1] * classes) * es
+        out[tag] = {"ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "hbm": _roofline("hbm", nbytes, ms)}
+        del x
+    return out
+
+
 def _bandwidth_probe():
     """What plain streaming kernels reach on this device, next to the published 8 TB/s: a 1 GiB device-to-device copy
     (read + write) and a 1 GiB fill (write only), both far beyond the 256 MB last-level cache."""
@@ -515,10 +549,19 @@ def main() -> int:
             entry = {"ms_per_step": round(ms, 4), "images_T_per_s": round(other.wl.batch * other.wl.T / (ms * 1e-3), 1),
                      "dtype": "f32" if name == "conv3x3_block" else args.dtype}
             try:
+                kms, how = _time_kernel(other.step, args.steps, max(3, args.warmup // 2))
+                entry["kernel_ms"], entry["timed"] = round(kms, 4), how
+            except Exception as exc:
+                entry["kernel_error"] = str(exc)[:200]
+            try:
                 entry["graph_ms_per_step"] = round(_time_graph(other.step, args.steps, max(3, args.warmup // 2)), 4)
             except Exception as exc:
                 entry["graph_error"] = str(exc)[:200]
             extra[name] = entry
+        try:
+            extra["streaming_operators"] = _streaming_operators(dtype, args.steps, args.warmup)
+        except Exception as exc:
+            extra["streaming_operators"] = {"error": str(exc)[:300]}
         for name in MODEL_CONFIGS:
             try:
                 extra[f"{name}_end_to_end"] = _model_forward(name, dtype, max(10, args.steps // 2), max(3, args.warmup // 2))

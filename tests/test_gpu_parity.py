@@ -126,7 +126,9 @@ def test_depthwise_residual_alias_and_membrane_chaining(hip_ops):
 # ---------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [F32, BF16, F16])
 @pytest.mark.parametrize("T,N,C,H,W,K,bias", [(4, 3, 32, 7, 7, 10, True), (4, 4, 512, 1, 1, 10, True), (4, 4, 512, 2, 2, 1000, True),
-                                               (4, 16, 512, 7, 7, 1000, True), (8, 2, 48, 5, 3, 17, False), (1, 1, 8, 32, 32, 3, True)])
+                                               (4, 16, 512, 7, 7, 1000, True), (8, 2, 48, 5, 3, 17, False), (1, 1, 8, 32, 32, 3, True),
+                                               (3, 1, 3, 3, 3, 5, True), (4, 50, 50, 5, 5, 7, True), (2, 2, 4, 25, 25, 6, True),
+                                               (16, 5, 64, 4, 4, 100, True)])
 def test_lif_avgpool_linear(hip_ops, dtype, T, N, C, H, W, K, bias):
     g = gen(300 + C)
     x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + 0.15, dtype)
@@ -140,6 +142,22 @@ def test_lif_avgpool_linear(hip_ops, dtype, T, N, C, H, W, K, bias):
     assert torch.equal(v.cpu(), ref_v)                              # elementwise LIF: exact
     tol = 1e-4 if dtype == F32 else (8e-3 if dtype == BF16 else 2e-3)   # out_sum is stored in the activation dtype
     assert torch.allclose(out.float().cpu(), ref_out, rtol=tol, atol=tol), (out.float().cpu() - ref_out).abs().max()
+    _no_fallback(hip_ops, 1)
+
+
+@pytest.mark.parametrize("N,C,H,W", [(6, 64, 7, 7), (3, 5, 3, 3), (40, 128, 1, 1)])
+def test_lif_avgpool_linear_tensor_v_init(hip_ops, N, C, H, W):
+    """A membrane tensor as initial state (vector and element-wise paths of the pooling kernel)."""
+    T, K = 4, 12
+    g = gen(340 + C)
+    x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + 0.15, BF16)
+    v0 = torch.rand(N, C, H, W, generator=g) * 0.9
+    w = q(torch.randn(K, C, generator=g) * 0.05, BF16)
+    b = q(torch.randn(K, generator=g) * 0.05, BF16)
+    ref_out, ref_v, _, _ = O.temporal_lif_avgpool_linear(x, v0, w, b, *LIF)
+    out, v = S.fused_temporal_lif_avgpool_linear(dev(x, BF16), dev(v0, F32), dev(w, BF16), dev(b, BF16), *LIF, False)
+    assert torch.equal(v.cpu(), ref_v)
+    assert torch.allclose(out.float().cpu(), ref_out, rtol=8e-3, atol=8e-3), (out.float().cpu() - ref_out).abs().max()
     _no_fallback(hip_ops, 1)
 
 

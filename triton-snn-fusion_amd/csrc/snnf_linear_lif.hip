@@ -3,8 +3,9 @@
 // Both operands are K-contiguous in memory (x rows and W rows), which is exactly the per-lane operand order of
 // v_mfma_f32_16x16x32 (8 consecutive k per lane), so fragments are loaded straight from global memory into registers.
 // All T timesteps of a row tile share one weight fragment load (the weight is streamed once per workgroup, not once per
-// timestep). The four waves of a workgroup split K; partial sums meet in LDS, then each thread runs the LIF recurrence
-// over T for its (row, output feature) pairs with the membrane in a register.
+// timestep). The 8 (or, beyond 8 timesteps, 4) waves of a workgroup split K and prefetch their next K step while the
+// current one multiplies; partial sums meet in LDS, then each thread runs the LIF recurrence over T for its (row, output
+// feature) pair with the membrane in a register.
 #include "snnf_common.h"
 
 namespace snnf {
@@ -15,8 +16,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
 constexpr int kTileOC = 16;   // output features per workgroup
 constexpr int kTileM = 16;    // rows per workgroup (per timestep)
 
@@ -83,12 +82,17 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     }
 }
 
+// Waves per workgroup: they split K, so more waves mean more loads in flight per CU; their partial sums (1 KiB per wave
+// and timestep) must fit the 64 KiB of static LDS.
+template <int TT> struct LinWaves { static constexpr int value = TT <= 8 ? 8 : 4; };
+
 template <typename XT, typename VT, int TT, bool FAST>
-__global__ __launch_bounds__(kThreads) void linear_lif_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
-                                                              const XT* __restrict__ bias,
-                                                              const VT* __restrict__ v_init, XT* __restrict__ spikes,
-                                                              VT* __restrict__ v_out, LifParams lif) {
-    __shared__ float partial[kWaves][TT][kTileOC * kTileM];
+__global__ __launch_bounds__(LinWaves<TT>::value * 64) void linear_lif_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
+                                                                              const XT* __restrict__ bias,
+                                                                              const VT* __restrict__ v_init, XT* __restrict__ spikes,
+                                                                              VT* __restrict__ v_out, LifParams lif) {
+    constexpr int NW = LinWaves<TT>::value;
+    __shared__ float partial[NW][TT][kTileOC * kTileM];
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int oc0 = blockIdx.x * kTileOC;
@@ -99,22 +103,35 @@ __global__ __launch_bounds__(kThreads) void linear_lif_kernel(StepPtrs xs, LinGe
     const int b_row = min(m0 + (lane & 15), g.M - 1);
     const int koff = (lane >> 4) * 8;
     const XT* __restrict__ wrow = W + static_cast<int64_t>(a_row) * g.Fin;
+    const XT* xrow[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) xrow[t] = static_cast<const XT*>(xs.p[t]) + static_cast<int64_t>(b_row) * g.x_row_stride;
 
     f32x4 acc[TT];
 #pragma unroll
     for (int t = 0; t < TT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int s = wave; s < g.ksteps; s += kWaves) {
+    // K step s (32 elements of K) belongs to wave s % NW. Two register sets: the loads of a wave's next step are in flight
+    // while the matrix instructions of the current one run.
+    u32x4 a0, a1, b0[TT], b1[TT];
+    auto fetch = [&](int s, u32x4& a, u32x4 (&b)[TT]) __attribute__((always_inline)) {
         const int k = s * 32 + koff;
-        const u32x4 a = load_octet<XT, FAST>(wrow, k, g.Fin);
-        u32x4 b[TT];
+        a = load_octet<XT, FAST>(wrow, k, g.Fin);
 #pragma unroll
-        for (int t = 0; t < TT; ++t) {
-            const XT* __restrict__ xrow = static_cast<const XT*>(xs.p[t]) + static_cast<int64_t>(b_row) * g.x_row_stride;
-            b[t] = load_octet<XT, FAST>(xrow, k, g.Fin);
-        }
+        for (int t = 0; t < TT; ++t) b[t] = load_octet<XT, FAST>(xrow[t], k, g.Fin);
+    };
+    auto multiply = [&](const u32x4& a, const u32x4 (&b)[TT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < TT; ++t) acc[t] = mfma16<XT>(a, b[t], acc[t]);
+    };
+    int s = wave;
+    if (s < g.ksteps) fetch(s, a0, b0);
+    for (; s < g.ksteps; s += 2 * NW) {
+        const bool more1 = s + NW < g.ksteps;
+        if (more1) fetch(s + NW, a1, b1);
+        multiply(a0, b0);
+        if (s + 2 * NW < g.ksteps) fetch(s + 2 * NW, a0, b0);
+        if (more1) multiply(a1, b1);
     }
 
     // D[i = oc][j = m]: lane holds column j = lane % 16, rows i = 4 * (lane / 16) + r.
@@ -124,8 +141,10 @@ __global__ __launch_bounds__(kThreads) void linear_lif_kernel(StepPtrs xs, LinGe
         for (int r = 0; r < 4; ++r) partial[wave][t][(lane & 15) * kTileOC + (lane >> 4) * 4 + r] = acc[t][r];
     __syncthreads();
 
-    // Thread e owns (row m_local = e / 16, feature oc_local = e % 16): consecutive threads write consecutive features.
+    // Thread e < 256 owns (row m_local = e / 16, feature oc_local = e % 16): consecutive threads write consecutive
+    // features. The partial sums are added in a fixed order.
     const int e = threadIdx.x;
+    if (e >= kTileOC * kTileM) return;
     const int m = m0 + (e >> 4);
     const int oc = oc0 + (e & 15);
     if (m >= g.M || oc >= g.Fout) return;
@@ -135,7 +154,10 @@ __global__ __launch_bounds__(kThreads) void linear_lif_kernel(StepPtrs xs, LinGe
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
         if (t >= g.T) break;
-        const float cur = ((partial[0][t][e] + partial[1][t][e]) + (partial[2][t][e] + partial[3][t][e])) + bv;
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; w += 2) sum += partial[w][t][e] + partial[w + 1][t][e];
+        const float cur = sum + bv;
         spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
     }
     v_out[o] = from_float<VT>(v);
@@ -151,11 +173,11 @@ int launch_tt(const StepPtrs& xs, const LinGeom& g, const void* W, const void* b
     const VT* vi = static_cast<const VT*>(v_init);
     XT* sp = static_cast<XT*>(spikes);
     VT* vo = static_cast<VT*>(v_out);
-    if (g.T <= 1) linear_lif_kernel<XT, VT, 1, FAST><<<grid, kThreads, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 2) linear_lif_kernel<XT, VT, 2, FAST><<<grid, kThreads, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 4) linear_lif_kernel<XT, VT, 4, FAST><<<grid, kThreads, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 8) linear_lif_kernel<XT, VT, 8, FAST><<<grid, kThreads, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else linear_lif_kernel<XT, VT, 16, FAST><<<grid, kThreads, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
+    if (g.T <= 1) linear_lif_kernel<XT, VT, 1, FAST><<<grid, LinWaves<1>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
+    else if (g.T <= 2) linear_lif_kernel<XT, VT, 2, FAST><<<grid, LinWaves<2>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
+    else if (g.T <= 4) linear_lif_kernel<XT, VT, 4, FAST><<<grid, LinWaves<4>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
+    else if (g.T <= 8) linear_lif_kernel<XT, VT, 8, FAST><<<grid, LinWaves<8>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
+    else linear_lif_kernel<XT, VT, 16, FAST><<<grid, LinWaves<16>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
     return check_launch("snnf_linear_lif");
 }
 

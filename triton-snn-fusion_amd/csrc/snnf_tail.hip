@@ -3,8 +3,9 @@
 //   out_sum[n, k] = sum_t ( W[k, :] . mean_hw(s_t[n, :, :, :]) + b[k] ) = (W[k, :] . count[n, :]) / HW + T * b[k]
 //
 // where count[n, c] is the number of spikes of plane (n, c) over all T steps: the pooled activations are never
-// materialised per step. Launch 1 streams x once (HBM-bound), keeps the membrane in registers, counts spikes per plane
-// with wave ballots and writes the integer counts to the workspace; launch 2 is a small GEMV over the counts.
+// materialised per step. Launch 1 streams x once (HBM-bound, 16-byte accesses where the operands allow), keeps the membrane
+// in registers, counts spikes per plane in LDS and writes the integer counts to the workspace; launch 2 is a small GEMV
+// over the counts with wave-shuffle reductions.
 #include "snnf_common.h"
 
 namespace snnf {
@@ -64,6 +65,98 @@ __global__ __launch_bounds__(kThreads) void lif_pool_kernel(StepPtrs xs, int T, 
     for (int i = threadIdx.x; i < planes_here; i += kThreads) counts[plane0 + i] = plane_count[i];
 }
 
+// Vector variant of the pooling kernel: a thread owns 8 consecutive neurons of the workgroup's planes per pass, fetched
+// with 16-byte loads, four timesteps in flight at a time; a thread's spikes are merged per plane before they reach the
+// LDS counters. The host guarantees that a workgroup's first neuron is a multiple of 8 and that all bases are 16-byte
+// aligned; only the last 8 neurons of the last workgroup may be ragged and are moved one by one.
+constexpr int kVec = 8;
+
+template <typename XT, typename VT>
+__global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int T, int planes, int HW, int planes_per_block,
+                                                                const VT* __restrict__ v_init, VT* __restrict__ v_out,
+                                                                int* __restrict__ counts, LifParams lif) {
+    __shared__ int plane_count[kMaxPlanes];
+    const int plane0 = blockIdx.x * planes_per_block;
+    const int planes_here = min(planes_per_block, planes - plane0);
+    const int elems = planes_here * HW;
+    const int64_t base = static_cast<int64_t>(plane0) * HW;
+    for (int i = threadIdx.x; i < planes_here; i += kThreads) plane_count[i] = 0;
+    __syncthreads();
+
+    for (int i0 = threadIdx.x * kVec; i0 < elems; i0 += kThreads * kVec) {
+        const bool whole = i0 + kVec <= elems;
+        float v[kVec];
+        int fired[kVec];
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+            v[j] = 0.0f;
+            fired[j] = 0;
+        }
+        if (v_init != nullptr) {
+            if (whole) {
+                const Pack<VT, kVec> pv = *reinterpret_cast<const Pack<VT, kVec>*>(v_init + base + i0);
+#pragma unroll
+                for (int j = 0; j < kVec; ++j) v[j] = to_float(pv.v[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < kVec; ++j)
+                    if (i0 + j < elems) v[j] = to_float(v_init[base + i0 + j]);
+            }
+        }
+        for (int t0 = 0; t0 < T; t0 += 4) {
+            Pack<XT, kVec> px[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (t0 + u < T) {
+                    const XT* __restrict__ x = static_cast<const XT*>(xs.p[t0 + u]) + base + i0;
+                    if (whole) {
+                        px[u] = *reinterpret_cast<const Pack<XT, kVec>*>(x);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < kVec; ++j) px[u].v[j] = i0 + j < elems ? x[j] : XT{};
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (t0 + u < T) {
+#pragma unroll
+                    for (int j = 0; j < kVec; ++j) fired[j] += lif_step(to_float(px[u].v[j]), v[j], lif) ? 1 : 0;
+                }
+            }
+        }
+        if (whole) {
+            Pack<VT, kVec> pv;
+#pragma unroll
+            for (int j = 0; j < kVec; ++j) pv.v[j] = from_float<VT>(v[j]);
+            *reinterpret_cast<Pack<VT, kVec>*>(v_out + base + i0) = pv;
+        } else {
+#pragma unroll
+            for (int j = 0; j < kVec; ++j)
+                if (i0 + j < elems) v_out[base + i0 + j] = from_float<VT>(v[j]);
+        }
+        // Spikes of consecutive neurons of one plane are summed before they go to that plane's counter.
+        int p = i0 / HW;
+        int rem = i0 - p * HW;
+        int run = 0;
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+            if (i0 + j < elems) {
+                run += fired[j];
+                if (++rem == HW) {
+                    if (run != 0) atomicAdd(&plane_count[p], run);
+                    run = 0;
+                    rem = 0;
+                    ++p;
+                }
+            }
+        }
+        if (run != 0) atomicAdd(&plane_count[p], run);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < planes_here; i += kThreads) counts[plane0 + i] = plane_count[i];
+}
+
 // One workgroup: one sample n, kWavesPerBlock * kRowsPerWave output rows; the sample's spike counts sit in LDS.
 constexpr int kRowsPerWave = 4;
 
@@ -95,9 +188,72 @@ __global__ __launch_bounds__(kThreads) void count_linear_kernel(const int* __res
     }
 }
 
+// Vector variant (C a multiple of 8, 16-byte aligned weight): no LDS and no barrier; a lane fetches 8 consecutive weights
+// of each of its wave's rows with 16-byte loads, all rows in flight together, and the 8 matching counts once.
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void count_linear_vec_kernel(const int* __restrict__ counts, int C, int K,
+                                                                    const XT* __restrict__ W, const XT* __restrict__ bias,
+                                                                    XT* __restrict__ out, float inv_hw, float steps) {
+    const int n = blockIdx.y;
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int k0 = (blockIdx.x * (kThreads / 64) + wave) * kRowsPerWave;
+    if (k0 >= K) return;
+    float acc[kRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
+    for (int c0 = lane * kVec; c0 < C; c0 += 64 * kVec) {
+        const Pack<int, kVec> pc = *reinterpret_cast<const Pack<int, kVec>*>(counts + static_cast<int64_t>(n) * C + c0);
+        Pack<XT, kVec> pw[kRowsPerWave];
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) {
+            const int k = min(k0 + r, K - 1);   // rows beyond K re-read the last one and are not stored
+            pw[r] = *reinterpret_cast<const Pack<XT, kVec>*>(W + static_cast<int64_t>(k) * C + c0);
+        }
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+            for (int j = 0; j < kVec; ++j) acc[r] = fmaf(to_float(pw[r].v[j]), static_cast<float>(pc.v[j]), acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc[r] += __shfl_xor(acc[r], off);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) {
+            const int k = k0 + r;
+            if (k < K) {
+                float o = acc[r] * inv_hw;
+                if (bias != nullptr) o += steps * to_float(bias[k]);
+                out[static_cast<int64_t>(n) * K + k] = from_float<XT>(o);
+            }
+        }
+    }
+}
+
 template <typename XT, typename VT>
 int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void* v_out, int* counts,
         const LifParams& lif, hipStream_t stream) {
+    // Vector variant: about kThreads * kVec neurons per workgroup, whole planes, every workgroup starting at a multiple
+    // of 8 neurons, all bases 16-byte aligned.
+    bool aligned = aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16));
+    for (int t = 0; t < T; ++t) aligned = aligned && aligned_to(xs.p[t], 16);
+    int vpb = (kThreads * kVec) / HW;
+    if (vpb < 1) vpb = 1;
+    if (vpb > kMaxPlanes) vpb = kMaxPlanes;
+    int tries = 0;
+    while (vpb > 1 && vpb < planes && (static_cast<int64_t>(vpb) * HW) % kVec != 0 && tries < kVec) {
+        --vpb;
+        ++tries;
+    }
+    if (aligned && (vpb >= planes || (static_cast<int64_t>(vpb) * HW) % kVec == 0)) {
+        const int blocks = (planes + vpb - 1) / vpb;
+        lif_pool_vec_kernel<XT, VT><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, static_cast<const VT*>(v_init),
+                                                                          static_cast<VT*>(v_out), counts, lif);
+        return check_launch("snnf_lif_pool_linear(pool)");
+    }
     int ppb = (kThreads * kItems) / HW;
     if (ppb < 1) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: H*W=%d exceeds %d", HW, kThreads * kItems);
     if (ppb > kMaxPlanes) ppb = kMaxPlanes;
@@ -105,6 +261,17 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
     lif_pool_kernel<XT, VT><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, ppb, static_cast<const VT*>(v_init),
                                                                   static_cast<VT*>(v_out), counts, lif);
     return check_launch("snnf_lif_pool_linear(pool)");
+}
+
+template <typename XT>
+void run_linear(bool vec, dim3 grid, size_t lds, hipStream_t hs, const int* counts, int C, int K, const void* W, const void* bias,
+                void* out, float inv_hw, float steps) {
+    if (vec)
+        count_linear_vec_kernel<XT><<<grid, kThreads, 0, hs>>>(counts, C, K, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                                              static_cast<XT*>(out), inv_hw, steps);
+    else
+        count_linear_kernel<XT><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                                            static_cast<XT*>(out), inv_hw, steps);
 }
 
 }  // namespace
@@ -169,14 +336,9 @@ extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, 
     const size_t lds = static_cast<size_t>(C) * sizeof(float);
     const float inv_hw = 1.0f / static_cast<float>(HW);
     const float steps = static_cast<float>(T);
-    if (x_dtype == SNNF_F32)
-        count_linear_kernel<float><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const float*>(fc_weight),
-                                                               static_cast<const float*>(fc_bias), static_cast<float*>(out_sum), inv_hw, steps);
-    else if (x_dtype == SNNF_BF16)
-        count_linear_kernel<bf16_t><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const bf16_t*>(fc_weight),
-                                                                static_cast<const bf16_t*>(fc_bias), static_cast<bf16_t*>(out_sum), inv_hw, steps);
-    else
-        count_linear_kernel<f16_t><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const f16_t*>(fc_weight),
-                                                               static_cast<const f16_t*>(fc_bias), static_cast<f16_t*>(out_sum), inv_hw, steps);
+    const bool vec = C % kVec == 0 && aligned_to(fc_weight, 16);
+    if (x_dtype == SNNF_F32) run_linear<float>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
+    else if (x_dtype == SNNF_BF16) run_linear<bf16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
+    else run_linear<f16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
     return check_launch("snnf_lif_pool_linear(linear)");
 }
