@@ -176,7 +176,9 @@ def _linear_case(seed, T, M, Fin, Fout, dtype, bias=True, p=0.1):
 
 @pytest.mark.parametrize("dtype,vdtype", [(BF16, F32), (F32, F32), (F16, F16), (BF16, BF16)])
 @pytest.mark.parametrize("T,M,Fin,Fout,bias", [(8, 64, 256, 128, True), (3, 5, 100, 37, True), (16, 1, 512, 512, False),
-                                                (4, 16, 1000, 48, True), (20, 3, 64, 16, True), (2, 33, 96, 130, True)])
+                                                (4, 16, 1000, 48, True), (20, 3, 64, 16, True), (2, 33, 96, 130, True),
+                                                (4, 64, 512, 1024, True), (16, 64, 256, 1024, True), (5, 40, 200, 64, True),
+                                                (12, 17, 264, 96, False)])
 def test_linear_lif_packed(hip_ops, dtype, vdtype, T, M, Fin, Fout, bias):
     x, w_dev, b_dev, w_ref, b_ref = _linear_case(400 + Fin, T, M, Fin, Fout, dtype, bias)
     ref = O.temporal_linear_lif(x, w_ref, b_ref, torch.tensor(0.0), *LIF)

@@ -1,11 +1,12 @@
 // Temporal Linear + LIF on the matrix cores: out^T[Fout, T*M] = W[Fout, Fin] . x^T, LIF recurrence in the epilogue.
 //
-// Both operands are K-contiguous in memory (x rows and W rows), which is exactly the per-lane operand order of
-// v_mfma_f32_16x16x32 (8 consecutive k per lane), so fragments are loaded straight from global memory into registers.
-// All T timesteps of a row tile share one weight fragment load (the weight is streamed once per workgroup, not once per
-// timestep). The 8 (or, beyond 8 timesteps, 4) waves of a workgroup split K and prefetch their next K step while the
-// current one multiplies; partial sums meet in LDS, then each thread runs the LIF recurrence over T for its (row, output
-// feature) pair with the membrane in a register.
+// Both operands are K-contiguous in memory (x rows and W rows), which is the per-lane operand order of
+// v_mfma_f32_16x16x32 (8 consecutive k per lane). All T timesteps of a row tile share one weight fragment (the weight is
+// streamed once per workgroup, not once per timestep), and each thread runs the LIF recurrence over T for its (row,
+// output feature) pair with the membrane in a register. Two kernels: the staged one (4 timesteps or more, aligned rows)
+// moves K slabs of all operand rows through LDS with coalesced loads; the direct one (everything else) loads fragments
+// straight from global memory, its 8 (beyond 8 timesteps, 4) waves splitting K in pairs of K steps with partial sums
+// meeting in LDS.
 #include "snnf_common.h"
 
 namespace snnf {
@@ -36,37 +37,41 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
 }
 
-// Loads k .. k+7 of `row`; elements at or beyond `kmax` read as zero. FAST requires 16-byte aligned rows.
+// Loads k .. k+7 of `row`; elements at or beyond `kmax` read as zero. FAST requires 16-byte aligned rows and kmax % 8 == 0
+// and is branch-free (an octet beyond kmax re-reads the row's first one and is zeroed): a branch around a load would make
+// the compiler wait for every load before it issues the next.
 template <typename XT, bool FAST>
 __device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, int kmax) {
     u32x4 out = {0u, 0u, 0u, 0u};
-    if constexpr (sizeof(XT) == 2) {
-        if (FAST && k + 8 <= kmax) {
-            out = *reinterpret_cast<const u32x4*>(row + k);
+    if constexpr (FAST) {
+        const bool inside = k < kmax;
+        const XT* __restrict__ src = row + (inside ? k : 0);
+        if constexpr (sizeof(XT) == 2) {
+            out = *reinterpret_cast<const u32x4*>(src);
         } else {
-            const uint16_t* p = reinterpret_cast<const uint16_t*>(row);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t lo = (k + 2 * j) < kmax ? p[k + 2 * j] : 0u;
-                const uint32_t hi = (k + 2 * j + 1) < kmax ? p[k + 2 * j + 1] : 0u;
-                out[j] = lo | (hi << 16);
-            }
-        }
-    } else {
-        if (FAST && k + 8 <= kmax) {
-            const f32x4 a = *reinterpret_cast<const f32x4*>(row + k);
-            const f32x4 b = *reinterpret_cast<const f32x4*>(row + k + 4);
+            const f32x4 a = *reinterpret_cast<const f32x4*>(src);
+            const f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
             out[0] = pack_bf16x2(a[0], a[1]);
             out[1] = pack_bf16x2(a[2], a[3]);
             out[2] = pack_bf16x2(b[0], b[1]);
             out[3] = pack_bf16x2(b[2], b[3]);
-        } else {
+        }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float lo = (k + 2 * j) < kmax ? to_float(row[k + 2 * j]) : 0.0f;
-                const float hi = (k + 2 * j + 1) < kmax ? to_float(row[k + 2 * j + 1]) : 0.0f;
-                out[j] = pack_bf16x2(lo, hi);
-            }
+        for (int j = 0; j < 4; ++j) out[j] = inside ? out[j] : 0u;
+    } else if constexpr (sizeof(XT) == 2) {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(row);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = (k + 2 * j) < kmax ? p[k + 2 * j] : 0u;
+            const uint32_t hi = (k + 2 * j + 1) < kmax ? p[k + 2 * j + 1] : 0u;
+            out[j] = lo | (hi << 16);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float lo = (k + 2 * j) < kmax ? to_float(row[k + 2 * j]) : 0.0f;
+            const float hi = (k + 2 * j + 1) < kmax ? to_float(row[k + 2 * j + 1]) : 0.0f;
+            out[j] = pack_bf16x2(lo, hi);
         }
     }
     return out;
@@ -82,103 +87,320 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     }
 }
 
-// Waves per workgroup: they split K, so more waves mean more loads in flight per CU; their partial sums (1 KiB per wave
-// and timestep) must fit the 64 KiB of static LDS.
+// Waves per workgroup: they split K, so more waves mean more loads in flight per CU.
 template <int TT> struct LinWaves { static constexpr int value = TT <= 8 ? 8 : 4; };
 
-template <typename XT, typename VT, int TT, bool FAST>
+// OCF: fragments of 16 output features per workgroup. Two fragments share every activation fragment (half the activation
+// traffic per output) at the price of half as many workgroups.
+template <typename XT, typename VT, int TT, bool FAST, int OCF>
 __global__ __launch_bounds__(LinWaves<TT>::value * 64) void linear_lif_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
                                                                               const XT* __restrict__ bias,
                                                                               const VT* __restrict__ v_init, XT* __restrict__ spikes,
                                                                               VT* __restrict__ v_out, LifParams lif) {
     constexpr int NW = LinWaves<TT>::value;
-    __shared__ float partial[NW][TT][kTileOC * kTileM];
+    constexpr int TILE_OC = OCF * kTileOC;
+    constexpr int OUTS = TILE_OC * kTileM;                    // outputs per workgroup and timestep
+    constexpr int PITCH = TILE_OC + 4;                        // floats per row of a partial tile: the 16-byte writes of
+                                                              // 8 consecutive lanes (8 rows) then fall into distinct banks
+    constexpr int SLAB = kTileM * PITCH;                      // floats per (wave, timestep)
+    extern __shared__ __align__(16) float partial[];          // [NW][TT][kTileM][PITCH]
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int oc0 = blockIdx.x * kTileOC;
+    const int oc0 = blockIdx.x * TILE_OC;
     const int m0 = blockIdx.y * kTileM;
 
     // Operand rows of this lane (clamped: out-of-range rows compute garbage that is never stored).
-    const int a_row = min(oc0 + (lane & 15), g.Fout - 1);
     const int b_row = min(m0 + (lane & 15), g.M - 1);
     const int koff = (lane >> 4) * 8;
-    const XT* __restrict__ wrow = W + static_cast<int64_t>(a_row) * g.Fin;
+    const XT* wrow[OCF];
+#pragma unroll
+    for (int f = 0; f < OCF; ++f) wrow[f] = W + static_cast<int64_t>(min(oc0 + f * kTileOC + (lane & 15), g.Fout - 1)) * g.Fin;
     const XT* xrow[TT];
 #pragma unroll
     for (int t = 0; t < TT; ++t) xrow[t] = static_cast<const XT*>(xs.p[t]) + static_cast<int64_t>(b_row) * g.x_row_stride;
 
-    f32x4 acc[TT];
+    f32x4 acc[OCF][TT];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < OCF; ++f)
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // K step s (32 elements of K) belongs to wave s % NW. Two register sets: the loads of a wave's next step are in flight
-    // while the matrix instructions of the current one run.
-    u32x4 a0, a1, b0[TT], b1[TT];
-    auto fetch = [&](int s, u32x4& a, u32x4 (&b)[TT]) __attribute__((always_inline)) {
+    // K steps (32 elements of K each) are dealt to the waves in pairs: the two steps of a pair read the two halves of the
+    // same 128-byte lines of every operand row back to back. The loads of both steps are issued before the first
+    // matrix instruction; the other wave of the SIMD covers the wait.
+    u32x4 a0[OCF], a1[OCF], b0[TT], b1[TT];
+    auto fetch = [&](int s, u32x4 (&a)[OCF], u32x4 (&b)[TT]) __attribute__((always_inline)) {
         const int k = s * 32 + koff;
-        a = load_octet<XT, FAST>(wrow, k, g.Fin);
+#pragma unroll
+        for (int f = 0; f < OCF; ++f) a[f] = load_octet<XT, FAST>(wrow[f], k, g.Fin);
 #pragma unroll
         for (int t = 0; t < TT; ++t) b[t] = load_octet<XT, FAST>(xrow[t], k, g.Fin);
     };
-    auto multiply = [&](const u32x4& a, const u32x4 (&b)[TT]) __attribute__((always_inline)) {
+    auto multiply = [&](const u32x4 (&a)[OCF], const u32x4 (&b)[TT]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < TT; ++t) acc[t] = mfma16<XT>(a, b[t], acc[t]);
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int f = 0; f < OCF; ++f) acc[f][t] = mfma16<XT>(a[f], b[t], acc[f][t]);
     };
-    int s = wave;
-    if (s < g.ksteps) fetch(s, a0, b0);
-    for (; s < g.ksteps; s += 2 * NW) {
-        const bool more1 = s + NW < g.ksteps;
-        if (more1) fetch(s + NW, a1, b1);
+    for (int s = 2 * wave; s < g.ksteps; s += 2 * NW) {
+        const bool second = s + 1 < g.ksteps;
+        fetch(s, a0, b0);
+        if (second) fetch(s + 1, a1, b1);
         multiply(a0, b0);
-        if (s + 2 * NW < g.ksteps) fetch(s + 2 * NW, a0, b0);
-        if (more1) multiply(a1, b1);
+        if (second) multiply(a1, b1);
     }
 
     // D[i = oc][j = m]: lane holds column j = lane % 16, rows i = 4 * (lane / 16) + r.
 #pragma unroll
     for (int t = 0; t < TT; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) partial[wave][t][(lane & 15) * kTileOC + (lane >> 4) * 4 + r] = acc[t][r];
+        for (int f = 0; f < OCF; ++f)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                partial[(wave * TT + t) * SLAB + (lane & 15) * PITCH + f * kTileOC + (lane >> 4) * 4 + r] = acc[f][t][r];
     __syncthreads();
 
-    // Thread e < 256 owns (row m_local = e / 16, feature oc_local = e % 16): consecutive threads write consecutive
-    // features. The partial sums are added in a fixed order.
-    const int e = threadIdx.x;
-    if (e >= kTileOC * kTileM) return;
-    const int m = m0 + (e >> 4);
-    const int oc = oc0 + (e & 15);
-    if (m >= g.M || oc >= g.Fout) return;
-    const float bv = bias != nullptr ? to_float(bias[oc]) : 0.0f;
-    const int64_t o = static_cast<int64_t>(m) * g.Fout + oc;
-    float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
+    // Output e of the tile = (row e / TILE_OC, feature e % TILE_OC): consecutive threads write consecutive features. The
+    // partial sums are added in a fixed order.
+    for (int e = threadIdx.x; e < OUTS; e += NW * 64) {
+        const int slot = (e / TILE_OC) * PITCH + e % TILE_OC;
+        const int m = m0 + e / TILE_OC;
+        const int oc = oc0 + e % TILE_OC;
+        if (m >= g.M || oc >= g.Fout) continue;
+        const float bv = bias != nullptr ? to_float(bias[oc]) : 0.0f;
+        const int64_t o = static_cast<int64_t>(m) * g.Fout + oc;
+        float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-        if (t >= g.T) break;
-        float sum = 0.0f;
+        for (int t = 0; t < TT; ++t) {
+            if (t >= g.T) break;
+            float sum = 0.0f;
 #pragma unroll
-        for (int w = 0; w < NW; w += 2) sum += partial[w][t][e] + partial[w + 1][t][e];
-        const float cur = sum + bv;
-        spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+            for (int w = 0; w < NW; w += 2) sum += partial[(w * TT + t) * SLAB + slot] + partial[((w + 1) * TT + t) * SLAB + slot];
+            const float cur = sum + bv;
+            spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+        }
+        v_out[o] = from_float<VT>(v);
     }
-    v_out[o] = from_float<VT>(v);
+}
+
+template <typename XT, typename VT, int TT, bool FAST, int OCF>
+int launch_one(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+               void* v_out, const LifParams& lif, hipStream_t stream) {
+    constexpr int NW = LinWaves<TT>::value;
+    constexpr size_t lds = static_cast<size_t>(NW) * TT * kTileM * (OCF * kTileOC + 4) * sizeof(float);
+    static_assert(lds <= 160 * 1024, "partial sums exceed LDS");
+    const dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
+    if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
+    auto kernel = linear_lif_kernel<XT, VT, TT, FAST, OCF>;
+    if (lds > 64 * 1024) {
+        static const hipError_t raised =
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (raised != hipSuccess) return fail(SNNF_ERR_LAUNCH, "snnf_linear_lif: cannot reserve %zu bytes of LDS", lds);
+    }
+    kernel<<<grid, NW * 64, lds, stream>>>(xs, g, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                           static_cast<const VT*>(v_init), static_cast<XT*>(spikes), static_cast<VT*>(v_out), lif);
+    return check_launch("snnf_linear_lif");
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Staged variant (4 timesteps or more, 16-byte aligned rows, Fin % 8 == 0). Operand fragments fetched straight from
+// global memory put the 16 rows of a fragment in 16 adjacent lanes, i.e. 16 different cache lines per 256 bytes
+// fetched, and the texture path then delivers about 16 bytes per clock and CU. Here a K slab of 128 elements of every
+// operand row (the 16 x TT activation rows and the 16 x OCF weight rows of the tile) is fetched with adjacent lanes on
+// adjacent 16 bytes, parked in LDS (row pitch 272 bytes: the 16-byte reads of 8 consecutive rows fall into distinct
+// banks), and the waves read their fragments from there. Wave w owns timesteps (w % TG) * TPW ... and, when fewer than 8
+// timesteps leave waves to spare, every KSPLIT-th K step of the slab. The next slab's loads are in flight while the
+// current one multiplies. The accumulators meet in LDS (aliasing the slab) for the LIF recurrence.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kStagedWaves = 8;
+constexpr int kSlabK = 128;                       // K elements per slab = 4 matrix K steps (256: +6 % on one workgroup per
+                                                  // CU, -25 % where several fit a CU)
+constexpr int kSlabOctets = kSlabK / 8;           // 16-byte staging items per operand row
+constexpr int kSlabPitch = kSlabK * 2 + 16;       // bytes per operand row in LDS
+
+template <int TT, int OCF> struct StagedShape {
+    static constexpr int TPW = TT >= 8 ? TT / 8 : 1;            // timesteps per wave
+    static constexpr int TG = TT / TPW;                          // wave groups along time
+    static constexpr int KSPLIT = kStagedWaves / TG;             // waves sharing the K steps of a slab
+    static constexpr int ROWS = TT * kTileM + OCF * kTileOC;     // operand rows per slab
+    static constexpr int ITEMS = (ROWS * (kSlabK / 8) + kStagedWaves * 64 - 1) / (kStagedWaves * 64);   // octets per thread
+    static constexpr int PITCH = OCF * kTileOC + 4;              // floats per row of an accumulator tile in LDS
+    static constexpr size_t slab_bytes = static_cast<size_t>(ROWS) * kSlabPitch;
+    static constexpr size_t acc_bytes = static_cast<size_t>(KSPLIT) * TT * kTileM * PITCH * sizeof(float);
+    static constexpr size_t lds_bytes = slab_bytes > acc_bytes ? slab_bytes : acc_bytes;
+};
+
+template <typename XT, typename VT, int TT, int OCF>
+__global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
+                                                                              const XT* __restrict__ bias,
+                                                                              const VT* __restrict__ v_init, XT* __restrict__ spikes,
+                                                                              VT* __restrict__ v_out, LifParams lif) {
+    using SH = StagedShape<TT, OCF>;
+    constexpr int NT = kStagedWaves * 64;
+    constexpr int TILE_OC = OCF * kTileOC;
+    constexpr int OUTS = TILE_OC * kTileM;
+    extern __shared__ __align__(16) unsigned char staged_lds[];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int oc0 = blockIdx.x * TILE_OC;
+    const int m0 = blockIdx.y * kTileM;
+
+    // Staging items of this thread: item i = tid + j * NT is octet i % 16 of operand row i / 16 (NT is a multiple of 16, so
+    // the octet is the same for all of a thread's items). Rows beyond M / Fout re-read the last real row; what they produce
+    // is never stored.
+    const int octet = tid % kSlabOctets;
+    const XT* item_row[SH::ITEMS];
+    uint32_t item_dst[SH::ITEMS];
+    bool item_live[SH::ITEMS];
+#pragma unroll
+    for (int j = 0; j < SH::ITEMS; ++j) {
+        const int row = tid / kSlabOctets + j * (NT / kSlabOctets);
+        item_live[j] = row < SH::ROWS;
+        const int r = item_live[j] ? row : 0;
+        const XT* ptr;
+        if (r < TT * kTileM) {
+            const int t = r / kTileM;
+            const void* base = xs.p[0];
+#pragma unroll
+            for (int u = 1; u < TT; ++u) base = t == u ? xs.p[u] : base;
+            ptr = static_cast<const XT*>(base) + static_cast<int64_t>(min(m0 + r % kTileM, g.M - 1)) * g.x_row_stride;
+        } else {
+            ptr = W + static_cast<int64_t>(min(oc0 + r - TT * kTileM, g.Fout - 1)) * g.Fin;
+        }
+        item_row[j] = ptr;
+        item_dst[j] = static_cast<uint32_t>(r * kSlabPitch + octet * 16);
+    }
+
+    const int tg = wave % SH::TG;
+    const int kp = wave / SH::TG;
+    f32x4 acc[OCF][SH::TPW];
+#pragma unroll
+    for (int f = 0; f < OCF; ++f)
+#pragma unroll
+        for (int u = 0; u < SH::TPW; ++u) acc[f][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // One slab ahead in registers (deeper rings measured slower: the slab loop is bound by LDS traffic and its two
+    // barriers, not by the latency of the loads).
+    constexpr int DEPTH = 1;
+    u32x4 pre[DEPTH][SH::ITEMS];
+    auto fetch = [&](int slab, u32x4 (&dst)[SH::ITEMS]) __attribute__((always_inline)) {
+        const int k = slab * kSlabK + octet * 8;
+#pragma unroll
+        for (int j = 0; j < SH::ITEMS; ++j)
+            if (item_live[j]) dst[j] = load_octet<XT, true>(item_row[j], k, g.Fin);
+    };
+    const int nslabs = (g.Fin + kSlabK - 1) / kSlabK;
+    // Fragment addresses in the slab: lane = 16 q + r reads K elements 8 q .. 8 q + 7 of row r of its fragment.
+    const uint32_t frag_off = static_cast<uint32_t>((lane & 15) * kSlabPitch + (lane >> 4) * 16);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < nslabs) fetch(d, pre[d]);
+    for (int slab0 = 0; slab0 < nslabs; slab0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int slab = slab0 + d;
+            if (slab < nslabs) {                                       // uniform
+#pragma unroll
+                for (int j = 0; j < SH::ITEMS; ++j)
+                    if (item_live[j]) *reinterpret_cast<u32x4*>(staged_lds + item_dst[j]) = pre[d][j];
+                __syncthreads();
+                if (slab + DEPTH < nslabs) fetch(slab + DEPTH, pre[d]);
+#pragma unroll
+                for (int ks = 0; ks < kSlabK / 32; ++ks) {
+                    if (ks % SH::KSPLIT != kp % SH::KSPLIT) continue;      // wave-uniform
+                    u32x4 a[OCF];
+#pragma unroll
+                    for (int f = 0; f < OCF; ++f)
+                        a[f] = *reinterpret_cast<const u32x4*>(staged_lds + (TT * kTileM + f * kTileOC) * kSlabPitch + frag_off + ks * 64);
+#pragma unroll
+                    for (int u = 0; u < SH::TPW; ++u) {
+                        const int t = tg * SH::TPW + u;
+                        const u32x4 b = *reinterpret_cast<const u32x4*>(staged_lds + t * kTileM * kSlabPitch + frag_off + ks * 64);
+#pragma unroll
+                        for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[f], b, acc[f][u]);
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    // Accumulators -> LDS as [K part][t][m][PITCH]; D[i = oc][j = m]: lane holds column j = lane % 16, rows 4 (lane / 16) + r.
+    float* partial = reinterpret_cast<float*>(staged_lds);
+    constexpr int SLAB_F = kTileM * SH::PITCH;
+#pragma unroll
+    for (int u = 0; u < SH::TPW; ++u)
+#pragma unroll
+        for (int f = 0; f < OCF; ++f)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                partial[(kp * TT + tg * SH::TPW + u) * SLAB_F + (lane & 15) * SH::PITCH + f * kTileOC + (lane >> 4) * 4 + r] = acc[f][u][r];
+    __syncthreads();
+
+    for (int e = tid; e < OUTS; e += NT) {
+        const int slot = (e / TILE_OC) * SH::PITCH + e % TILE_OC;
+        const int m = m0 + e / TILE_OC;
+        const int oc = oc0 + e % TILE_OC;
+        if (m >= g.M || oc >= g.Fout) continue;
+        const float bv = bias != nullptr ? to_float(bias[oc]) : 0.0f;
+        const int64_t o = static_cast<int64_t>(m) * g.Fout + oc;
+        float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+            if (t >= g.T) break;
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+            const float cur = sum + bv;
+            spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+        }
+        v_out[o] = from_float<VT>(v);
+    }
+}
+
+template <typename XT, typename VT, int TT, int OCF>
+int launch_staged(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+                  void* v_out, const LifParams& lif, hipStream_t stream) {
+    using SH = StagedShape<TT, OCF>;
+    static_assert(SH::lds_bytes <= 160 * 1024, "slab exceeds LDS");
+    const dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
+    if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
+    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF>;
+    if (SH::lds_bytes > 64 * 1024) {
+        static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(SH::lds_bytes));
+        if (raised != hipSuccess) return fail(SNNF_ERR_LAUNCH, "snnf_linear_lif: cannot reserve %zu bytes of LDS", SH::lds_bytes);
+    }
+    kernel<<<grid, kStagedWaves * 64, SH::lds_bytes, stream>>>(xs, g, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                                               static_cast<const VT*>(v_init), static_cast<XT*>(spikes),
+                                                               static_cast<VT*>(v_out), lif);
+    return check_launch("snnf_linear_lif");
 }
 
 template <typename XT, typename VT, bool FAST>
 int launch_tt(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
               void* v_out, const LifParams& lif, hipStream_t stream) {
-    const dim3 grid((g.Fout + kTileOC - 1) / kTileOC, (g.M + kTileM - 1) / kTileM);
-    if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
-    const XT* w = static_cast<const XT*>(W);
-    const XT* b = static_cast<const XT*>(bias);
-    const VT* vi = static_cast<const VT*>(v_init);
-    XT* sp = static_cast<XT*>(spikes);
-    VT* vo = static_cast<VT*>(v_out);
-    if (g.T <= 1) linear_lif_kernel<XT, VT, 1, FAST><<<grid, LinWaves<1>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 2) linear_lif_kernel<XT, VT, 2, FAST><<<grid, LinWaves<2>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 4) linear_lif_kernel<XT, VT, 4, FAST><<<grid, LinWaves<4>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else if (g.T <= 8) linear_lif_kernel<XT, VT, 8, FAST><<<grid, LinWaves<8>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    else linear_lif_kernel<XT, VT, 16, FAST><<<grid, LinWaves<16>::value * 64, 0, stream>>>(xs, g, w, b, vi, sp, vo, lif);
-    return check_launch("snnf_linear_lif");
+    // Two feature fragments per workgroup (half the activation traffic) when that still leaves at least 128 workgroups.
+    const bool wide = g.Fout % (2 * kTileOC) == 0 &&
+                      static_cast<int64_t>(g.Fout / (2 * kTileOC)) * ((g.M + kTileM - 1) / kTileM) >= 128;
+    if constexpr (FAST) {
+        if (g.T > 2) {
+            if (wide) {
+                if (g.T <= 4) return launch_staged<XT, VT, 4, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                if (g.T <= 8) return launch_staged<XT, VT, 8, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                return launch_staged<XT, VT, 16, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            }
+            if (g.T <= 4) return launch_staged<XT, VT, 4, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            if (g.T <= 8) return launch_staged<XT, VT, 8, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            return launch_staged<XT, VT, 16, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+        }
+    }
+    if (g.T <= 1) return launch_one<XT, VT, 1, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    if (g.T <= 2) return launch_one<XT, VT, 2, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    if (g.T <= 4) return launch_one<XT, VT, 4, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    if (g.T <= 8) return launch_one<XT, VT, 8, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_one<XT, VT, 16, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 template <typename XT, typename VT>
@@ -221,7 +443,7 @@ extern "C" int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int
         int tt = 1;
         while (tt < tw) tt *= 2;
         StepPtrs ptrs = {};
-        bool fast = Fin % per16 == 0 && x_row_stride % per16 == 0 && aligned_to(weight, 16);
+        bool fast = Fin % 8 == 0 && x_row_stride % per16 == 0 && aligned_to(weight, 16);
         for (int t = 0; t < tt; ++t) {
             ptrs.p[t] = xs[t0 + (t < tw ? t : 0)];  // padded steps re-read step 0 and are never stored
             fast = fast && aligned_to(ptrs.p[t], 16);
