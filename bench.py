@@ -42,6 +42,8 @@ def _parse():
     ap.add_argument("--model", default=None, choices=["resnet18", "vgg11"],
                     help="end-to-end forward of the spiking ResNet-18 (T=4, B=16, 224x224) or VGG-11 (T=4, B=64, 32x32) "
                          "network through the fused operators, replayed as one HIP graph")
+    ap.add_argument("--streaming", action="store_true",
+                    help="time only the temporal LIF scan and the LIF -> average pool -> linear tail, each alone")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only copy 256 MiB device to device three times: the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -457,6 +459,14 @@ def main() -> int:
         stats = ops.get_fused_op_call_stats()
         sweep["native_calls"], sweep["fallback_calls"] = stats["triton"], stats["fallback"]
         print(json.dumps(sweep))
+        return 0 if stats["fallback"] == 0 else 1
+
+    if args.streaming:
+        res = {"metric": METRIC, "workload": "streaming_operators", "dtype": args.dtype,
+               "operators": _streaming_operators(dtype, args.steps, args.warmup)}
+        stats = ops.get_fused_op_call_stats()
+        res["native_calls"], res["fallback_calls"] = stats["triton"], stats["fallback"]
+        print(json.dumps(res))
         return 0 if stats["fallback"] == 0 else 1
 
     if args.model is not None:

@@ -6,6 +6,9 @@
 // materialised per step. Launch 1 streams x once (HBM-bound, 16-byte accesses where the operands allow), keeps the membrane
 // in registers, counts spikes per plane in LDS and writes the integer counts to the workspace; launch 2 is a small GEMV
 // over the counts with wave-shuffle reductions.
+#include <algorithm>
+#include <type_traits>
+
 #include "snnf_common.h"
 
 namespace snnf {
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void lif_pool_kernel(StepPtrs xs, int T, 
 // aligned; only the last 8 neurons of the last workgroup may be ragged and are moved one by one.
 constexpr int kVec = 8;
 
-template <typename XT, typename VT>
+template <typename XT, typename VT, int TC>
 __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int T, int planes, int HW, int planes_per_block,
                                                                 const VT* __restrict__ v_init, VT* __restrict__ v_out,
                                                                 int* __restrict__ counts, LifParams lif) {
@@ -83,8 +86,10 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
     for (int i = threadIdx.x; i < planes_here; i += kThreads) plane_count[i] = 0;
     __syncthreads();
 
-    for (int i0 = threadIdx.x * kVec; i0 < elems; i0 += kThreads * kVec) {
-        const bool whole = i0 + kVec <= elems;
+    // A workgroup whose neuron count is a multiple of 8 (all but, at most, the last one) moves whole vectors only; its
+    // loop body has no branch around a load, so all loads of a pass are in flight together.
+    auto pass = [&](int i0, auto whole_tag) __attribute__((always_inline)) {
+        constexpr bool whole = decltype(whole_tag)::value;
         float v[kVec];
         int fired[kVec];
 #pragma unroll
@@ -93,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
             fired[j] = 0;
         }
         if (v_init != nullptr) {
-            if (whole) {
+            if constexpr (whole) {
                 const Pack<VT, kVec> pv = *reinterpret_cast<const Pack<VT, kVec>*>(v_init + base + i0);
 #pragma unroll
                 for (int j = 0; j < kVec; ++j) v[j] = to_float(pv.v[j]);
@@ -103,29 +108,41 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
                     if (i0 + j < elems) v[j] = to_float(v_init[base + i0 + j]);
             }
         }
-        for (int t0 = 0; t0 < T; t0 += 4) {
-            Pack<XT, kVec> px[4];
+        if constexpr (whole && TC > 0) {
+            // T == TC known at compile time: every timestep's load is issued before the recurrence starts. (Fetching
+            // the next pass ahead as well measured no faster.)
+            Pack<XT, kVec> px[TC > 0 ? TC : 1];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (t0 + u < T) {
-                    const XT* __restrict__ x = static_cast<const XT*>(xs.p[t0 + u]) + base + i0;
-                    if (whole) {
-                        px[u] = *reinterpret_cast<const Pack<XT, kVec>*>(x);
-                    } else {
+            for (int t = 0; t < TC; ++t) px[t] = *reinterpret_cast<const Pack<XT, kVec>*>(static_cast<const XT*>(xs.p[t]) + base + i0);
 #pragma unroll
-                        for (int j = 0; j < kVec; ++j) px[u].v[j] = i0 + j < elems ? x[j] : XT{};
+            for (int t = 0; t < TC; ++t)
+#pragma unroll
+                for (int j = 0; j < kVec; ++j) fired[j] += lif_step(to_float(px[t].v[j]), v[j], lif) ? 1 : 0;
+        } else {
+            for (int t0 = 0; t0 < T; t0 += 4) {
+                Pack<XT, kVec> px[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (t0 + u < T) {
+                        const XT* __restrict__ x = static_cast<const XT*>(xs.p[t0 + u]) + base + i0;
+                        if constexpr (whole) {
+                            px[u] = *reinterpret_cast<const Pack<XT, kVec>*>(x);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < kVec; ++j) px[u].v[j] = i0 + j < elems ? x[j] : XT{};
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (t0 + u < T) {
+#pragma unroll
+                        for (int j = 0; j < kVec; ++j) fired[j] += lif_step(to_float(px[u].v[j]), v[j], lif) ? 1 : 0;
                     }
                 }
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (t0 + u < T) {
-#pragma unroll
-                    for (int j = 0; j < kVec; ++j) fired[j] += lif_step(to_float(px[u].v[j]), v[j], lif) ? 1 : 0;
-                }
-            }
         }
-        if (whole) {
+        if constexpr (whole) {
             Pack<VT, kVec> pv;
 #pragma unroll
             for (int j = 0; j < kVec; ++j) pv.v[j] = from_float<VT>(v[j]);
@@ -135,23 +152,42 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
             for (int j = 0; j < kVec; ++j)
                 if (i0 + j < elems) v_out[base + i0 + j] = from_float<VT>(v[j]);
         }
-        // Spikes of consecutive neurons of one plane are summed before they go to that plane's counter.
+        // Spikes of consecutive neurons of one plane are summed before they go to that plane's counter; a wave whose
+        // neurons all lie in one plane adds them up with shuffles first (one LDS atomic per wave instead of 64 on the
+        // same address).
         int p = i0 / HW;
         int rem = i0 - p * HW;
-        int run = 0;
+        const bool one_plane = rem + kVec <= HW && whole;      // this thread's 8 neurons lie inside plane p
+        const int lead = __shfl(p, 0);
+        const bool full_wave = __builtin_amdgcn_ballot_w64(true) == ~0ull;   // the shuffles below need all 64 lanes
+        if (full_wave && __all(one_plane && p == lead)) {
+            int sum = 0;
 #pragma unroll
-        for (int j = 0; j < kVec; ++j) {
-            if (i0 + j < elems) {
-                run += fired[j];
-                if (++rem == HW) {
-                    if (run != 0) atomicAdd(&plane_count[p], run);
-                    run = 0;
-                    rem = 0;
-                    ++p;
+            for (int j = 0; j < kVec; ++j) sum += fired[j];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+            if ((threadIdx.x & 63) == 0 && sum != 0) atomicAdd(&plane_count[lead], sum);
+        } else {
+            int run = 0;
+#pragma unroll
+            for (int j = 0; j < kVec; ++j) {
+                if (i0 + j < elems) {
+                    run += fired[j];
+                    if (++rem == HW) {
+                        if (run != 0) atomicAdd(&plane_count[p], run);
+                        run = 0;
+                        rem = 0;
+                        ++p;
+                    }
                 }
             }
+            if (run != 0) atomicAdd(&plane_count[p], run);
         }
-        if (run != 0) atomicAdd(&plane_count[p], run);
+    };
+    if (elems % kVec == 0) {
+        for (int i0 = threadIdx.x * kVec; i0 < elems; i0 += kThreads * kVec) pass(i0, std::true_type{});
+    } else {
+        for (int i0 = threadIdx.x * kVec; i0 < elems; i0 += kThreads * kVec) pass(i0, std::false_type{});
     }
     __syncthreads();
     for (int i = threadIdx.x; i < planes_here; i += kThreads) counts[plane0 + i] = plane_count[i];
@@ -189,21 +225,32 @@ __global__ __launch_bounds__(kThreads) void count_linear_kernel(const int* __res
 }
 
 // Vector variant (C a multiple of 8, 16-byte aligned weight): no LDS and no barrier; a lane fetches 8 consecutive weights
-// of each of its wave's rows with 16-byte loads, all rows in flight together, and the 8 matching counts once.
+// of each of its wave's kRowsPerWave rows with 16-byte loads, all rows in flight together, and the 8 matching counts of
+// kSamplesPerWave samples (1: sharing a weight vector among 4 samples saved 2 % at 64 samples x 1000 classes and cost
+// 15-20 % at the sizes of the network tails, where the shuffle reductions of a wave then run one after the other).
+constexpr int kSamplesPerWave = 1;
+
 template <typename XT>
-__global__ __launch_bounds__(kThreads) void count_linear_vec_kernel(const int* __restrict__ counts, int C, int K,
+__global__ __launch_bounds__(kThreads) void count_linear_vec_kernel(const int* __restrict__ counts, int N, int C, int K,
                                                                     const XT* __restrict__ W, const XT* __restrict__ bias,
                                                                     XT* __restrict__ out, float inv_hw, float steps) {
-    const int n = blockIdx.y;
+    const int n0 = blockIdx.y * kSamplesPerWave;
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int k0 = (blockIdx.x * (kThreads / 64) + wave) * kRowsPerWave;
     if (k0 >= K) return;
-    float acc[kRowsPerWave];
+    float acc[kRowsPerWave][kSamplesPerWave];
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+        for (int i = 0; i < kSamplesPerWave; ++i) acc[r][i] = 0.0f;
     for (int c0 = lane * kVec; c0 < C; c0 += 64 * kVec) {
-        const Pack<int, kVec> pc = *reinterpret_cast<const Pack<int, kVec>*>(counts + static_cast<int64_t>(n) * C + c0);
+        Pack<int, kVec> pc[kSamplesPerWave];
+#pragma unroll
+        for (int i = 0; i < kSamplesPerWave; ++i) {
+            const int n = min(n0 + i, N - 1);   // samples beyond N re-read the last one and are not stored
+            pc[i] = *reinterpret_cast<const Pack<int, kVec>*>(counts + static_cast<int64_t>(n) * C + c0);
+        }
         Pack<XT, kVec> pw[kRowsPerWave];
 #pragma unroll
         for (int r = 0; r < kRowsPerWave; ++r) {
@@ -213,21 +260,29 @@ __global__ __launch_bounds__(kThreads) void count_linear_vec_kernel(const int* _
 #pragma unroll
         for (int r = 0; r < kRowsPerWave; ++r)
 #pragma unroll
-            for (int j = 0; j < kVec; ++j) acc[r] = fmaf(to_float(pw[r].v[j]), static_cast<float>(pc.v[j]), acc[r]);
+            for (int j = 0; j < kVec; ++j) {
+                const float w = to_float(pw[r].v[j]);
+#pragma unroll
+                for (int i = 0; i < kSamplesPerWave; ++i) acc[r][i] = fmaf(w, static_cast<float>(pc[i].v[j]), acc[r][i]);
+            }
     }
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r) {
+    for (int r = 0; r < kRowsPerWave; ++r)
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) acc[r] += __shfl_xor(acc[r], off);
-    }
+        for (int i = 0; i < kSamplesPerWave; ++i) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc[r][i] += __shfl_xor(acc[r][i], off);
+        }
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < kRowsPerWave; ++r) {
             const int k = k0 + r;
-            if (k < K) {
-                float o = acc[r] * inv_hw;
-                if (bias != nullptr) o += steps * to_float(bias[k]);
-                out[static_cast<int64_t>(n) * K + k] = from_float<XT>(o);
+            if (k >= K) continue;
+            const float bv = bias != nullptr ? steps * to_float(bias[k]) : 0.0f;
+#pragma unroll
+            for (int i = 0; i < kSamplesPerWave; ++i) {
+                const int n = n0 + i;
+                if (n < N) out[static_cast<int64_t>(n) * K + k] = from_float<XT>(acc[r][i] * inv_hw + bv);
             }
         }
     }
@@ -240,18 +295,33 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
     // of 8 neurons, all bases 16-byte aligned.
     bool aligned = aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16));
     for (int t = 0; t < T; ++t) aligned = aligned && aligned_to(xs.p[t], 16);
-    int vpb = (kThreads * kVec) / HW;
-    if (vpb < 1) vpb = 1;
-    if (vpb > kMaxPlanes) vpb = kMaxPlanes;
-    int tries = 0;
-    while (vpb > 1 && vpb < planes && (static_cast<int64_t>(vpb) * HW) % kVec != 0 && tries < kVec) {
-        --vpb;
-        ++tries;
+    // Planes per workgroup: whole planes, a multiple of 8 neurons per workgroup, up to 4 passes of kThreads * kVec neurons,
+    // chosen for the fewest idle lanes in the last pass (the first candidate wins unless a smaller one is 2 % better).
+    const int pass_elems = kThreads * kVec;
+    int vpb = 0;
+    double best_eff = 0.0;
+    // Several passes per workgroup only while that leaves 1024 workgroups or more.
+    const int64_t one_pass = std::max<int64_t>(1, pass_elems / HW);
+    const int64_t cand_max = std::min<int64_t>(std::max<int64_t>(1, (4 * pass_elems) / HW), std::max<int64_t>(one_pass, planes / 1024));
+    for (int cand = static_cast<int>(std::min<int64_t>(kMaxPlanes, cand_max)); cand >= 1; --cand) {
+        const int64_t e = static_cast<int64_t>(cand) * HW;
+        if (cand < planes && e % kVec != 0) continue;
+        const int64_t passes = (e + pass_elems - 1) / pass_elems;
+        const double eff = static_cast<double>(e) / static_cast<double>(passes * pass_elems);
+        if (eff > best_eff + 0.02) {
+            best_eff = eff;
+            vpb = cand;
+        }
+        if (cand >= planes) break;   // one workgroup holds everything: nothing smaller to consider
     }
-    if (aligned && (vpb >= planes || (static_cast<int64_t>(vpb) * HW) % kVec == 0)) {
+    if (aligned && vpb > 0) {
+        if (vpb > planes) vpb = planes;
         const int blocks = (planes + vpb - 1) / vpb;
-        lif_pool_vec_kernel<XT, VT><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, static_cast<const VT*>(v_init),
-                                                                          static_cast<VT*>(v_out), counts, lif);
+        const VT* vi = static_cast<const VT*>(v_init);
+        VT* vo = static_cast<VT*>(v_out);
+        if (T == 4) lif_pool_vec_kernel<XT, VT, 4><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
+        else if (T == 8) lif_pool_vec_kernel<XT, VT, 8><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
+        else lif_pool_vec_kernel<XT, VT, 0><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
         return check_launch("snnf_lif_pool_linear(pool)");
     }
     int ppb = (kThreads * kItems) / HW;
@@ -266,10 +336,12 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
 template <typename XT>
 void run_linear(bool vec, dim3 grid, size_t lds, hipStream_t hs, const int* counts, int C, int K, const void* W, const void* bias,
                 void* out, float inv_hw, float steps) {
-    if (vec)
-        count_linear_vec_kernel<XT><<<grid, kThreads, 0, hs>>>(counts, C, K, static_cast<const XT*>(W), static_cast<const XT*>(bias),
-                                                              static_cast<XT*>(out), inv_hw, steps);
-    else
+    if (vec) {
+        const int N = static_cast<int>(grid.y);
+        const dim3 vgrid(grid.x, (N + kSamplesPerWave - 1) / kSamplesPerWave);
+        count_linear_vec_kernel<XT><<<vgrid, kThreads, 0, hs>>>(counts, N, C, K, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                                               static_cast<XT*>(out), inv_hw, steps);
+    } else
         count_linear_kernel<XT><<<grid, kThreads, lds, hs>>>(counts, C, K, static_cast<const XT*>(W), static_cast<const XT*>(bias),
                                                             static_cast<XT*>(out), inv_hw, steps);
 }
