@@ -113,9 +113,11 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw
     for (int wk_log2 = 0; wk_log2 <= nw_log2; ++wk_log2) {
         if ((1 << wk_log2) > g0.npairs) break;
         // Measured on layers that fill the machine without it: splitting pays from K of about 1152 on. A layer of real size
-        // (4096 output pixels or more) whose unsplit tiles occupy less than half of the CUs splits at any K.
-        const double unsplit_groups = static_cast<double>(g0.N) * g0.Ho * g0.Wo * g0.Cout / (nw * 64.0 * 32.0);
-        const bool starved = static_cast<int64_t>(g0.N) * g0.Ho * g0.Wo >= 4096 && unsplit_groups * 2.0 < cus;
+        // (2^18 outputs per timestep or more) whose unsplit tiles occupy less than a quarter of the CUs splits at any K
+        // (with the bar at a half, the 3x3/2 and 1x1/2 64->128 layers at 56x56 lost 25-35 %).
+        const double outputs = static_cast<double>(g0.N) * g0.Ho * g0.Wo * g0.Cout;
+        const double unsplit_groups = outputs / (nw * 64.0 * 32.0);
+        const bool starved = outputs >= 262144.0 && unsplit_groups * 4.0 < cus;
         if (wk_log2 > 0 && g0.nchunks * g0.npairs < 72 && !starved) break;
         const int max_items = nw * 64 * ((wk_log2 > 0 && load_mode == LOAD_PAIR32 && tt >= 2) ? slots / 2 : slots);
         for (int wn_log2 = 0; wn_log2 + wk_log2 <= nw_log2; ++wn_log2) {
