@@ -230,7 +230,7 @@ template <int TT, int OCF> struct StagedShape {
     static constexpr size_t lds_bytes = slab_bytes > acc_bytes ? slab_bytes : acc_bytes;
 };
 
-template <typename XT, typename VT, int TT, int OCF>
+template <typename XT, typename VT, int TT, int OCF, bool DB>
 __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
                                                                               const XT* __restrict__ bias,
                                                                               const VT* __restrict__ v_init, XT* __restrict__ spikes,
@@ -280,51 +280,46 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
 #pragma unroll
         for (int u = 0; u < SH::TPW; ++u) acc[f][u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // One slab ahead in registers (deeper rings measured slower: the slab loop is bound by LDS traffic and its two
-    // barriers, not by the latency of the loads).
-    constexpr int DEPTH = 1;
-    u32x4 pre[DEPTH][SH::ITEMS];
-    auto fetch = [&](int slab, u32x4 (&dst)[SH::ITEMS]) __attribute__((always_inline)) {
+    // One slab ahead in registers (deeper rings measured slower: the slab loop is bound by LDS traffic and its barriers,
+    // not by the latency of the loads). DB: two slab buffers in LDS, so that a slab costs one barrier instead of two
+    // (writing buffer b for slab s + 1 cannot overtake the reads of slab s - 1, which every wave finished before the
+    // barrier of slab s).
+    u32x4 pre[SH::ITEMS];
+    auto fetch = [&](int slab) __attribute__((always_inline)) {
         const int k = slab * kSlabK + octet * 8;
 #pragma unroll
         for (int j = 0; j < SH::ITEMS; ++j)
-            if (item_live[j]) dst[j] = load_octet<XT, true>(item_row[j], k, g.Fin);
+            if (item_live[j]) pre[j] = load_octet<XT, true>(item_row[j], k, g.Fin);
     };
     const int nslabs = (g.Fin + kSlabK - 1) / kSlabK;
     // Fragment addresses in the slab: lane = 16 q + r reads K elements 8 q .. 8 q + 7 of row r of its fragment.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 15) * kSlabPitch + (lane >> 4) * 16);
+    fetch(0);
+    for (int slab = 0; slab < nslabs; ++slab) {
+        unsigned char* buf = staged_lds + (DB ? (slab & 1) * SH::slab_bytes : 0);
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d)
-        if (d < nslabs) fetch(d, pre[d]);
-    for (int slab0 = 0; slab0 < nslabs; slab0 += DEPTH) {
+        for (int j = 0; j < SH::ITEMS; ++j)
+            if (item_live[j]) *reinterpret_cast<u32x4*>(buf + item_dst[j]) = pre[j];
+        __syncthreads();
+        if (slab + 1 < nslabs) fetch(slab + 1);
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int slab = slab0 + d;
-            if (slab < nslabs) {                                       // uniform
+        for (int ks = 0; ks < kSlabK / 32; ++ks) {
+            if (ks % SH::KSPLIT != kp % SH::KSPLIT) continue;      // wave-uniform
+            u32x4 a[OCF];
 #pragma unroll
-                for (int j = 0; j < SH::ITEMS; ++j)
-                    if (item_live[j]) *reinterpret_cast<u32x4*>(staged_lds + item_dst[j]) = pre[d][j];
-                __syncthreads();
-                if (slab + DEPTH < nslabs) fetch(slab + DEPTH, pre[d]);
+            for (int f = 0; f < OCF; ++f)
+                a[f] = *reinterpret_cast<const u32x4*>(buf + (TT * kTileM + f * kTileOC) * kSlabPitch + frag_off + ks * 64);
 #pragma unroll
-                for (int ks = 0; ks < kSlabK / 32; ++ks) {
-                    if (ks % SH::KSPLIT != kp % SH::KSPLIT) continue;      // wave-uniform
-                    u32x4 a[OCF];
+            for (int u = 0; u < SH::TPW; ++u) {
+                const int t = tg * SH::TPW + u;
+                const u32x4 b = *reinterpret_cast<const u32x4*>(buf + t * kTileM * kSlabPitch + frag_off + ks * 64);
 #pragma unroll
-                    for (int f = 0; f < OCF; ++f)
-                        a[f] = *reinterpret_cast<const u32x4*>(staged_lds + (TT * kTileM + f * kTileOC) * kSlabPitch + frag_off + ks * 64);
-#pragma unroll
-                    for (int u = 0; u < SH::TPW; ++u) {
-                        const int t = tg * SH::TPW + u;
-                        const u32x4 b = *reinterpret_cast<const u32x4*>(staged_lds + t * kTileM * kSlabPitch + frag_off + ks * 64);
-#pragma unroll
-                        for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[f], b, acc[f][u]);
-                    }
-                }
-                __syncthreads();
+                for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[f], b, acc[f][u]);
             }
         }
+        if (!DB) __syncthreads();
     }
+    if (DB) __syncthreads();
 
     // Accumulators -> LDS as [K part][t][m][PITCH]; D[i = oc][j = m]: lane holds column j = lane % 16, rows 4 (lane / 16) + r.
     float* partial = reinterpret_cast<float*>(staged_lds);
@@ -359,23 +354,37 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     }
 }
 
+template <typename XT, typename VT, int TT, int OCF, bool DB>
+int launch_staged_db(dim3 grid, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+                     void* v_out, const LifParams& lif, hipStream_t stream) {
+    using SH = StagedShape<TT, OCF>;
+    constexpr size_t lds = DB ? 2 * SH::slab_bytes : SH::lds_bytes;
+    static_assert(lds <= 160 * 1024 && SH::acc_bytes <= lds, "slabs exceed LDS");
+    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB>;
+    if (lds > 64 * 1024) {
+        static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (raised != hipSuccess) return fail(SNNF_ERR_LAUNCH, "snnf_linear_lif: cannot reserve %zu bytes of LDS", lds);
+    }
+    kernel<<<grid, kStagedWaves * 64, lds, stream>>>(xs, g, static_cast<const XT*>(W), static_cast<const XT*>(bias),
+                                                     static_cast<const VT*>(v_init), static_cast<XT*>(spikes),
+                                                     static_cast<VT*>(v_out), lif);
+    return check_launch("snnf_linear_lif");
+}
+
 template <typename XT, typename VT, int TT, int OCF>
 int launch_staged(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
                   void* v_out, const LifParams& lif, hipStream_t stream) {
     using SH = StagedShape<TT, OCF>;
-    static_assert(SH::lds_bytes <= 160 * 1024, "slab exceeds LDS");
     const dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
     if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
-    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF>;
-    if (SH::lds_bytes > 64 * 1024) {
-        static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(SH::lds_bytes));
-        if (raised != hipSuccess) return fail(SNNF_ERR_LAUNCH, "snnf_linear_lif: cannot reserve %zu bytes of LDS", SH::lds_bytes);
+    // Two slab buffers where a CU gets one workgroup anyway (they would cost occupancy otherwise) and both fit LDS.
+    constexpr bool can_double = 2 * SH::slab_bytes <= 160 * 1024;
+    if constexpr (can_double) {
+        if (static_cast<int64_t>(grid.x) * grid.y <= compute_units())
+            return launch_staged_db<XT, VT, TT, OCF, true>(grid, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     }
-    kernel<<<grid, kStagedWaves * 64, SH::lds_bytes, stream>>>(xs, g, static_cast<const XT*>(W), static_cast<const XT*>(bias),
-                                                               static_cast<const VT*>(v_init), static_cast<XT*>(spikes),
-                                                               static_cast<VT*>(v_out), lif);
-    return check_launch("snnf_linear_lif");
+    return launch_staged_db<XT, VT, TT, OCF, false>(grid, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 template <typename XT, typename VT, bool FAST>
