@@ -68,14 +68,21 @@ __global__ __launch_bounds__(kThreads) void pool2d_s2_vec_kernel(const XT* __res
     for (int j = 0; j < 4; ++j) acc[j] = IS_MAX ? -3.0e38f : 0.0f;
 #pragma unroll
     for (int ky = 0; ky < K; ++ky) {
-        const int iy = oy * 2 - PAD + ky;
-        if (iy < 0 || iy >= H) continue;
+        // No branch around a load (the compiler would wait for each load before issuing the next): a window row outside
+        // the plane re-reads the nearest row inside, which belongs to the same window and leaves a maximum unchanged
+        // (unpadded 2x2 windows never leave the plane); the column left of the first one re-reads the first.
+        const int iy = min(max(oy * 2 - PAD + ky, 0), H - 1);
         const XT* __restrict__ line = src + static_cast<int64_t>(iy) * W;
         const Pack<XT, 8> eight = *reinterpret_cast<const Pack<XT, 8>*>(line);
         float v[9];
 #pragma unroll
         for (int c = 0; c < 8; ++c) v[1 + c] = to_float(eight.v[c]);
-        v[0] = (PAD == 1 && ox0 > 0) ? to_float(line[-1]) : -3.0e38f;
+        if constexpr (PAD == 1) {
+            const float left = to_float(line[ox0 > 0 ? -1 : 0]);
+            v[0] = ox0 > 0 ? left : -3.0e38f;
+        } else {
+            v[0] = -3.0e38f;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             if constexpr (K == 3) acc[j] = fmaxf(fmaxf(acc[j], v[2 * j]), fmaxf(v[2 * j + 1], v[2 * j + 2]));
