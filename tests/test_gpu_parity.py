@@ -257,6 +257,25 @@ def test_conv_lif_kernel_keys(hip_ops, dtype, vdtype, k, s, p, Cin, Cout, H, W, 
     _no_fallback(hip_ops, 1)
 
 
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p", [(32, 64, 12, 12, 3, 1, 1), (64, 64, 9, 9, 3, 1, 1), (16, 32, 8, 10, 1, 2, 0)])
+def test_conv_lif_activations_at_two_byte_alignment(hip_ops, Cin, Cout, H, W, k, s, p):
+    """Timestep tensors that start one element into their storage: even widths then take the two-loads-per-pair path, odd
+    widths the paired 4-byte loads at 2-byte alignment."""
+    T, N = 4, 2
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(650 + H, T, N, Cin, Cout, H, W, k, BF16)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, torch.tensor(0.0), (s, s), (p, p), (1, 1), 1, *LIF)
+    shifted = []
+    for x in xs:
+        store = torch.zeros(x.numel() + 1, device=DEV, dtype=BF16)
+        view = store[1:].view(x.shape)
+        view.copy_(x.to(DEV, BF16))
+        assert view.data_ptr() % 4 == 2 and view.is_contiguous()
+        shifted.append(view)
+    sp, v = S.fused_temporal_conv_lif_state(shifted, dev(w_dev, BF16), dev(b_dev, BF16), zero_v(), [s, s], [p, p], [1, 1], 1, *LIF, False)
+    check(sp, v, ref, what="conv, activations at 2-byte alignment")
+    _no_fallback(hip_ops, 1)
+
+
 @pytest.mark.parametrize("T", [1, 2, 3, 4, 5, 8, 16])
 def test_conv_lif_timestep_counts_and_windows(hip_ops, T):
     xs, w_dev, b_dev, w_ref, b_ref = _conv_case(600 + T, T, 2, 32, 48, 10, 10, 3, BF16)

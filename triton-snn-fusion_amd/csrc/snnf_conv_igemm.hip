@@ -313,6 +313,8 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         if (residuals != nullptr) vec4_ok = vec4_ok && aligned_to(residuals[t], 8);
     }
     const int load_mode = xsize == 4 ? LOAD_2XF32 : (pair_aligned ? LOAD_PAIR32 : LOAD_2X16);
+    // The matrix kernel also pairs the pixels of planes of odd width (2 columns or more): 4-byte loads at 2-byte alignment.
+    const int mm_load_mode = (xsize == 2 && g.W % 2 == 1 && g.W >= 3) ? LOAD_PAIR32 : load_mode;
 
     // Kernel choice. Layers whose arithmetic intensity is far below the matrix-core / HBM ridge (about 300 flop/byte)
     // run the time-outer kernel (small footprint, two workgroups per CU, membrane resident for any T); the others
@@ -339,11 +341,11 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         const int vec = vec_ok ? 8 : (vec4_ok ? 4 : 0);
         for (; w2 >= 1 && !mm_kernel; w2 >>= 1) {
             MmPlan p8 = {}, p4 = {};
-            const bool ok8 = plan_mm(g, w2, load_mode, vec, 8, p8);
+            const bool ok8 = plan_mm(g, w2, mm_load_mode, vec, 8, p8);
             // One shared frame: a single short matrix stage, then T steps of epilogue per tile. Two 4-wave workgroups per
             // CU (fast variant only) overlap one's epilogue with the other's loads and matrix work; measured 15 % faster on
             // a 7x7/2 stem, slower on every layer with a deep matrix loop.
-            const bool ok4 = all_shared && fast_layer && plan_mm(g, w2, load_mode, vec, 4, p4) && p4.all_full && p4.run >= 4;
+            const bool ok4 = all_shared && fast_layer && plan_mm(g, w2, mm_load_mode, vec, 4, p4) && p4.all_full && p4.run >= 4;
             if (!ok8 && !ok4) continue;
             mp = ok4 ? p4 : p8;
             // The masked variant with 4 timesteps of accumulators spills registers (and every reload then waits behind
@@ -513,9 +515,10 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         L.stream = hs;
         int rc;
         const int tt = parts[part].tt;
-        if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, load_mode);
-        else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, load_mode);
-        else rc = launch_conv_f16(L, tt, load_mode);
+        const int lm = mm_kernel ? mm_load_mode : load_mode;
+        if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, lm);
+        else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, lm);
+        else rc = launch_conv_f16(L, tt, lm);
         if (rc != SNNF_OK) return rc;
       }
     }

@@ -130,6 +130,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     // ---- the stage in flight.
     uint32_t pre[SS][TT][8][RPE];
     uint32_t pre_zero0 = 0, pre_zero1 = 0;                   // bit s: first / second column of item s is padding or beyond Cin
+    uint32_t pre_edge = 0;                                   // paired loads, odd widths: bit s: item s is a row's last column, fetched
+                                                             // together with the column to its left (it sits in the upper half)
 
     // Loads of stage `stg` (stage_chunks channel chunks) of the tile whose halo starts at input (row ih_lo, column iw_lo)
     // of image n.
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
         const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
         uint32_t off0[SS], off1[SS];
-        uint32_t z0 = 0, z1 = 0;
+        uint32_t z0 = 0, z1 = 0, edges = 0;
 #pragma unroll
         for (int s = 0; s < SS; ++s) {
             const int ih = ih_lo + item_r[s];
@@ -147,13 +149,25 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             const bool ok0 = cok && iw >= 0 && iw < g.W;
             const bool ok1 = cok && iw + 1 >= 0 && iw + 1 < g.W;
             const uint32_t src = static_cast<uint32_t>(item_src[s] + tile_rel) * ES;
-            off0[s] = ok0 ? src : 0u;
+            if constexpr (LM == LOAD_PAIR32) {
+                // A pair is one 4-byte load (2-byte aligned in the odd rows of a plane of odd width). The last column of such
+                // a plane has no right neighbour in its row, and at the very end of the tensor none at all: it is fetched
+                // as the upper half of the pair that starts one column to its left. (Planes of even width never meet this
+                // case; confining the three extra instructions per item to odd widths behind uniform branches measured
+                // slower on every layer.)
+                const bool edge = ok0 && !ok1;
+                off0[s] = ok0 ? (edge ? src - ES : src) : 0u;
+                edges |= edge ? (1u << s) : 0u;
+            } else {
+                off0[s] = ok0 ? src : 0u;
+            }
             off1[s] = ok1 ? src + ES : 0u;
             z0 |= ok0 ? 0u : (1u << s);
             z1 |= ok1 ? 0u : (1u << s);
         }
         pre_zero0 = z0;
         pre_zero1 = z1;
+        pre_edge = edges;
         // A load address is a uniform base (timestep, image, chunk) plus a 32-bit lane offset that walks the 8 channels of
         // the group: one vector add per load. Fewer than 8 input channels in all: the absent ones re-read the last real
         // one (their weights are 0).
@@ -195,9 +209,10 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 for (int t = 0; t < TT; ++t) {
                     cv_u32x4 lo, hi;
                     if constexpr (LM == LOAD_PAIR32) {
+                        const uint32_t first = ((pre_edge >> s) & 1u) ? 0x07060302u : 0x05040100u;   // halves that hold the item's first column
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
-                            lo[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], 0x05040100u);
+                            lo[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], first);
                             hi[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], 0x07060302u);
                         }
                     } else {
