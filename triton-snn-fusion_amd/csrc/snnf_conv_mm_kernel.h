@@ -130,8 +130,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     // ---- the stage in flight.
     uint32_t pre[SS][TT][8][RPE];
     uint32_t pre_zero0 = 0, pre_zero1 = 0;                   // bit s: first / second column of item s is padding or beyond Cin
-    uint32_t pre_edge = 0;                                   // paired loads, odd widths: bit s: item s is a row's last column, fetched
-                                                             // together with the column to its left (it sits in the upper half)
 
     // Loads of stage `stg` (stage_chunks channel chunks) of the tile whose halo starts at input (row ih_lo, column iw_lo)
     // of image n.
@@ -140,7 +138,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
         const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
         uint32_t off0[SS], off1[SS];
-        uint32_t z0 = 0, z1 = 0, edges = 0;
+        uint32_t z0 = 0, z1 = 0;
 #pragma unroll
         for (int s = 0; s < SS; ++s) {
             const int ih = ih_lo + item_r[s];
@@ -153,11 +151,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 // A pair is one 4-byte load (2-byte aligned in the odd rows of a plane of odd width). The last column of such
                 // a plane has no right neighbour in its row, and at the very end of the tensor none at all: it is fetched
                 // as the upper half of the pair that starts one column to its left. (Planes of even width never meet this
-                // case; confining the three extra instructions per item to odd widths behind uniform branches measured
-                // slower on every layer.)
-                const bool edge = ok0 && !ok1;
-                off0[s] = ok0 ? (edge ? src - ES : src) : 0u;
-                edges |= edge ? (1u << s) : 0u;
+                // case; confining the extra instructions per item to odd widths behind uniform branches measured slower
+                // on every layer.)
+                off0[s] = ok0 ? (ok1 ? src : src - ES) : 0u;
             } else {
                 off0[s] = ok0 ? src : 0u;
             }
@@ -167,7 +163,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         }
         pre_zero0 = z0;
         pre_zero1 = z1;
-        pre_edge = edges;
         // A load address is a uniform base (timestep, image, chunk) plus a 32-bit lane offset that walks the 8 channels of
         // the group: one vector add per load. Fewer than 8 input channels in all: the absent ones re-read the last real
         // one (their weights are 0).
@@ -209,7 +204,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 for (int t = 0; t < TT; ++t) {
                     cv_u32x4 lo, hi;
                     if constexpr (LM == LOAD_PAIR32) {
-                        const uint32_t first = ((pre_edge >> s) & 1u) ? 0x07060302u : 0x05040100u;   // halves that hold the item's first column
+                        // An item whose first column is real and whose second is not is a row's last column: its first
+                        // column sits in the upper halves.
+                        const uint32_t first = (!zero0 && zero1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
                             lo[k] = __builtin_amdgcn_perm(pre[s][t][2 * k + 1][0], pre[s][t][2 * k][0], first);
