@@ -331,6 +331,7 @@ POINTWISE_CASES = [  # Cin, Cout, H, W, dtype, vdtype, lif, T, residual, tensor 
     (128, 64, 8, 8, F32, F32, (1.0, 0.0, 2.0), 4, True, False),        # fp32 activations (rounded to bf16 on the way in)
     (128, 96, 8, 16, F16, F16, (1.0, 0.0, 2.0), 4, False, True),       # f16 with an f16 membrane
     (192, 64, 16, 8, F16, F32, (1.0, 0.0, 2.0), 17, False, False),     # channel tail in the second chunk, two launch windows
+    (128, 64, 16, 16, BF16, F32, (1.0, 0.0, 1.5), 4, False, True),     # tau not a power of two: true division
 ]
 
 
@@ -371,6 +372,8 @@ DENSE_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, re
     (256, 128, 4, 4, 3, 1, 1, BF16, F32, (1.0, -1.0, 2.0), 3, 5, True, False),    # several images per tile, K split, masked variant, soft reset
     (64, 64, 8, 8, 3, 2, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 8, False, False),      # stride 2 onto 4x4 planes, several images per tile
     (32, 64, 6, 6, 5, 1, 2, F16, F32, (1.0, 0.0, 2.0), 2, 7, True, True),         # 6x6 planes (no aligned runs), 5x5 kernel, f16
+    (64, 64, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 3.0), 4, 2, False, True),     # tau not a power of two: true division
+    (128, 64, 8, 8, 3, 1, 1, BF16, F32, (0.75, -1.0, 1.5), 4, 2, True, False),    # + soft reset, K split
 ]
 
 
@@ -391,6 +394,65 @@ def test_dense_conv_lif_matrix_kernel_variants(hip_ops, Cin, Cout, H, W, k, stri
         sp, v = S.fused_temporal_conv_lif_state(dx, dw, db, dv, *geo, *lif, False)
     assert sp.dtype == dtype and v.dtype == vdtype and tuple(sp.shape) == (T, N, Cout, Ho, Wo)
     check(sp, v, ref, v_threshold=lif[0], v_dtype=vdtype, what=f"dense {Cin}->{Cout} k{k} s{stride} {H}x{W}")
+    _no_fallback(hip_ops, 1)
+
+
+FALLBACK_KERNEL_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, residual, tensor v_init, kernel family
+    (12, 32, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "time_outer"),    # partial channel group
+    (20, 48, 14, 14, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True, "time_outer"),      # + residual, v_init
+    (36, 64, 9, 11, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 5, 3, False, True, "time_outer"),      # ragged planes, T = 5
+    (12, 32, 13, 13, 3, 2, 1, F16, F16, (1.0, -1.0, 2.0), 3, 2, True, False, "time_outer"),     # stride 2, f16 membrane, soft reset
+    (20, 40, 10, 10, 3, 1, 1, F32, F32, (0.5, 0.0, 1.0), 4, 2, False, False, "time_outer"),     # fp32, IF neuron
+    (12, 32, 12, 12, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "time_outer"),    # 1x1 with Cin % 8 != 0
+    (20, 64, 7, 9, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 3, True, True, "time_outer"),        # 1x1, odd plane, residual, v_init
+    (44, 256, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "t_in_m"),      # high intensity, Cin % 8 != 0
+    (44, 256, 9, 9, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 3, True, True, "t_in_m"),          # + odd plane, residual, v_init
+    (52, 320, 10, 10, 3, 1, 1, F16, F32, (1.0, 0.0, 4.0), 6, 2, False, True, "t_in_m"),        # two launch windows, f16
+    (512, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "t_in_m"),     # deep pointwise layer (AI 205)
+    (1024, 1024, 7, 7, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True, "t_in_m"),       # deep pointwise layer (AI 410)
+    (12, 32, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 3.0), 4, 2, False, True, "time_outer"),     # tau not a power of two
+    (44, 256, 12, 12, 3, 1, 1, BF16, F32, (0.75, 0.0, 1.5), 4, 2, False, True, "t_in_m"),      # tau not a power of two
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,stride,pad,dtype,vdtype,lif,T,N,residual,tensor_v,family", FALLBACK_KERNEL_CASES)
+def test_dense_conv_lif_shapes_outside_the_matrix_and_pointwise_kernels(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N,
+                                                                        residual, tensor_v, family):
+    """Layers the 8-wave matrix kernel and the pointwise kernel do not take (input channels that are not whole groups of 8,
+    plain 1x1 layers of high arithmetic intensity) run the time-outer kernel or the 4-wave T-in-M kernel."""
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(1600 + Cin + Cout + H + k, T, N, Cin, Cout, H, W, k, dtype, p=0.25)
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    g = gen(1601 + Cin)
+    rs = [q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, vdtype) if tensor_v else torch.tensor(0.0)
+    geo = ([stride, stride], [pad, pad], [1, 1], 1)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (stride, stride), (pad, pad), (1, 1), 1, *lif, residuals=rs)
+    dx, dw, db = [dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype)
+    dv = dev(v0, vdtype) if tensor_v else zero_v(vdtype)
+    if residual:
+        sp, v = S.fused_temporal_conv_add_lif_state(dx, [dev(r, dtype) for r in rs], dw, db, dv, *geo, *lif, False)
+    else:
+        sp, v = S.fused_temporal_conv_lif_state(dx, dw, db, dv, *geo, *lif, False)
+    assert last_conv_plan()["kernel"] == family, last_conv_plan()
+    check(sp, v, ref, v_threshold=lif[0], v_dtype=vdtype, what=f"{family} {Cin}->{Cout} k{k} s{stride} {H}x{W}")
+    _no_fallback(hip_ops, 1)
+
+
+def test_planes_of_four_pixels_with_several_images_per_tile(hip_ops):
+    """2x2 planes, two images per tile: a lane's run of 8 pixels spans two images (each half is one whole plane)."""
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    Cin, Cout, T, N = 256, 512, 4, 40
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(1700, T, N, Cin, Cout, 2, 2, 3, BF16, p=0.25)
+    g = gen(1701)
+    rs = [q(torch.randn(N, Cout, 2, 2, generator=g) * 0.3, BF16) for _ in range(T)]
+    v0 = torch.randn(N, Cout, 2, 2, generator=g) * 0.3
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (1, 1), (1, 1), (1, 1), 1, *LIF, residuals=rs)
+    sp, v = S.fused_temporal_conv_add_lif_state([dev(x, BF16) for x in xs], [dev(r, BF16) for r in rs], dev(w_dev, BF16), dev(b_dev, BF16),
+                                                dev(v0, F32), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+    plan = last_conv_plan()
+    assert plan["kernel"] == "matrix" and plan["tile"] == "2x2x2" and plan["variant"] == 24, plan
+    check(sp, v, ref, what="2x2 planes, two images per tile")
     _no_fallback(hip_ops, 1)
 
 
@@ -576,3 +638,57 @@ def test_unsupported_configurations_fall_back_to_eager_ops_on_the_gpu_and_are_co
             S.fused_temporal_conv_lif_state([dev(x, F32) for x in xs], dev(w, F32), dev(b, F32), zero_v(), [1, 1], [2, 2], [2, 2], 1, *LIF, False)
     finally:
         ops.configure_fused_op("torch")
+
+
+def test_fallback_chains_a_float32_membrane_next_to_16_bit_activations(snnf_lib):
+    """A call the kernels do not take (dilation 2) with bf16 activations and a full-shape fp32 membrane: the eager ops step in
+    fp32 and return an fp32 membrane, as the kernels do, so two chained fallback windows equal one long oracle call."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd.runtime import snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=False)
+    ops.reset_fused_op_call_stats()
+    try:
+        g = gen(5)
+        T, N, C, H = 4, 2, 8, 9
+        xs = [spikes((N, C, H, H), 0.3, g) for _ in range(T)]
+        w, b = q(torch.randn(C, C, 3, 3, generator=g) * 0.4, BF16), q(torch.randn(C, generator=g) * 0.1, BF16)
+        v0 = torch.randn(N, C, H, H, generator=g) * 0.3
+        geo = ([1, 1], [2, 2], [2, 2], 1)
+        ref = O.temporal_conv_lif(xs, w, b, v0, (1, 1), (2, 2), (2, 2), 1, *LIF)
+        dx, dw, db = [dev(x, BF16) for x in xs], dev(w, BF16), dev(b, BF16)
+        s1, v1 = S.fused_temporal_conv_lif_state(dx[:2], dw, db, dev(v0, F32), *geo, *LIF, False)
+        assert v1.dtype == F32 and s1.dtype == BF16
+        s2, v2 = S.fused_temporal_conv_lif_state(dx[2:], dw, db, v1, *geo, *LIF, False)
+        assert v2.dtype == F32
+        check(torch.cat([s1, s2]), v2, ref, what="chained dilated fallback, fp32 membrane")
+        stats = ops.get_fused_op_call_stats()
+        assert stats["fallback"] == 2 and stats["triton"] == 0
+        # a 0-dim fp32 zero on the device also selects an fp32 membrane; a host-side placeholder the activation dtype
+        _, v3 = S.fused_temporal_conv_lif_state(dx[:2], dw, db, zero_v(F32), *geo, *LIF, False)
+        _, v4 = S.fused_temporal_conv_lif_state(dx[:2], dw, db, torch.tensor(0.0), *geo, *LIF, False)
+        assert v3.dtype == F32 and v4.dtype == BF16
+        # the native path follows the same rule
+        _, v5 = S.fused_temporal_conv_lif_state(dx[:2], dw, db, zero_v(F32), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+        _, v6 = S.fused_temporal_conv_lif_state(dx[:2], dw, db, torch.tensor(0.0), [1, 1], [1, 1], [1, 1], 1, *LIF, False)
+        assert v5.dtype == F32 and v6.dtype == BF16
+        assert ops.get_fused_op_call_stats()["triton"] == 2
+    finally:
+        ops.configure_fused_op("torch")
+
+
+def test_single_step_lif_runs_the_scan_kernel_on_the_gpu(hip_ops):
+    """`lif_forward_state` on GPU tensors of any rank: one launch of the scan kernel, bit exact against the oracle, state
+    chained through a module-style loop."""
+    g = gen(6)
+    for shape, dtype, vdtype in (((3, 50), F32, F32), ((2, 8, 7, 7), BF16, BF16), ((2, 8, 7, 7), BF16, F32), ((5,), F16, F16)):
+        xs = q(torch.randn((3,) + shape, generator=g) * 0.9 + 0.2, dtype)
+        v = zero_v(vdtype)
+        ref = O.temporal_lif(xs, torch.tensor(0.0), *LIF)
+        got = []
+        for t in range(3):
+            s, v = S.lif_forward_state(dev(xs[t], dtype), v, *LIF, False)
+            assert s.dtype == dtype and v.dtype == vdtype
+            got.append(s)
+        check(torch.stack(got), v, ref, v_dtype=vdtype, what=f"single-step lif {shape} {dtype}")
+        assert torch.equal(torch.stack(got).float().cpu(), ref[0])

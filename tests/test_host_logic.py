@@ -270,3 +270,30 @@ def test_workloads_are_seeded_and_bn_fold_is_exact_algebra():
     nbytes = W.algorithmic_conv_bytes(4, 8, 64, 32, 32, 64, 32, 32, 3, 3, 1, 4, 4)
     assert abs(nbytes - 19.02e6) < 0.02e6
     assert W.conv_flops(4, 8, 64, 64, 32, 32, 3, 3, 1) == 2415919104
+
+
+def test_eager_and_meta_functions_agree_on_the_membrane_dtype():
+    """One rule for native kernels, eager functions and meta functions: a v_init on the activations' device with dtype
+    float32 or the activation dtype chooses the membrane dtype, anything else gives the activation dtype."""
+    import torch
+    from triton_snn_fusion_amd.runtime import snn_custom_ops as ops
+    S = torch.ops.snn_custom
+    x = [(torch.rand(2, 4, 6, 6) < 0.3).to(torch.bfloat16) for _ in range(3)]
+    w, b = torch.randn(4, 4, 3, 3).to(torch.bfloat16), torch.zeros(4, dtype=torch.bfloat16)
+    geo = ([1, 1], [1, 1], [1, 1], 1)
+    lif = (1.0, 0.0, 2.0, False)
+    for v_init, want in ((torch.zeros(2, 4, 6, 6), torch.float32), (torch.zeros(()), torch.float32),
+                         (torch.zeros((), dtype=torch.bfloat16), torch.bfloat16), (torch.zeros(2, 4, 6, 6, dtype=torch.bfloat16), torch.bfloat16),
+                         (torch.zeros((), dtype=torch.float64), torch.bfloat16)):
+        s, v = S.fused_temporal_conv_lif_state(x, w, b, v_init, *geo, *lif)
+        ms, mv = S.fused_temporal_conv_lif_state([t.to("meta") for t in x], w.to("meta"), b.to("meta"), v_init.to("meta"), *geo, *lif)
+        assert v.dtype == want == mv.dtype and s.dtype == torch.bfloat16 == ms.dtype and mv.shape == v.shape
+        s1, v1 = S.lif_forward_state(x[0], v_init, *lif)
+        m1 = S.lif_forward_state(x[0].to("meta"), v_init.to("meta"), *lif)
+        assert v1.dtype == want == m1[1].dtype
+    # a float32 membrane next to 16-bit activations is stepped in float32: chaining two windows equals one call
+    v0 = torch.randn(2, 4, 6, 6) * 0.3
+    s_all, v_all = S.fused_temporal_conv_lif_state(x, w, b, v0, *geo, *lif)
+    s_a, v_a = S.fused_temporal_conv_lif_state(x[:1], w, b, v0, *geo, *lif)
+    s_b, v_b = S.fused_temporal_conv_lif_state(x[1:], w, b, v_a, *geo, *lif)
+    assert torch.equal(torch.cat([s_a, s_b]), s_all) and torch.equal(v_b, v_all) and v_all.dtype == torch.float32

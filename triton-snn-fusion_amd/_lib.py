@@ -80,6 +80,18 @@ def lib() -> ctypes.CDLL:
     return _LIB
 
 
+def membrane_dtype(x: torch.Tensor, v_init) -> torch.dtype:
+    """dtype of the membrane an operator call returns. A `v_init` on the activations' device whose dtype is float32 or
+    the activation dtype chooses it (a full-shape state to continue from, or a 0-dim zero placed there on purpose:
+    16-bit activations with a float32 membrane); anything else - in particular the host-side 0-dim `torch.tensor(0.0)`
+    placeholder the reference's rewriter emits (compiler/fx_lif_temporal_rewrite.py:2593) - gives the activation dtype,
+    as in the reference (runtime/snn_custom_ops.py:378-381). Native kernels, eager functions and meta functions all
+    use this one rule."""
+    if (isinstance(v_init, torch.Tensor) and v_init.dtype in (torch.float32, x.dtype) and v_init.device == x.device):
+        return v_init.dtype
+    return x.dtype
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPE_CODES[dtype]

@@ -3,6 +3,10 @@
 
 #include "snnf_common.h"
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 namespace snnf {
 
 constexpr int kConvThreads = 256;   // 4 waves
@@ -137,6 +141,26 @@ struct ConvLaunch {
     size_t lds_bytes;
     hipStream_t stream;
 };
+
+// Lets `kernel` use more than 64 KiB of dynamic LDS. The attribute belongs to one kernel function on one device, so
+// what has been raised already is remembered per (function, device).
+inline int reserve_lds(const void* kernel, size_t bytes, const char* who) {
+    if (bytes <= 64 * 1024) return SNNF_OK;
+    static std::mutex mu;
+    static std::set<std::pair<const void*, int>> raised;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const std::pair<const void*, int> key(kernel, dev);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (raised.count(key)) return SNNF_OK;
+    }
+    const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
+    if (err != hipSuccess) return fail(SNNF_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS: %s", who, bytes, hipGetErrorString(err));
+    std::lock_guard<std::mutex> lock(mu);
+    raised.insert(key);
+    return SNNF_OK;
+}
 
 // One launcher per activation dtype (each in its own translation unit so they compile in parallel).
 // tt: 1, 2, 4 = timesteps accumulated side by side (4-wave kernel); 10 + tt / 20 + tt = 8-wave matrix kernel, general /

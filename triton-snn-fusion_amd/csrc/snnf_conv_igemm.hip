@@ -257,8 +257,6 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     if (v_dtype != SNNF_F32 && v_dtype != x_dtype)
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: unsupported_dtype: membrane dtype must be fp32 or the activation dtype");
     if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: unsupported_tau: tau must be nonzero");
-    if (make_lif_params(v_threshold, v_reset, tau).charge_mode == CHARGE_DIVIDE)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: unsupported_tau: tau must be <= 1 or a power of two, got %g", tau);
     if (H + 2 * pad_h < KH || W + 2 * pad_w < KW)
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_lif: unsupported_kernel: kernel larger than padded input");
     if (2 * pad_h > KH || 2 * pad_w > KW)

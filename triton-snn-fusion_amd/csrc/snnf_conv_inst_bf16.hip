@@ -14,9 +14,3 @@ int launch_conv_bf16(const ConvLaunch& L, int tt, int load_mode) {
     return launch_conv_tt<bf16_t>(L, tt, load_mode);
 }
 }  // namespace snnf
-
-#ifdef SNNF_MM_TRACE
-extern "C" int snnf_debug_mm_trace(unsigned long long* host_out) {
-    return static_cast<int>(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(snnf::mm_trace), sizeof(unsigned long long) * 64 * 16));
-}
-#endif

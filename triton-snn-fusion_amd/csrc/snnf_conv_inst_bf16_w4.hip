@@ -8,9 +8,3 @@ int launch_conv_mm_w4_bf16(const ConvLaunch& L, int tt, int load_mode) {
     return launch_conv_mm_tt<bf16_t, 1, 4>(L, load_mode, true);
 }
 }  // namespace snnf
-
-#ifdef SNNF_MM_TRACE
-extern "C" int snnf_debug_mm_trace_w4(unsigned long long* host_out) {
-    return static_cast<int>(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(snnf::mm_trace), sizeof(unsigned long long) * 64 * 16));
-}
-#endif

@@ -356,6 +356,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
             const bool fast = g.vec8 && okmask == 0xffu && (pxoff[7] - pxoff[0]) == 7 && (pxoff[0] & 7) == 0;
             const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
             const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+            const bool divide = lif.charge_mode == CHARGE_DIVIDE;   // tau is not a power of two: a true division
             const int po = static_cast<int>(plane_out);
 
 #pragma unroll
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
                                 Pack<XT, 8> sp;
 #pragma unroll
                                 for (int k = 0; k < 8; ++k) {
-                                    const float h = v[k] + (x[k] - v[k] * c0f) * c1f;
+                                    const float h = divide ? v[k] + __fdiv_rn(x[k] - v[k], lif.tau) : v[k] + (x[k] - v[k] * c0f) * c1f;
                                     const bool fired = h >= lif.v_threshold;
                                     v[k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
                                     sp.v[k] = spike_value<XT>(fired);
@@ -463,19 +464,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
 template <typename XT, int TT>
 int launch_conv_lm(const ConvLaunch& L, int load_mode) {
     auto run = [&](auto kernel) -> int {
-        if (L.lds_bytes > 64 * 1024) {
-            // Opt in to the full 160 KiB of LDS once per kernel instantiation and device.
-            static bool raised[64] = {};
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-            if (!raised[dev]) {
-                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                     static_cast<int>(kMaxLds));
-                if (err != hipSuccess)
-                    return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: cannot reserve %zu bytes of LDS: %s", L.lds_bytes, hipGetErrorString(err));
-                raised[dev] = true;
-            }
-        }
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif"); rc != SNNF_OK) return rc;
         kernel<<<dim3(L.grid), kConvThreads, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
                                                                       static_cast<XT*>(L.spikes), L.v_out, L.lif);
         return check_launch("snnf_conv_lif");

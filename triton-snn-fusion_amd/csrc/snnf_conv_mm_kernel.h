@@ -38,19 +38,6 @@ __host__ __device__ constexpr int mm_staging_slots(int load_mode, int tt, bool s
 }
 typedef float cv_f32x4 __attribute__((ext_vector_type(4)));
 
-// Phase timestamps of the first tile of the first 64 workgroups (development builds with -DSNNF_MM_TRACE only): slot 0
-// kernel start, 1 first loads issued, 2 + 2 s / 3 + 2 s stage s in LDS / stage s multiplied (s < 4), 10 / 11 epilogue
-// start / end. Read back with snnf_debug_mm_trace() of the translation unit that launched the kernel.
-#ifdef SNNF_MM_TRACE
-__device__ unsigned long long mm_trace[64 * 16];
-#define SNNF_MM_STAMP(slot)                                                                                  \
-    do {                                                                                                     \
-        if (threadIdx.x == 0 && blockIdx.x < 64 && trace_on) mm_trace[blockIdx.x * 16 + (slot)] = __builtin_amdgcn_s_memtime(); \
-    } while (0)
-#else
-#define SNNF_MM_STAMP(slot) do {} while (0)
-#endif
-
 // NW waves per workgroup: 8 (one workgroup per CU) or 4 (two independent workgroups per CU, whose load, matrix and
 // epilogue phases overlap each other instead of running in lockstep across the whole CU).
 template <typename XT, int TT, int LM, bool FAST, bool SK, int NW>
@@ -65,11 +52,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
     constexpr int NT = NW * 64;                               // threads per workgroup
     const int tid = threadIdx.x;
-#ifdef SNNF_MM_TRACE
-    bool trace_on = true;
-    int trace_tile = 0;
-#endif
-    SNNF_MM_STAMP(0);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int half = lane >> 5;
@@ -79,7 +61,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     const int wk = SK ? (wave >> (g.wm_log2 + g.wn_log2)) : 0;     // K slice of this wave (split-K variant)
     const int WK = SK ? (1 << g.wk_log2) : 1;
 
-    if (g.wm_log2 >= 0) SNNF_MM_STAMP(12);
     const int groups = 1 << g.groups_log2;                   // channel groups of 8 per packed chunk
     const int stage_groups = groups * g.stage_chunks;        // ... per LDS stage (a stage holds stage_chunks chunks)
     const int nstages = (g.nchunks + g.stage_chunks - 1) / g.stage_chunks;
@@ -270,14 +251,12 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         if (pair_shift && (iw_lo & 1)) iw_lo -= 1;
     };
     bool have_tile = decode(work, oc_tile, img, oh0, ow0);
-    if (oh0 != -12345) SNNF_MM_STAMP(14);
     if (have_tile) {
         int ih_lo, iw_lo;
         halo_origin(oh0, ow0, ih_lo, iw_lo);
         issue_loads(0, img, ih_lo, iw_lo);
         fetch_bias(oc_tile);
     }
-    SNNF_MM_STAMP(1);
 
     // ---- kernel constants of the matrix loop: this lane's pixel (block pixel wm * 32 + l32) inside the halo tile.
     const int mpix = wm * 32 + l32;
@@ -300,10 +279,17 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     const bool hi_inside = epix + 8 <= g.TI * tile_px;       // each half of a lane's run of 8 pixels is inside or outside as a whole
     const uint32_t image_out = static_cast<uint32_t>(g.Cout) * static_cast<uint32_t>(g.Ho * g.Wo);
     const uint32_t lane_px = static_cast<uint32_t>(epi) * image_out + static_cast<uint32_t>(epr * g.Wo + epc);
+    // The second half of the lane's run of 8 (pixels epix + 4 .. + 7): contiguous with the first half inside an image, but
+    // with tiles of several whole planes of 4 pixels (2x2 planes) it lies in the next image of the tile.
+    const int epi_hi = fast_div(epix + 4, g.d_tile_px);
+    const int erem_hi = epix + 4 - epi_hi * tile_px;
+    const int epr_hi = fast_div(erem_hi, g.d_TW);
+    const uint32_t lane_px_hi = static_cast<uint32_t>(epi_hi) * image_out + static_cast<uint32_t>(epr_hi * g.Wo + (erem_hi - epr_hi * g.TW));
     float* __restrict__ stage_wr = stage + (half * 4) * kMmStagePitch + l32;
     const float* __restrict__ stage_rd = stage + row16 * kMmStagePitch + pcx * 8;
     const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
     const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+    const bool divide = lif.charge_mode == CHARGE_DIVIDE;   // tau is not a power of two: a true division
 
     while (have_tile) {
         int ih_lo, iw_lo;
@@ -348,9 +334,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         };
         // Weight fragments stream from L2 two pairs ahead of their use, through three register sets.
         auto load_frags = [&](int gpair, cv_u32x4& a0, cv_u32x4& a1) __attribute__((always_inline)) {
-#ifdef SNNF_MM_EXPERIMENT_NO_WEIGHT_STREAM
-            if (gpair >= 2 * WK) return;   // timing experiment (wrong results): only the first fragments of a tile are loaded
-#endif
             const int64_t o = static_cast<int64_t>(min(gpair, total_pairs - 1)) * (kFragBytes / 2);
             a0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + o);
             a1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + o);
@@ -365,7 +348,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             write_lds();       // waits for the stage's loads
             if (chunk == 0 && tid < (64 << g.wn_log2)) bias_lds[tid] = bias_pre;
             __syncthreads();
-            if (chunk < 4) SNNF_MM_STAMP(2 + 2 * chunk);
             // ---- the stage after this one: next chunk, or the first chunk of the next tile.
             {
                 int nc = chunk + 1, nimg = img, nih = ih_lo, niw = iw_lo;
@@ -399,12 +381,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                     }
                 }
             }
-            if (chunk < 4) SNNF_MM_STAMP(3 + 2 * chunk);
         }
-        SNNF_MM_STAMP(10);
-#ifdef SNNF_MM_TRACE
-        if (trace_tile == 1 && threadIdx.x == 0 && blockIdx.x < 64) mm_trace[blockIdx.x * 16 + 13] = __builtin_amdgcn_s_memtime();
-#endif
 
         // ---- epilogue. h = v + (x - v * c0) * c1 covers tau <= 1 and power-of-two tau exactly.
         // FAST: 16 channel rows x 32 pixels at a time go through the wave's LDS stage, so that a lane owns 8 consecutive pixels
@@ -418,6 +395,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                                      : ((m_inside && img + mpi < g.N && oh0 + mpr < g.Ho && ow0 + mpc < g.Wo) ? 0xffu : 0u);
         // Element offset of the lane's first pixel (FAST: of its run of 8) from the tile origin of its channel row.
         const uint32_t px0 = FAST ? lane_px : static_cast<uint32_t>(mpi) * image_out + static_cast<uint32_t>(mpr * g.Wo + mpc);
+        const uint32_t px4 = lane_px_hi;   // FAST: offset of the run's second half
         const int64_t tile_off = static_cast<int64_t>(img) * g.Cout * po + oh0 * g.Wo + ow0;   // uniform, elements
         const bool analog = g.analog_out != 0;   // neuron-free output: conv + bias (+ residual) where the spikes would go
 
@@ -456,7 +434,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                     for (int k = 0; k < 4; ++k) v[k] = lo.v[k];
                 }
                 if (okmask & 0xf0u) {
-                    const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src + 4);
+                    const Pack<float, 4> hi = *reinterpret_cast<const Pack<float, 4>*>(src - px0 + px4);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) v[4 + k] = hi.v[k];
                 }
@@ -480,7 +458,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int k = 0; k < 4; ++k) { lo.v[k] = v[k]; hi.v[k] = v[4 + k]; }
                 if (okmask & 0x0fu) *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
-                if (okmask & 0xf0u) *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
+                if (okmask & 0xf0u) *reinterpret_cast<Pack<float, 4>*>(dst - px0 + px4) = hi;
             } else {
                 const int oc = first_row(gidx);
                 if (group_full(gidx)) {
@@ -513,7 +491,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 fired = h >= lif.v_threshold;
                 v = fired ? lif.v_reset : h;
             } else {
-                const float h = v + (x - v * c0f) * c1f;
+                const float h = divide ? v + __fdiv_rn(x - v, lif.tau) : v + (x - v * c0f) * c1f;
                 fired = h >= lif.v_threshold;
                 v = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
             }
@@ -548,7 +526,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                             for (int k = 0; k < 4; ++k) x[k] += to_float(ra.v[k]);
                         }
                         if (okmask & 0xf0u) {
-                            const Pack<XT, 4> rb = *reinterpret_cast<const Pack<XT, 4>*>(res_t + px0 + 4);
+                            const Pack<XT, 4> rb = *reinterpret_cast<const Pack<XT, 4>*>(res_t + px4);
 #pragma unroll
                             for (int k = 0; k < 4; ++k) x[4 + k] += to_float(rb.v[k]);
                         }
@@ -570,7 +548,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                         for (int k = 0; k < 4; ++k) { sa.v[k] = sp.v[k]; sb.v[k] = sp.v[4 + k]; }
                         if (okmask & 0x0fu) *reinterpret_cast<Pack<XT, 4>*>(out_t + px0) = sa;
-                        if (okmask & 0xf0u) *reinterpret_cast<Pack<XT, 4>*>(out_t + px0 + 4) = sb;
+                        if (okmask & 0xf0u) *reinterpret_cast<Pack<XT, 4>*>(out_t + px4) = sb;
                     }
                 }
             } else {
@@ -695,12 +673,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                 if (owner == wk) store_membrane(gidx, row_ok[gidx & 1], row_off[gidx & 1], v[gidx & 1]);
             }
         }
-        SNNF_MM_STAMP(11);
-#ifdef SNNF_MM_TRACE
-        if (trace_tile == 1 && threadIdx.x == 0 && blockIdx.x < 64) mm_trace[blockIdx.x * 16 + 15] = __builtin_amdgcn_s_memtime();
-        trace_on = false;
-        ++trace_tile;
-#endif
         if (SK && next_tile) {
             int nih, niw;
             halo_origin(next_oh0, next_ow0, nih, niw);
@@ -720,18 +692,7 @@ template <typename XT, int TT, int NW>
 int launch_conv_mm_tt(const ConvLaunch& L, int load_mode, bool fast) {
     const bool split_k = L.g.wk_log2 > 0;
     auto run = [&](auto kernel) -> int {
-        if (L.lds_bytes > 64 * 1024) {
-            static bool raised[64] = {};   // per kernel instantiation and device
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-            if (!raised[dev]) {
-                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                     static_cast<int>(kMaxLds));
-                if (err != hipSuccess)
-                    return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: cannot reserve %zu bytes of LDS: %s", L.lds_bytes, hipGetErrorString(err));
-                raised[dev] = true;
-            }
-        }
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif"); rc != SNNF_OK) return rc;
         kernel<<<dim3(L.grid), NW * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
                                                                     static_cast<XT*>(L.spikes), L.v_out, L.lif);
         return check_launch("snnf_conv_lif");

@@ -232,6 +232,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
     const float* __restrict__ stage_rd = stage + rg * kPwStagePitch + pcx * 4;
     const float c0f = lif.charge_mode == CHARGE_IF ? 0.0f : 1.0f;
     const float c1f = lif.charge_mode == CHARGE_IF ? 1.0f : lif.inv_tau;
+    const bool divide = lif.charge_mode == CHARGE_DIVIDE;   // tau is not a power of two: a true division
 
     // Bias fragment: row l32 of the weight operand carries the fp32 bias as three 16-bit terms (exact to 24 bits) in its
     // first k-slots; the activation fragments of ones differ in slots the bias fragment leaves zero, only so that the
@@ -514,7 +515,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                             fired = h >= lif.v_threshold;
                             v[gi][k] = fired ? lif.v_reset : h;
                         } else {
-                            const float h = v[gi][k] + (x[k] - v[gi][k] * c0f) * c1f;
+                            const float h = divide ? v[gi][k] + __fdiv_rn(x[k] - v[gi][k], lif.tau) : v[gi][k] + (x[k] - v[gi][k] * c0f) * c1f;
                             fired = h >= lif.v_threshold;
                             v[gi][k] = fired ? (lif.soft_reset ? h - lif.v_threshold : lif.v_reset) : h;
                         }
@@ -565,18 +566,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 template <typename XT>
 int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     auto run = [&](auto kernel) -> int {
-        if (L.lds_bytes > 64 * 1024) {
-            static bool raised[64] = {};   // per kernel instantiation and device
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-            if (!raised[dev]) {
-                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                     static_cast<int>(kMaxLds));
-                if (err != hipSuccess)
-                    return fail(SNNF_ERR_LAUNCH, "snnf_conv_lif: cannot reserve %zu bytes of LDS: %s", L.lds_bytes, hipGetErrorString(err));
-                raised[dev] = true;
-            }
-        }
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif"); rc != SNNF_OK) return rc;
         kernel<<<dim3(L.grid), kConvThreads, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.has_residual, L.g, L.wpacked, L.bias, L.v_init,
                                                                       static_cast<XT*>(L.spikes), L.v_out, L.lif);
         return check_launch("snnf_conv_lif");

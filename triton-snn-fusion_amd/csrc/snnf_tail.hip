@@ -28,41 +28,44 @@ __global__ __launch_bounds__(kThreads) void lif_pool_kernel(StepPtrs xs, int T, 
     const int elems = planes_here * HW;
     const int64_t base = static_cast<int64_t>(plane0) * HW;
     for (int i = threadIdx.x; i < planes_here; i += kThreads) plane_count[i] = 0;
+    __syncthreads();
 
-    float v[kItems];
-    int plane_of[kItems];
-    int fired_total[kItems];
-#pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        const int i = threadIdx.x + k * kThreads;
-        plane_of[k] = i < elems ? i / HW : -1;
-        fired_total[k] = 0;
-        v[k] = (i < elems && v_init != nullptr) ? to_float(v_init[base + i]) : 0.0f;
-    }
-    for (int t = 0; t < T; ++t) {
-        const XT* __restrict__ x = static_cast<const XT*>(xs.p[t]) + base;
+    // Chunks of kThreads * kItems neurons: one chunk unless a single plane is larger than that.
+    for (int c0 = 0; c0 < elems; c0 += kThreads * kItems) {
+        float v[kItems];
+        int plane_of[kItems];
+        int fired_total[kItems];
 #pragma unroll
         for (int k = 0; k < kItems; ++k) {
-            const int i = threadIdx.x + k * kThreads;
-            if (i < elems) fired_total[k] += lif_step(to_float(x[i]), v[k], lif) ? 1 : 0;
+            const int i = c0 + threadIdx.x + k * kThreads;
+            plane_of[k] = i < elems ? i / HW : -1;
+            fired_total[k] = 0;
+            v[k] = (i < elems && v_init != nullptr) ? to_float(v_init[base + i]) : 0.0f;
         }
-    }
-    __syncthreads();
+        for (int t = 0; t < T; ++t) {
+            const XT* __restrict__ x = static_cast<const XT*>(xs.p[t]) + base;
 #pragma unroll
-    for (int k = 0; k < kItems; ++k) {
-        const int i = threadIdx.x + k * kThreads;
-        // Wave-level reduction when the whole wave sits in one plane, LDS atomics otherwise.
-        const int my_plane = plane_of[k];
-        const int lead_plane = __shfl(my_plane, 0);
-        if (__all(my_plane == lead_plane)) {
-            int sum = fired_total[k];
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-            if ((threadIdx.x & 63) == 0 && lead_plane >= 0) atomicAdd(&plane_count[lead_plane], sum);
-        } else if (my_plane >= 0 && fired_total[k] != 0) {
-            atomicAdd(&plane_count[my_plane], fired_total[k]);
+            for (int k = 0; k < kItems; ++k) {
+                const int i = c0 + threadIdx.x + k * kThreads;
+                if (i < elems) fired_total[k] += lif_step(to_float(x[i]), v[k], lif) ? 1 : 0;
+            }
         }
-        if (i < elems) v_out[base + i] = from_float<VT>(v[k]);
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            const int i = c0 + threadIdx.x + k * kThreads;
+            // Wave-level reduction when the whole wave sits in one plane, LDS atomics otherwise.
+            const int my_plane = plane_of[k];
+            const int lead_plane = __shfl(my_plane, 0);
+            if (__all(my_plane == lead_plane)) {
+                int sum = fired_total[k];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+                if ((threadIdx.x & 63) == 0 && lead_plane >= 0) atomicAdd(&plane_count[lead_plane], sum);
+            } else if (my_plane >= 0 && fired_total[k] != 0) {
+                atomicAdd(&plane_count[my_plane], fired_total[k]);
+            }
+            if (i < elems) v_out[base + i] = from_float<VT>(v[k]);
+        }
     }
     __syncthreads();
     for (int i = threadIdx.x; i < planes_here; i += kThreads) counts[plane0 + i] = plane_count[i];
@@ -325,7 +328,7 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
         return check_launch("snnf_lif_pool_linear(pool)");
     }
     int ppb = (kThreads * kItems) / HW;
-    if (ppb < 1) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: H*W=%d exceeds %d", HW, kThreads * kItems);
+    if (ppb < 1) ppb = 1;   // a plane larger than one chunk: the workgroup walks it chunk by chunk
     if (ppb > kMaxPlanes) ppb = kMaxPlanes;
     const int blocks = (planes + ppb - 1) / ppb;
     lif_pool_kernel<XT, VT><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, ppb, static_cast<const VT*>(v_init),
@@ -354,42 +357,38 @@ extern "C" size_t snnf_lif_pool_linear_workspace_bytes(int N, int C) {
     return static_cast<size_t>(N) * static_cast<size_t>(C) * sizeof(int);
 }
 
-extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
-                                    const void* v_init, int v_dtype, const void* fc_weight, const void* fc_bias, int K,
-                                    int w_dtype, void* out_sum, void* v_out, void* workspace, size_t workspace_bytes,
-                                    float v_threshold, float v_reset, float tau, void* stream) {
-    using namespace snnf;
-    if (xs == nullptr || fc_weight == nullptr || out_sum == nullptr || v_out == nullptr)
-        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: xs, fc_weight, out_sum and v_out must be non-null");
-    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1)
-        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: T=%d N=%d C=%d H=%d W=%d K=%d", T, N, C, H, W, K);
+namespace snnf {
+namespace {
+
+// Shared body of the two entry points: `counts` is N * C ints of device memory (the caller's workspace or the library's
+// own static array).
+int lif_pool_linear_impl(const char* who, const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                         const void* v_init, int v_dtype, const void* fc_weight, const void* fc_bias, int K,
+                         int w_dtype, void* out_sum, void* v_out, int* counts,
+                         float v_threshold, float v_reset, float tau, void* stream) {
     if (T > SNNF_MAX_T_PER_LAUNCH)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_temporal_length: T=%d exceeds %d", T, SNNF_MAX_T_PER_LAUNCH);
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_temporal_length: T=%d exceeds %d", who, T, SNNF_MAX_T_PER_LAUNCH);
     if (!valid_dtype(x_dtype) || !valid_dtype(v_dtype) || !valid_dtype(w_dtype))
-        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: unknown dtype code");
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: unknown dtype code", who);
     if (w_dtype != x_dtype)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_dtype: fc_weight/fc_bias dtype must match x");
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: fc_weight/fc_bias dtype must match x", who);
     if (v_dtype != SNNF_F32 && v_dtype != x_dtype)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_dtype: membrane dtype must be fp32 or the activation dtype");
-    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: unsupported_tau: tau must be nonzero");
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: membrane dtype must be fp32 or the activation dtype", who);
+    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_tau: tau must be nonzero", who);
     const int64_t planes64 = static_cast<int64_t>(N) * C;
     const int64_t hw64 = static_cast<int64_t>(H) * W;
-    if (planes64 > 0x7fffffffLL || hw64 > kThreads * kItems)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: N*C=%lld or H*W=%lld too large", (long long)planes64, (long long)hw64);
-    if (N > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: N=%d exceeds 65535", N);
+    if (planes64 > 0x7fffffffLL || hw64 > (1 << 24) || planes64 * hw64 > 0x7fffffffLL)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: N*C=%lld or H*W=%lld too large", who, (long long)planes64, (long long)hw64);
+    if (N > 65535) return fail(SNNF_ERR_UNSUPPORTED, "%s: N=%d exceeds 65535", who, N);
     if (static_cast<size_t>(C) * sizeof(float) > 64 * 1024)
-        return fail(SNNF_ERR_UNSUPPORTED, "snnf_lif_pool_linear: C=%d exceeds LDS capacity", C);
-    if (workspace == nullptr || workspace_bytes < snnf_lif_pool_linear_workspace_bytes(N, C) || !aligned_to(workspace, 16))
-        return fail(SNNF_ERR_WORKSPACE, "snnf_lif_pool_linear: workspace of %zu bytes (16-byte aligned) required",
-                    snnf_lif_pool_linear_workspace_bytes(N, C));
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: C=%d exceeds LDS capacity", who, C);
     StepPtrs ptrs = {};
     for (int t = 0; t < T; ++t) {
-        if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: xs[%d] is null", t);
+        if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs[%d] is null", who, t);
         ptrs.p[t] = xs[t];
     }
     const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
     hipStream_t hs = as_stream(stream);
-    int* counts = static_cast<int*>(workspace);
     const int planes = static_cast<int>(planes64);
     const int HW = static_cast<int>(hw64);
 
@@ -412,5 +411,24 @@ extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, 
     if (x_dtype == SNNF_F32) run_linear<float>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
     else if (x_dtype == SNNF_BF16) run_linear<bf16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
     else run_linear<f16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
-    return check_launch("snnf_lif_pool_linear(linear)");
+    return check_launch(who);
+}
+
+}  // namespace
+}  // namespace snnf
+
+extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                                    const void* v_init, int v_dtype, const void* fc_weight, const void* fc_bias, int K,
+                                    int w_dtype, void* out_sum, void* v_out, void* workspace, size_t workspace_bytes,
+                                    float v_threshold, float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    if (xs == nullptr || fc_weight == nullptr || out_sum == nullptr || v_out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: xs, fc_weight, out_sum and v_out must be non-null");
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear: T=%d N=%d C=%d H=%d W=%d K=%d", T, N, C, H, W, K);
+    if (workspace == nullptr || workspace_bytes < snnf_lif_pool_linear_workspace_bytes(N, C) || !aligned_to(workspace, 16))
+        return fail(SNNF_ERR_WORKSPACE, "snnf_lif_pool_linear: workspace of %zu bytes (16-byte aligned) required",
+                    snnf_lif_pool_linear_workspace_bytes(N, C));
+    return lif_pool_linear_impl("snnf_lif_pool_linear", xs, T, N, C, H, W, x_dtype, v_init, v_dtype, fc_weight, fc_bias, K, w_dtype,
+                                out_sum, v_out, static_cast<int*>(workspace), v_threshold, v_reset, tau, stream);
 }

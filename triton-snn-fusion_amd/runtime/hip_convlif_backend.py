@@ -305,9 +305,7 @@ def _packed_weight(weight: torch.Tensor, bias: Optional[torch.Tensor], x_dtype: 
 
 
 def _membrane_dtype(x: torch.Tensor, v_init) -> torch.dtype:
-    if isinstance(v_init, torch.Tensor) and v_init.dtype in (torch.float32, x.dtype):
-        return v_init.dtype
-    return x.dtype
+    return _lib.membrane_dtype(x, v_init)
 
 
 def _v_init_pointer(v_init, out_shape, v_dtype, device):

@@ -16,7 +16,7 @@ from .. import _lib
 
 SUPPORTED_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 MAX_TIMESTEPS = _lib.SNNF_MAX_T_PER_LAUNCH
-MAX_PLANE_ELEMENTS = 1024
+MAX_PLANE_ELEMENTS = 1 << 24
 
 
 @dataclass
@@ -93,7 +93,7 @@ def run_triton_fused_temporal_lif_avgpool_linear(x_seq, v_init, fc_weight, fc_bi
     x = x_seq if x_seq.is_contiguous() else x_seq.contiguous()
     T, N, C, H, W = (int(d) for d in x.shape)
     K = int(fc_weight.shape[0])
-    v_dtype = v_init.dtype if v_init.dtype in (torch.float32, x.dtype) else x.dtype
+    v_dtype = _lib.membrane_dtype(x, v_init)
     vi = None
     if v_init.dim() != 0:
         vi = v_init if v_init.is_contiguous() else v_init.contiguous()

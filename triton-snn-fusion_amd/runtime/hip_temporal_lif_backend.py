@@ -87,9 +87,7 @@ def run_triton_fused_temporal_lif_state(x_seq, v_init, v_threshold: float, v_res
     x = x_seq if x_seq.is_contiguous() else x_seq.contiguous()
     T = int(x.shape[0])
     numel = int(x[0].numel())
-    v_dtype = v_init.dtype if v_init.dim() != 0 or v_init.dtype in (torch.float32, x.dtype) else x.dtype
-    if v_dtype not in (torch.float32, x.dtype):
-        v_dtype = x.dtype
+    v_dtype = _lib.membrane_dtype(x, v_init)
     vi = None
     if v_init.dim() != 0:
         vi = v_init if v_init.is_contiguous() else v_init.contiguous()
@@ -111,3 +109,28 @@ def run_triton_fused_temporal_lif_state(x_seq, v_init, v_threshold: float, v_res
     }
     return TritonTemporalLIFResult(spikes=spikes, v_next=v_next, used_triton=True, kernel_key="temporal_lif",
                                    kernel_temporal_config=config, kernel_diagnostics=diagnostics)
+
+
+def run_hip_lif_forward_state(x, v_prev, v_threshold: float, v_reset: float, tau: float):
+    """One LIF step on a tensor of any rank (the single-step operator `lif_forward_state`, which the reference always
+    evaluates with eager ops, runtime/snn_custom_ops.py:878-879): snnf_lif_scan with T = 1. A `v_prev` that is not a
+    membrane of x's shape on x's device starts from zeros (runtime/snn_custom_ops.py:378-381). Returns (spikes, v_next);
+    raises RuntimeError for tensors the kernel does not take."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype not in SUPPORTED_DTYPES or x.numel() == 0:
+        raise RuntimeError("unsupported_device: lif_forward_state on the HIP kernels needs a non-empty fp32/bf16/fp16 GPU tensor")
+    if float(tau) == 0.0:
+        raise RuntimeError("unsupported_tau: tau must be nonzero")
+    xc = x if x.is_contiguous() else x.contiguous()
+    v_dtype = _lib.membrane_dtype(xc, v_prev)
+    vi = None
+    if (isinstance(v_prev, torch.Tensor) and v_prev.dim() != 0 and tuple(v_prev.shape) == tuple(x.shape)
+            and v_prev.device == x.device and v_prev.dtype == v_dtype):
+        vi = v_prev if v_prev.is_contiguous() else v_prev.contiguous()
+    spikes = torch.empty_like(xc)
+    v_next = torch.empty(xc.shape, dtype=v_dtype, device=x.device)
+    numel = int(xc.numel())
+    _lib.check("snnf_lif_scan", _lib.lib().snnf_lif_scan(
+        _lib.step_pointers([xc]), 1, numel, _lib.dtype_code(x.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype),
+        spikes.data_ptr(), numel, v_next.data_ptr(), float(v_threshold), float(v_reset), float(tau),
+        _lib.current_stream(x.device)))
+    return spikes, v_next

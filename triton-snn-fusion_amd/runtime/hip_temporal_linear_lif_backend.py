@@ -104,7 +104,7 @@ def _run_steps(steps: List[torch.Tensor], weight, bias, v_init, v_threshold, v_r
     T = len(steps)
     M, Fin = int(first.shape[0]), int(first.shape[1])
     Fout = int(weight.shape[0])
-    v_dtype = v_init.dtype if v_init.dtype in (torch.float32, first.dtype) else first.dtype
+    v_dtype = _lib.membrane_dtype(first, v_init)
     row_stride = int(first.stride(0)) if M > 1 else Fin
     fixed = []
     for s in steps:

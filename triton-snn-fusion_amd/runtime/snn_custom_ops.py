@@ -36,7 +36,7 @@ from .hip_convlif_backend import (
     run_triton_fused_temporal_pointwise_conv_lif_state,
 )
 from .hip_temporal_lif_avgpool_linear_backend import run_triton_fused_temporal_lif_avgpool_linear
-from .hip_temporal_lif_backend import run_triton_fused_temporal_lif_state
+from .hip_temporal_lif_backend import run_hip_lif_forward_state, run_triton_fused_temporal_lif_state
 from .hip_temporal_linear_lif_backend import (
     run_triton_fused_temporal_linear_lif_state,
     run_triton_fused_temporal_linear_lif_state_packed,
@@ -266,29 +266,52 @@ def _require_library() -> None:
 # -----------------------------------------------------------------------------------------------------------------
 # Eager implementations (CPU tensors, "torch" backend, and calls outside the kernels' coverage)
 # -----------------------------------------------------------------------------------------------------------------
-def _ensure_v_prev(x: torch.Tensor, v_prev: torch.Tensor) -> torch.Tensor:
-    if (v_prev.dim() == 0 or tuple(v_prev.shape) != tuple(x.shape) or v_prev.device != x.device
-            or v_prev.dtype != x.dtype):
-        return torch.zeros_like(x)
+def _ensure_v_prev(x: torch.Tensor, v_prev: torch.Tensor, shape=None) -> torch.Tensor:
+    """The membrane a step starts from (runtime/snn_custom_ops.py:378-381): `v_prev` when it has the neurons' shape
+    (`shape`, default that of `x`), the device of `x` and the membrane dtype of the call (the activation dtype, or
+    float32 next to 16-bit activations, which the native kernels honour as well), zeros of that dtype otherwise."""
+    shape = tuple(x.shape if shape is None else shape)
+    v_dtype = _lib.membrane_dtype(x, v_prev)
+    if (not isinstance(v_prev, torch.Tensor) or v_prev.dim() == 0 or tuple(v_prev.shape) != shape
+            or v_prev.device != x.device or v_prev.dtype != v_dtype):
+        return torch.zeros(shape, dtype=v_dtype, device=x.device)
     return v_prev
 
 
-def lif_forward_state_torch(x, v_prev, v_threshold: float, v_reset: float, tau: float, detach_reset: bool):
-    v = _ensure_v_prev(x, v_prev)
-    h = v + x if float(tau) <= 1.0 else v + (x - v) / float(tau)
-    spike = (h >= float(v_threshold)).to(x.dtype)
+def _lif_step_torch(cur, v, spike_dtype, v_threshold: float, v_reset: float, tau: float, detach_reset: bool):
+    """One LIF update (runtime/snn_custom_ops.py:384-409) of the input current `cur` on the membrane `v` (same dtype)."""
+    h = v + cur if float(tau) <= 1.0 else v + (cur - v) / float(tau)
+    spike = (h >= float(v_threshold)).to(spike_dtype)
     gate = spike.detach() if bool(detach_reset) else spike
     if float(v_reset) < 0:
-        v_next = h - gate * float(v_threshold)
+        v_next = h - gate.to(h.dtype) * float(v_threshold)
     else:
         v_next = torch.where(gate.bool(), torch.full_like(h, float(v_reset)), h)
     return spike, v_next
 
 
+def lif_forward_state_torch(x, v_prev, v_threshold: float, v_reset: float, tau: float, detach_reset: bool):
+    v = _ensure_v_prev(x, v_prev)
+    cur = x if x.dtype == v.dtype else x.to(v.dtype)     # float32 membrane next to 16-bit activations: step in float32
+    return _lif_step_torch(cur, v, x.dtype, v_threshold, v_reset, tau, detach_reset)
+
+
+def _wide(x, v_prev, *operands):
+    """Operands of a layer whose membrane is float32 while its activations are 16 bit, converted to float32: the eager
+    path then accumulates and steps in float32 like the kernels (16-bit operands, float32 accumulator and membrane)."""
+    if _lib.membrane_dtype(x, v_prev) == x.dtype:
+        return (x,) + operands
+    return (x.float(),) + tuple(None if t is None else t.float() for t in operands)
+
+
 def fused_conv_lif_state_torch(x, weight, bias, v_prev, stride, padding, dilation, groups: int, v_threshold: float,
-                               v_reset: float, tau: float, detach_reset: bool):
-    cur = F.conv2d(x, weight, bias, stride, padding, dilation, groups)
-    return lif_forward_state_torch(cur, v_prev, v_threshold, v_reset, tau, detach_reset)
+                               v_reset: float, tau: float, detach_reset: bool, residual=None):
+    xw, ww, bw, rw = _wide(x, v_prev, weight, bias, residual)
+    cur = F.conv2d(xw, ww, bw, stride, padding, dilation, groups)
+    if rw is not None:
+        cur = cur + rw
+    v = _ensure_v_prev(x, v_prev, cur.shape)
+    return _lif_step_torch(cur, v, x.dtype, v_threshold, v_reset, tau, detach_reset)
 
 
 def fused_temporal_conv_lif_state_torch(xs, weight, bias, v_init, stride, padding, dilation, groups: int,
@@ -323,8 +346,8 @@ def fused_temporal_conv_add_lif_state_torch(xs, residuals, weight, bias, v_init,
         raise RuntimeError("xs and residuals must have the same temporal length")
     v, spikes = v_init, []
     for x, residual in zip(xs, residuals):
-        cur = F.conv2d(x, weight, bias, stride, padding, dilation, groups) + residual
-        s, v = lif_forward_state_torch(cur, v, v_threshold, v_reset, tau, detach_reset)
+        s, v = fused_conv_lif_state_torch(x, weight, bias, v, stride, padding, dilation, groups, v_threshold, v_reset, tau,
+                                          detach_reset, residual=residual)
         spikes.append(s)
     return torch.stack(spikes, dim=0), v
 
@@ -364,8 +387,10 @@ def fused_temporal_linear_lif_state_torch(xs, weight, bias, v_init, v_threshold:
         raise RuntimeError("fused_temporal_linear_lif_state requires at least one input tensor")
     v, spikes = v_init, []
     for x in xs:
-        s, v = lif_forward_state_torch(F.linear(x, weight, _optional_bias(bias)), v, v_threshold, v_reset, tau,
-                                       detach_reset)
+        xw, ww, bw = _wide(x, v, weight, _optional_bias(bias))
+        cur = F.linear(xw, ww, bw)
+        vv = _ensure_v_prev(x, v, cur.shape)
+        s, v = _lif_step_torch(cur, vv, x.dtype, v_threshold, v_reset, tau, detach_reset)
         spikes.append(s)
     return torch.stack(spikes, dim=0), v
 
@@ -401,9 +426,7 @@ def fused_temporal_linear_lif_state_packed_out_torch(x_seq, weight, bias, v_init
 # float32 or the activation dtype, which is x.dtype in every configuration the reference supports.
 # -----------------------------------------------------------------------------------------------------------------
 def _v_dtype(x, v_init) -> torch.dtype:
-    if isinstance(v_init, torch.Tensor) and v_init.dtype in (torch.float32, x.dtype):
-        return v_init.dtype
-    return x.dtype
+    return _lib.membrane_dtype(x, v_init)
 
 
 def _conv_out_shape(x, weight, stride, padding, dilation):
@@ -415,7 +438,7 @@ def _conv_out_shape(x, weight, stride, padding, dilation):
 
 
 def _lif_forward_state_meta(x, v_prev, v_threshold, v_reset, tau, detach_reset):
-    return x.new_empty(x.shape), x.new_empty(x.shape)
+    return x.new_empty(x.shape), x.new_empty(x.shape, dtype=_v_dtype(x, v_prev))
 
 
 def _fused_conv_lif_state_meta(x, weight, bias, v_prev, stride, padding, dilation, groups, v_threshold, v_reset, tau,
@@ -517,6 +540,18 @@ def _run(first, counters: Sequence[str], fallback_kind: str, shape_desc: str, na
 
 
 def _lif_forward_state_impl(x, v_prev, v_threshold, v_reset, tau, detach_reset):
+    """Single LIF step. The reference keeps this operator on eager ops and counts nothing for it
+    (runtime/snn_custom_ops.py:878-879); with the native backend selected a GPU tensor goes through the scan kernel
+    (one launch instead of seven elementwise ones), uncounted as well."""
+    if _native(x):
+        _require_library()
+        try:
+            return run_hip_lif_forward_state(x, v_prev, v_threshold, v_reset, tau)
+        except _lib.SnnfError:
+            raise
+        except RuntimeError:
+            if _strict():
+                raise
     return lif_forward_state_torch(x, v_prev, v_threshold, v_reset, tau, detach_reset)
 
 
