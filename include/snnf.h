@@ -101,6 +101,23 @@ int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int 
                          float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * snnf_lif_pool_linear without a workspace argument and without any allocation, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in
+ * the reference. The per-(n, c) spike counts between the two launches live in a static device array of the library
+ * (SNNF_LIF_POOL_LINEAR_STATIC_MAX_PLANES ints = 1 MiB per GPU the library runs on, held until the process ends);
+ * N * C beyond that returns SNNF_ERR_WORKSPACE. Arguments, kernels and results are those of snnf_lif_pool_linear.
+ * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race; calls on one stream
+ * are ordered and safe. The array's address is looked up on the first call on a device (not a stream operation; make
+ * that first call outside a graph capture).
+ */
+#define SNNF_LIF_POOL_LINEAR_STATIC_MAX_PLANES (256 * 1024)
+int snnf_lif_pool_linear_static(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                                const void* v_init, int v_dtype,
+                                const void* fc_weight, const void* fc_bias, int K, int w_dtype,
+                                void* out_sum, void* v_out,
+                                float v_threshold, float v_reset, float tau, void* stream);
+
+/*
  * Temporal Linear + LIF: for each t, s_t, v = LIF(x_t . W^T + b, v).
  * Replaces run_fused_temporal_linear_lif_state_kernel (kernels/generated_temporal_linear_lif_kernel.py:205-363) as
  * called by runtime/triton_temporal_linear_lif_backend.py:185-274.

@@ -7,6 +7,7 @@
 // in registers, counts spikes per plane in LDS and writes the integer counts to the workspace; launch 2 is a small GEMV
 // over the counts with wave-shuffle reductions.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "snnf_common.h"
@@ -431,4 +432,61 @@ extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, 
                     snnf_lif_pool_linear_workspace_bytes(N, C));
     return lif_pool_linear_impl("snnf_lif_pool_linear", xs, T, N, C, H, W, x_dtype, v_init, v_dtype, fc_weight, fc_bias, K, w_dtype,
                                 out_sum, v_out, static_cast<int*>(workspace), v_threshold, v_reset, tau, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same operator for callers that cannot allocate: the spike counts live in a static device array of the library.
+// ---------------------------------------------------------------------------------------------------------------
+namespace snnf {
+namespace {
+
+constexpr int kStaticCounts = SNNF_LIF_POOL_LINEAR_STATIC_MAX_PLANES;   // N * C of one call, at most
+constexpr int kMaxDevices = 64;
+
+// One copy per GPU the library runs on, held until the process ends. In host code this name is only a handle for
+// hipGetSymbolAddress: the device address it yields is what kernels and memory calls get.
+static __device__ __align__(256) int scratch[kStaticCounts];
+
+// Device address of `scratch` on the current device (looked up once per device), or nullptr after reporting why not.
+int* static_counts() {
+    static std::mutex mu;
+    static int* address[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        fail(SNNF_ERR_LAUNCH, "snnf_lif_pool_linear_static: cannot identify the current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (address[dev] == nullptr) {
+        void* p = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || p == nullptr) {
+            fail(SNNF_ERR_LAUNCH, "snnf_lif_pool_linear_static: hipGetSymbolAddress failed: %s", hipGetErrorString(err));
+            return nullptr;
+        }
+        address[dev] = static_cast<int*>(p);
+    }
+    return address[dev];
+}
+
+}  // namespace
+}  // namespace snnf
+
+extern "C" int snnf_lif_pool_linear_static(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
+                                           const void* v_init, int v_dtype, const void* fc_weight, const void* fc_bias,
+                                           int K, int w_dtype, void* out_sum, void* v_out,
+                                           float v_threshold, float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    if (xs == nullptr || fc_weight == nullptr || out_sum == nullptr || v_out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear_static: xs, fc_weight, out_sum and v_out must be non-null");
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_lif_pool_linear_static: T=%d N=%d C=%d H=%d W=%d K=%d", T, N, C, H, W, K);
+    if (static_cast<int64_t>(N) * C > kStaticCounts)
+        return fail(SNNF_ERR_WORKSPACE, "snnf_lif_pool_linear_static: N*C=%lld exceeds the static scratch of %d planes; "
+                    "use snnf_lif_pool_linear with a workspace", static_cast<long long>(N) * C, kStaticCounts);
+    int* counts = static_counts();
+    if (counts == nullptr) return SNNF_ERR_LAUNCH;
+    // Every plane count the second launch reads is written by the first, so nothing of an earlier call needs clearing.
+    return lif_pool_linear_impl("snnf_lif_pool_linear_static", xs, T, N, C, H, W, x_dtype, v_init, v_dtype, fc_weight, fc_bias, K,
+                                w_dtype, out_sum, v_out, counts, v_threshold, v_reset, tau, stream);
 }
