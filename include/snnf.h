@@ -41,6 +41,18 @@ typedef enum snnf_dtype {
     SNNF_F16 = 2
 } snnf_dtype;
 
+/* Activation layouts. NCHW is the layout of the reference's operators and of every entry point that takes no layout
+ * argument. C8 and BITS are internal layouts for tensors that travel between consecutive fused operators of one
+ * network without being seen by anyone else (the `*_blocked` entry points); no operator of the reference has them.
+ *   C8   : [N, ceil(C / 8), H, W, 8] elements of the activation dtype (16 bytes per pixel and group of 8 channels);
+ *          channels beyond C hold zeros.
+ *   BITS : [N, ceil(C / 8), H, W] bytes; bit j of a byte is the spike of channel 8 * c8 + j; bits beyond C are zero. */
+typedef enum snnf_layout {
+    SNNF_LAYOUT_NCHW = 0,
+    SNNF_LAYOUT_C8 = 1,
+    SNNF_LAYOUT_BITS = 2
+} snnf_layout;
+
 typedef enum snnf_status {
     SNNF_OK = 0,
     SNNF_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive extent, unknown dtype code */
@@ -179,6 +191,50 @@ int snnf_conv_bias(const void* const* xs, const void* const* residuals /* nullab
  *   x : [planes, H, W] x_dtype;  y : [planes, Ho, Wo] x_dtype */
 int snnf_pool2d(const void* x, void* y, int64_t planes, int H, int W, int kernel, int stride, int pad, int is_max,
                 int x_dtype, void* stream);
+
+/*
+ * Internal activation layouts between consecutive fused operators (see snnf_layout). The reference stores every spike as
+ * a dense 0/1 element of the activation dtype (kernels/benchmark_conv_lif_temporal_general.py:707-708) and copies the T
+ * inputs of a layer into one stack (runtime/triton_convlif_backend.py:579); its executor's fast path hands pooled
+ * caller-owned buffers to the `_packed_out` operator (runtime/fx_standalone_executor.py:900-952). The entry points below
+ * are this library's counterpart of that producer-consumer plumbing: a network executor keeps spikes at one bit each
+ * (16 times fewer bytes than bf16) and analog activations channel-blocked, in matrix-operand order.
+ *
+ * snnf_layout_bytes: bytes of `frames` frames of [C, H, W] in a layout (0 for invalid arguments).
+ * snnf_layout_convert: frames of [C, H, W] from one layout to another (any pair). Values written to BITS are
+ *   (element != 0); elements read from BITS are 0 / 1 in the activation dtype.
+ * snnf_pool2d_blocked: 2-D pooling of frames in C8 or BITS: max k x k / stride s / padding p (k in {2, 3}, s = 2) and
+ *   average 2 x 2 / 2. BITS -> BITS for max (a bitwise OR), BITS -> C8 for average (quarters are exact in 16 bits),
+ *   C8 -> C8 for both; SNNF_ERR_UNSUPPORTED otherwise. Same window rules as snnf_pool2d.
+ */
+size_t snnf_layout_bytes(int layout, int64_t frames, int C, int H, int W, int x_dtype);
+int snnf_layout_convert(const void* src, int src_layout, void* dst, int dst_layout, int64_t frames, int C, int H, int W,
+                        int x_dtype, void* stream);
+int snnf_pool2d_blocked(const void* x, int x_layout, void* y, int y_layout, int64_t frames, int C, int H, int W,
+                        int kernel, int stride, int pad, int is_max, int x_dtype, void* stream);
+
+/*
+ * snnf_conv_lif / snnf_conv_bias on the internal layouts: dense convolution + bias (+ residual) (+ LIF) over T steps
+ * with inputs in C8 or BITS, the residual in any layout, the output in any layout (BITS only with a neuron). Same
+ * operator semantics, packed weight (snnf_conv_pack_weight for the same activation dtype) and LIF rule as
+ * snnf_conv_lif, which replaces run_fused_temporal_general[_residual][_autotuned]
+ * (kernels/benchmark_conv_lif_temporal_general.py:971-1323) as called from runtime/triton_convlif_backend.py:513-817.
+ *   xs[t]        : N frames [Cin, H, W] in `x_layout` (C8, 16-byte aligned, or BITS); all T pointers equal = one frame
+ *                  shared by every timestep (convolved once)
+ *   residuals[t] : N frames [Cout, Ho, Wo] in `res_layout`, or residuals == NULL
+ *   x_dtype      : SNNF_BF16 or SNNF_F16 (dtype of C8 / NCHW elements and of the matrix operands)
+ *   out          : T x N frames [Cout, Ho, Wo] in `out_layout`, `out_step_stride` BYTES between timesteps
+ *   v_init       : [N, Cout, Ho, Wo] fp32 NCHW or NULL (zeros);  v_out : the same or NULL (final membrane not stored;
+ *                  only allowed when all T timesteps fit one window: T <= 4, or a shared frame)
+ *   neuron       : 1 = LIF and spikes; 0 = write conv + bias (+ residual) itself (out_layout C8 or NCHW), v_* ignored
+ * T <= SNNF_MAX_T_PER_LAUNCH, Cin and Cout arbitrary (groups of 8 are padded with zeros), dilation 1.
+ */
+int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
+                          int N, int Cin, int H, int W, int x_dtype,
+                          const void* packed_weight, int Cout, int KH, int KW,
+                          int stride_h, int stride_w, int pad_h, int pad_w,
+                          const void* v_init, void* out, int out_layout, int64_t out_step_stride, void* v_out,
+                          int neuron, float v_threshold, float v_reset, float tau, void* stream);
 
 /* Describes what the most recent snnf_conv_lif / snnf_conv_bias call on this thread selected: kernel family, timesteps per launch, tile
  * and wave decomposition, LDS bytes, grid ("key=value" pairs, empty before the first call). Plays the role of the

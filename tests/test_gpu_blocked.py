@@ -1,0 +1,222 @@
+"""GPU parity of the internal activation layouts (channel-blocked C8, bit-packed BITS): layout conversion and pooling are
+exact against plain tensor arithmetic; the blocked convolution + LIF kernel is gated against the CPU oracle like the dense
+operators (tests/helpers.py:check), with its bit-packed / blocked outputs converted back to dense tensors first, and
+bit for bit against the dense operator of the same library where both run the same arithmetic order is not required:
+the gate is the oracle's.
+"""
+import pytest
+import torch
+
+from helpers import DEV, LIF, check, dev, gen, q, spikes
+from oracle import snn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16, F16 = torch.float32, torch.bfloat16, torch.float16
+
+
+@pytest.fixture()
+def B(snnf_lib):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend
+    from triton_snn_fusion_amd.runtime import hip_convlif_backend
+    hip_convlif_backend.clear_packed_weight_cache()
+    return hip_blocked_backend
+
+
+def _ref_groups(x):
+    """[T, N, C, H, W] -> [T, N, C8, 8, H, W] with zero channels appended."""
+    T, N, C, H, W = x.shape
+    c8 = (C + 7) // 8
+    pad = torch.zeros(T, N, c8 * 8 - C, H, W, dtype=x.dtype)
+    return torch.cat([x, pad], 2).reshape(T, N, c8, 8, H, W)
+
+
+def _ref_bits(x):
+    g = (_ref_groups(x) != 0).to(torch.int32)
+    weights = (2 ** torch.arange(8, dtype=torch.int32)).reshape(1, 1, 1, 8, 1, 1)
+    return (g * weights).sum(3).to(torch.uint8)
+
+
+def _ref_c8(x):
+    return _ref_groups(x).permute(0, 1, 2, 4, 5, 3).contiguous()
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("shape", [(2, 3, 16, 5, 7), (1, 2, 20, 9, 9), (4, 1, 3, 8, 8), (1, 1, 64, 14, 14), (3, 2, 8, 1, 1)])
+def test_layout_conversions_are_exact(B, shape, dtype):
+    g = gen(3000 + shape[2])
+    s = spikes(shape, 0.3, g)
+    a = q(torch.randn(shape, generator=g), dtype)
+    ds, da = dev(s, dtype), dev(a, dtype)
+    bits = B.from_dense(ds, B.BITS)
+    assert bits.data.dtype == torch.uint8 and torch.equal(bits.data.cpu(), _ref_bits(s))
+    c8 = B.from_dense(da, B.C8)
+    assert torch.equal(c8.data.float().cpu(), _ref_c8(a))
+    assert torch.equal(B.to_dense(bits).float().cpu(), s)
+    assert torch.equal(B.to_dense(c8).float().cpu(), a)
+    # between the internal layouts
+    assert torch.equal(B.convert(B.from_dense(ds, B.C8), B.BITS).data.cpu(), _ref_bits(s))
+    assert torch.equal(B.convert(bits, B.C8).data.float().cpu(), _ref_c8(s))
+
+
+@pytest.mark.parametrize("kind,k,p,shape", [("max", 3, 1, (4, 2, 64, 16, 16)), ("max", 3, 1, (2, 1, 20, 9, 11)), ("max", 2, 0, (1, 3, 8, 6, 10)),
+                                            ("avg", 2, 0, (4, 2, 64, 8, 8)), ("avg", 2, 0, (2, 2, 12, 7, 9))])
+def test_pooling_on_the_internal_layouts_is_exact(B, kind, k, p, shape):
+    g = gen(3100 + shape[2] + k)
+    s = spikes(shape, 0.3, g)
+    a = q(torch.randn(shape, generator=g), BF16)
+    module = torch.nn.MaxPool2d(k, 2, p) if kind == "max" else torch.nn.AvgPool2d(2)
+    want_s = module(s.flatten(0, 1)).reshape(shape[0], shape[1], shape[2], *module(s.flatten(0, 1)).shape[-2:])
+    want_a = module(a.flatten(0, 1)).reshape(want_s.shape)
+    bits = B.from_dense(dev(s, BF16), B.BITS)
+    ps = B.pool_blocked(bits, kind == "max", k, 2, p)
+    assert ps.layout == (B.BITS if kind == "max" else B.C8)
+    assert torch.equal(B.to_dense(ps).float().cpu(), want_s)             # quarters are exact in bf16
+    pa = B.pool_blocked(B.from_dense(dev(a, BF16), B.C8), kind == "max", k, 2, p)
+    assert pa.layout == B.C8
+    assert torch.allclose(B.to_dense(pa).float().cpu(), q(want_a, BF16), rtol=2 ** -8, atol=1e-6)
+
+
+def _case(seed, T, N, Cin, Cout, H, W, k, dtype, analog=False, p=0.25, gain=2.0, shared=False):
+    g = gen(seed)
+    if analog:
+        frames = 1 if shared else T
+        xs = q(torch.randn(frames, N, Cin, H, W, generator=g), dtype)
+    else:
+        xs = spikes((T, N, Cin, H, W), p, g)
+    w = q(torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * k * k)) ** 0.5 * gain, dtype)
+    b = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    return xs, w, b
+
+
+BLOCKED_CASES = [  # Cin, Cout, H, W, k, s, p, dtype, lif, T, N, in layout, residual layout, out layout, tensor v_init
+    (64, 64, 16, 16, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 2, "bits", None, "bits", False),     # the common layer
+    (64, 64, 16, 16, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 2, "bits", "bits", "bits", True),    # + bit-packed residual, v_init
+    (32, 96, 12, 12, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 3, 2, "bits", "c8", "c8", False),       # 3 of 4 steps, blocked residual and output
+    (64, 72, 9, 11, 3, 1, 1, BF16, (1.0, -1.0, 2.0), 2, 3, "bits", "nchw", "nchw", True),    # ragged planes, Cout % 8 == 0 only, soft reset, dense ends
+    (20, 44, 10, 10, 3, 1, 1, BF16, (0.5, 0.0, 1.0), 1, 2, "bits", None, "bits", False),     # channel counts that are no multiples of 8, IF neuron
+    (64, 128, 16, 16, 3, 2, 1, BF16, (1.0, 0.0, 2.0), 4, 2, "bits", None, "bits", False),    # stride 2: windows of 2 steps
+    (64, 128, 16, 16, 1, 2, 0, BF16, (1.0, 0.0, 2.0), 4, 2, "bits", None, "bits", False),    # strided 1x1
+    (128, 64, 8, 8, 1, 1, 0, BF16, (1.0, 0.0, 3.0), 4, 2, "bits", None, "bits", True),       # plain 1x1, tau not a power of two
+    (64, 64, 12, 12, 5, 1, 2, F16, (1.0, 0.0, 2.0), 4, 2, "bits", None, "bits", False),      # 5x5, fp16
+    (64, 64, 14, 14, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 6, 2, "bits", "bits", "bits", False),   # two windows (4 + 2)
+    (64, 64, 8, 8, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 2, "c8", None, "bits", False),         # analog blocked input
+    (256, 128, 7, 7, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 4, "bits", "bits", "bits", True),    # 7x7 planes, K split over waves
+    (512, 128, 4, 4, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 6, "bits", None, "bits", False),     # 4x4 planes: two images per patch, K split
+    (128, 128, 2, 2, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 20, "bits", "c8", "bits", True),     # 2x2 planes: eight images per patch
+    (512, 512, 7, 7, 3, 1, 1, BF16, (1.0, 0.0, 2.0), 4, 4, "bits", None, "nchw", False),     # deep layer, dense output
+]
+
+
+def _to_layout(B, t, name, dtype):
+    return B.from_dense(dev(t, dtype), {"nchw": B.NCHW, "c8": B.C8, "bits": B.BITS}[name])
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p,dtype,lif,T,N,inl,resl,outl,tensor_v", BLOCKED_CASES)
+def test_blocked_conv_lif_against_the_oracle(B, Cin, Cout, H, W, k, s, p, dtype, lif, T, N, inl, resl, outl, tensor_v):
+    xs, w, b = _case(3200 + Cin + Cout + H + k + T, T, N, Cin, Cout, H, W, k, dtype, analog=inl == "c8")
+    Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    g = gen(3201 + Cin)
+    if resl == "bits":
+        rs = spikes((T, N, Cout, Ho, Wo), 0.3, g)
+    elif resl is not None:
+        rs = q(torch.randn(T, N, Cout, Ho, Wo, generator=g) * 0.3, dtype)
+    else:
+        rs = None
+    v0 = torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3 if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif([xs[t] for t in range(T)], w, b, v0, (s, s), (p, p), (1, 1), 1, *lif,
+                              residuals=None if rs is None else [rs[t] for t in range(T)])
+    x = _to_layout(B, xs, inl, dtype)
+    res = None if rs is None else _to_layout(B, rs, resl, dtype)
+    out_layout = {"nchw": B.NCHW, "c8": B.C8, "bits": B.BITS}[outl]
+    print(f"blocked conv {Cin}->{Cout} {H}x{W} k{k} s{s} T={T} N={N} {inl}/{resl}/{outl}", flush=True)
+    out, v = B.conv_lif_blocked(x, dev(w, dtype), dev(b, dtype), [s, s], [p, p], lif, residual=res, out_layout=out_layout,
+                                v_init=dev(v0, F32) if tensor_v else None, want_v=True)
+    torch.cuda.synchronize()
+    assert B.last_conv_plan()["kernel"] == "blocked"
+    assert out.layout == out_layout and out.shape == (T, N, Cout, Ho, Wo) and v.dtype == F32
+    rep = check(B.to_dense(out), v, ref, v_threshold=lif[0], what=f"blocked {Cin}->{Cout} k{k} s{s} {inl}->{outl}")
+    assert 0.001 < float(ref[0].mean()) < 0.9, float(ref[0].mean())
+    assert rep["neurons_with_matching_history"] >= 0.999 * rep["neurons"]
+    if outl != "nchw" and Cout % 8:       # padded channels of the internal layouts hold zeros
+        c8 = (Cout + 7) // 8
+        if outl == "bits":
+            assert int((out.data[:, :, c8 - 1] >> (Cout % 8)).max()) == 0
+        else:
+            assert float(out.data[:, :, c8 - 1, :, :, Cout % 8:].abs().max()) == 0.0
+
+
+def test_blocked_conv_without_membrane_output_and_chained_windows(B):
+    """The final membrane is optional; two calls chained through it equal one call of all steps, bit for bit."""
+    T, N, C, H = 4, 2, 64, 12
+    xs, w, b = _case(3300, T, N, C, C, H, H, 3, BF16)
+    x = B.from_dense(dev(xs, BF16), B.BITS)
+    dw, db = dev(w, BF16), dev(b, BF16)
+    out, v = B.conv_lif_blocked(x, dw, db, [1, 1], [1, 1], LIF, want_v=True)
+    out2, v2 = B.conv_lif_blocked(x, dw, db, [1, 1], [1, 1], LIF, want_v=False)
+    assert v2 is None and torch.equal(out.data, out2.data)
+    xa = B.from_dense(dev(xs[:1], BF16), B.BITS)
+    xb = B.from_dense(dev(xs[1:], BF16), B.BITS)
+    oa, va = B.conv_lif_blocked(xa, dw, db, [1, 1], [1, 1], LIF, want_v=True)
+    ob, vb = B.conv_lif_blocked(xb, dw, db, [1, 1], [1, 1], LIF, v_init=va, want_v=True)
+    assert torch.equal(torch.cat([oa.data, ob.data]), out.data) and torch.equal(vb, v)
+
+
+SHARED_CASES = [  # Cin, Cout, H, W, k, s, p, T, N
+    (3, 64, 32, 32, 7, 2, 3, 4, 2),      # ResNet stem: one analog frame, taps paired inside a single channel group
+    (3, 64, 16, 16, 3, 1, 1, 16, 2),     # VGG stem, 16 LIF steps on one convolution
+    (64, 64, 8, 8, 3, 1, 1, 5, 2),       # whole channel groups
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p,T,N", SHARED_CASES)
+def test_blocked_conv_with_one_analog_frame_for_all_timesteps(B, Cin, Cout, H, W, k, s, p, T, N):
+    xs, w, b = _case(3400 + Cin + H, T, N, Cin, Cout, H, W, k, BF16, analog=True, shared=True, gain=1.5)
+    ref = O.temporal_conv_lif([xs[0]] * T, w, b, torch.tensor(0.0), (s, s), (p, p), (1, 1), 1, *LIF)
+    x = B.from_dense(dev(xs[0], BF16), B.C8, shared=True)
+    x.T = T
+    out, v = B.conv_lif_blocked(x, dev(w, BF16), dev(b, BF16), [s, s], [p, p], LIF, want_v=True)
+    plan = B.last_conv_plan()
+    assert plan["kernel"] == "blocked" and plan["window"] == T
+    check(B.to_dense(out), v, ref, what=f"blocked shared frame {Cin}->{Cout} k{k}")
+    assert 0.001 < float(ref[0].mean()) < 0.9
+
+
+CONV_BIAS_CASES = [  # Cin, Cout, H, W, k, s, p, T, N, residual layout, out layout
+    (64, 128, 16, 16, 1, 2, 0, 4, 2, None, "c8"),        # downsample shortcut: spikes in, analog blocked out
+    (64, 64, 7, 7, 3, 1, 1, 4, 3, "c8", "nchw"),         # pre-tail sum: conv + blocked residual, dense out
+    (128, 96, 7, 7, 3, 1, 1, 3, 2, "bits", "c8"),        # spike residual
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p,T,N,resl,outl", CONV_BIAS_CASES)
+def test_blocked_conv_without_neuron(B, Cin, Cout, H, W, k, s, p, T, N, resl, outl):
+    """No neuron: conv + bias (+ residual) in fp32 from bf16 operands, one rounding to bf16 at the store."""
+    xs, w, b = _case(3500 + Cin + Cout, T, N, Cin, Cout, H, W, k, BF16)
+    Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    g = gen(3501)
+    rs = None if resl is None else (spikes((T, N, Cout, Ho, Wo), 0.3, g) if resl == "bits" else q(torch.randn(T, N, Cout, Ho, Wo, generator=g), BF16))
+    want = torch.stack([torch.nn.functional.conv2d(xs[t], w, b, s, p) for t in range(T)])
+    if rs is not None:
+        want = want + rs
+    out, v = B.conv_lif_blocked(B.from_dense(dev(xs, BF16), B.BITS), dev(w, BF16), dev(b, BF16), [s, s], [p, p], None,
+                                residual=None if rs is None else _to_layout(B, rs, resl, BF16),
+                                out_layout={"nchw": B.NCHW, "c8": B.C8}[outl])
+    assert v is None
+    got = B.to_dense(out).float().cpu()
+    assert torch.allclose(got, want, rtol=2 ** -8, atol=1e-3), (got - want).abs().max()
+
+
+def test_blocked_conv_rejects_what_it_does_not_take(B):
+    x = B.from_dense(torch.zeros(4, 2, 64, 8, 8, device=DEV, dtype=BF16), B.BITS)
+    w = torch.zeros(64, 64, 3, 3, device=DEV, dtype=BF16)
+    with pytest.raises(RuntimeError, match="unsupported_layout"):
+        B.conv_lif_blocked(x, w, None, [1, 1], [1, 1], None, out_layout=B.BITS)          # bits without a neuron
+    with pytest.raises(RuntimeError, match="unsupported_layout"):
+        B.conv_lif_blocked(B.from_dense(torch.zeros(4, 2, 64, 8, 8, device=DEV, dtype=BF16), B.NCHW), w, None, [1, 1], [1, 1], LIF)
+    with pytest.raises(RuntimeError, match="unsupported_groups"):
+        B.conv_lif_blocked(x, torch.zeros(64, 1, 3, 3, device=DEV, dtype=BF16), None, [1, 1], [1, 1], LIF)
+    with pytest.raises(RuntimeError, match="unsupported_padding"):
+        B.conv_lif_blocked(x, w, None, [1, 1], [2, 2], LIF)

@@ -192,16 +192,19 @@ def test_fx_rewrite_leaves_a_layer_alone_when_its_state_chain_is_broken():
 # ---------------------------------------------------------------------------------------------------------------
 # Fused form (GPU)
 # ---------------------------------------------------------------------------------------------------------------
-def _fused(name, T=4, gain=5.0):
+def _fused(name, T=4, gain=5.0, internal=False):
     model = M.build_network(name, width=SMALL[name]["width"], gain=gain)
-    return model, M.fuse_network(model, T, BF16, DEV)
+    return model, M.fuse_network(model, T, BF16, DEV, internal_layouts=internal)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
 @pytest.mark.parametrize("name", ["vgg11", "resnet18"])
-def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name):
+def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
+    """`internal`: spikes bit-packed and analog activations channel-blocked between the network's own operators; the
+    executor records every operator's operands and results converted back to dense tensors."""
     T = 4
-    model, fused = _fused(name, T)
+    model, fused = _fused(name, T, internal=internal)
     fused.record = []
     out = fused(_frame(name))
     torch.cuda.synchronize()
@@ -236,7 +239,11 @@ def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name):
             assert torch.allclose(out.float().cpu(), ref_out / T, rtol=8e-3, atol=8e-3)
     assert active >= 5, "the test network is nearly silent"
     stats = hip_ops.get_fused_op_call_stats()
-    assert stats["fallback"] == 0 and stats["triton"] == kinds.count("conv_lif") + 1, stats
+    if internal:      # only the tail goes through the dense operator layer
+        assert all(e.get("blocked") for e in fused.record if e["kind"] != "tail")
+        assert stats["fallback"] == 0 and stats["triton"] == 1, stats
+    else:
+        assert stats["fallback"] == 0 and stats["triton"] == kinds.count("conv_lif") + 1, stats
 
 
 @pytest.mark.gpu
@@ -267,9 +274,28 @@ def test_fused_network_tracks_the_eager_network(hip_ops, name):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["vgg11", "resnet18"])
-def test_fused_network_graph_replay_matches_eager_launches(hip_ops, name):
+def test_internal_layouts_track_the_dense_executor(hip_ops, name):
+    """Same network, same operands: the two executors differ in summation order only, so the first layer agrees up to
+    near-threshold flips and the logits point the same way."""
     T = 4
-    _, fused = _fused(name, T)
+    _, dense = _fused(name, T)
+    _, internal = _fused(name, T, internal=True)
+    x = _frame(name)
+    dense.record, internal.record = [], []
+    want, got = dense(x).float().cpu(), internal(x).float().cpu()
+    mismatch = (dense.record[0]["spikes"].float().cpu() != internal.record[0]["spikes"].float().cpu()).float().mean()
+    assert float(mismatch) <= 1e-4, float(mismatch)
+    cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
+    print(f"{name}: internal layouts vs dense executor, cosine similarity of the logits {cos:.5f}")
+    assert cos > 0.8, cos
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fused_network_graph_replay_matches_eager_launches(hip_ops, name, internal):
+    T = 4
+    _, fused = _fused(name, T, internal=internal)
     frames = [_frame(name, seed=20 + i) for i in range(3)]
     replay, static_in, static_out = fused.capture(frames[0])
     for f in frames + [frames[0]]:

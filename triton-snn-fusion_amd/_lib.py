@@ -15,6 +15,7 @@ PKG_DIR = Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "lib" / "libsnnf.so"
 
 SNNF_F32, SNNF_BF16, SNNF_F16 = 0, 1, 2
+SNNF_LAYOUT_NCHW, SNNF_LAYOUT_C8, SNNF_LAYOUT_BITS = 0, 1, 2
 SNNF_MAX_T_PER_LAUNCH = 16
 
 _DTYPE_CODES = {torch.float32: SNNF_F32, torch.bfloat16: SNNF_BF16, torch.float16: SNNF_F16}
@@ -44,6 +45,11 @@ SIGNATURES = {
     "snnf_conv_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "snnf_conv_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i64,
                            _vp, _f, _f, _f, _vp]),
+    "snnf_layout_bytes": (_sz, [_i, _i64, _i, _i, _i, _i]),
+    "snnf_layout_convert": (_i, [_vp, _i, _vp, _i, _i64, _i, _i, _i, _i, _vp]),
+    "snnf_pool2d_blocked": (_i, [_vp, _i, _vp, _i, _i64, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "snnf_conv_lif_blocked": (_i, [_pp, _i, _pp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i64,
+                                   _vp, _i, _f, _f, _f, _vp]),
     "snnf_pool2d": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "snnf_conv_bias": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
 }

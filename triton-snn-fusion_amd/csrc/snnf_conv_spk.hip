@@ -1,0 +1,207 @@
+// Host side of the convolution + LIF operator on the internal activation layouts (channel-blocked C8, bit-packed BITS):
+// argument validation, patch planning and launch of conv_spk_kernel.
+#include <algorithm>
+#include <cstdio>
+
+#include "snnf_conv_spk_kernel.h"
+
+namespace snnf {
+namespace {
+
+constexpr int kWaveLds = static_cast<int>(kMaxLds) / kSpkWaves;   // private staging bytes of a wave
+
+struct SpkPlan {
+    int PR, PC, PI, RR, RC, region, G, patches_x, patches_y, img_groups;
+    double score;
+};
+
+// Patch of a wave (PR x PC output pixels of one image, or PI whole planes when a plane has at most 32 pixels) and the
+// channel groups per LDS stage G: the patch with the most useful matrix lanes and the smallest halo whose stage fits the
+// wave's LDS region and its staging slots; the largest such G (fewer, longer stages).
+bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best) {
+    best.score = -1.0;
+    for (int pc = 1; pc <= 32 && pc <= g0.Wo; ++pc) {
+        const int pr = std::min(32 / pc, g0.Ho);
+        const bool whole = pr == g0.Ho && pc == g0.Wo;
+        const int pi = whole ? std::max(1, std::min(g0.N, 32 / (pr * pc))) : 1;
+        const int rr = (pr - 1) * g0.sh + g0.KH;
+        const int rc = (pc - 1) * g0.sw + g0.KW;
+        if (rr > 255 || rc > 255) continue;
+        const int region = pi * rr * rc;
+        int G = 0;
+        if (g0.tap_pairs) {
+            if (region <= 64 * kSpkSlots && tt * region * 16 <= kWaveLds) G = 1;
+        } else {
+            for (int cand = g0.gpc; cand >= 2; cand >>= 1) {
+                if (cand * region <= 64 * kSpkSlots && tt * cand * region * 16 <= kWaveLds) {
+                    G = cand;
+                    break;
+                }
+            }
+        }
+        if (G == 0) continue;
+        const int patches_x = (g0.Wo + pc - 1) / pc;
+        const int patches_y = (g0.Ho + pr - 1) / pr;
+        const int img_groups = (g0.N + pi - 1) / pi;
+        const double lanes = static_cast<double>(img_groups) * patches_x * patches_y * 32.0;
+        const double eff = static_cast<double>(g0.N) * g0.Ho * g0.Wo / lanes;
+        const double halo = static_cast<double>(region) / (static_cast<double>(pi) * pr * pc);
+        // Wide patches store longer runs of a row; stages of 4 slots move in one batch.
+        double score = eff / (1.0 + 0.08 * (halo - 1.0)) * (1.0 + 0.004 * std::min(pc, 16));
+        if (G * region > 256) score *= 0.97;
+        if (score > best.score) best = SpkPlan{pr, pc, pi, rr, rc, region, G, patches_x, patches_y, img_groups, score};
+    }
+    return best.score > 0.0;
+}
+
+bool valid_layout(int layout) { return layout == SNNF_LAYOUT_NCHW || layout == SNNF_LAYOUT_C8 || layout == SNNF_LAYOUT_BITS; }
+
+}  // namespace
+
+char* conv_plan_buffer();   // the thread's plan text (snnf_conv_igemm.hip), shared with snnf_conv_last_plan()
+
+}  // namespace snnf
+
+extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
+                                     int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
+                                     int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
+                                     int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
+                                     float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    const char* who = "snnf_conv_lif_blocked";
+    if (xs == nullptr || packed_weight == nullptr || out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs, packed_weight and out must be non-null", who);
+    if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: bad extent (T=%d N=%d Cin=%d H=%d W=%d Cout=%d K=%dx%d s=%dx%d p=%dx%d)", who,
+                    T, N, Cin, H, W, Cout, KH, KW, stride_h, stride_w, pad_h, pad_w);
+    if (T > SNNF_MAX_T_PER_LAUNCH)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_temporal_length: T=%d exceeds %d", who, T, SNNF_MAX_T_PER_LAUNCH);
+    if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: the internal layouts hold bf16 or fp16 activations", who);
+    if (x_layout != SNNF_LAYOUT_C8 && x_layout != SNNF_LAYOUT_BITS)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: inputs must be in C8 or BITS layout", who);
+    if (!valid_layout(out_layout) || (residuals != nullptr && !valid_layout(res_layout)))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: unknown layout code", who);
+    if (!neuron && out_layout == SNNF_LAYOUT_BITS)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: an output without a neuron cannot be bit-packed", who);
+    if (neuron && !(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_tau: tau must be nonzero", who);
+    if (H + 2 * pad_h < KH || W + 2 * pad_w < KW)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_kernel: kernel larger than padded input", who);
+    if (2 * pad_h > KH || 2 * pad_w > KW)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_padding: padding %dx%d too large for kernel %dx%d", who, pad_h, pad_w, KH, KW);
+    // Bytes a tensor in a layout is accessed by: bit-packed tensors by single bytes, blocked inputs by 16-byte groups, blocked
+    // outputs and residuals by 4 channels (8 bytes), dense tensors by elements.
+    auto need_align = [](int layout, bool as_input) -> size_t { return layout == SNNF_LAYOUT_BITS ? 1 : (layout == SNNF_LAYOUT_C8 ? (as_input ? 16 : 8) : 2); };
+    if (!aligned_to(packed_weight, 16) || !aligned_to(out, need_align(out_layout, false)) || (out_step_stride % need_align(out_layout, false)) != 0 ||
+        (v_init != nullptr && !aligned_to(v_init, 4)) || (v_out != nullptr && !aligned_to(v_out, 4)))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: packed_weight, out (and its step stride) or a membrane pointer is misaligned", who);
+    bool shared = T > 1;
+    for (int t = 0; t < T; ++t) {
+        if (xs[t] == nullptr || !aligned_to(xs[t], need_align(x_layout, true)))
+            return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs[%d] is null or misaligned for its layout", who, t);
+        if (residuals != nullptr && (residuals[t] == nullptr || !aligned_to(residuals[t], need_align(res_layout, false))))
+            return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: residuals[%d] is null or misaligned for its layout", who, t);
+        shared = shared && xs[t] == xs[0];
+    }
+
+    SpkGeom g = {};
+    g.N = N; g.Cin = Cin; g.H = H; g.W = W; g.Cout = Cout; g.KH = KH; g.KW = KW;
+    g.sh = stride_h; g.sw = stride_w; g.ph = pad_h; g.pw = pad_w;
+    g.Ho = (H + 2 * pad_h - KH) / stride_h + 1;
+    g.Wo = (W + 2 * pad_w - KW) / stride_w + 1;
+    g.C8in = (Cin + 7) / 8;
+    g.C8out = (Cout + 7) / 8;
+    const int64_t in_items = static_cast<int64_t>(N) * g.C8in * H * W;
+    const int64_t out_elems = static_cast<int64_t>(N) * g.C8out * 8 * g.Ho * g.Wo;
+    if (in_items >= (1LL << 27) || out_elems >= (1LL << 30) || static_cast<int64_t>(T) * N * g.C8out * g.Ho * g.Wo >= (1LL << 31))
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: tensor too large for 32-bit offsets", who);
+    if (out_layout == SNNF_LAYOUT_BITS && (out_step_stride < 0 || out_step_stride >= (1LL << 31) / T))
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: bit-packed output beyond 2 GiB", who);
+    const PackGeom pg = make_pack_geom(Cout, Cin, KH, KW, false);
+    g.gpc = pg.CK / 8;
+    g.npairs = pg.npairs;
+    g.nocf = pg.nocf;
+    g.tap_pairs = pg.CK == 8 ? 1 : 0;
+    g.taps = KH * KW;
+    g.frag_stride = static_cast<int64_t>(pg.nchunks) * pg.npairs * (kFragBytes / 2);
+    g.T = T;
+    g.shared_x = shared ? 1 : 0;
+    g.in_layout = x_layout;
+    g.res_layout = residuals != nullptr ? res_layout : -1;
+    g.out_layout = out_layout;
+    g.analog_out = neuron ? 0 : 1;
+    g.out_step_stride = out_step_stride;
+
+    // Timesteps side by side: 4 (2 for T == 2, 1 for a single step or a shared frame), fewer when the halo does not fit.
+    int tt = shared || T == 1 ? 1 : (T == 2 ? 2 : 4);
+    SpkPlan pl = {};
+    bool planned = false;
+    for (; tt >= 1; tt >>= 1) {
+        planned = plan_spk(g, tt, pl);
+        if (planned) break;
+    }
+    if (!planned)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: no patch of this layer fits a wave's LDS region (kernel %dx%d, stride %dx%d)",
+                    who, KH, KW, stride_h, stride_w);
+    const int windows = shared ? 1 : (T + tt - 1) / tt;
+    if (neuron && windows > 1 && v_out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: v_out is required when the timesteps take %d windows of %d (it carries the membrane between them)",
+                    who, windows, tt);
+    g.PR = pl.PR; g.PC = pl.PC; g.PI = pl.PI; g.RR = pl.RR; g.RC = pl.RC; g.region = pl.region; g.G = pl.G;
+    g.patches_x = pl.patches_x;
+    g.patches_img = pl.patches_x * pl.patches_y;
+    g.n_patches = pl.img_groups * g.patches_img;
+    g.nstages = (g.C8in + g.G - 1) / g.G;
+    g.IT = g.G * g.region;
+    g.JT = (g.IT + 63) / 64;
+    g.lds_wave_bytes = tt * g.IT * 16;
+    const int oc_tiles = (Cout + 63) / 64;
+    g.n_items = g.n_patches * oc_tiles;
+    // Split K over waves of a workgroup while the layer has fewer items than the machine has SIMDs (one wave each) and
+    // every wave still gets at least two stages.
+    const int cus = compute_units();
+    int wk_log2 = 0;
+    while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 4 && g.nstages >= (4 << wk_log2)) ++wk_log2;
+    g.wk_log2 = wk_log2;
+    const int tiles_per_block = kSpkWaves >> wk_log2;
+    int grid = (g.n_items + tiles_per_block - 1) / tiles_per_block;
+    if (grid > cus) grid = cus;
+    g.iters = (g.n_items + grid * tiles_per_block - 1) / (grid * tiles_per_block);
+    g.d_ppx = make_fast_div(g.PR * g.PC);
+    g.d_PC = make_fast_div(g.PC);
+    g.d_region = make_fast_div(g.region);
+    g.d_rrrc = make_fast_div(g.RR * g.RC);
+    g.d_RC = make_fast_div(g.RC);
+    g.d_n_patches = make_fast_div(g.n_patches);
+    g.d_patches_img = make_fast_div(g.patches_img);
+    g.d_patches_x = make_fast_div(g.patches_x);
+    g.d_gpc = make_fast_div(g.gpc);
+    const int hg = g.tap_pairs ? 1 : g.G / 2;
+    const int nst = g.tap_pairs ? g.npairs : g.taps * hg;
+    g.d_hg = make_fast_div(hg);
+    g.d_nst = make_fast_div(nst);
+    g.d_KW = make_fast_div(KW);
+
+    SpkLaunch L = {};
+    for (int t = 0; t < T; ++t) {
+        L.xs.p[t] = xs[t];
+        if (residuals != nullptr) L.residuals.p[t] = residuals[t];
+    }
+    L.g = g;
+    L.wpacked = static_cast<const uint16_t*>(packed_weight);
+    L.bias = reinterpret_cast<const float*>(L.wpacked + packed_weight_elems(pg));
+    L.v_init = neuron ? static_cast<const float*>(v_init) : nullptr;
+    L.out = out;
+    L.v_out = neuron ? static_cast<float*>(v_out) : nullptr;
+    L.lif = make_lif_params(v_threshold, v_reset, tau);
+    L.grid = grid;
+    L.lds_bytes = static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes;
+    if (wk_log2 > 0 && L.lds_bytes < kSpkPartialBytes) L.lds_bytes = kSpkPartialBytes;
+    L.stream = as_stream(stream);
+    snprintf(snnf::conv_plan_buffer(), 256,
+             "kernel=blocked variant=%d window=%d launches=1 tile=%dx%dx%d halo=%dx%d waves=8x1x%d oc_tiles=%d px_tiles=%d "
+             "stage_chunks=%d run=0 lds=%zu grid=%d",
+             (wk_log2 > 0 ? 50 : 40) + tt, shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
+             L.lds_bytes, grid);
+    return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16(L, tt) : launch_conv_spk_f16(L, tt);
+}

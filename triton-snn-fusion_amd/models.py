@@ -263,7 +263,8 @@ class _FusedNetwork(nn.Module):
     """Shared plumbing: parameter folding, operator calls, optional recording of every operator call (inputs and
     outputs, for layer-by-layer verification), and whole-forward HIP graph capture."""
 
-    def __init__(self, T: int, dtype: torch.dtype, device, v_dtype: torch.dtype = torch.float32):
+    def __init__(self, T: int, dtype: torch.dtype, device, v_dtype: torch.dtype = torch.float32,
+                 internal_layouts: bool = False):
         super().__init__()
         from .runtime import snn_custom_ops
         if torch.device(device).type == "cuda":
@@ -276,6 +277,11 @@ class _FusedNetwork(nn.Module):
         self.record: Optional[List[Dict]] = None
         self.native_plain_conv = True        # False: LIF-free convolutions always go to the framework's convolution
         self.native_pool = True              # False: pooling layers always go to the framework's modules
+        # True: between the network's own operators spikes travel bit-packed and analog activations channel-blocked
+        # (runtime/hip_blocked_backend.py); the dense `snn_custom` operators then only serve the tail. GPU, 16-bit only.
+        self.internal_layouts = bool(internal_layouts)
+        self.keep_membranes = False          # internal layouts: also write every layer's final membrane (nobody reads it:
+                                             # the harness resets all neurons between forwards, like the reference's)
         self._graph = None
 
     # -- operator calls ------------------------------------------------------------------------------------------
@@ -328,6 +334,36 @@ class _FusedNetwork(nn.Module):
         self._log(kind="pool", name=name, x=x_seq, pool=pool, y=y, native=config is not None)
         return y
 
+    # -- the same operators on the internal layouts ----------------------------------------------------------------
+    def conv_lif_b(self, name: str, x, layer: _FusedLayer, residual=None, out_layout=None):
+        """Conv + folded BN (+ residual) + LIF (`layer.lif`), or without a neuron when the layer has none, on Blocked tensors."""
+        from .runtime import hip_blocked_backend as B
+        if out_layout is None:
+            out_layout = B.BITS if layer.lif is not None else B.C8
+        out, v = B.conv_lif_blocked(x, layer.weight, layer.bias, layer.stride, layer.padding, layer.lif, residual=residual,
+                                    out_layout=out_layout, want_v=self.keep_membranes or self.record is not None)
+        if self.record is not None:
+            T = x.T
+            xs = list(B.to_dense(x).unbind(0)) if not x.shared else [B.to_dense(x)[0]] * T
+            rs = None if residual is None else list(B.to_dense(residual).unbind(0))
+            if layer.lif is not None:
+                self._log(kind="conv_lif", name=name, xs=xs, residuals=rs, layer=layer, spikes=B.to_dense(out), v=v, blocked=True)
+            else:
+                self._log(kind="plain_conv", name=name, x=torch.stack(xs), layer=layer, residual=None if rs is None else torch.stack(rs),
+                          y=B.to_dense(out), native=True, blocked=True)
+        return out
+
+    def pooled_b(self, name: str, x, pool: nn.Module):
+        from .runtime import hip_blocked_backend as B
+        from .runtime.hip_pool_backend import pool_config
+        config = pool_config(pool)
+        if config is None:
+            raise RuntimeError(f"unsupported_kernel: no blocked pooling kernel for {pool}")
+        y = B.pool_blocked(x, *config)
+        if self.record is not None:
+            self._log(kind="pool", name=name, x=B.to_dense(x), pool=pool, y=B.to_dense(y), native=True, blocked=True)
+        return y
+
     def tail(self, x_seq: torch.Tensor, lif, fc_weight, fc_bias) -> torch.Tensor:
         out_sum, v = torch.ops.snn_custom.fused_temporal_lif_avgpool_linear(x_seq, self.zero_v, fc_weight, fc_bias, *lif, False)
         self._log(kind="tail", name="tail", x=x_seq, lif=lif, fc_weight=fc_weight, fc_bias=fc_bias, out_sum=out_sum, v=v)
@@ -339,7 +375,15 @@ class _FusedNetwork(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         with torch.no_grad():
-            return self.run(self._prepare(x))
+            x = self._prepare(x)
+            if self.internal_layouts:
+                if not x.is_cuda or x.dtype not in (torch.bfloat16, torch.float16):
+                    raise RuntimeError("unsupported_dtype: the internal layouts need bfloat16 / float16 tensors on the GPU")
+                return self.run_blocked(x)
+            return self.run(x)
+
+    def run_blocked(self, x: torch.Tensor) -> torch.Tensor:     # pragma: no cover - implemented by the subclasses
+        raise NotImplementedError
 
     def run(self, x: torch.Tensor) -> torch.Tensor:     # pragma: no cover - implemented by the subclasses
         raise NotImplementedError
@@ -366,8 +410,8 @@ class _FusedNetwork(nn.Module):
 
 
 class FusedSpikingVGG11(_FusedNetwork):
-    def __init__(self, model: SpikingVGG11, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0"):
-        super().__init__(T, dtype, device)
+    def __init__(self, model: SpikingVGG11, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0", internal_layouts: bool = False):
+        super().__init__(T, dtype, device, internal_layouts=internal_layouts)
         self.steps: List[Tuple[str, object]] = []
         for i, m in enumerate(model.features):
             if isinstance(m, ConvBNNeuron):
@@ -390,10 +434,25 @@ class FusedSpikingVGG11(_FusedNetwork):
                 seq = self.plain_conv(f"features.{i}", seq, item)
         return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
 
+    def run_blocked(self, x):
+        """The same layer sequence with the frame channel-blocked, every spike tensor bit-packed (2x2 average pools turn
+        bits into blocked quarters) and only the last, neuron-free convolution writing the dense tensor the tail reads."""
+        from .runtime import hip_blocked_backend as B
+        seq = B.from_dense(x, B.C8, shared=True)
+        seq.T = self.T
+        for i, (kind, item) in enumerate(self.steps):
+            if kind == "conv":
+                seq = self.conv_lif_b(f"features.{i}", seq, item)
+            elif kind == "pool":
+                seq = self.pooled_b(f"features.{i}", seq, item)
+            else:
+                seq = self.conv_lif_b(f"features.{i}", seq, item, out_layout=B.NCHW)
+        return self.tail(B.to_dense(seq), self.tail_lif, self.fc_weight, self.fc_bias)
+
 
 class FusedSpikingResNet18(_FusedNetwork):
-    def __init__(self, model: SpikingResNet18, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0"):
-        super().__init__(T, dtype, device)
+    def __init__(self, model: SpikingResNet18, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0", internal_layouts: bool = False):
+        super().__init__(T, dtype, device, internal_layouts=internal_layouts)
         self.stem = _FusedLayer(model.stem, dtype, self.device_)
         self.maxpool = copy.deepcopy(model.maxpool)
         self.block_layers = []
@@ -418,6 +477,23 @@ class FusedSpikingResNet18(_FusedNetwork):
                 seq = self.plain_conv(f"blocks.{i}.conv2", hidden, conv2, residual=identity)
         return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
 
+    def run_blocked(self, x):
+        """Stem on the channel-blocked frame, everything after it on bit-packed spikes; the LIF-free shortcuts produce
+        blocked analog residuals; the last block's sum is written dense for the tail."""
+        from .runtime import hip_blocked_backend as B
+        frame = B.from_dense(x, B.C8, shared=True)
+        frame.T = self.T
+        seq = self.conv_lif_b("stem", frame, self.stem)
+        seq = self.pooled_b("maxpool", seq, self.maxpool)
+        for i, (conv1, conv2, down) in enumerate(self.block_layers):
+            identity = seq if down is None else self.conv_lif_b(f"blocks.{i}.downsample", seq, down)
+            hidden = self.conv_lif_b(f"blocks.{i}.conv1", seq, conv1)
+            if conv2.lif is not None:
+                seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity)
+            else:   # last block: its neuron is the tail's
+                seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity, out_layout=B.NCHW)
+        return self.tail(B.to_dense(seq), self.tail_lif, self.fc_weight, self.fc_bias)
+
 
 def build_network(name: str, width: int = 64, num_classes: Optional[int] = None, seed: int = 0, gain: float = 1.0) -> nn.Module:
     """`vgg11` (10 classes) or `resnet18` (1000 classes) with the synthetic initialisation."""
@@ -430,9 +506,12 @@ def build_network(name: str, width: int = 64, num_classes: Optional[int] = None,
     return init_synthetic_(model, seed=seed, gain=gain)
 
 
-def fuse_network(model: nn.Module, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0") -> _FusedNetwork:
+def fuse_network(model: nn.Module, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0",
+                 internal_layouts: bool = False) -> _FusedNetwork:
+    """`internal_layouts`: run the network's own operator-to-operator tensors bit-packed / channel-blocked instead of
+    through the dense `snn_custom` operators (same operators, same arithmetic; GPU and 16-bit activations only)."""
     if isinstance(model, SpikingVGG11):
-        return FusedSpikingVGG11(model, T, dtype, device)
+        return FusedSpikingVGG11(model, T, dtype, device, internal_layouts)
     if isinstance(model, SpikingResNet18):
-        return FusedSpikingResNet18(model, T, dtype, device)
+        return FusedSpikingResNet18(model, T, dtype, device, internal_layouts)
     raise TypeError(f"no fused executor for {type(model).__name__}")

@@ -1,0 +1,161 @@
+"""Internal activation layouts between consecutive fused operators of one network, on libsnnf.
+
+The reference hands dense [T, N, C, H, W] tensors of 0/1 elements from one fused operator to the next
+(kernels/benchmark_conv_lif_temporal_general.py:707-708), stacks a layer's T inputs into one tensor
+(runtime/triton_convlif_backend.py:579) and, in its executor's fast path, writes into pooled caller-owned buffers
+(runtime/fx_standalone_executor.py:900-952). This module is the counterpart of that producer-consumer plumbing for a
+network executor that owns both ends of a tensor: spikes travel at one bit each (`BITS`: [T, N, ceil(C/8), H, W] bytes,
+bit j = channel 8*c8 + j), analog activations channel-blocked (`C8`: [T, N, ceil(C/8), H, W, 8] elements), which is the
+operand order of the matrix instruction. Tensors at the operator boundary (`torch.ops.snn_custom.*`) stay dense NCHW.
+
+Everything here raises when libsnnf.so is missing or a call is outside what the kernels take (RuntimeError with an
+`unsupported_*:` reason): there is no eager substitute.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from .. import _lib
+from .hip_convlif_backend import _as_pair, _packed_weight, last_conv_plan  # noqa: F401  (last_conv_plan re-exported)
+
+NCHW, C8, BITS = _lib.SNNF_LAYOUT_NCHW, _lib.SNNF_LAYOUT_C8, _lib.SNNF_LAYOUT_BITS
+LAYOUT_NAMES = {NCHW: "nchw", C8: "c8", BITS: "bits"}
+
+
+@dataclass
+class Blocked:
+    """T x N frames of [C, H, W] in one of the layouts. `data` is [T, N, C, H, W] (NCHW), [T, N, C8, H, W, 8] (C8) in the
+    activation dtype, or [T, N, C8, H, W] uint8 (BITS). `shared`: every timestep is the same frame (data holds one)."""
+
+    data: torch.Tensor
+    layout: int
+    T: int
+    N: int
+    C: int
+    H: int
+    W: int
+    dtype: torch.dtype
+    shared: bool = False
+
+    @property
+    def shape(self) -> Tuple[int, int, int, int, int]:
+        return (self.T, self.N, self.C, self.H, self.W)
+
+    def step_pointers(self):
+        if self.shared:
+            return _lib.step_pointers([self.data[0]] * self.T)
+        return _lib.packed_step_pointers(self.data)
+
+    def step_stride_bytes(self) -> int:
+        return int(self.data.stride(0)) * self.data.element_size()
+
+
+def _check_dtype(dtype: torch.dtype) -> None:
+    if dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError(f"unsupported_dtype: the internal layouts hold bfloat16 or float16 activations, got {dtype}")
+
+
+def empty_blocked(layout: int, T: int, N: int, C: int, H: int, W: int, dtype: torch.dtype, device) -> Blocked:
+    _check_dtype(dtype)
+    c8 = (C + 7) // 8
+    if layout == NCHW:
+        data = torch.empty((T, N, C, H, W), dtype=dtype, device=device)
+    elif layout == C8:
+        data = torch.empty((T, N, c8, H, W, 8), dtype=dtype, device=device)
+    elif layout == BITS:
+        data = torch.empty((T, N, c8, H, W), dtype=torch.uint8, device=device)
+    else:
+        raise RuntimeError(f"unknown layout code {layout}")
+    return Blocked(data, layout, T, N, C, H, W, dtype)
+
+
+def from_dense(x_seq: torch.Tensor, layout: int = BITS, shared: bool = False) -> Blocked:
+    """Dense [T, N, C, H, W] (or one [N, C, H, W] frame with `shared`) -> the layout (BITS: element != 0)."""
+    if shared and x_seq.dim() == 4:
+        x_seq = x_seq.unsqueeze(0)
+    if x_seq.dim() != 5 or not x_seq.is_cuda:
+        raise RuntimeError("unsupported_rank: from_dense takes a [T, N, C, H, W] tensor on the GPU")
+    _check_dtype(x_seq.dtype)
+    x = x_seq if x_seq.is_contiguous() else x_seq.contiguous()
+    T, N, C, H, W = (int(d) for d in x.shape)
+    src = Blocked(x, NCHW, T, N, C, H, W, x.dtype, shared)
+    return src if layout == NCHW else convert(src, layout)
+
+
+def convert(x: Blocked, layout: int) -> Blocked:
+    if x.layout == layout:
+        return x
+    frames = int(x.data.shape[0]) * x.N
+    out = empty_blocked(layout, int(x.data.shape[0]), x.N, x.C, x.H, x.W, x.dtype, x.data.device)
+    out.T, out.shared = x.T, x.shared
+    _lib.check("snnf_layout_convert", _lib.lib().snnf_layout_convert(
+        x.data.data_ptr(), x.layout, out.data.data_ptr(), layout, frames, x.C, x.H, x.W, _lib.dtype_code(x.dtype),
+        _lib.current_stream(x.data.device)))
+    return out
+
+
+def to_dense(x: Blocked) -> torch.Tensor:
+    """The dense [T, N, C, H, W] tensor (spikes as 0 / 1 in the activation dtype)."""
+    d = convert(x, NCHW).data
+    return d.expand(x.T, -1, -1, -1, -1) if x.shared and d.shape[0] == 1 else d
+
+
+def pool_blocked(x: Blocked, is_max: bool, kernel: int, stride: int, padding: int, out_layout: Optional[int] = None) -> Blocked:
+    """Max (2x2 or 3x3, stride 2) or average (2x2 / 2) pooling of every frame. Max pooling keeps the layout (BITS: a bitwise
+    OR); average pooling of BITS yields C8 (quarters)."""
+    if x.layout == NCHW:
+        raise RuntimeError("unsupported_layout: pool_blocked takes C8 or BITS tensors (dense ones go to snnf_pool2d)")
+    if out_layout is None:
+        out_layout = x.layout if is_max else C8
+    ho = (x.H + 2 * padding - kernel) // stride + 1
+    wo = (x.W + 2 * padding - kernel) // stride + 1
+    frames_t = int(x.data.shape[0])
+    out = empty_blocked(out_layout, frames_t, x.N, x.C, ho, wo, x.dtype, x.data.device)
+    out.T, out.shared = x.T, x.shared
+    _lib.check("snnf_pool2d_blocked", _lib.lib().snnf_pool2d_blocked(
+        x.data.data_ptr(), x.layout, out.data.data_ptr(), out_layout, frames_t * x.N, x.C, x.H, x.W, int(kernel), int(stride),
+        int(padding), 1 if is_max else 0, _lib.dtype_code(x.dtype), _lib.current_stream(x.data.device)))
+    return out
+
+
+def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding,
+                     lif: Optional[Sequence[float]], residual: Optional[Blocked] = None, out_layout: int = BITS,
+                     v_init: Optional[torch.Tensor] = None, want_v: bool = False):
+    """Dense convolution + bias (+ residual) + LIF over the T steps of `x` (C8 or BITS), or without a neuron when `lif` is
+    None (output C8 or NCHW). Returns (Blocked output, final membrane [N, Cout, Ho, Wo] fp32 or None). The membrane is
+    only written when asked for (`want_v`) or when the timesteps take more than one window of the kernel."""
+    if x.layout not in (C8, BITS):
+        raise RuntimeError("unsupported_layout: conv_lif_blocked takes inputs in C8 or BITS layout")
+    if weight.dim() != 4 or int(weight.shape[1]) != x.C:
+        raise RuntimeError(f"unsupported_groups: weight {tuple(weight.shape)} does not match {x.C} input channels (dense convolutions only)")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise RuntimeError("unsupported_dtype: weight / bias dtype must be the activation dtype")
+    cout, _, kh, kw = (int(d) for d in weight.shape)
+    sh, sw = _as_pair(stride)
+    ph, pw = _as_pair(padding)
+    ho, wo = (x.H + 2 * ph - kh) // sh + 1, (x.W + 2 * pw - kw) // sw + 1
+    dev = x.data.device
+    if bias is None:
+        bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    packed = _packed_weight(weight, bias, x.dtype)
+    out = empty_blocked(out_layout, x.T, x.N, cout, ho, wo, x.dtype, dev)
+    neuron = lif is not None
+    windows = 1 if (x.shared or x.T <= 4) else (x.T + 3) // 4
+    v_out = torch.empty((x.N, cout, ho, wo), dtype=torch.float32, device=dev) if neuron and (want_v or windows > 1) else None
+    if residual is not None and (residual.shape != (x.T, x.N, cout, ho, wo) or residual.dtype != x.dtype or residual.shared):
+        raise RuntimeError(f"unsupported_residual_shape: residual {residual.shape} does not match the output {(x.T, x.N, cout, ho, wo)}")
+    vi = None
+    if v_init is not None and isinstance(v_init, torch.Tensor) and v_init.dim() != 0:
+        if tuple(v_init.shape) != (x.N, cout, ho, wo) or v_init.dtype != torch.float32 or v_init.device != dev:
+            raise RuntimeError("unsupported_membrane_state: v_init must be a float32 [N, Cout, Ho, Wo] tensor on the activations' device")
+        vi = v_init if v_init.is_contiguous() else v_init.contiguous()
+    v_th, v_reset, tau = (float(lif[0]), float(lif[1]), float(lif[2])) if neuron else (1.0, 0.0, 2.0)
+    _lib.check("snnf_conv_lif_blocked", _lib.lib().snnf_conv_lif_blocked(
+        x.step_pointers(), x.layout, residual.step_pointers() if residual is not None else None,
+        residual.layout if residual is not None else 0, x.T, x.N, x.C, x.H, x.W, _lib.dtype_code(x.dtype),
+        packed.data_ptr(), cout, kh, kw, sh, sw, ph, pw, _lib.ptr(vi), out.data.data_ptr(), out_layout, out.step_stride_bytes(),
+        _lib.ptr(v_out), 1 if neuron else 0, v_th, v_reset, tau, _lib.current_stream(dev)))
+    return out, v_out
