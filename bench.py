@@ -39,6 +39,8 @@ def _parse():
     ap.add_argument("--layers", default=None, choices=["resnet18", "vgg11"],
                     help="instead of a workload: time every fused conv layer shape of the spiking ResNet-18 (T=4, B=16, "
                          "224x224) or VGG-11 (T=4, B=64, 32x32) configuration on its own, synthetic spike inputs")
+    ap.add_argument("--internal", action="store_true",
+                    help="with --layers: time the layers as the network executor runs them, on the bit-packed / channel-blocked internal layouts")
     ap.add_argument("--model", default=None, choices=["resnet18", "vgg11"],
                     help="end-to-end forward of the spiking ResNet-18 (T=4, B=16, 224x224) or VGG-11 (T=4, B=64, 32x32) "
                          "network through the fused operators, replayed as one HIP graph")
@@ -130,13 +132,10 @@ def _time_kernel(fn, steps: int, warmup: int, reps: int = 10):
         return _time_gpu(fn, steps, warmup)[0], "eager"
 
 
-# HBM bytes per launch of the default workload's kernels, from rocprofv3 FETCH_SIZE / WRITE_SIZE (KiB per dispatch),
-# each scaled by what the same counter reads for a plain 256 MiB device copy (FETCH_SIZE reads half the bytes copied,
-# factor 2.0; WRITE_SIZE reads them exactly, factor 1.0). Valid for mobilenet_block in bf16 only.
-MEASURED_TRAFFIC_BYTES = {
-    ("mobilenet_block", "bf16", "layer0_depthwise3x3"): (50262.5 * 2.0 + 150532.5) * 1024,
-    ("mobilenet_block", "bf16", "layer1_pointwise1x1"): (50522.2 * 2.0 + 301076.0) * 1024,
-}
+# `roofline.traffic` (HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE) is not measured inside this script: a
+# counter run needs the profiler around the process. The line therefore carries null and names the committed summary of
+# the counter run of this same command.
+TRAFFIC_PROFILE = "profiles/mobilenet_block_hbm_traffic.md"
 
 
 class Prepared:
@@ -237,10 +236,13 @@ VGG11_LAYERS = [
 ]
 
 
-def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
-    """Times every fused conv(+residual)+LIF layer shape of a network configuration on its own (graph replay, HIP events)."""
+def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, internal: bool = False):
+    """Times every fused conv(+residual)+LIF layer shape of a network configuration on its own (graph replay, HIP events).
+    `internal`: the layer as it runs inside the network executor, spikes bit-packed on both sides (an analog frame
+    channel-blocked), final membrane not written; otherwise through the dense operator (NCHW in and out, fp32 membrane)."""
     import torch
     from triton_snn_fusion_amd import workloads as W
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
     ops = torch.ops.snn_custom
     layers, batch = (RESNET18_LAYERS, 16) if which == "resnet18" else (VGG11_LAYERS, 64)
     T, dev = 4, torch.device("cuda:0")
@@ -259,23 +261,44 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int):
         b = (torch.randn(cout, generator=g) * 0.1).to(dev, dtype)
         out = (size + 2 * pad - k) // stride + 1
         rs = [(torch.rand(batch, cout, out, out, generator=g) < 0.15).to(dev, dtype) for _ in range(T)] if residual else None
-        if residual:
+        if internal:
+            if analog:
+                bx = B.from_dense(xs[0], B.C8, shared=True)
+                bx.T = T
+            else:
+                bx = B.from_dense(torch.stack(xs), B.BITS)
+            br = B.from_dense(torch.stack(rs), B.BITS) if residual else None
+            fn = lambda: B.conv_lif_blocked(bx, w, b, [stride, stride], [pad, pad], (1.0, 0.0, 2.0), residual=br, out_layout=B.BITS)
+        elif residual:
             fn = lambda: ops.fused_temporal_conv_add_lif_state(xs, rs, w, b, v0, [stride, stride], [pad, pad], [1, 1], 1, 1.0, 0.0, 2.0, False)
         else:
             fn = lambda: ops.fused_temporal_conv_lif_state(xs, w, b, v0, [stride, stride], [pad, pad], [1, 1], 1, 1.0, 0.0, 2.0, False)
         ms, how = _time_kernel(fn, steps, warmup)
         flops = W.conv_flops(T, batch, cin, cout, out, out, k, k, 1)
+        # Algorithmic bytes are those of the dense operator in both modes (x once, spikes once in the activation dtype, fp32
+        # membrane once), so that the two modes' figures compare; `internal_bytes` is what the bit-packed form moves.
         nbytes = W.algorithmic_conv_bytes(T, batch, cin, size, size, cout, out, out, k, k, 1, esize, 4, shared_input=analog)
         if residual:
             nbytes += T * batch * cout * out * out * esize
-        rows.append({"layer": name, "count": count, "ms": round(ms, 4), "timed": how,
+        c8i, c8o = (cin + 7) // 8, (cout + 7) // 8
+        internal_bytes = ((batch * c8i * size * size * 16) if analog else (T * batch * c8i * size * size)) + T * batch * c8o * out * out * (2 if residual else 1) \
+            + cout * cin * k * k * esize
+        rows.append({"layer": name, "count": count, "ms": round(ms, 4), "timed": how, "plan": _plan_summary(),
+                     **({"internal_bytes": internal_bytes} if internal else {}),
                      "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
         total_ms += ms * count
         total_flops += flops * count
-    return {"metric": METRIC, "workload": f"{which}_layers", "dtype": dtype_name, "T": T, "batch": batch,
+    return {"metric": METRIC, "workload": f"{which}_layers" + ("_internal_layouts" if internal else ""), "dtype": dtype_name, "T": T, "batch": batch,
             "conv_ms_per_forward": round(total_ms, 4), "images_T_per_s_conv_only": round(batch * T / (total_ms * 1e-3), 1),
             "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
+
+
+def _plan_summary() -> str:
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    plan = last_conv_plan()
+    keys = ("kernel", "variant", "window", "tile", "waves", "stage_chunks", "grid")
+    return " ".join(f"{k}={plan[k]}" for k in keys if k in plan)
 
 
 def _streaming_operators(dtype, steps: int, warmup: int):
@@ -372,7 +395,30 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
             out["fx_rewrite"]["graph_ms_per_forward"] = round(_time_graph(lambda: gm(x), steps, warmup), 4)
     except Exception as exc:  # pragma: no cover - reported, the executor numbers stand
         out.setdefault("fx_rewrite", {})["error"] = str(exc)[:200]
+    # The same network with bit-packed spikes / channel-blocked activations between its own operators.
     best = ms_graph if ms_graph is not None else ms_eager
+    try:
+        net_i = M.fuse_network(M.build_network(name, seed=0), cfg["T"], dtype, "cuda:0", internal_layouts=True)
+        net_i(frame)
+        torch.cuda.synchronize()
+        ms_i, wall_i = _time_gpu(lambda: net_i(x), max(5, steps // 2), max(2, warmup // 2))
+        entry = {"eager_launch_ms_per_forward": round(ms_i, 4), "host_ms_per_forward": round(wall_i, 4)}
+        replay_i, _, _ = net_i.capture(frame)
+        ms_ig, _ = _time_gpu(replay_i, steps, warmup)
+        entry["graph_ms_per_forward"] = round(ms_ig, 4)
+        entry["images_T_per_s"] = round(cfg["batch"] * cfg["T"] / (ms_ig * 1e-3), 1)
+        out["internal_layouts"] = entry
+        best = min(best, ms_ig)
+    except Exception as exc:  # pragma: no cover - reported, the dense executor's numbers stand
+        out.setdefault("internal_layouts", {})["error"] = str(exc)[:300]
+    layers = RESNET18_LAYERS if name == "resnet18" else VGG11_LAYERS
+    from triton_snn_fusion_amd import workloads as W
+    conv_flops = 0
+    for _n, cin, cout, size, k, stride, pad, _res, _analog, count in layers:
+        o = (size + 2 * pad - k) // stride + 1
+        conv_flops += count * W.conv_flops(cfg["T"], cfg["batch"], cin, cout, o, o, k, k, 1)
+    out["conv_flops_per_forward"] = conv_flops
+    out["roofline"] = _roofline("mfma", conv_flops, best)
     out["ms_per_forward"] = round(best, 4)
     out["images_T_per_s"] = round(cfg["batch"] * cfg["T"] / (best * 1e-3), 1)
     out["images_per_s"] = round(cfg["batch"] / (best * 1e-3), 1)
@@ -406,16 +452,27 @@ def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
             xs = [out[0][t] for t in range(wl.T)]
         return out
 
-    run()  # warm-up
-    times = []
-    t_begin = time.perf_counter()
-    while len(times) < 3 or (len(times) < 20 and time.perf_counter() - t_begin < seconds_budget):
-        t0 = time.perf_counter()
-        run()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    median = times[len(times) // 2]
+    def median_ms(budget):
+        run()  # warm-up
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 3 or (len(times) < 20 and time.perf_counter() - t_begin < budget):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    median, count = median_ms(seconds_budget * 0.6)
+    threads = int(torch.get_num_threads())
+    torch.set_num_threads(1)
+    try:
+        median_1, count_1 = median_ms(seconds_budget * 0.4)
+    finally:
+        torch.set_num_threads(threads)
+    times = [0.0] * count
     return {
+        "single_thread": {"value": round(sample_batch * wl.T / median_1, 2), "cores": 1, "ms_per_step": round(median_1 * 1e3, 3), "runs": count_1},
         "value": round(sample_batch * wl.T / median, 2),
         "unit": "images*T/s",
         "cores": int(torch.get_num_threads()),
@@ -455,7 +512,7 @@ def main() -> int:
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
 
     if args.layers is not None:
-        sweep = _layer_sweep(args.layers, dtype, args.dtype, args.steps, args.warmup)
+        sweep = _layer_sweep(args.layers, dtype, args.dtype, args.steps, args.warmup, internal=args.internal)
         stats = ops.get_fused_op_call_stats()
         sweep["native_calls"], sweep["fallback_calls"] = stats["triton"], stats["fallback"]
         print(json.dumps(sweep))
@@ -515,8 +572,7 @@ def main() -> int:
             nbytes, flops = prep.layer_work(i, xs)
             groups = prep.layers[i][5]
             kind = "depthwise3x3" if groups > 1 else ("pointwise1x1" if tuple(prep.layers[i][1].shape[2:]) == (1, 1) else "conv")
-            traffic = MEASURED_TRAFFIC_BYTES.get((args.workload, args.dtype, f"layer{i}_{kind}"))
-            traffic = None if traffic is None else int(traffic)
+            traffic = None
             kernels[f"layer{i}_{kind}"] = {
                 "ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "flops": flops,
                 "hbm": _roofline("hbm", nbytes, ms, traffic),
@@ -525,7 +581,7 @@ def main() -> int:
         dominant = max(kernels.items(), key=lambda kv: kv[1]["ms"])
         ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
         bound = "mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS and dominant[1]["mfma"] is not None else "hbm"
-        result["roofline"] = dict(dominant[1][bound], kernel=dominant[0])
+        result["roofline"] = dict(dominant[1][bound], kernel=dominant[0], traffic_measured_in=TRAFFIC_PROFILE)
     else:
         T, M, fin, fout = wl.T, wl.batch, int(wl.linear_weight.shape[1]), int(wl.linear_weight.shape[0])
         nbytes = (T * M * fin + fout * fin + fout) * prep.esize + T * M * fout * prep.esize + M * fout * 4
@@ -562,6 +618,17 @@ def main() -> int:
             try:
                 kms, how = _time_kernel(other.step, args.steps, max(3, args.warmup // 2))
                 entry["kernel_ms"], entry["timed"] = round(kms, 4), how
+                if other.layers:
+                    nbytes, flops = other.layer_work(0, other.xs)
+                else:
+                    T_, M_, fin_, fout_ = other.wl.T, other.wl.batch, int(other.wl.linear_weight.shape[1]), int(other.wl.linear_weight.shape[0])
+                    nbytes = (T_ * M_ * fin_ + fout_ * fin_ + fout_) * other.esize + T_ * M_ * fout_ * other.esize + M_ * fout_ * 4
+                    flops = 2 * T_ * M_ * fin_ * fout_
+                ai = flops / nbytes
+                entry["algorithmic_bytes"], entry["flops"] = nbytes, flops
+                entry["matrix_operand_dtype"] = "f16" if args.dtype == "f16" and name != "conv3x3_block" else "bf16"
+                entry["roofline"] = _roofline("mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm", flops if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else nbytes, kms)
+                entry["hbm"], entry["mfma"] = _roofline("hbm", nbytes, kms), _roofline("mfma", flops, kms)
             except Exception as exc:
                 entry["kernel_error"] = str(exc)[:200]
             try:
@@ -589,7 +656,10 @@ def main() -> int:
         return 1
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = _cpu_baseline(args.workload)
+        result["cpu_baseline"] = _cpu_baseline(args.workload, 14.0)
+        if args.workload != "conv3x3_block" and not args.no_extra:
+            # BASELINE's config 0 (the reference's own CPU-runnable case) at its full size, next to its GPU figure above.
+            result["extra"]["conv3x3_block"]["cpu_baseline"] = _cpu_baseline("conv3x3_block", 8.0)
     print(json.dumps(result))
     return 0
 

@@ -8,7 +8,7 @@
 namespace snnf {
 namespace {
 
-constexpr int kWaveLds = static_cast<int>(kMaxLds) / kSpkWaves;   // private staging bytes of a wave
+constexpr int kWaveLds = (static_cast<int>(kMaxLds) - static_cast<int>(kSpkTableBytes)) / kSpkWaves / 16 * 16;   // private staging bytes of a wave
 
 struct SpkPlan {
     int PR, PC, PI, RR, RC, region, G, patches_x, patches_y, img_groups;
@@ -178,6 +178,17 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     g.d_gpc = make_fast_div(g.gpc);
     const int hg = g.tap_pairs ? 1 : g.G / 2;
     const int nst = g.tap_pairs ? g.npairs : g.taps * hg;
+    g.kw_mul = (KW & (KW - 1)) == 0 ? 65536 / KW : 65536 / KW + 1;
+    for (int tap = 0; tap < KH * KW; ++tap)
+        if (((tap * g.kw_mul) >> 16) != tap / KW)
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_kernel: kernel %dx%d too large", who, KH, KW);
+    g.gpc_log2 = 0;
+    while ((1 << g.gpc_log2) < g.gpc) ++g.gpc_log2;
+    g.hg_log2 = 0;
+    while ((1 << g.hg_log2) < hg) ++g.hg_log2;
+    g.pair_tap_stride = g.tap_pairs ? 1 : g.gpc / 2;
+    if (nst > kSpkMaxSteps)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_kernel: %d matrix steps per stage exceed %d (kernel %dx%d)", who, nst, kSpkMaxSteps, KH, KW);
     g.d_hg = make_fast_div(hg);
     g.d_nst = make_fast_div(nst);
     g.d_KW = make_fast_div(KW);
@@ -195,13 +206,17 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     L.v_out = neuron ? static_cast<float*>(v_out) : nullptr;
     L.lif = make_lif_params(v_threshold, v_reset, tau);
     L.grid = grid;
-    L.lds_bytes = static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes;
-    if (wk_log2 > 0 && L.lds_bytes < kSpkPartialBytes) L.lds_bytes = kSpkPartialBytes;
+    L.lds_bytes = kSpkTableBytes + static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes;
+    if (wk_log2 > 0 && L.lds_bytes < kSpkTableBytes + kSpkPartialBytes) L.lds_bytes = kSpkTableBytes + kSpkPartialBytes;
     L.stream = as_stream(stream);
+    const bool fast_epi = neuron && out_layout == SNNF_LAYOUT_BITS && (residuals == nullptr || res_layout == SNNF_LAYOUT_BITS) &&
+                          L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset && v_init == nullptr && windows == 1 && Cout % 8 == 0;
     snprintf(snnf::conv_plan_buffer(), 256,
              "kernel=blocked variant=%d window=%d launches=1 tile=%dx%dx%d halo=%dx%d waves=8x1x%d oc_tiles=%d px_tiles=%d "
              "stage_chunks=%d run=0 lds=%zu grid=%d",
-             (wk_log2 > 0 ? 50 : 40) + tt, shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
+             (wk_log2 > 0 ? 50 : 40) + tt + (fast_epi ? 20 : 0), shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
              L.lds_bytes, grid);
-    return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16(L, tt) : launch_conv_spk_f16(L, tt);
+    L.fast_epilogue = fast_epi;
+    if (x_layout == SNNF_LAYOUT_BITS) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_bits(L, tt) : launch_conv_spk_f16_bits(L, tt);
+    return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_c8(L, tt) : launch_conv_spk_f16_c8(L, tt);
 }

@@ -34,6 +34,8 @@ constexpr int kSpkWaves = 8;                      // waves per workgroup, one wo
 #endif
 constexpr int kSpkSlots = SPK_SLOTS;                      // staging items per lane and timestep, at most
 constexpr size_t kSpkPartialBytes = kSpkWaves * 8 * 64 * 16;   // split-K: one timestep's partial sums of all waves
+constexpr int kSpkMaxSteps = 60;                  // matrix steps per stage, at most (the step table holds 4 more)
+constexpr size_t kSpkTableBytes = (kSpkMaxSteps + 4) * 16;      // the workgroup's step table at the start of LDS
 
 struct SpkGeom {
     int N, Cin, H, W, Cout, KH, KW, sh, sw, ph, pw, Ho, Wo;
@@ -53,6 +55,10 @@ struct SpkGeom {
     int taps;
     int T;                       // timesteps
     int shared_x;                // one input frame for all T timesteps (TT == 1): convolved once
+    int kw_mul;                  // tap / KW == (tap * kw_mul) >> 16 for every tap of the kernel (branch-free on the scalar unit)
+    int gpc_log2;                // log2(gpc)
+    int hg_log2;                 // log2 of the k-slot pairs per tap and stage (G / 2; 0 with tap pairs)
+    int pair_tap_stride;         // packed pairs between consecutive taps of one group pair (gpc / 2; 1 with tap pairs)
     int wk_log2;                 // split-K: waves per tile
     int n_items, iters;          // (patch, 64-channel tile) pairs; loop trips per wave
     int in_layout, res_layout, out_layout;   // snnf_layout codes; res_layout < 0: no residual
@@ -76,6 +82,8 @@ struct SpkLaunch {
     int grid;
     size_t lds_bytes;
     hipStream_t stream;
+    bool fast_epilogue;   // the straight-line epilogue applies: bit-packed output, no or a bit-packed residual, the common neuron,
+                          // zero initial membrane, one window, whole channel groups
 };
 
 template <bool F16>
@@ -110,7 +118,7 @@ __device__ __forceinline__ sk_u32x4 sk_expand_bits(uint32_t byte) {
     return d;
 }
 
-template <typename XT, int TT, int IN, bool SK>
+template <typename XT, int TT, int IN, bool SK, bool FAST>
 __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_spk_kernel(
     const StepPtrs xs, const StepPtrs residuals, const SpkGeom g, const uint16_t* __restrict__ wpacked,
     const float* __restrict__ bias, const float* __restrict__ v_init, unsigned char* __restrict__ out,
@@ -124,7 +132,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const int lane = tid & 63;
     const int half = lane >> 5;
     const int l32 = lane & 31;
-    unsigned char* const wlds = lds + wave * g.lds_wave_bytes;
+    unsigned char* const wlds = lds + kSpkTableBytes + wave * g.lds_wave_bytes;
     const int region16 = g.region * 16;        // bytes of one channel group of the halo
     const int tile_t = g.G * region16;         // bytes of one timestep's stage
 
@@ -146,6 +154,37 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const uint16_t* __restrict__ wlane = wpacked + lane * 8;
     const int hg = g.tap_pairs ? 1 : (g.G >> 1);        // k-slot pairs per tap and stage
     const int nst = g.tap_pairs ? g.npairs : g.taps * hg;   // matrix steps per stage
+    const bool common_lif = lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+
+    // ---- step table of the workgroup: for step i of a stage, the byte offset of its weight fragments from the stage's
+    // first pair and the LDS offset of its activations for the lower / upper half of a wave (tap and channel group of
+    // the half's k-slot). The matrix loop then needs no index arithmetic. Steps beyond the last repeat it (prefetch only).
+    {
+        sk_u32x4* __restrict__ table = reinterpret_cast<sk_u32x4*>(lds);
+        if (tid < nst + 4) {
+            const int i = min(tid, nst - 1);
+            sk_u32x4 e;
+            if (g.tap_pairs) {
+                const int tap0 = 2 * i, tap1 = min(2 * i + 1, g.taps - 1);   // an odd tap count leaves the last k-slot empty (zero weights)
+                const int kh0 = tap0 / g.KW, kh1 = tap1 / g.KW;
+                e[0] = static_cast<uint32_t>(i * kFragBytes);
+                e[1] = static_cast<uint32_t>((kh0 * g.RC + (tap0 - kh0 * g.KW)) * 16);
+                e[2] = static_cast<uint32_t>((kh1 * g.RC + (tap1 - kh1 * g.KW)) * 16);
+            } else {
+                const int tap = i >> g.hg_log2;
+                const int gp = i & (hg - 1);
+                const int kh = tap / g.KW;
+                const int tapoff = (kh * g.RC + (tap - kh * g.KW)) * 16;
+                e[0] = static_cast<uint32_t>((tap * g.pair_tap_stride + gp) * kFragBytes);
+                e[1] = static_cast<uint32_t>(tapoff + (2 * gp) * region16);
+                e[2] = static_cast<uint32_t>(tapoff + (2 * gp + 1) * region16);
+            }
+            e[3] = 0u;
+            table[tid] = e;
+        }
+        __syncthreads();
+    }
+    const sk_u32x4* __restrict__ table = reinterpret_cast<const sk_u32x4*>(lds);
 
     for (int it = 0; it < g.iters; ++it) {
         // Consecutive items go to consecutive workgroups, so that a layer with fewer items than wave slots still uses every compute unit.
@@ -176,13 +215,24 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         const int n_c = px_ok ? n : 0;
 
         for (int t0 = 0; t0 < nsteps_t; t0 += TT) {
+            // The accumulators start from the bias (requested now, needed at the first matrix instruction): register 4 q + k of
+            // fragment f is channel 64 oc_tile + 32 f + 8 q + 4 half + k. With K split over waves only the first one adds it.
             sk_f32x16 acc[TT][2];
-#pragma unroll
-            for (int t = 0; t < TT; ++t)
+            {
+                const int nbias = g.nocf * 32;               // bias values behind the packed weight (zero beyond Cout)
 #pragma unroll
                 for (int f = 0; f < 2; ++f)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[t][f][r] = 0.0f;
+                    for (int q = 0; q < 4; ++q) {
+                        const int ch0 = oc_tile * 64 + f * 32 + q * 8 + 4 * half;
+                        sk_f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                        if (ch0 < nbias && (!SK || wk == 0)) b4 = *reinterpret_cast<const sk_f32x4*>(bias + ch0);
+#pragma unroll
+                        for (int t = 0; t < TT; ++t)
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) acc[t][f][4 * q + k] = b4[k];
+                    }
+            }
 
             // One LDS stage: G channel groups of the patch's halo for TT timesteps, from global memory into this wave's region.
             // Item e = slot * 64 + lane of a timestep = (group, image, row, column) of the halo; its LDS address is 16 e. Items
@@ -192,6 +242,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const int gg0 = s * g.G;
                 const int base_u = ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
                 __builtin_amdgcn_wave_barrier();   // the matrix steps of the previous stage have read their operands
+                int lane_s = lane;                 // opaque: the decode below stays here instead of being hoisted out of every loop
+                asm volatile("" : "+v"(lane_s));   // (its results would sit in registers, or in scratch memory, across the matrix loop)
 #pragma unroll
                 for (int jb = 0; jb < kSpkSlots; jb += 4) {
                     if (jb < g.JT) {
@@ -199,7 +251,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         uint32_t ok_bits = 0;       // bit j: the item is real data; bit 4 + j: the item exists (is written)
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
-                            const int e = (jb + j) * 64 + lane;
+                            const int e = (jb + j) * 64 + lane_s;
                             const int gq = fast_div(e, g.d_region);
                             const int rem = e - gq * g.region;
                             const int ii = fast_div(rem, g.d_rrrc);
@@ -227,7 +279,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 #pragma unroll
                                 for (int j = 0; j < 4; ++j) {
                                     const sk_u32x4 d = sk_expand_bits<ONE>(((ok_bits >> j) & 1u) ? raw[t][j] : 0u);
-                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane) * 16) = d;
+                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
                                 }
                         } else {
 #pragma unroll
@@ -242,7 +294,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                                     sk_u32x4 d;
 #pragma unroll
                                     for (int k = 0; k < 4; ++k) d[k] = ((ok_bits >> j) & 1u) ? raw[j][k] : 0u;
-                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane) * 16) = d;
+                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
                                 }
                             }
                         }
@@ -252,76 +304,82 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             };
 
             // ---- matrix loop over this wave's stages. Step = one pair of k-slots = one matrix instruction per (timestep,
-            // 32-channel fragment); weight fragments stream from L2 two steps ahead through three register sets, across stages.
+            // 32-channel fragment). Per stage: the first weight fragments are requested from L2, the stage is brought into LDS,
+            // then the steps run four at a time without a branch: weight fragments three steps ahead through four register
+            // sets, activation fragments one step ahead through two.
             if (have) {
                 const int s_first = SK ? wk : 0;
                 const int s_step = SK ? WK : 1;
-                const int my_stages = s_first < g.nstages ? (g.nstages - s_first + s_step - 1) / s_step : 0;
-                const int total = my_stages * nst;
-                // Weight fragment of flat step `fs` of this wave (clamped to its last step).
-                auto load_a = [&](int fs, sk_u32x4& a0, sk_u32x4& a1) __attribute__((always_inline)) {
-                    fs = min(fs, total - 1);
-                    const int si = fast_div(fs, g.d_nst);
-                    const int st = fs - si * nst;
-                    const int gg0 = (s_first + si * s_step) * g.G;
-                    const int chunk = fast_div(gg0, g.d_gpc);
-                    int pair;
-                    if (g.tap_pairs) {
-                        pair = chunk * g.npairs + st;
-                    } else {
-                        const int tap = fast_div(st, g.d_hg);
-                        const int gp = st - tap * hg;
-                        pair = chunk * g.npairs + ((tap * g.gpc + (gg0 - chunk * g.gpc) + 2 * gp) >> 1);
-                    }
-                    const int64_t o = static_cast<int64_t>(pair) * (kFragBytes / 2);
-                    a0 = *reinterpret_cast<const sk_u32x4*>(wlane + w_off0 + o);
-                    a1 = *reinterpret_cast<const sk_u32x4*>(wlane + w_off1 + o);
-                };
-                // Matrix work of step `st` of the stage in LDS.
-                auto mma_step = [&](int st, const sk_u32x4& a0, const sk_u32x4& a1) __attribute__((always_inline)) {
-                    const unsigned char* __restrict__ bq;
-                    if (g.tap_pairs) {
-                        const int tap0 = 2 * st, tap1 = min(2 * st + 1, g.taps - 1);   // an odd tap count leaves the last k-slot empty (zero weights)
-                        const int kh0 = fast_div(tap0, g.d_KW), kh1 = fast_div(tap1, g.d_KW);
-                        const int off0 = (kh0 * g.RC + (tap0 - kh0 * g.KW)) * 16;
-                        const int off1 = (kh1 * g.RC + (tap1 - kh1 * g.KW)) * 16;
-                        bq = wlds + lane_b + (half ? off1 : off0);
-                    } else {
-                        const int tap = fast_div(st, g.d_hg);
-                        const int gp = st - tap * hg;
-                        const int kh = fast_div(tap, g.d_KW);
-                        bq = wlds + lane_b + (kh * g.RC + (tap - kh * g.KW)) * 16 + (2 * gp + half) * region16;
-                    }
+                const uint32_t lane16 = static_cast<uint32_t>(lane) * 16u;
+                const unsigned char* __restrict__ bl = wlds + lane_b;
+                for (int stage = s_first; stage < g.nstages; stage += s_step) {
+                    const int gg0 = stage * g.G;
+                    const int chunk = gg0 >> g.gpc_log2;
+                    const int pbase = chunk * g.npairs + ((gg0 - (chunk << g.gpc_log2)) >> 1);   // pair of (tap 0, the stage's first two groups)
+                    const unsigned char* __restrict__ pa0 = reinterpret_cast<const unsigned char*>(wpacked + w_off0 + static_cast<int64_t>(pbase) * (kFragBytes / 2));
+                    const unsigned char* __restrict__ pa1 = reinterpret_cast<const unsigned char*>(wpacked + w_off1 + static_cast<int64_t>(pbase) * (kFragBytes / 2));
+                    sk_u32x4 wa[4][2];
+                    sk_u32x4 wb[2][TT];
+                    uint32_t bo[4];
+                    // Requests the weight fragments of the step described by table entry `e` and notes where its activations are.
+                    auto req_a = [&](int slot, const sk_u32x4& e) __attribute__((always_inline)) {
+                        const uint32_t voff = lane16 + e[0];
+                        wa[slot][0] = *reinterpret_cast<const sk_u32x4*>(pa0 + voff);
+                        wa[slot][1] = *reinterpret_cast<const sk_u32x4*>(pa1 + voff);
+                        bo[slot] = half ? e[2] : e[1];
+                    };
+                    auto read_b = [&](int slot, uint32_t boff) __attribute__((always_inline)) {
 #pragma unroll
-                    for (int t = 0; t < TT; ++t) {
-                        const sk_u32x4 b = *reinterpret_cast<const sk_u32x4*>(bq + t * tile_t);
-                        acc[t][0] = sk_mfma<F16>(a0, b, acc[t][0]);
-                        acc[t][1] = sk_mfma<F16>(a1, b, acc[t][1]);
+                        for (int t = 0; t < TT; ++t) wb[slot][t] = *reinterpret_cast<const sk_u32x4*>(bl + boff + t * tile_t);
+                    };
+                    auto mma = [&](int sa, int sb) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int t = 0; t < TT; ++t) {
+                            acc[t][0] = sk_mfma<F16>(wa[sa][0], wb[sb][t], acc[t][0]);
+                            acc[t][1] = sk_mfma<F16>(wa[sa][1], wb[sb][t], acc[t][1]);
+                        }
+                    };
+                    req_a(0, table[0]);
+                    req_a(1, table[1]);
+                    req_a(2, table[2]);
+                    sk_u32x4 ent = table[3];       // entry of the step whose weights are requested next
+                    stage_in(stage);
+                    read_b(0, bo[0]);
+                    int st = 0;
+                    // Four steps per trip, no branch inside: weights three steps ahead (4 register sets), activations one step
+                    // ahead (2 sets). The scheduling fences keep each step's operand requests ahead of the previous step's
+                    // matrix instructions; left alone the compiler sinks them below, where their latency is exposed.
+                    for (; st + 4 <= nst; st += 4) {
+                        req_a(3, ent);
+                        ent = table[st + 4];
+                        read_b(1, bo[1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(0, 0);
+                        req_a(0, ent);
+                        ent = table[st + 5];
+                        read_b(0, bo[2]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(1, 1);
+                        req_a(1, ent);
+                        ent = table[st + 6];
+                        read_b(1, bo[3]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(2, 0);
+                        req_a(2, ent);
+                        ent = table[st + 7];
+                        read_b(0, bo[0]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma(3, 1);
                     }
-                };
-                sk_u32x4 wa[3][2];
-                if (total > 0) {
-                    load_a(0, wa[0][0], wa[0][1]);
-                    load_a(1, wa[1][0], wa[1][1]);
-                }
-                int st = 0;            // step inside the current stage
-                int stage = s_first;
-                for (int fs = 0; fs < total; fs += 3) {
-                    load_a(fs + 2, wa[2][0], wa[2][1]);
-                    if (st == 0) stage_in(stage);
-                    mma_step(st, wa[0][0], wa[0][1]);
-                    if (++st == nst) { st = 0; stage += s_step; }
-                    if (fs + 1 < total) {
-                        load_a(fs + 3, wa[0][0], wa[0][1]);
-                        if (st == 0) stage_in(stage);
-                        mma_step(st, wa[1][0], wa[1][1]);
-                        if (++st == nst) { st = 0; stage += s_step; }
-                    }
-                    if (fs + 2 < total) {
-                        load_a(fs + 4, wa[1][0], wa[1][1]);
-                        if (st == 0) stage_in(stage);
-                        mma_step(st, wa[2][0], wa[2][1]);
-                        if (++st == nst) { st = 0; stage += s_step; }
+                    // The last nst % 4 steps: wa[0..2] hold their weight fragments, wb[0] the first one's activations.
+                    if (st < nst) {
+                        if (st + 1 < nst) read_b(1, bo[1]);
+                        mma(0, 0);
+                        if (st + 1 < nst) {
+                            if (st + 2 < nst) read_b(0, bo[2]);
+                            mma(1, 1);
+                            if (st + 2 < nst) mma(2, 0);
+                        }
                     }
                 }
             }
@@ -330,24 +388,22 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // pixel: a "quad" (f, q) is the lane's half of channel group j8 = 8 oc_tile + 4 f + q. One quad at a time: its bias
             // and membrane (4 + 4 registers) live across its timesteps; a lane's addresses are 32-bit offsets from uniform bases.
             const float* __restrict__ v_src = t0 == 0 ? v_init : v_out;   // later windows continue from the stored membrane
-            // The epilogue's loop-invariant loads (bias values of 8 quads) must not be hoisted above the matrix loop, where
-            // they would hold registers: the pointer is made opaque here.
-            const float* bias_e = bias;
-            asm volatile("" : "+s"(bias_e));
             const int t_count = g.shared_x ? g.T : min(TT, g.T - t0);      // LIF steps of this window
-            const uint32_t lane_nchw = static_cast<uint32_t>((n_c * g.Cout + 4 * half) * po + pxo);        // elements
-            const uint32_t lane_c8 = static_cast<uint32_t>(((n_c * g.C8out) * po + pxo) * 8 + 4 * half);   // elements
-            const uint32_t lane_bits = static_cast<uint32_t>((n_c * g.C8out) * po + pxo);                  // bytes
+            // (Made opaque here: everything derived from the lane's pixel offset is then computed after the matrix loop instead of
+            // before it, where the compiler would otherwise park two dozen store addresses in registers or scratch memory.)
+            int pxo_e = pxo, n_e = n_c;
+            asm volatile("" : "+v"(pxo_e), "+v"(n_e));
+            const uint32_t lane_nchw = static_cast<uint32_t>((n_e * g.Cout + 4 * half) * po + pxo_e);        // elements
+            const uint32_t lane_c8 = static_cast<uint32_t>(((n_e * g.C8out) * po + pxo_e) * 8 + 4 * half);   // elements
+            const uint32_t lane_bits = static_cast<uint32_t>((n_e * g.C8out) * po + pxo_e);                  // bytes
 
-            // Bias, valid-channel mask and initial membrane of the quad of channel group j8.
-            auto quad_begin = [&](int j8, float (&bv)[4], float (&v)[4], uint32_t& chm) __attribute__((always_inline)) {
+            // Valid-channel mask and initial membrane of the quad of channel group j8.
+            auto quad_begin = [&](int j8, float (&v)[4], uint32_t& chm) __attribute__((always_inline)) {
                 const int ch0 = j8 * 8 + 4 * half;
                 chm = 0;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const bool ch_ok = ch0 + k < g.Cout;
-                    chm |= ch_ok ? (1u << k) : 0u;
-                    bv[k] = ch_ok ? bias_e[ch0 + k] : 0.0f;
+                    chm |= ch0 + k < g.Cout ? (1u << k) : 0u;
                     v[k] = 0.0f;
                 }
                 if (v_src != nullptr && !g.analog_out && px_ok) {
@@ -357,52 +413,95 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         if ((chm >> k) & 1u) v[k] = vp[lane_nchw + static_cast<uint32_t>(k * po)];
                 }
             };
-            // One step of a quad at absolute timestep `ta`: x = sums + bias (+ residual), then the neuron (its spikes are the
-            // returned nibble) or, without a neuron, x itself; dense output layouts are written here.
-            auto quad_step = [&](int ta, int j8, const float (&x_in)[4], const float (&bv)[4], float (&v)[4], uint32_t chm) __attribute__((always_inline)) -> uint32_t {
+            // The residual of a quad at timestep `ta`, raw (two registers in any layout), and its addition to the quad's sums.
+            auto res_load = [&](int ta, int j8, uint32_t (&raw)[2]) __attribute__((always_inline)) {
+                raw[0] = 0u;
+                raw[1] = 0u;
+                if (g.res_layout < 0 || !(j8 < g.C8out && px_ok)) return;
+                const unsigned char* __restrict__ res_t = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, ta));
+                if (g.res_layout == SNNF_LAYOUT_BITS) {
+                    raw[0] = (res_t + static_cast<int64_t>(j8) * po)[lane_bits];
+                } else if (g.res_layout == SNNF_LAYOUT_C8) {
+                    const Pack<uint32_t, 2> r2 = *reinterpret_cast<const Pack<uint32_t, 2>*>(reinterpret_cast<const XT*>(res_t) + static_cast<int64_t>(j8) * po * 8 + lane_c8);
+                    raw[0] = r2.v[0];
+                    raw[1] = r2.v[1];
+                } else {
+                    const uint16_t* __restrict__ rp = reinterpret_cast<const uint16_t*>(res_t) + static_cast<int64_t>(j8) * 8 * po;
+                    const int ch0 = j8 * 8 + 4 * half;
+                    uint32_t e[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) e[k] = ch0 + k < g.Cout ? rp[lane_nchw + static_cast<uint32_t>(k * po)] : 0u;
+                    raw[0] = e[0] | (e[1] << 16);
+                    raw[1] = e[2] | (e[3] << 16);
+                }
+            };
+            auto res_add = [&](const uint32_t (&raw)[2], float (&x)[4]) __attribute__((always_inline)) {
+                if (g.res_layout < 0) return;
+                if (g.res_layout == SNNF_LAYOUT_BITS) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) x[k] += ((raw[0] >> (4 * half + k)) & 1u) ? 1.0f : 0.0f;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t bits = (raw[k >> 1] >> (16 * (k & 1))) & 0xffffu;
+                        x[k] += to_float(XT{static_cast<uint16_t>(bits)});
+                    }
+                }
+            };
+            // Store of 4 channel values of the lane's pixel at timestep `ta` in a dense layout (C8: one 8-byte store).
+            auto quad_store_dense = [&](int ta, int j8, const Pack<XT, 4>& o, uint32_t chm) __attribute__((always_inline)) {
+                unsigned char* __restrict__ out_t = out + static_cast<int64_t>(ta) * g.out_step_stride;
+                if (g.out_layout == SNNF_LAYOUT_C8) {
+                    *reinterpret_cast<Pack<XT, 4>*>(reinterpret_cast<XT*>(out_t) + static_cast<int64_t>(j8) * po * 8 + lane_c8) = o;
+                } else {
+                    XT* __restrict__ op = reinterpret_cast<XT*>(out_t) + static_cast<int64_t>(j8) * 8 * po;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if ((chm >> k) & 1u) op[lane_nchw + static_cast<uint32_t>(k * po)] = o.v[k];
+                }
+            };
+            // One step of a quad at absolute timestep `ta`: x = sums (bias included) (+ residual), then the neuron (its spikes are the
+            // returned nibble) or, without a neuron, x itself written to the dense output.
+            auto quad_step = [&](int ta, int j8, const float (&x_in)[4], const uint32_t (&res_raw)[2], float (&v)[4], uint32_t chm) __attribute__((always_inline)) -> uint32_t {
                 const bool grp_ok = j8 < g.C8out && px_ok;
                 float x[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) x[k] = x_in[k] + bv[k];
-                if (g.res_layout >= 0 && grp_ok) {
-                    const unsigned char* __restrict__ res_t = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, ta));
-                    if (g.res_layout == SNNF_LAYOUT_BITS) {
-                        const uint32_t byte = (res_t + static_cast<int64_t>(j8) * po)[lane_bits];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) x[k] += ((byte >> (4 * half + k)) & 1u) ? 1.0f : 0.0f;
-                    } else if (g.res_layout == SNNF_LAYOUT_C8) {
-                        const Pack<XT, 4> r4 = *reinterpret_cast<const Pack<XT, 4>*>(reinterpret_cast<const XT*>(res_t) + static_cast<int64_t>(j8) * po * 8 + lane_c8);
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) x[k] += to_float(r4.v[k]);
-                    } else {
-                        const XT* __restrict__ rp = reinterpret_cast<const XT*>(res_t) + static_cast<int64_t>(j8) * 8 * po;
-#pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                            if ((chm >> k) & 1u) x[k] += to_float(rp[lane_nchw + static_cast<uint32_t>(k * po)]);
-                    }
-                }
+                for (int k = 0; k < 4; ++k) x[k] = x_in[k];
+                res_add(res_raw, x);
                 uint32_t nib = 0;
                 if (!g.analog_out) {
+                    if (common_lif) {   // power-of-two tau, hard reset: one test per quad step instead of two per neuron step
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) nib |= lif_step(x[k], v[k], lif) ? (1u << k) : 0u;
+                        for (int k = 0; k < 4; ++k) {
+                            const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
+                            const bool fired = h >= lif.v_threshold;
+                            v[k] = fired ? lif.v_reset : h;
+                            nib |= fired ? (1u << k) : 0u;
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) nib |= lif_step(x[k], v[k], lif) ? (1u << k) : 0u;
+                    }
                     nib &= chm;
-                }
-                if (grp_ok && g.out_layout != SNNF_LAYOUT_BITS) {
-                    unsigned char* __restrict__ out_t = out + static_cast<int64_t>(ta) * g.out_step_stride;
+                } else if (grp_ok) {
                     Pack<XT, 4> o;
 #pragma unroll
-                    for (int k = 0; k < 4; ++k)
-                        o.v[k] = g.analog_out ? from_float<XT>(((chm >> k) & 1u) ? x[k] : 0.0f) : spike_value<XT>((nib >> k) & 1u);
-                    if (g.out_layout == SNNF_LAYOUT_C8) {
-                        *reinterpret_cast<Pack<XT, 4>*>(reinterpret_cast<XT*>(out_t) + static_cast<int64_t>(j8) * po * 8 + lane_c8) = o;
-                    } else {
-                        XT* __restrict__ op = reinterpret_cast<XT*>(out_t) + static_cast<int64_t>(j8) * 8 * po;
-#pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                            if ((chm >> k) & 1u) op[lane_nchw + static_cast<uint32_t>(k * po)] = o.v[k];
-                    }
+                    for (int k = 0; k < 4; ++k) o.v[k] = from_float<XT>(((chm >> k) & 1u) ? x[k] : 0.0f);
+                    quad_store_dense(ta, j8, o, chm);
                 }
                 return nib;
+            };
+            // Dense spike output of up to 8 consecutive steps [ta0, ta0 + cnt) of a quad from their nibbles, one step at a time
+            // (a loop: dense spikes only leave at the network's boundary, and unrolled stores would cost the common path registers).
+            auto quad_store_spikes = [&](int ta0, int cnt, int j8, uint32_t nibw, uint32_t chm) __attribute__((always_inline)) {
+                if (j8 < g.C8out && px_ok) {
+                    for (int i = 0; i < cnt; ++i) {
+                        Pack<XT, 4> o;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) o.v[k] = spike_value<XT>((nibw >> (4 * i + k)) & 1u);
+                        quad_store_dense(ta0 + i, j8, o, chm);
+                    }
+                }
             };
             // Bit-packed output of up to 8 consecutive steps [ta0, ta0 + cnt) of a quad: nibble i of `nibw` = step ta0 + i. The
             // other half of the wave holds the other nibble of every byte (lanes l and l + 32 own the same pixel); even
@@ -432,100 +531,193 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 }
             };
 
+            // FAST: the layer as it runs inside a network - bit-packed output, no or a bit-packed residual, the common neuron
+            // (power-of-two tau, hard reset), zero initial membrane, one window, whole channel groups. Straight-line code.
+            // One LIF step of 4 neurons: sums x (+ the residual bits of this half of the byte), returns the spike nibble.
+            auto fast_lif4 = [&](const float (&x)[4], uint32_t res_half, bool with_res, float (&v)[4]) __attribute__((always_inline)) -> uint32_t {
+                uint32_t nib = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float xx = x[k];
+                    if (with_res) xx += __uint_as_float(static_cast<uint32_t>(static_cast<int32_t>(res_half << (31 - k)) >> 31) & 0x3f800000u);
+                    const float h = v[k] + (xx - v[k]) * lif.inv_tau;
+                    const bool fired = h >= lif.v_threshold;
+                    v[k] = fired ? lif.v_reset : h;
+                    nib |= fired ? (1u << k) : 0u;
+                }
+                return nib;
+            };
+            // Residual byte of channel group j8 at timestep ta for this lane's pixel, shifted to this half's nibble. Lanes
+            // without a pixel read pixel 0 of image 0 (their result is never stored).
+            auto fast_res = [&](int ta, int j8) __attribute__((always_inline)) -> uint32_t {
+                const unsigned char* __restrict__ res_t = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, ta));
+                const uint32_t byte = (res_t + static_cast<int64_t>(min(j8, g.C8out - 1)) * po)[lane_bits];
+                return byte >> (4 * half);
+            };
+            // All steps of one quad whose sums are xq[tw][k]: residual, LIF, bit-packed store, optional membrane store.
+            auto fast_quad = [&](int j8, const float (&xq)[TT][4], const uint32_t (&rb)[TT], bool with_res) __attribute__((always_inline)) {
+                float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                if constexpr (TT == 1) {
+                    for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
+                        const int cnt = min(8, t_count - ta0);
+                        uint32_t nibw = 0;
+                        for (int i = 0; i < cnt; ++i) {
+                            const uint32_t r = with_res ? fast_res(ta0 + i, j8) : 0u;
+                            nibw |= fast_lif4(xq[0], r, with_res, v) << (4 * i);
+                        }
+                        quad_store_bits(ta0, cnt, j8, nibw);
+                    }
+                } else {
+                    uint32_t nibw = 0;
+                    if (with_res) {
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw)
+                            if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw], true, v) << (4 * tw);
+                    } else {
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw)
+                            if (tw < t_count) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                    }
+                    quad_store_bits(0, t_count, j8, nibw);
+                }
+                if (v_out != nullptr && px_ok && j8 < g.C8out) {
+                    float* __restrict__ vp = v_out + static_cast<int64_t>(j8) * 8 * po;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) vp[lane_nchw + static_cast<uint32_t>(k * po)] = v[k];
+                }
+            };
+            // All steps of one quad, any layouts and neuron (the general path).
+            auto general_quad = [&](int j8, const float (&xq)[TT][4]) __attribute__((always_inline)) {
+                float v[4];
+                uint32_t chm;
+                quad_begin(j8, v, chm);
+                if constexpr (TT == 1) {
+                    // One convolution result, t_count LIF steps on it (one step, or one frame shared by all T timesteps).
+                    for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
+                        const int cnt = min(8, t_count - ta0);
+                        uint32_t nibw = 0;
+                        for (int i = 0; i < cnt; ++i) {
+                            uint32_t rr[2];
+                            res_load(t0 + ta0 + i, j8, rr);
+                            nibw |= quad_step(t0 + ta0 + i, j8, xq[0], rr, v, chm) << (4 * i);
+                        }
+                        if (g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0 + ta0, cnt, j8, nibw);
+                        else if (!g.analog_out) quad_store_spikes(t0 + ta0, cnt, j8, nibw, chm);
+                    }
+                } else {
+                    uint32_t rr[TT][2];
+#pragma unroll
+                    for (int tw = 0; tw < TT; ++tw) res_load(min(t0 + tw, g.T - 1), j8, rr[tw]);
+                    uint32_t nibw = 0;
+#pragma unroll
+                    for (int tw = 0; tw < TT; ++tw)
+                        if (tw < t_count) nibw |= quad_step(t0 + tw, j8, xq[tw], rr[tw], v, chm) << (4 * tw);
+                    if (g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0, t_count, j8, nibw);
+                    else if (!g.analog_out) quad_store_spikes(t0, t_count, j8, nibw, chm);
+                }
+                quad_end(j8, v, chm);
+            };
+
             if constexpr (!SK) {
-                // A runtime loop over the wave's 8 quads keeps the code small; a quad's sums are copied out of the accumulators
-                // by a switch (constant register indices), so the accumulators stay in registers.
-                for (int fq = 0; fq < 8; ++fq) {
-                    const int j8 = oc_tile * 8 + fq;
-                    float xq[TT][4];
+                if constexpr (FAST) {
+                    const bool with_res = g.res_layout >= 0;
+                    // The residual bytes of a quad are requested two quads ahead, through three register sets.
+                    uint32_t rb[3][TT];
+#pragma unroll
+                    for (int i = 0; i < 3; ++i)
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw) rb[i][tw] = 0u;
+                    auto req_res = [&](int set, int fq) __attribute__((always_inline)) {
+                        if (with_res && TT > 1) {
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw) rb[set][tw] = fast_res(min(tw, t_count - 1), oc_tile * 8 + fq);
+                        }
+                    };
+                    req_res(0, 0);
+                    req_res(1, 1);
+                    auto do_quad = [&](auto fq_tag) __attribute__((always_inline)) {
+                        constexpr int fq = decltype(fq_tag)::value;
+                        if constexpr (fq + 2 < 8) req_res((fq + 2) % 3, fq + 2);
+                        float xq[TT][4];
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw)
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) xq[tw][k] = acc[tw][fq >> 2][4 * (fq & 3) + k];
+                        fast_quad(oc_tile * 8 + fq, xq, rb[fq % 3], with_res);
+                    };
+                    do_quad(std::integral_constant<int, 0>{});
+                    do_quad(std::integral_constant<int, 1>{});
+                    do_quad(std::integral_constant<int, 2>{});
+                    do_quad(std::integral_constant<int, 3>{});
+                    do_quad(std::integral_constant<int, 4>{});
+                    do_quad(std::integral_constant<int, 5>{});
+                    do_quad(std::integral_constant<int, 6>{});
+                    do_quad(std::integral_constant<int, 7>{});
+                } else {
+                    // A runtime loop over the wave's 8 quads keeps the code small; a quad's sums are copied out of the accumulators
+                    // by a switch (constant register indices), so the accumulators stay in registers.
+                    for (int fq = 0; fq < 8; ++fq) {
+                        float xq[TT][4];
 #define SNNF_SPK_COPY_QUAD(F, Q)                                          \
     _Pragma("unroll") for (int tw = 0; tw < TT; ++tw)                     \
         _Pragma("unroll") for (int k = 0; k < 4; ++k) xq[tw][k] = acc[tw][F][4 * (Q) + k]
-                    switch (fq) {
-                        case 0: SNNF_SPK_COPY_QUAD(0, 0); break;
-                        case 1: SNNF_SPK_COPY_QUAD(0, 1); break;
-                        case 2: SNNF_SPK_COPY_QUAD(0, 2); break;
-                        case 3: SNNF_SPK_COPY_QUAD(0, 3); break;
-                        case 4: SNNF_SPK_COPY_QUAD(1, 0); break;
-                        case 5: SNNF_SPK_COPY_QUAD(1, 1); break;
-                        case 6: SNNF_SPK_COPY_QUAD(1, 2); break;
-                        default: SNNF_SPK_COPY_QUAD(1, 3); break;
-                    }
-#undef SNNF_SPK_COPY_QUAD
-                    float bv[4], v[4];
-                    uint32_t chm;
-                    quad_begin(j8, bv, v, chm);
-                    if constexpr (TT == 1) {
-                        // One convolution result, t_count LIF steps on it (one step, or one frame shared by all T timesteps).
-                        for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
-                            const int cnt = min(8, t_count - ta0);
-                            uint32_t nibw = 0;
-                            for (int i = 0; i < cnt; ++i) nibw |= quad_step(t0 + ta0 + i, j8, xq[0], bv, v, chm) << (4 * i);
-                            if (g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0 + ta0, cnt, j8, nibw);
+                        switch (fq) {
+                            case 0: SNNF_SPK_COPY_QUAD(0, 0); break;
+                            case 1: SNNF_SPK_COPY_QUAD(0, 1); break;
+                            case 2: SNNF_SPK_COPY_QUAD(0, 2); break;
+                            case 3: SNNF_SPK_COPY_QUAD(0, 3); break;
+                            case 4: SNNF_SPK_COPY_QUAD(1, 0); break;
+                            case 5: SNNF_SPK_COPY_QUAD(1, 1); break;
+                            case 6: SNNF_SPK_COPY_QUAD(1, 2); break;
+                            default: SNNF_SPK_COPY_QUAD(1, 3); break;
                         }
-                    } else {
-                        uint32_t nibw = 0;
-#pragma unroll
-                        for (int tw = 0; tw < TT; ++tw)
-                            if (tw < t_count) nibw |= quad_step(t0 + tw, j8, xq[tw], bv, v, chm) << (4 * tw);
-                        if (g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0, t_count, j8, nibw);
+#undef SNNF_SPK_COPY_QUAD
+                        general_quad(oc_tile * 8 + fq, xq);
                     }
-                    quad_end(j8, v, chm);
                 }
             } else {
-                // Split K: every wave parks one timestep's 32 partial sums per lane in LDS (the staging regions are dead by
-                // then); the owner of a quad adds the WK partial sums in a fixed order and runs that step's LIF right away, so
-                // only the owned quads' membranes stay in registers between rounds.
-                float* __restrict__ part = reinterpret_cast<float*>(lds);      // [wave][quad 0..7][lane][4]
-                const int nq = 8 >> g.wk_log2;                                 // quads this wave owns: quad0 .. quad0 + nq - 1
-                const int quad0 = wk * nq;
-                float bv[4][4], v[4][4];
-                uint32_t chm[4], nibw[4];
+                // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then), two
+                // quads per round for all TT timesteps; quad 2 r + e of round r is finished by wave (2 r + e) mod WK of the tile,
+                // which adds the WK partial sums in a fixed order and then runs that quad's timesteps like the unsplit kernel.
+                float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkTableBytes);      // [wave][e 0..1][tw][lane][4]
+                for (int r = 0; r < 4; ++r) {
+                    __syncthreads();   // the previous round's sums are consumed (first round: every wave is done with its staging region)
+#define SNNF_SPK_PARK_QUAD(E, F, Q)                                                                                              \
+    _Pragma("unroll") for (int tw = 0; tw < TT; ++tw) {                                                                          \
+        const sk_f32x4 four = {acc[tw][F][4 * (Q)], acc[tw][F][4 * (Q) + 1], acc[tw][F][4 * (Q) + 2], acc[tw][F][4 * (Q) + 3]};  \
+        *reinterpret_cast<sk_f32x4*>(part + (((wave * 2 + (E)) * TT + tw) * 64 + lane) * 4) = four;                             \
+    }
+                    switch (r) {
+                        case 0: SNNF_SPK_PARK_QUAD(0, 0, 0) SNNF_SPK_PARK_QUAD(1, 0, 1) break;
+                        case 1: SNNF_SPK_PARK_QUAD(0, 0, 2) SNNF_SPK_PARK_QUAD(1, 0, 3) break;
+                        case 2: SNNF_SPK_PARK_QUAD(0, 1, 0) SNNF_SPK_PARK_QUAD(1, 1, 1) break;
+                        default: SNNF_SPK_PARK_QUAD(0, 1, 2) SNNF_SPK_PARK_QUAD(1, 1, 3) break;
+                    }
+#undef SNNF_SPK_PARK_QUAD
+                    const int e_own = (wk - 2 * r) & (WK - 1);      // this wave finishes quad 2 r + e_own of the round, if that is 0 or 1
+                    const int j8 = oc_tile * 8 + 2 * r + e_own;
+                    uint32_t rb[TT];
 #pragma unroll
-                for (int qi = 0; qi < 4; ++qi) {
-                    nibw[qi] = 0;
-                    if (qi < nq) quad_begin(oc_tile * 8 + quad0 + qi, bv[qi], v[qi], chm[qi]);
-                }
+                    for (int tw = 0; tw < TT; ++tw) rb[tw] = 0u;
+                    if constexpr (FAST) {
+                        if (e_own < 2 && g.res_layout >= 0 && TT > 1) {
 #pragma unroll
-                for (int tw = 0; tw < TT; ++tw) {
-                    if (tw < (TT == 1 ? 1 : t_count)) {   // uniform over the workgroup
-                        __syncthreads();
-#pragma unroll
-                        for (int f = 0; f < 2; ++f)
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) {
-                                const sk_f32x4 four = {acc[tw][f][4 * q], acc[tw][f][4 * q + 1], acc[tw][f][4 * q + 2], acc[tw][f][4 * q + 3]};
-                                *reinterpret_cast<sk_f32x4*>(part + ((wave * 8 + f * 4 + q) * 64 + lane) * 4) = four;
-                            }
-                        __syncthreads();
-#pragma unroll
-                        for (int qi = 0; qi < 4; ++qi) {
-                            if (qi < nq) {
-                                const int j8 = oc_tile * 8 + quad0 + qi;
-                                sk_f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-                                for (int k = 0; k < WK; ++k)
-                                    sum += *reinterpret_cast<const sk_f32x4*>(part + (((tile_in_block * WK + k) * 8 + quad0 + qi) * 64 + lane) * 4);
-                                const float x_in[4] = {sum[0], sum[1], sum[2], sum[3]};
-                                if constexpr (TT == 1) {
-                                    for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
-                                        const int cnt = min(8, t_count - ta0);
-                                        uint32_t w8 = 0;
-                                        for (int i = 0; i < cnt; ++i) w8 |= quad_step(t0 + ta0 + i, j8, x_in, bv[qi], v[qi], chm[qi]) << (4 * i);
-                                        if (g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0 + ta0, cnt, j8, w8);
-                                    }
-                                } else {
-                                    nibw[qi] |= quad_step(t0 + tw, j8, x_in, bv[qi], v[qi], chm[qi]) << (4 * tw);
-                                }
-                            }
+                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), j8);
                         }
                     }
-                }
+                    __syncthreads();
+                    if (e_own < 2) {
+                        float xq[TT][4];
 #pragma unroll
-                for (int qi = 0; qi < 4; ++qi) {
-                    if (qi < nq) {
-                        const int j8 = oc_tile * 8 + quad0 + qi;
-                        if (TT > 1 && g.out_layout == SNNF_LAYOUT_BITS) quad_store_bits(t0, t_count, j8, nibw[qi]);
-                        quad_end(j8, v[qi], chm[qi]);
+                        for (int tw = 0; tw < TT; ++tw) {
+                            sk_f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+                            for (int k = 0; k < WK; ++k)
+                                sum += *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 2 + e_own) * TT + tw) * 64 + lane) * 4);
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) xq[tw][k] = sum[k];
+                        }
+                        if constexpr (FAST) fast_quad(j8, xq, rb, g.res_layout >= 0);
+                        else general_quad(j8, xq);
                     }
                 }
             }
@@ -542,22 +734,21 @@ int launch_conv_spk_variant(const SpkLaunch& L) {
                                                                         static_cast<unsigned char*>(L.out), L.v_out, L.lif);
         return check_launch("snnf_conv_lif_blocked");
     };
-    return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true>) : run(conv_spk_kernel<XT, TT, IN, false>);
+    if (L.fast_epilogue) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true, true>) : run(conv_spk_kernel<XT, TT, IN, false, true>);
+    return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true, false>) : run(conv_spk_kernel<XT, TT, IN, false, false>);
 }
 
-template <typename XT>
+template <typename XT, int IN>
 int launch_conv_spk_tt(const SpkLaunch& L, int tt) {
-    if (L.g.in_layout == SNNF_LAYOUT_BITS) {
-        if (tt == 4) return launch_conv_spk_variant<XT, 4, SNNF_LAYOUT_BITS>(L);
-        if (tt == 2) return launch_conv_spk_variant<XT, 2, SNNF_LAYOUT_BITS>(L);
-        return launch_conv_spk_variant<XT, 1, SNNF_LAYOUT_BITS>(L);
-    }
-    if (tt == 4) return launch_conv_spk_variant<XT, 4, SNNF_LAYOUT_C8>(L);
-    if (tt == 2) return launch_conv_spk_variant<XT, 2, SNNF_LAYOUT_C8>(L);
-    return launch_conv_spk_variant<XT, 1, SNNF_LAYOUT_C8>(L);
+    if (tt == 4) return launch_conv_spk_variant<XT, 4, IN>(L);
+    if (tt == 2) return launch_conv_spk_variant<XT, 2, IN>(L);
+    return launch_conv_spk_variant<XT, 1, IN>(L);
 }
 
-int launch_conv_spk_bf16(const SpkLaunch& L, int tt);
-int launch_conv_spk_f16(const SpkLaunch& L, int tt);
+// One launcher per activation dtype and input layout (each in its own translation unit, so that they compile in parallel).
+int launch_conv_spk_bf16_bits(const SpkLaunch& L, int tt);
+int launch_conv_spk_bf16_c8(const SpkLaunch& L, int tt);
+int launch_conv_spk_f16_bits(const SpkLaunch& L, int tt);
+int launch_conv_spk_f16_c8(const SpkLaunch& L, int tt);
 
 }  // namespace snnf
