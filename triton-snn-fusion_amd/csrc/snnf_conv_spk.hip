@@ -161,7 +161,7 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     // every wave still gets at least two stages.
     const int cus = compute_units();
     int wk_log2 = 0;
-    while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 4 && g.nstages >= (4 << wk_log2)) ++wk_log2;
+    while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 6 && g.nstages >= (4 << wk_log2)) ++wk_log2;
     g.wk_log2 = wk_log2;
     const int tiles_per_block = kSpkWaves >> wk_log2;
     int grid = (g.n_items + tiles_per_block - 1) / tiles_per_block;

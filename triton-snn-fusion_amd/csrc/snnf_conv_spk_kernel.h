@@ -33,7 +33,7 @@ constexpr int kSpkWaves = 8;                      // waves per workgroup, one wo
 #define SPK_SLOTS 8
 #endif
 constexpr int kSpkSlots = SPK_SLOTS;                      // staging items per lane and timestep, at most
-constexpr size_t kSpkPartialBytes = kSpkWaves * 8 * 64 * 16;   // split-K: one timestep's partial sums of all waves
+constexpr size_t kSpkPartialBytes = kSpkWaves * 16 * 64 * 16;  // split-K: every wave parks 4 quads x up to 4 timesteps of partial sums per round
 constexpr int kSpkMaxSteps = 60;                  // matrix steps per stage, at most (the step table holds 4 more)
 constexpr size_t kSpkTableBytes = (kSpkMaxSteps + 4) * 16;      // the workgroup's step table at the start of LDS
 
@@ -215,9 +215,11 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         const int n_c = px_ok ? n : 0;
 
         for (int t0 = 0; t0 < nsteps_t; t0 += TT) {
-            // The accumulators start from the bias (requested now, needed at the first matrix instruction): register 4 q + k of
-            // fragment f is channel 64 oc_tile + 32 f + 8 q + 4 half + k. With K split over waves only the first one adds it.
+            // The accumulators start from the bias: register 4 q + k of fragment f is channel 64 oc_tile + 32 f + 8 q + 4 half + k.
+            // With K split over waves only the first one adds it. The bias is requested here and copied into the accumulators
+            // after the first stage's activations have been requested, so that both round trips to memory overlap.
             sk_f32x16 acc[TT][2];
+            sk_f32x4 bias4[2][4];
             {
                 const int nbias = g.nocf * 32;               // bias values behind the packed weight (zero beyond Cout)
 #pragma unroll
@@ -225,12 +227,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int ch0 = oc_tile * 64 + f * 32 + q * 8 + 4 * half;
-                        sk_f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
-                        if (ch0 < nbias && (!SK || wk == 0)) b4 = *reinterpret_cast<const sk_f32x4*>(bias + ch0);
-#pragma unroll
-                        for (int t = 0; t < TT; ++t)
-#pragma unroll
-                            for (int k = 0; k < 4; ++k) acc[t][f][4 * q + k] = b4[k];
+                        bias4[f][q] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                        if (ch0 < nbias && (!SK || wk == 0)) bias4[f][q] = *reinterpret_cast<const sk_f32x4*>(bias + ch0);
                     }
             }
 
@@ -238,49 +236,84 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // Item e = slot * 64 + lane of a timestep = (group, image, row, column) of the halo; its LDS address is 16 e. Items
             // are decoded on the fly (nothing about them is kept in registers across the matrix loop) and move in batches of 4
             // slots x TT timesteps: all loads of a batch are in flight together.
-            auto stage_in = [&](int s) __attribute__((always_inline)) {
+            // PRE (bit-packed inputs, lean epilogue): the first batch of the NEXT stage is requested before the matrix steps of the
+            // current one and sits in registers meanwhile, so that its latency hides behind them.
+            constexpr bool PRE = FAST && IN == SNNF_LAYOUT_BITS;
+            uint32_t pre_raw[TT][4];
+            uint32_t pre_ok = 0;
+            // Decodes the 4 items of batch jb of stage s: their global index (0 when they are padding) and the two flag nibbles
+            // (bit j: real data; bit 4 + j: the item exists and is written).
+            auto batch_decode = [&](int s, int jb, int lane_s, int (&idx)[4]) __attribute__((always_inline)) -> uint32_t {
                 const int gg0 = s * g.G;
                 const int base_u = ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
+                uint32_t ok_bits = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = (jb + j) * 64 + lane_s;
+                    const int gq = fast_div(e, g.d_region);
+                    const int rem = e - gq * g.region;
+                    const int ii = fast_div(rem, g.d_rrrc);
+                    const int rem2 = rem - ii * (g.RR * g.RC);
+                    const int r = fast_div(rem2, g.d_RC);
+                    const int c = rem2 - r * g.RC;
+                    const int ih = ih_lo + r, iw = iw_lo + c;
+                    const bool exists = e < g.IT;
+                    const bool ok = exists && n0 + ii < g.N && gg0 + gq < g.C8in && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
+                                    static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
+                    idx[j] = ok ? base_u + ((ii * g.C8in + gq) * g.H + r) * g.W + c : 0;
+                    ok_bits |= (ok ? (1u << j) : 0u) | (exists ? (16u << j) : 0u);
+                }
+                return ok_bits;
+            };
+            auto batch_load_bits = [&](const int (&idx)[4], uint32_t (&raw)[TT][4]) __attribute__((always_inline)) {
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const int ts = t0 + t < nsteps_t ? t0 + t : t0;   // steps beyond T repeat the window's first and are never stored
+                    const unsigned char* __restrict__ src = static_cast<const unsigned char*>(sk_kernarg_ptr(0, ts));
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) raw[t][j] = src[idx[j]];
+                }
+            };
+            auto batch_put_bits = [&](int jb, int lane_s, uint32_t ok_bits, const uint32_t (&raw)[TT][4]) __attribute__((always_inline)) {
+#pragma unroll
+                for (int t = 0; t < TT; ++t)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const sk_u32x4 d = sk_expand_bits<ONE>(((ok_bits >> j) & 1u) ? raw[t][j] : 0u);
+                        if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
+                    }
+            };
+            // Requests the first batch of stage s (PRE only).
+            auto stage_req = [&](int s) __attribute__((always_inline)) {
+                int lane_s = lane;
+                asm volatile("" : "+v"(lane_s));
+                int idx[4];
+                pre_ok = batch_decode(s, 0, lane_s, idx);
+                batch_load_bits(idx, pre_raw);
+            };
+            // One LDS stage: G channel groups of the patch's halo for TT timesteps, from global memory into this wave's region.
+            // Item e = slot * 64 + lane of a timestep = (group, image, row, column) of the halo; its LDS address is 16 e. Items
+            // are decoded on the fly (nothing about them is kept in registers across the matrix loop) and move in batches of 4
+            // slots x TT timesteps: all loads of a batch are in flight together.
+            auto stage_in = [&](int s) __attribute__((always_inline)) {
                 __builtin_amdgcn_wave_barrier();   // the matrix steps of the previous stage have read their operands
                 int lane_s = lane;                 // opaque: the decode below stays here instead of being hoisted out of every loop
                 asm volatile("" : "+v"(lane_s));   // (its results would sit in registers, or in scratch memory, across the matrix loop)
 #pragma unroll
                 for (int jb = 0; jb < kSpkSlots; jb += 4) {
                     if (jb < g.JT) {
-                        int idx[4];
-                        uint32_t ok_bits = 0;       // bit j: the item is real data; bit 4 + j: the item exists (is written)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int e = (jb + j) * 64 + lane_s;
-                            const int gq = fast_div(e, g.d_region);
-                            const int rem = e - gq * g.region;
-                            const int ii = fast_div(rem, g.d_rrrc);
-                            const int rem2 = rem - ii * (g.RR * g.RC);
-                            const int r = fast_div(rem2, g.d_RC);
-                            const int c = rem2 - r * g.RC;
-                            const int ih = ih_lo + r, iw = iw_lo + c;
-                            const bool exists = e < g.IT;
-                            const bool ok = exists && n0 + ii < g.N && gg0 + gq < g.C8in && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
-                                            static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
-                            idx[j] = ok ? base_u + ((ii * g.C8in + gq) * g.H + r) * g.W + c : 0;
-                            ok_bits |= (ok ? (1u << j) : 0u) | (exists ? (16u << j) : 0u);
+                        if constexpr (PRE) {
+                            if (jb == 0) {
+                                batch_put_bits(0, lane_s, pre_ok, pre_raw);
+                                continue;
+                            }
                         }
+                        int idx[4];
+                        const uint32_t ok_bits = batch_decode(s, jb, lane_s, idx);
                         if constexpr (IN == SNNF_LAYOUT_BITS) {
                             uint32_t raw[TT][4];
-#pragma unroll
-                            for (int t = 0; t < TT; ++t) {
-                                const int ts = t0 + t < nsteps_t ? t0 + t : t0;   // steps beyond T repeat the window's first and are never stored
-                                const unsigned char* __restrict__ src = static_cast<const unsigned char*>(sk_kernarg_ptr(0, ts));
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) raw[t][j] = src[idx[j]];
-                            }
-#pragma unroll
-                            for (int t = 0; t < TT; ++t)
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) {
-                                    const sk_u32x4 d = sk_expand_bits<ONE>(((ok_bits >> j) & 1u) ? raw[t][j] : 0u);
-                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
-                                }
+                            batch_load_bits(idx, raw);
+                            batch_put_bits(jb, lane_s, ok_bits, raw);
                         } else {
 #pragma unroll
                             for (int t = 0; t < TT; ++t) {
@@ -307,9 +340,26 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // 32-channel fragment). Per stage: the first weight fragments are requested from L2, the stage is brought into LDS,
             // then the steps run four at a time without a branch: weight fragments three steps ahead through four register
             // sets, activation fragments one step ahead through two.
+            const int s_first = SK ? wk : 0;
+            const int s_step = SK ? WK : 1;
+            if constexpr (PRE) {
+                if (have && s_first < g.nstages) stage_req(s_first);
+            }
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int t = 0; t < TT; ++t)
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) acc[t][f][4 * q + k] = bias4[f][q][k];
+            if constexpr (!SK) {
+                // The two waves of a SIMD unit (waves w and w + 4 of the workgroup) run out of phase: the first has the matrix
+                // cores to itself and then runs its epilogue, on the vector unit, under the second one's matrix instructions.
+                if (wave < 4) __builtin_amdgcn_s_setprio(2);
+                else __builtin_amdgcn_s_setprio(1);
+            }
             if (have) {
-                const int s_first = SK ? wk : 0;
-                const int s_step = SK ? WK : 1;
                 const uint32_t lane16 = static_cast<uint32_t>(lane) * 16u;
                 const unsigned char* __restrict__ bl = wlds + lane_b;
                 for (int stage = s_first; stage < g.nstages; stage += s_step) {
@@ -344,6 +394,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     req_a(2, table[2]);
                     sk_u32x4 ent = table[3];       // entry of the step whose weights are requested next
                     stage_in(stage);
+                    if constexpr (PRE) {
+                        if (stage + s_step < g.nstages) stage_req(stage + s_step);
+                    }
                     read_b(0, bo[0]);
                     int st = 0;
                     // Four steps per trip, no branch inside: weights three steps ahead (4 register sets), activations one step
@@ -387,6 +440,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // ---- epilogue. Accumulator register 4 q + k of fragment f holds channel 32 f + 8 q + 4 half + k of the lane's
             // pixel: a "quad" (f, q) is the lane's half of channel group j8 = 8 oc_tile + 4 f + q. One quad at a time: its bias
             // and membrane (4 + 4 registers) live across its timesteps; a lane's addresses are 32-bit offsets from uniform bases.
+            if constexpr (!SK) {
+                if (wave < 4) __builtin_amdgcn_s_setprio(0);
+            }
             const float* __restrict__ v_src = t0 == 0 ? v_init : v_out;   // later windows continue from the stored membrane
             const int t_count = g.shared_x ? g.T : min(TT, g.T - t0);      // LIF steps of this window
             // (Made opaque here: everything derived from the lane's pixel offset is then computed after the matrix loop instead of
@@ -547,12 +603,12 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 }
                 return nib;
             };
-            // Residual byte of channel group j8 at timestep ta for this lane's pixel, shifted to this half's nibble. Lanes
-            // without a pixel read pixel 0 of image 0 (their result is never stored).
+            // Residual byte of channel group j8 at timestep ta for this lane's pixel (this half's nibble is picked at the use,
+            // so that nothing waits on the load where it is issued). Lanes without a pixel read pixel 0 of image 0 (their
+            // result is never stored).
             auto fast_res = [&](int ta, int j8) __attribute__((always_inline)) -> uint32_t {
                 const unsigned char* __restrict__ res_t = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, ta));
-                const uint32_t byte = (res_t + static_cast<int64_t>(min(j8, g.C8out - 1)) * po)[lane_bits];
-                return byte >> (4 * half);
+                return (res_t + static_cast<int64_t>(min(j8, g.C8out - 1)) * po)[lane_bits];
             };
             // All steps of one quad whose sums are xq[tw][k]: residual, LIF, bit-packed store, optional membrane store.
             auto fast_quad = [&](int j8, const float (&xq)[TT][4], const uint32_t (&rb)[TT], bool with_res) __attribute__((always_inline)) {
@@ -562,7 +618,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         const int cnt = min(8, t_count - ta0);
                         uint32_t nibw = 0;
                         for (int i = 0; i < cnt; ++i) {
-                            const uint32_t r = with_res ? fast_res(ta0 + i, j8) : 0u;
+                            const uint32_t r = with_res ? fast_res(ta0 + i, j8) >> (4 * half) : 0u;
                             nibw |= fast_lif4(xq[0], r, with_res, v) << (4 * i);
                         }
                         quad_store_bits(ta0, cnt, j8, nibw);
@@ -572,7 +628,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     if (with_res) {
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw)
-                            if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw], true, v) << (4 * tw);
+                            if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
                     } else {
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw)
@@ -621,29 +677,43 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             if constexpr (!SK) {
                 if constexpr (FAST) {
                     const bool with_res = g.res_layout >= 0;
-                    // The residual bytes of a quad are requested two quads ahead, through three register sets.
-                    uint32_t rb[3][TT];
+                    // The residual bytes of all 8 quads are requested up front (the matrix loop's operand registers are free now):
+                    // one round trip to memory for the whole epilogue. The fence keeps the compiler from sinking each request
+                    // to its use, where every one of them would be waited for in turn.
+                    uint32_t rb[8][TT];
 #pragma unroll
-                    for (int i = 0; i < 3; ++i)
+                    for (int fq = 0; fq < 8; ++fq)
 #pragma unroll
-                        for (int tw = 0; tw < TT; ++tw) rb[i][tw] = 0u;
-                    auto req_res = [&](int set, int fq) __attribute__((always_inline)) {
-                        if (with_res && TT > 1) {
+                        for (int tw = 0; tw < TT; ++tw) rb[fq][tw] = 0u;
+                    if (with_res && TT > 1) {
+                        const unsigned char* res_ptr[TT];
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw) rb[set][tw] = fast_res(min(tw, t_count - 1), oc_tile * 8 + fq);
-                        }
-                    };
-                    req_res(0, 0);
-                    req_res(1, 1);
+                        for (int tw = 0; tw < TT; ++tw)
+                            res_ptr[tw] = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, min(tw, t_count - 1))) + static_cast<int64_t>(oc_tile) * 8 * po;
+                        auto req_res = [&](auto fq_tag) __attribute__((always_inline)) {
+                            constexpr int fq = decltype(fq_tag)::value;
+                            const uint32_t off = lane_bits + static_cast<uint32_t>(min(fq, g.C8out - 1 - oc_tile * 8) * po);
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw) rb[fq][tw] = res_ptr[tw][off];
+                        };
+                        req_res(std::integral_constant<int, 0>{});
+                        req_res(std::integral_constant<int, 1>{});
+                        req_res(std::integral_constant<int, 2>{});
+                        req_res(std::integral_constant<int, 3>{});
+                        req_res(std::integral_constant<int, 4>{});
+                        req_res(std::integral_constant<int, 5>{});
+                        req_res(std::integral_constant<int, 6>{});
+                        req_res(std::integral_constant<int, 7>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     auto do_quad = [&](auto fq_tag) __attribute__((always_inline)) {
                         constexpr int fq = decltype(fq_tag)::value;
-                        if constexpr (fq + 2 < 8) req_res((fq + 2) % 3, fq + 2);
                         float xq[TT][4];
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw)
 #pragma unroll
                             for (int k = 0; k < 4; ++k) xq[tw][k] = acc[tw][fq >> 2][4 * (fq & 3) + k];
-                        fast_quad(oc_tile * 8 + fq, xq, rb[fq % 3], with_res);
+                        fast_quad(oc_tile * 8 + fq, xq, rb[fq], with_res);
                     };
                     do_quad(std::integral_constant<int, 0>{});
                     do_quad(std::integral_constant<int, 1>{});
@@ -676,48 +746,55 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     }
                 }
             } else {
-                // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then), two
-                // quads per round for all TT timesteps; quad 2 r + e of round r is finished by wave (2 r + e) mod WK of the tile,
+                // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then), four
+                // quads per round for all TT timesteps; quad 4 r + e of round r is finished by wave (4 r + e) mod WK of the tile,
                 // which adds the WK partial sums in a fixed order and then runs that quad's timesteps like the unsplit kernel.
-                float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkTableBytes);      // [wave][e 0..1][tw][lane][4]
-                for (int r = 0; r < 4; ++r) {
+                float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkTableBytes);      // [wave][e 0..3][tw][lane][4]
+                for (int r = 0; r < 2; ++r) {
                     __syncthreads();   // the previous round's sums are consumed (first round: every wave is done with its staging region)
-#define SNNF_SPK_PARK_QUAD(E, F, Q)                                                                                              \
+#define SNNF_SPK_PARK_QUAD(E, F)                                                                                                 \
     _Pragma("unroll") for (int tw = 0; tw < TT; ++tw) {                                                                          \
-        const sk_f32x4 four = {acc[tw][F][4 * (Q)], acc[tw][F][4 * (Q) + 1], acc[tw][F][4 * (Q) + 2], acc[tw][F][4 * (Q) + 3]};  \
-        *reinterpret_cast<sk_f32x4*>(part + (((wave * 2 + (E)) * TT + tw) * 64 + lane) * 4) = four;                             \
+        const sk_f32x4 four = {acc[tw][F][4 * (E)], acc[tw][F][4 * (E) + 1], acc[tw][F][4 * (E) + 2], acc[tw][F][4 * (E) + 3]};  \
+        *reinterpret_cast<sk_f32x4*>(part + (((wave * 4 + (E)) * TT + tw) * 64 + lane) * 4) = four;                             \
     }
-                    switch (r) {
-                        case 0: SNNF_SPK_PARK_QUAD(0, 0, 0) SNNF_SPK_PARK_QUAD(1, 0, 1) break;
-                        case 1: SNNF_SPK_PARK_QUAD(0, 0, 2) SNNF_SPK_PARK_QUAD(1, 0, 3) break;
-                        case 2: SNNF_SPK_PARK_QUAD(0, 1, 0) SNNF_SPK_PARK_QUAD(1, 1, 1) break;
-                        default: SNNF_SPK_PARK_QUAD(0, 1, 2) SNNF_SPK_PARK_QUAD(1, 1, 3) break;
+                    if (r == 0) {
+                        SNNF_SPK_PARK_QUAD(0, 0) SNNF_SPK_PARK_QUAD(1, 0) SNNF_SPK_PARK_QUAD(2, 0) SNNF_SPK_PARK_QUAD(3, 0)
+                    } else {
+                        SNNF_SPK_PARK_QUAD(0, 1) SNNF_SPK_PARK_QUAD(1, 1) SNNF_SPK_PARK_QUAD(2, 1) SNNF_SPK_PARK_QUAD(3, 1)
                     }
 #undef SNNF_SPK_PARK_QUAD
-                    const int e_own = (wk - 2 * r) & (WK - 1);      // this wave finishes quad 2 r + e_own of the round, if that is 0 or 1
-                    const int j8 = oc_tile * 8 + 2 * r + e_own;
+                    const int e_first = (wk - 4 * r) & (WK - 1);      // this wave finishes quads 4 r + e, e = e_first, e_first + WK, ... < 4
+                    // The residual bytes of the wave's first quad travel while the workgroup meets.
                     uint32_t rb[TT];
 #pragma unroll
                     for (int tw = 0; tw < TT; ++tw) rb[tw] = 0u;
                     if constexpr (FAST) {
-                        if (e_own < 2 && g.res_layout >= 0 && TT > 1) {
+                        if (e_first < 4 && g.res_layout >= 0 && TT > 1) {
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), j8);
+                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), oc_tile * 8 + 4 * r + e_first);
                         }
                     }
                     __syncthreads();
-                    if (e_own < 2) {
+                    for (int e_own = e_first; e_own < 4; e_own += WK) {
+                        const int j8 = oc_tile * 8 + 4 * r + e_own;
                         float xq[TT][4];
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw) {
                             sk_f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
                             for (int k = 0; k < WK; ++k)
-                                sum += *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 2 + e_own) * TT + tw) * 64 + lane) * 4);
+                                sum += *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 4 + e_own) * TT + tw) * 64 + lane) * 4);
 #pragma unroll
                             for (int k = 0; k < 4; ++k) xq[tw][k] = sum[k];
                         }
-                        if constexpr (FAST) fast_quad(j8, xq, rb, g.res_layout >= 0);
-                        else general_quad(j8, xq);
+                        if constexpr (FAST) {
+                            if (e_own != e_first && g.res_layout >= 0 && TT > 1) {
+#pragma unroll
+                                for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), j8);
+                            }
+                            fast_quad(j8, xq, rb, g.res_layout >= 0);
+                        } else {
+                            general_quad(j8, xq);
+                        }
                     }
                 }
             }
