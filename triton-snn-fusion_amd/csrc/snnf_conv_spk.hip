@@ -158,15 +158,20 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     const int oc_tiles = (Cout + 63) / 64;
     g.n_items = g.n_patches * oc_tiles;
     // Split K over waves of a workgroup while the layer has fewer items than the machine has SIMDs (one wave each) and
-    // every wave still gets at least two stages.
+    // every wave still gets at least one stage.
     const int cus = compute_units();
     int wk_log2 = 0;
-    while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 6 && g.nstages >= (4 << wk_log2)) ++wk_log2;
+    while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 6 && g.nstages >= (2 << wk_log2)) ++wk_log2;
     g.wk_log2 = wk_log2;
     const int tiles_per_block = kSpkWaves >> wk_log2;
-    int grid = (g.n_items + tiles_per_block - 1) / tiles_per_block;
-    if (grid > cus) grid = cus;
-    g.iters = (g.n_items + grid * tiles_per_block - 1) / (grid * tiles_per_block);
+    // Workgroups that are resident together: one per compute unit, or two where a wave needs at most a quarter of a SIMD's
+    // registers (one timestep's accumulators) and two staging areas fit the LDS. The tiles are dealt evenly over as many
+    // rounds as that takes.
+    const size_t lds_bytes = std::max(kSpkTableBytes + static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes, wk_log2 > 0 ? kSpkTableBytes + kSpkPartialBytes : size_t{0});
+    const int resident = cus * ((tt == 1 && 2 * (lds_bytes + 1024) <= kMaxLds) ? 2 : 1);
+    const int blocks = (g.n_items + tiles_per_block - 1) / tiles_per_block;
+    g.iters = (blocks + resident - 1) / resident;
+    const int grid = (blocks + g.iters - 1) / g.iters;
     g.d_ppx = make_fast_div(g.PR * g.PC);
     g.d_PC = make_fast_div(g.PC);
     g.d_region = make_fast_div(g.region);
@@ -206,8 +211,7 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     L.v_out = neuron ? static_cast<float*>(v_out) : nullptr;
     L.lif = make_lif_params(v_threshold, v_reset, tau);
     L.grid = grid;
-    L.lds_bytes = kSpkTableBytes + static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes;
-    if (wk_log2 > 0 && L.lds_bytes < kSpkTableBytes + kSpkPartialBytes) L.lds_bytes = kSpkTableBytes + kSpkPartialBytes;
+    L.lds_bytes = lds_bytes;
     L.stream = as_stream(stream);
     const bool fast_epi = neuron && out_layout == SNNF_LAYOUT_BITS && (residuals == nullptr || res_layout == SNNF_LAYOUT_BITS) &&
                           L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset && v_init == nullptr && windows == 1 && Cout % 8 == 0;

@@ -119,11 +119,26 @@ __device__ __forceinline__ sk_u32x4 sk_expand_bits(uint32_t byte) {
 }
 
 template <typename XT, int TT, int IN, bool SK, bool FAST>
-__global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_spk_kernel(
+__global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_eu(TT == 1 ? 4 : 2, TT == 1 ? 4 : 2))) void conv_spk_kernel(
     const StepPtrs xs, const StepPtrs residuals, const SpkGeom g, const uint16_t* __restrict__ wpacked,
     const float* __restrict__ bias, const float* __restrict__ v_init, unsigned char* __restrict__ out,
     float* __restrict__ v_out, const LifParams lif) {
     extern __shared__ __align__(16) unsigned char lds[];
+    // ---- every cache line of the kernel arguments is touched once, in one round trip: the compiler loads the arguments
+    // where they are used, all over the prologue, and each of those loads then hits the scalar cache instead of waiting
+    // for memory in turn.
+    {
+        auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+        uint32_t d0, d1, d2, d3, d4, d5, d6, d7, d8, d9, d10;
+        asm volatile(
+            "s_load_dword %0, %11, 0x40\n\ts_load_dword %1, %11, 0x80\n\ts_load_dword %2, %11, 0xc0\n\ts_load_dword %3, %11, 0x100\n\t"
+            "s_load_dword %4, %11, 0x140\n\ts_load_dword %5, %11, 0x180\n\ts_load_dword %6, %11, 0x1c0\n\ts_load_dword %7, %11, 0x200\n\t"
+            "s_load_dword %8, %11, 0x240\n\ts_load_dword %9, %11, 0x280\n\ts_load_dword %10, %11, 0x2c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(d0), "=&s"(d1), "=&s"(d2), "=&s"(d3), "=&s"(d4), "=&s"(d5), "=&s"(d6), "=&s"(d7), "=&s"(d8), "=&s"(d9), "=&s"(d10)
+            : "s"(ka));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr uint32_t ONE = F16 ? 0x3c00u : 0x3f80u;
     constexpr int kResTable = static_cast<int>(sizeof(StepPtrs));
