@@ -144,6 +144,25 @@ int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int64_t x_row_
                     float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * The same operator with a caller-owned workspace, which lets the library split the K dimension of a tile over
+ * several workgroups (partial sums in the workspace, added in the order of their K ranges by the workgroup that
+ * finishes last: results do not depend on scheduling and equal those of snnf_linear_lif up to the order of the fp32
+ * additions). Layers with few output tiles or a long Fin are bound by memory latency without it. The reference has no
+ * counterpart (its Triton kernel, kernels/generated_temporal_linear_lif_kernel.py:138-182, walks K inside one program).
+ *   snnf_linear_lif_workspace_bytes : bytes that let this shape split as far as it pays (0: the shape does not split).
+ *   workspace : NULL (then this is snnf_linear_lif), or `workspace_bytes` of device memory, 256-byte aligned, whose first
+ *               64 KiB were zero before the first call that used it; every call leaves them zero again. A smaller
+ *               workspace than asked for splits less. Calls that share a workspace must not overlap in time.
+ */
+size_t snnf_linear_lif_workspace_bytes(int T, int M, int Fin, int Fout);
+int snnf_linear_lif_ws(const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
+                       const void* weight, const void* bias, int Fout, int w_dtype,
+                       const void* v_init, int v_dtype,
+                       void* spikes, int64_t spike_step_stride, void* v_out,
+                       float v_threshold, float v_reset, float tau,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Dense (groups == 1) convolution + bias (+ residual) + LIF over T steps as an implicit GEMM on the matrix cores.
  * Replaces run_fused_temporal_general[_residual][_autotuned] with kernel keys k1_s1_p0, k3_s1_p1, k3_s2_p1, k5_s1_p2,
  * k7_s2_p3, k11_s4_p2 (kernels/benchmark_conv_lif_temporal_general.py:971-1323, emitter :561-710) as called from

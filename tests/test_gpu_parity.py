@@ -202,10 +202,11 @@ def test_linear_lif_list_out_and_leading_dims_forms_agree(hip_ops):
     assert torch.equal(so, s) and torch.equal(vo, v)
     s4, v4 = S.fused_temporal_linear_lif_state_packed(dx.reshape(T, 3, 4, Fin), dw, db, zero_v(), *LIF, False)
     assert tuple(s4.shape) == (T, 3, 4, Fout) and torch.equal(s4.reshape(T, M, Fout), s) and torch.equal(v4.reshape(M, Fout), v)
-    # window chaining through a full-shape fp32 v_init
+    # window chaining through a full-shape fp32 v_init. One timestep runs on the kernel without staging, which adds the
+    # same products in another order than the staged kernel of the 4-step call: same spikes, membrane to the last bit or two.
     s1, v1 = S.fused_temporal_linear_lif_state_packed(dx[:1], dw, db, zero_v(), *LIF, False)
     s2, v2 = S.fused_temporal_linear_lif_state_packed(dx[1:], dw, db, v1, *LIF, False)
-    assert torch.equal(torch.cat([s1, s2]), s) and torch.equal(v2, v)
+    assert torch.equal(torch.cat([s1, s2]), s) and torch.allclose(v2, v, rtol=0, atol=1e-6)
     _no_fallback(hip_ops, 6)
     assert hip_ops.get_fused_op_call_stats()["temporal_linear_lif_stack_materialized"] == 0
 

@@ -41,6 +41,8 @@ SIGNATURES = {
                                   _f, _f, _f, _vp]),
     "snnf_lif_pool_linear_static": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _f, _f, _f, _vp]),
     "snnf_linear_lif": (_i, [_pp, _i, _i, _i, _i64, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _i64, _vp, _f, _f, _f, _vp]),
+    "snnf_linear_lif_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "snnf_linear_lif_ws": (_i, [_pp, _i, _i, _i, _i64, _i, _vp, _vp, _i, _i, _vp, _i, _vp, _i64, _vp, _f, _f, _f, _vp, _sz, _vp]),
     "snnf_conv_packed_weight_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "snnf_conv_pack_weight": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "snnf_conv_lif": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i64,

@@ -7,6 +7,8 @@
 // moves K slabs of all operand rows through LDS with coalesced loads; the direct one (everything else) loads fragments
 // straight from global memory, its 8 (beyond 8 timesteps, 4) waves splitting K in pairs of K steps with partial sums
 // meeting in LDS.
+#include <algorithm>
+
 #include "snnf_common.h"
 
 namespace snnf {
@@ -74,6 +76,38 @@ __device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, i
             out[j] = pack_bf16x2(lo, hi);
         }
     }
+    return out;
+}
+
+// The same octet in two steps, for loads that stay in flight over other work: the raw 16 (fp32 storage: 32) bytes as
+// loaded, and their conversion to a matrix operand (zero when the octet lies beyond K) at the point of use. Converting
+// where the load is issued would make the wave wait for it there.
+template <typename XT> struct RawOctet { u32x4 lo; };
+template <> struct RawOctet<float> { f32x4 lo, hi; };
+template <typename XT>
+__device__ __forceinline__ RawOctet<XT> load_raw_octet(const XT* __restrict__ src) {
+    RawOctet<XT> r;
+    if constexpr (sizeof(XT) == 2) {
+        r.lo = *reinterpret_cast<const u32x4*>(src);
+    } else {
+        r.lo = *reinterpret_cast<const f32x4*>(src);
+        r.hi = *reinterpret_cast<const f32x4*>(src + 4);
+    }
+    return r;
+}
+template <typename XT>
+__device__ __forceinline__ u32x4 finish_octet(const RawOctet<XT>& r, bool inside) {
+    u32x4 out;
+    if constexpr (sizeof(XT) == 2) {
+        out = r.lo;
+    } else {
+        out[0] = pack_bf16x2(r.lo[0], r.lo[1]);
+        out[1] = pack_bf16x2(r.lo[2], r.lo[3]);
+        out[2] = pack_bf16x2(r.hi[0], r.hi[1]);
+        out[3] = pack_bf16x2(r.hi[2], r.hi[3]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = inside ? out[j] : 0u;
     return out;
 }
 
@@ -213,35 +247,40 @@ int launch_one(const StepPtrs& xs, const LinGeom& g, const void* W, const void* 
 // current one multiplies. The accumulators meet in LDS (aliasing the slab) for the LIF recurrence.
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kStagedWaves = 8;
-constexpr int kSlabK = 128;                       // K elements per slab = 4 matrix K steps (256: +6 % on one workgroup per
-                                                  // CU, -25 % where several fit a CU)
-constexpr int kSlabOctets = kSlabK / 8;           // 16-byte staging items per operand row
-constexpr int kSlabPitch = kSlabK * 2 + 16;       // bytes per operand row in LDS
+constexpr int kSlabK = 128;                       // K elements per slab = 4 matrix K steps (wider slabs measured no faster once
+                                                  // several slabs are in flight; they cost LDS and registers)
 
-template <int TT, int OCF> struct StagedShape {
-    static constexpr int TPW = TT >= 8 ? TT / 8 : 1;            // timesteps per wave
+template <int TT, int OCF, int SLABK> struct StagedShape {
+    static constexpr int TPW = TT >= 8 ? 4 : 2;                 // timesteps per wave: its weight fragments serve all of them (LDS reads per
+                                                                 // matrix instruction fall with the size of a wave's register tile)
     static constexpr int TG = TT / TPW;                          // wave groups along time
     static constexpr int KSPLIT = kStagedWaves / TG;             // waves sharing the K steps of a slab
     static constexpr int ROWS = TT * kTileM + OCF * kTileOC;     // operand rows per slab
-    static constexpr int ITEMS = (ROWS * (kSlabK / 8) + kStagedWaves * 64 - 1) / (kStagedWaves * 64);   // octets per thread
+    static constexpr int PITCH_B = SLABK * 2 + 16;               // bytes per operand row in LDS (the 16-byte reads of 8 consecutive rows fall into distinct banks)
+    static constexpr int ITEMS = (ROWS * (SLABK / 8) + kStagedWaves * 64 - 1) / (kStagedWaves * 64);   // octets per thread
+    static constexpr int RING = ITEMS <= 3 ? 4 : 2;              // slabs in flight per thread (even; ITEMS x 4 registers each, 8 for fp32 storage)
     static constexpr int PITCH = OCF * kTileOC + 4;              // floats per row of an accumulator tile in LDS
-    static constexpr size_t slab_bytes = static_cast<size_t>(ROWS) * kSlabPitch;
+    static constexpr size_t slab_bytes = static_cast<size_t>(ROWS) * PITCH_B;
     static constexpr size_t acc_bytes = static_cast<size_t>(KSPLIT) * TT * kTileM * PITCH * sizeof(float);
     static constexpr size_t lds_bytes = slab_bytes > acc_bytes ? slab_bytes : acc_bytes;
 };
 
-template <typename XT, typename VT, int TT, int OCF, bool DB>
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK>
 __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
                                                                               const XT* __restrict__ bias,
                                                                               const VT* __restrict__ v_init, XT* __restrict__ spikes,
-                                                                              VT* __restrict__ v_out, LifParams lif) {
-    using SH = StagedShape<TT, OCF>;
+                                                                              VT* __restrict__ v_out, LifParams lif,
+                                                                              float* __restrict__ ws_partial, int* __restrict__ ws_count,
+                                                                              int slabs_per_part) {
+    using SH = StagedShape<TT, OCF, SLABK>;
+    constexpr int kSlabOctets = SLABK / 8;            // 16-byte staging items per operand row
+    constexpr int kSlabPitch = SH::PITCH_B;
     constexpr int NT = kStagedWaves * 64;
     constexpr int TILE_OC = OCF * kTileOC;
     constexpr int OUTS = TILE_OC * kTileM;
     extern __shared__ __align__(16) unsigned char staged_lds[];
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int oc0 = blockIdx.x * TILE_OC;
     const int m0 = blockIdx.y * kTileM;
@@ -280,44 +319,71 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
 #pragma unroll
         for (int u = 0; u < SH::TPW; ++u) acc[f][u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // One slab ahead in registers (deeper rings measured slower: the slab loop is bound by LDS traffic and its barriers,
-    // not by the latency of the loads). DB: two slab buffers in LDS, so that a slab costs one barrier instead of two
-    // (writing buffer b for slab s + 1 cannot overtake the reads of slab s - 1, which every wave finished before the
-    // barrier of slab s).
-    u32x4 pre[SH::ITEMS];
-    auto fetch = [&](int slab) __attribute__((always_inline)) {
-        const int k = slab * kSlabK + octet * 8;
+    // RING slabs ahead in registers: a slab's loads have the time of RING - 1 other slabs to arrive, so the loop runs at
+    // the rate of its LDS traffic and barriers instead of one memory latency per slab. Every load is unconditional and
+    // the ring is walked by a fully unrolled inner loop (static register indices; the compiler can then wait for exactly
+    // the oldest slab): the slab count is rounded up to a multiple of RING, and slabs beyond K read zeros (load_octet)
+    // and add nothing. DB: two slab buffers in LDS, so that a slab costs one barrier instead of two (writing buffer b for
+    // slab s + 1 cannot overtake the reads of slab s - 1, which every wave finished before the barrier of slab s).
+    constexpr int RING = SH::RING;
+    RawOctet<XT> pre[RING][SH::ITEMS];
+    bool pre_inside[RING];
+    // K split over workgroups: workgroup z of a tile takes slabs [z * slabs_per_part, ...) (all of them without a split).
+    const int slab0 = static_cast<int>(blockIdx.z) * slabs_per_part;
+    const int kend = min(g.Fin, (slab0 + slabs_per_part) * SLABK);      // this part's K range ends here: beyond it, zeros
+    const int rounds = (slabs_per_part + RING - 1) / RING;
+    auto fetch = [&](int slab, int r) __attribute__((always_inline)) {
+        const int k = slab * SLABK + octet * 8;
+        pre_inside[r] = k < kend;
+        const int ks = pre_inside[r] ? k : 0;
 #pragma unroll
-        for (int j = 0; j < SH::ITEMS; ++j)
-            if (item_live[j]) pre[j] = load_octet<XT, true>(item_row[j], k, g.Fin);
+        for (int j = 0; j < SH::ITEMS; ++j) pre[r][j] = load_raw_octet<XT>(item_row[j] + ks);   // items beyond the rows re-read row 0
     };
-    const int nslabs = (g.Fin + kSlabK - 1) / kSlabK;
     // Fragment addresses in the slab: lane = 16 q + r reads K elements 8 q .. 8 q + 7 of row r of its fragment.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 15) * kSlabPitch + (lane >> 4) * 16);
-    fetch(0);
-    for (int slab = 0; slab < nslabs; ++slab) {
-        unsigned char* buf = staged_lds + (DB ? (slab & 1) * SH::slab_bytes : 0);
 #pragma unroll
-        for (int j = 0; j < SH::ITEMS; ++j)
-            if (item_live[j]) *reinterpret_cast<u32x4*>(buf + item_dst[j]) = pre[j];
-        __syncthreads();
-        if (slab + 1 < nslabs) fetch(slab + 1);
+    for (int r = 0; r < RING; ++r) {
+        fetch(slab0 + r, r);
+        __builtin_amdgcn_sched_barrier(0);      // oldest slab first, as in the loop: its wait then leaves the others in flight
+    }
+    for (int round = 0; round < rounds; ++round) {
 #pragma unroll
-        for (int ks = 0; ks < kSlabK / 32; ++ks) {
-            if (ks % SH::KSPLIT != kp % SH::KSPLIT) continue;      // wave-uniform
-            u32x4 a[OCF];
+        for (int r = 0; r < RING; ++r) {
+            const int slab = slab0 + round * RING + r;
+            unsigned char* buf = staged_lds + (DB ? (r & 1) * SH::slab_bytes : 0);      // RING is even
 #pragma unroll
-            for (int f = 0; f < OCF; ++f)
-                a[f] = *reinterpret_cast<const u32x4*>(buf + (TT * kTileM + f * kTileOC) * kSlabPitch + frag_off + ks * 64);
+            for (int j = 0; j < SH::ITEMS; ++j)
+                if (item_live[j]) *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r]);
+            __syncthreads();
+            fetch(slab + RING, r);
+            // This wave's K steps of the slab (every KSPLIT-th), four at a time: their operand reads go out together.
+            constexpr int OWN = SLABK / 32 / SH::KSPLIT;
+            const unsigned char* own = buf + frag_off + (kp % SH::KSPLIT) * 64;
 #pragma unroll
-            for (int u = 0; u < SH::TPW; ++u) {
-                const int t = tg * SH::TPW + u;
-                const u32x4 b = *reinterpret_cast<const u32x4*>(buf + t * kTileM * kSlabPitch + frag_off + ks * 64);
+            for (int i0 = 0; i0 < OWN; i0 += 4) {
+                u32x4 a[4][OCF], b[4][SH::TPW];
 #pragma unroll
-                for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[f], b, acc[f][u]);
+                for (int i = 0; i < 4; ++i) {
+                    if (i0 + i < OWN) {
+                        const int off = (i0 + i) * SH::KSPLIT * 64;
+#pragma unroll
+                        for (int f = 0; f < OCF; ++f) a[i][f] = *reinterpret_cast<const u32x4*>(own + (TT * kTileM + f * kTileOC) * kSlabPitch + off);
+#pragma unroll
+                        for (int u = 0; u < SH::TPW; ++u) b[i][u] = *reinterpret_cast<const u32x4*>(own + (tg * SH::TPW + u) * kTileM * kSlabPitch + off);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (i0 + i < OWN) {
+#pragma unroll
+                        for (int u = 0; u < SH::TPW; ++u)
+#pragma unroll
+                            for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[i][f], b[i][u], acc[f][u]);
+                    }
+                }
             }
+            if (!DB) __syncthreads();
         }
-        if (!DB) __syncthreads();
     }
     if (DB) __syncthreads();
 
@@ -333,6 +399,38 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
                 partial[(kp * TT + tg * SH::TPW + u) * SLAB_F + (lane & 15) * SH::PITCH + f * kTileOC + (lane >> 4) * 4 + r] = acc[f][u][r];
     __syncthreads();
 
+    // K split over workgroups: every workgroup of a tile leaves its sums in the workspace and counts itself in; the one
+    // that arrives last adds all parts in the order of their K ranges (so the result does not depend on who was last)
+    // and runs the recurrence. It leaves the counter at zero for the next launch. The sums and the counter travel as
+    // device-scope atomic stores, loads and adds (relaxed): those go through to memory, past the L2 caches of the chip's
+    // partitions, which do not see each other's lines. A device-scope fence would do too, but it writes back a whole L2
+    // per wave that executes it and costs more than the kernel. Order: a workgroup barrier waits for each thread's stores
+    // to be acknowledged before one thread counts the workgroup in.
+    const int parts = static_cast<int>(gridDim.z);
+    const int tile = static_cast<int>(blockIdx.y * gridDim.x + blockIdx.x);
+    if (parts > 1) {
+        __shared__ int arrived_last;
+        float* __restrict__ mine = ws_partial + (static_cast<int64_t>(tile) * parts + blockIdx.z) * (TT * OUTS);
+        for (int e = tid; e < OUTS; e += NT) {
+            const int slot = (e / TILE_OC) * SH::PITCH + e % TILE_OC;
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+                __hip_atomic_store(mine + t * OUTS + e, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const int before = __hip_atomic_fetch_add(ws_count + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            arrived_last = before == parts - 1 ? 1 : 0;
+            if (arrived_last) __hip_atomic_store(ws_count + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!arrived_last) return;
+    }
+
     for (int e = tid; e < OUTS; e += NT) {
         const int slot = (e / TILE_OC) * SH::PITCH + e % TILE_OC;
         const int m = m0 + e / TILE_OC;
@@ -341,12 +439,17 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         const float bv = bias != nullptr ? to_float(bias[oc]) : 0.0f;
         const int64_t o = static_cast<int64_t>(m) * g.Fout + oc;
         float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
+        const float* __restrict__ all = ws_partial + static_cast<int64_t>(tile) * parts * (TT * OUTS) + e;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
             if (t >= g.T) break;
             float sum = 0.0f;
+            if (parts > 1) {
+                for (int z = 0; z < parts; ++z) sum += __hip_atomic_load(all + (static_cast<int64_t>(z) * TT + t) * OUTS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
 #pragma unroll
-            for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+                for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+            }
             const float cur = sum + bv;
             spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
         }
@@ -354,13 +457,20 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     }
 }
 
-template <typename XT, typename VT, int TT, int OCF, bool DB>
-int launch_staged_db(dim3 grid, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
-                     void* v_out, const LifParams& lif, hipStream_t stream) {
-    using SH = StagedShape<TT, OCF>;
+// Workspace of the split: one counter per tile (zero between launches), then [tile][part][t][16 x TILE_OC] sums.
+struct LinWorkspace {
+    void* base;
+    size_t bytes;
+};
+constexpr size_t kLinCounterBytes = 64 * 1024;     // 16384 tiles
+
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK>
+int launch_staged_db(dim3 grid, int slabs_per_part, const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias,
+                     const void* v_init, void* spikes, void* v_out, const LifParams& lif, hipStream_t stream) {
+    using SH = StagedShape<TT, OCF, SLABK>;
     constexpr size_t lds = DB ? 2 * SH::slab_bytes : SH::lds_bytes;
     static_assert(lds <= 160 * 1024 && SH::acc_bytes <= lds, "slabs exceed LDS");
-    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB>;
+    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB, SLABK>;
     if (lds > 64 * 1024) {
         static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -368,27 +478,46 @@ int launch_staged_db(dim3 grid, const StepPtrs& xs, const LinGeom& g, const void
     }
     kernel<<<grid, kStagedWaves * 64, lds, stream>>>(xs, g, static_cast<const XT*>(W), static_cast<const XT*>(bias),
                                                      static_cast<const VT*>(v_init), static_cast<XT*>(spikes),
-                                                     static_cast<VT*>(v_out), lif);
+                                                     static_cast<VT*>(v_out), lif,
+                                                     reinterpret_cast<float*>(static_cast<char*>(ws.base) + kLinCounterBytes),
+                                                     static_cast<int*>(ws.base), slabs_per_part);
     return check_launch("snnf_linear_lif");
 }
 
+// Parts the K dimension of a tile is split into: two, for a layer with a long K whose tiles leave half of the compute
+// units idle (the classifier layers at small batch), when the workspace takes it. Splitting costs three trips to memory
+// at the end of a tile; measured, it pays from K = 4096 on (4096 -> 4096 at 16 rows: 16.5 -> 13.9 us, 25088 -> 4096:
+// 75 -> 47 us) and more than two parts gain nothing.
+inline int linear_split_parts(int64_t tiles, int unit_slabs, size_t part_bytes, size_t ws_bytes) {
+    if (tiles > static_cast<int64_t>(kLinCounterBytes / sizeof(int)) || tiles * 2 > compute_units() || unit_slabs < 32) return 1;
+    if (ws_bytes < kLinCounterBytes + 2 * part_bytes * static_cast<size_t>(tiles)) return 1;
+    return 2;
+}
+
 template <typename XT, typename VT, int TT, int OCF>
-int launch_staged(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
                   void* v_out, const LifParams& lif, hipStream_t stream) {
-    using SH = StagedShape<TT, OCF>;
-    const dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
+    dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
     if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
+    const int unit_slabs = (g.Fin + kSlabK - 1) / kSlabK;
+    const int64_t tiles = static_cast<int64_t>(grid.x) * grid.y;
+    const size_t part_bytes = static_cast<size_t>(TT) * OCF * kTileOC * kTileM * sizeof(float);
+    int parts = ws.base != nullptr ? linear_split_parts(tiles, unit_slabs, part_bytes, ws.bytes) : 1;
+    const int unit_slabs_per_part = (unit_slabs + parts - 1) / parts;
+    using SH = StagedShape<TT, OCF, kSlabK>;
+    parts = (unit_slabs + unit_slabs_per_part - 1) / unit_slabs_per_part;      // no empty part
+    grid.z = parts;
     // Two slab buffers where a CU gets one workgroup anyway (they would cost occupancy otherwise) and both fit LDS.
     constexpr bool can_double = 2 * SH::slab_bytes <= 160 * 1024;
     if constexpr (can_double) {
-        if (static_cast<int64_t>(grid.x) * grid.y <= compute_units())
-            return launch_staged_db<XT, VT, TT, OCF, true>(grid, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+        if (tiles * parts <= compute_units())
+            return launch_staged_db<XT, VT, TT, OCF, true, kSlabK>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     }
-    return launch_staged_db<XT, VT, TT, OCF, false>(grid, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_staged_db<XT, VT, TT, OCF, false, kSlabK>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 template <typename XT, typename VT, bool FAST>
-int launch_tt(const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+int launch_tt(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
               void* v_out, const LifParams& lif, hipStream_t stream) {
     // Two feature fragments per workgroup (half the activation traffic) when that still leaves at least 128 workgroups.
     const bool wide = g.Fout % (2 * kTileOC) == 0 &&
@@ -396,13 +525,13 @@ int launch_tt(const StepPtrs& xs, const LinGeom& g, const void* W, const void* b
     if constexpr (FAST) {
         if (g.T > 2) {
             if (wide) {
-                if (g.T <= 4) return launch_staged<XT, VT, 4, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-                if (g.T <= 8) return launch_staged<XT, VT, 8, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-                return launch_staged<XT, VT, 16, 2>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                if (g.T <= 4) return launch_staged<XT, VT, 4, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                if (g.T <= 8) return launch_staged<XT, VT, 8, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                return launch_staged<XT, VT, 16, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
             }
-            if (g.T <= 4) return launch_staged<XT, VT, 4, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-            if (g.T <= 8) return launch_staged<XT, VT, 8, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-            return launch_staged<XT, VT, 16, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            if (g.T <= 4) return launch_staged<XT, VT, 4, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            if (g.T <= 8) return launch_staged<XT, VT, 8, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            return launch_staged<XT, VT, 16, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
         }
     }
     if (g.T <= 1) return launch_one<XT, VT, 1, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
@@ -413,20 +542,61 @@ int launch_tt(const StepPtrs& xs, const LinGeom& g, const void* W, const void* b
 }
 
 template <typename XT, typename VT>
-int launch(bool fast, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init,
+int launch(bool fast, const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init,
            void* spikes, void* v_out, const LifParams& lif, hipStream_t stream) {
-    return fast ? launch_tt<XT, VT, true>(xs, g, W, bias, v_init, spikes, v_out, lif, stream)
-                : launch_tt<XT, VT, false>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return fast ? launch_tt<XT, VT, true>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream)
+                : launch_tt<XT, VT, false>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 }  // namespace
 }  // namespace snnf
 
+extern "C" size_t snnf_linear_lif_workspace_bytes(int T, int M, int Fin, int Fout) {
+    using namespace snnf;
+    if (T < 3 || M < 1 || Fin < 1 || Fout < 1) return 0;      // one or two timesteps run on the kernel without staging
+    int tt = 4;
+    while (tt < T && tt < SNNF_MAX_T_PER_LAUNCH) tt *= 2;
+    const int64_t m_tiles = (M + kTileM - 1) / kTileM;
+    const int64_t tiles = ((Fout + kTileOC - 1) / kTileOC) * m_tiles;          // the narrow tiling has the most tiles
+    const int all_slabs = (Fin + kSlabK - 1) / kSlabK;
+    if (tiles > compute_units() || all_slabs < 32 || tiles > static_cast<int64_t>(kLinCounterBytes / sizeof(int))) return 0;
+    const int64_t parts = 2;
+    // Sums of one part of one tile: TT x 16 rows x 16 features x 4 bytes for the narrow tiling, twice that for half as many wide tiles.
+    const size_t sums = static_cast<size_t>(tiles) * parts * tt * kTileM * kTileOC * sizeof(float);
+    return kLinCounterBytes + sums;
+}
+
+static int linear_lif_impl(const char* who, const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
+                           const void* weight, const void* bias, int Fout, int w_dtype, const void* v_init,
+                           int v_dtype, void* spikes, int64_t spike_step_stride, void* v_out, float v_threshold,
+                           float v_reset, float tau, void* workspace, size_t workspace_bytes, void* stream);
+
 extern "C" int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
                                const void* weight, const void* bias, int Fout, int w_dtype, const void* v_init,
                                int v_dtype, void* spikes, int64_t spike_step_stride, void* v_out, float v_threshold,
                                float v_reset, float tau, void* stream) {
+    return linear_lif_impl("snnf_linear_lif", xs, T, M, Fin, x_row_stride, x_dtype, weight, bias, Fout, w_dtype, v_init, v_dtype, spikes,
+                           spike_step_stride, v_out, v_threshold, v_reset, tau, nullptr, 0, stream);
+}
+
+extern "C" int snnf_linear_lif_ws(const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
+                                  const void* weight, const void* bias, int Fout, int w_dtype, const void* v_init,
+                                  int v_dtype, void* spikes, int64_t spike_step_stride, void* v_out, float v_threshold,
+                                  float v_reset, float tau, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace snnf;
+    if (workspace != nullptr && !aligned_to(workspace, 256))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_ws: workspace must be 256-byte aligned");
+    return linear_lif_impl("snnf_linear_lif_ws", xs, T, M, Fin, x_row_stride, x_dtype, weight, bias, Fout, w_dtype, v_init, v_dtype, spikes,
+                           spike_step_stride, v_out, v_threshold, v_reset, tau, workspace, workspace != nullptr ? workspace_bytes : 0, stream);
+}
+
+static int linear_lif_impl(const char* who, const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
+                           const void* weight, const void* bias, int Fout, int w_dtype, const void* v_init,
+                           int v_dtype, void* spikes, int64_t spike_step_stride, void* v_out, float v_threshold,
+                           float v_reset, float tau, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace snnf;
+    (void)who;
+    const LinWorkspace ws = {workspace, workspace_bytes};
     if (xs == nullptr || weight == nullptr || spikes == nullptr || v_out == nullptr)
         return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif: xs, weight, spikes and v_out must be non-null");
     if (T < 1 || M < 1 || Fin < 1 || Fout < 1 || x_row_stride < Fin)
@@ -468,13 +638,13 @@ extern "C" int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int
         const void* vi = t0 == 0 ? v_init : v_out;
         void* sp = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
         int rc;
-        if (x_dtype == SNNF_F32) rc = launch<float, float>(fast, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
+        if (x_dtype == SNNF_F32) rc = launch<float, float>(fast, ws, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
         else if (x_dtype == SNNF_BF16)
-            rc = v_dtype == SNNF_F32 ? launch<bf16_t, float>(fast, ptrs, g, weight, bias, vi, sp, v_out, lif, hs)
-                                     : launch<bf16_t, bf16_t>(fast, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
+            rc = v_dtype == SNNF_F32 ? launch<bf16_t, float>(fast, ws, ptrs, g, weight, bias, vi, sp, v_out, lif, hs)
+                                     : launch<bf16_t, bf16_t>(fast, ws, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
         else
-            rc = v_dtype == SNNF_F32 ? launch<f16_t, float>(fast, ptrs, g, weight, bias, vi, sp, v_out, lif, hs)
-                                     : launch<f16_t, f16_t>(fast, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
+            rc = v_dtype == SNNF_F32 ? launch<f16_t, float>(fast, ws, ptrs, g, weight, bias, vi, sp, v_out, lif, hs)
+                                     : launch<f16_t, f16_t>(fast, ws, ptrs, g, weight, bias, vi, sp, v_out, lif, hs);
         if (rc != SNNF_OK) return rc;
     }
     return SNNF_OK;

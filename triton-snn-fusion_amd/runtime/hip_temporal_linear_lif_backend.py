@@ -133,10 +133,12 @@ def _run_steps(steps: List[torch.Tensor], weight, bias, v_init, v_threshold, v_r
         if not spike_out.is_contiguous() or not v_out.is_contiguous():
             raise RuntimeError("spike_out and v_out must be contiguous")
         spikes, v_next = spike_out, v_out
-    _lib.check("snnf_linear_lif", lib.snnf_linear_lif(
+    workspace = _split_workspace(lib, first.device, T, M, Fin, Fout)
+    _lib.check("snnf_linear_lif_ws", lib.snnf_linear_lif_ws(
         _lib.step_pointers(fixed), T, M, Fin, row_stride, _lib.dtype_code(first.dtype), w.data_ptr(), _lib.ptr(b), Fout,
         _lib.dtype_code(w.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype), spikes.data_ptr(), M * Fout,
-        v_next.data_ptr(), float(v_threshold), float(v_reset), float(tau), _lib.current_stream(first.device)))
+        v_next.data_ptr(), float(v_threshold), float(v_reset), float(tau), _lib.ptr(workspace),
+        0 if workspace is None else workspace.numel(), _lib.current_stream(first.device)))
     diagnostics = {
         "kernel_kind": "temporal_linear_lif",
         "compute_dtype": "float16" if first.dtype == torch.float16 else "float32",
@@ -155,6 +157,30 @@ def _run_steps(steps: List[torch.Tensor], weight, bias, v_init, v_threshold, v_r
     return TritonTemporalLinearLIFResult(spikes=spikes, v_next=v_next, used_triton=True,
                                          kernel_key="temporal_linear_lif", kernel_temporal_config=diagnostics,
                                          kernel_diagnostics=diagnostics)
+
+
+# Workspaces that let the kernel split K over workgroups: one per (device, stream), zeroed when allocated (the kernel
+# leaves its counters zero). A call under stream capture cannot allocate, and its stream exists only for the capture, so
+# captured calls share one workspace per device that the eager calls before the capture (the warm-up every capture
+# needs anyway) have prepared; without one they run unsplit. Graphs that share it must not replay concurrently.
+_WORKSPACES: Dict = {}
+
+
+def _split_workspace(lib, device, T: int, M: int, Fin: int, Fout: int):
+    need = int(lib.snnf_linear_lif_workspace_bytes(T, M, Fin, Fout))
+    if need == 0:
+        return None
+    capturing = torch.cuda.is_current_stream_capturing()
+    graph_key = (device.index, "captured")
+    key = graph_key if capturing else (device.index, int(torch.cuda.current_stream(device).cuda_stream))
+    keys = (key,) if capturing else (key, graph_key)
+    for k in keys:
+        have = _WORKSPACES.get(k)
+        if have is None or have.numel() < need:
+            if capturing:
+                return None
+            _WORKSPACES[k] = torch.zeros(need, dtype=torch.uint8, device=device)
+    return _WORKSPACES[key]
 
 
 def _run_packed(x_seq, weight, bias, v_init, v_threshold, v_reset, tau, detach_reset, strict, verbose,
