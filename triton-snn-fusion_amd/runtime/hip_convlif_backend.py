@@ -248,7 +248,23 @@ def last_conv_plan() -> Dict:
     return plan
 
 
-def _planned_temporal_config(kernel_key: str, residual_add: bool, T: int) -> Dict:
+# The temporal configuration of a launch depends only on the layer (shapes, dtypes, window); the planner's answer is read
+# back and parsed once per distinct layer.
+_TEMPORAL_CONFIGS: Dict[tuple, Dict] = {}
+
+
+def _planned_temporal_config(kernel_key: str, residual_add: bool, T: int, memo: Optional[tuple] = None) -> Dict:
+    if memo is not None:
+        known = _TEMPORAL_CONFIGS.get(memo)
+        if known is not None:
+            return dict(known)
+    config = _read_planned_temporal_config(kernel_key, residual_add, T)
+    if memo is not None and len(_TEMPORAL_CONFIGS) < 4096:
+        _TEMPORAL_CONFIGS[memo] = dict(config)
+    return config
+
+
+def _read_planned_temporal_config(kernel_key: str, residual_add: bool, T: int) -> Dict:
     config = get_autotune_best_config(kernel_key, residual_add=residual_add, T=T)
     if kernel_key.startswith("depthwise_"):
         return config
@@ -446,7 +462,10 @@ def _run_temporal(kind: str, xs, residuals, weight, bias, v_init, stride, paddin
         diagnostics["kernel_kind"] = "temporal_residual"
     return TritonConvLIFResult(
         spikes, v_next, True, kernel_key=kernel_key,
-        kernel_temporal_config=_planned_temporal_config(kernel_key, residuals is not None, T),
+        kernel_temporal_config=_planned_temporal_config(
+            kernel_key, residuals is not None, T,
+            (kernel_key, residuals is not None, T, first.shape, weight.shape, tuple(_as_pair(stride)), tuple(_as_pair(padding)),
+             first.dtype, v_dtype, isinstance(v_init, torch.Tensor) and v_init.dim() > 0)),
         kernel_diagnostics=diagnostics,
     )
 

@@ -180,6 +180,18 @@ def _as_pair(value) -> Tuple[int, int]:
     return int(value[0]), int(value[1])
 
 
+class _Lazy:
+    """A description that is only formatted if somebody prints it (verbose mode, fallback reports): building the string
+    on every operator call costs more host time than the rest of the dispatch."""
+    __slots__ = ("fn", "args", "kwargs")
+
+    def __init__(self, fn, *args, **kwargs):
+        self.fn, self.args, self.kwargs = fn, args, kwargs
+
+    def __str__(self) -> str:
+        return self.fn(*self.args, **self.kwargs)
+
+
 def _shape_tuple(x):
     return tuple(x.shape) if isinstance(x, torch.Tensor) else None
 
@@ -194,10 +206,30 @@ def _conv_shape_desc(x, weight, bias, v, stride, padding, dilation, groups, temp
     )
 
 
+_SIGNATURE_KEYS: Dict[tuple, str] = {}
+
+
 def _conv_signature_key(x, weight, stride, padding, dilation, groups) -> str:
-    """Same key format as runtime/snn_custom_ops.py:275-297 (summaries of reference drivers parse it)."""
+    """Same key format as runtime/snn_custom_ops.py:275-297 (summaries of reference drivers parse it). Formatted once per
+    distinct layer."""
     if not isinstance(weight, torch.Tensor) or weight.dim() != 4:
         return "unknown_conv_signature"
+    try:
+        memo = (x.shape[1] if isinstance(x, torch.Tensor) and x.dim() >= 2 else None, weight.shape,
+                stride if isinstance(stride, int) else tuple(stride), padding if isinstance(padding, int) else tuple(padding),
+                dilation if isinstance(dilation, int) else tuple(dilation), groups)
+        known = _SIGNATURE_KEYS.get(memo)
+    except TypeError:
+        memo, known = None, None
+    if known is not None:
+        return known
+    key = _format_conv_signature_key(x, weight, stride, padding, dilation, groups)
+    if memo is not None and len(_SIGNATURE_KEYS) < 4096:
+        _SIGNATURE_KEYS[memo] = key
+    return key
+
+
+def _format_conv_signature_key(x, weight, stride, padding, dilation, groups) -> str:
     s, p, d = _as_pair(stride), _as_pair(padding), _as_pair(dilation)
     oc, wic, kh, kw = (int(v) for v in weight.shape)
     groups = int(groups)
@@ -258,9 +290,15 @@ def _dispatch_reason(what: str) -> str:
     return "backend is not triton" if _CONFIG.backend not in NATIVE_BACKENDS else what
 
 
+_LIBRARY_SEEN = False
+
+
 def _require_library() -> None:
-    if not _lib.library_available():
-        _lib.lib()  # raises with the build instruction
+    global _LIBRARY_SEEN
+    if not _LIBRARY_SEEN:
+        if not _lib.library_available():
+            _lib.lib()  # raises with the build instruction
+        _LIBRARY_SEEN = True
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -557,7 +595,7 @@ def _lif_forward_state_impl(x, v_prev, v_threshold, v_reset, tau, detach_reset):
 
 def _fused_conv_lif_state_impl(x, weight, bias, v_prev, stride, padding, dilation, groups, v_threshold, v_reset, tau,
                                detach_reset):
-    desc = _conv_shape_desc(x, weight, bias, v_prev, stride, padding, dilation, groups)
+    desc = _Lazy(_conv_shape_desc, x, weight, bias, v_prev, stride, padding, dilation, groups)
     args = (x, weight, bias, v_prev, stride, padding, dilation, groups, v_threshold, v_reset, tau, detach_reset)
 
     def hit(result):
@@ -578,7 +616,7 @@ def _temporal_conv_impl(op_name: str, runner, stats_kind: str):
 
     def impl(xs, weight, bias, v_init, stride, padding, dilation, groups, v_threshold, v_reset, tau, detach_reset):
         first = xs[0] if len(xs) > 0 else None
-        desc = _conv_shape_desc(first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=len(xs))
+        desc = _Lazy(_conv_shape_desc, first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=len(xs))
         signature = _conv_signature_key(first, weight, stride, padding, dilation, groups)
         args = (xs, weight, bias, v_init, stride, padding, dilation, groups, v_threshold, v_reset, tau, detach_reset)
 
@@ -617,7 +655,7 @@ def _fused_temporal_conv_lif_state_packed_out_impl(x_seq, weight, bias, v_init, 
                                                    v_threshold, v_reset, tau, detach_reset, spike_out, v_out):
     first = x_seq[0] if isinstance(x_seq, torch.Tensor) and x_seq.dim() == 5 else None
     T = int(x_seq.shape[0]) if isinstance(x_seq, torch.Tensor) and x_seq.dim() > 0 else None
-    desc = _conv_shape_desc(first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=T)
+    desc = _Lazy(_conv_shape_desc, first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=T)
     signature = _conv_signature_key(first, weight, stride, padding, dilation, groups)
     args = (x_seq, weight, bias, v_init, stride, padding, dilation, groups, v_threshold, v_reset, tau, detach_reset,
             spike_out, v_out)
@@ -654,7 +692,7 @@ def _temporal_conv_add_impl(require_depthwise: bool):
     def impl(xs, residuals, weight, bias, v_init, stride, padding, dilation, groups, v_threshold, v_reset, tau,
              detach_reset):
         first = xs[0] if len(xs) > 0 else None
-        desc = _conv_shape_desc(first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=len(xs))
+        desc = _Lazy(_conv_shape_desc, first, weight, bias, v_init, stride, padding, dilation, groups, temporal_len=len(xs))
         signature = _conv_signature_key(first, weight, stride, padding, dilation, groups)
         args = (xs, residuals, weight, bias, v_init, stride, padding, dilation, groups, v_threshold, v_reset, tau,
                 detach_reset)
@@ -700,7 +738,7 @@ def _lif_shape_desc(x_seq, v_init) -> str:
 
 
 def _fused_temporal_lif_state_impl(x_seq, v_init, v_threshold, v_reset, tau, detach_reset):
-    desc = _lif_shape_desc(x_seq, v_init)
+    desc = _Lazy(_lif_shape_desc, x_seq, v_init)
     args = (x_seq, v_init, v_threshold, v_reset, tau, detach_reset)
 
     def hit(result):
@@ -719,7 +757,7 @@ def _fused_temporal_lif_state_impl(x_seq, v_init, v_threshold, v_reset, tau, det
 
 
 def _fused_temporal_lif_avgpool_linear_impl(x_seq, v_init, fc_weight, fc_bias, v_threshold, v_reset, tau, detach_reset):
-    desc = _lif_shape_desc(x_seq, v_init)
+    desc = _Lazy(_lif_shape_desc, x_seq, v_init)
     args = (x_seq, v_init, fc_weight, fc_bias, v_threshold, v_reset, tau, detach_reset)
     out, native = _run(x_seq, ("temporal", "temporal_lif_avgpool_linear", "temporal_lif_tail"),
                        "temporal_lif_avgpool_linear", desc,
@@ -756,7 +794,7 @@ def _fused_temporal_linear_lif_state_impl(xs, weight, bias, v_init, v_threshold,
     first = xs[0] if isinstance(xs, torch.Tensor) or (isinstance(xs, (tuple, list)) and len(xs) > 0) else None
     args = (xs, weight, bias, v_init, v_threshold, v_reset, tau, detach_reset)
     out, native = _run(first, ("temporal", "temporal_linear_lif"), "temporal_linear_lif",
-                       _linear_shape_desc(xs, weight, bias, v_init),
+                       _Lazy(_linear_shape_desc, xs, weight, bias, v_init),
                        lambda: run_triton_fused_temporal_linear_lif_state(*args, strict=_CONFIG.strict_triton,
                                                                           verbose=_CONFIG.verbose),
                        lambda: fused_temporal_linear_lif_state_torch(*args),
@@ -768,7 +806,7 @@ def _fused_temporal_linear_lif_state_impl(xs, weight, bias, v_init, v_threshold,
 def _fused_temporal_linear_lif_state_packed_impl(x_seq, weight, bias, v_init, v_threshold, v_reset, tau, detach_reset):
     args = (x_seq, weight, bias, v_init, v_threshold, v_reset, tau, detach_reset)
     out, native = _run(x_seq, ("temporal", "temporal_linear_lif", "temporal_linear_lif_packed"),
-                       "temporal_linear_lif_packed", _linear_shape_desc(x_seq, weight, bias, v_init),
+                       "temporal_linear_lif_packed", _Lazy(_linear_shape_desc, x_seq, weight, bias, v_init),
                        lambda: run_triton_fused_temporal_linear_lif_state_packed(*args, strict=_CONFIG.strict_triton,
                                                                                  verbose=_CONFIG.verbose),
                        lambda: fused_temporal_linear_lif_state_packed_torch(*args),
@@ -781,7 +819,7 @@ def _fused_temporal_linear_lif_state_packed_out_impl(x_seq, weight, bias, v_init
                                                      detach_reset, spike_out, v_out):
     args = (x_seq, weight, bias, v_init, v_threshold, v_reset, tau, detach_reset, spike_out, v_out)
     _run(x_seq, ("temporal", "temporal_linear_lif", "temporal_linear_lif_packed"), "temporal_linear_lif_packed_out",
-         _linear_shape_desc(x_seq, weight, bias, v_init),
+         _Lazy(_linear_shape_desc, x_seq, weight, bias, v_init),
          lambda: run_triton_fused_temporal_linear_lif_state_packed_out(*args, strict=_CONFIG.strict_triton,
                                                                        verbose=_CONFIG.verbose,
                                                                        use_autotune=_CONFIG.use_triton_autotune),
