@@ -217,25 +217,6 @@ def _roofline(bound: str, work: float, ms: float, traffic=None):
             "frac": round(achieved / peak, 4), "traffic": traffic}
 
 
-# (name, Cin, Cout, input size, kernel, stride, padding, residual added before the LIF, one analog frame for all T, count)
-RESNET18_LAYERS = [
-    ("stem 7x7/2 3->64", 3, 64, 224, 7, 2, 3, False, True, 1),
-    ("3x3 64->64 @56", 64, 64, 56, 3, 1, 1, False, False, 2), ("3x3 64->64 @56 +res", 64, 64, 56, 3, 1, 1, True, False, 2),
-    ("3x3/2 64->128 @56", 64, 128, 56, 3, 2, 1, False, False, 1), ("1x1/2 64->128 @56", 64, 128, 56, 1, 2, 0, False, False, 1),
-    ("3x3 128->128 @28", 128, 128, 28, 3, 1, 1, False, False, 1), ("3x3 128->128 @28 +res", 128, 128, 28, 3, 1, 1, True, False, 2),
-    ("3x3/2 128->256 @28", 128, 256, 28, 3, 2, 1, False, False, 1), ("1x1/2 128->256 @28", 128, 256, 28, 1, 2, 0, False, False, 1),
-    ("3x3 256->256 @14", 256, 256, 14, 3, 1, 1, False, False, 1), ("3x3 256->256 @14 +res", 256, 256, 14, 3, 1, 1, True, False, 2),
-    ("3x3/2 256->512 @14", 256, 512, 14, 3, 2, 1, False, False, 1), ("1x1/2 256->512 @14", 256, 512, 14, 1, 2, 0, False, False, 1),
-    ("3x3 512->512 @7", 512, 512, 7, 3, 1, 1, False, False, 1), ("3x3 512->512 @7 +res", 512, 512, 7, 3, 1, 1, True, False, 2),
-]
-VGG11_LAYERS = [
-    ("3x3 3->64 @32", 3, 64, 32, 3, 1, 1, False, True, 1), ("3x3 64->128 @16", 64, 128, 16, 3, 1, 1, False, False, 1),
-    ("3x3 128->256 @8", 128, 256, 8, 3, 1, 1, False, False, 1), ("3x3 256->256 @8", 256, 256, 8, 3, 1, 1, False, False, 1),
-    ("3x3 256->512 @4", 256, 512, 4, 3, 1, 1, False, False, 1), ("3x3 512->512 @4", 512, 512, 4, 3, 1, 1, False, False, 1),
-    ("3x3 512->512 @2", 512, 512, 2, 3, 1, 1, False, False, 2),
-]
-
-
 def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, internal: bool = False):
     """Times every fused conv(+residual)+LIF layer shape of a network configuration on its own (graph replay, HIP events).
     `internal`: the layer as it runs inside the network executor, spikes bit-packed on both sides (an analog frame
@@ -244,7 +225,7 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
     from triton_snn_fusion_amd import workloads as W
     from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
     ops = torch.ops.snn_custom
-    layers, batch = (RESNET18_LAYERS, 16) if which == "resnet18" else (VGG11_LAYERS, 64)
+    layers, batch = (W.RESNET18_LAYERS, W.RESNET18_BATCH) if which == "resnet18" else (W.VGG11_LAYERS, W.VGG11_BATCH)
     T, dev = 4, torch.device("cuda:0")
     esize = torch.empty((), dtype=dtype).element_size()
     g = torch.Generator(device="cpu")
@@ -411,8 +392,8 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
         best = min(best, ms_ig)
     except Exception as exc:  # pragma: no cover - reported, the dense executor's numbers stand
         out.setdefault("internal_layouts", {})["error"] = str(exc)[:300]
-    layers = RESNET18_LAYERS if name == "resnet18" else VGG11_LAYERS
     from triton_snn_fusion_amd import workloads as W
+    layers = W.RESNET18_LAYERS if name == "resnet18" else W.VGG11_LAYERS
     conv_flops = 0
     for _n, cin, cout, size, k, stride, pad, _res, _analog, count in layers:
         o = (size + 2 * pad - k) // stride + 1

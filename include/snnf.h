@@ -255,6 +255,18 @@ int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const
                           const void* v_init, void* out, int out_layout, int64_t out_step_stride, void* v_out,
                           int neuron, float v_threshold, float v_reset, float tau, void* stream);
 
+/*
+ * Registers a measured launch choice for snnf_conv_lif_blocked on one layer shape (the counterpart of the per-kernel-key
+ * "best config" the reference's autotuner keeps, kernels/benchmark_conv_lif_temporal_general.py:524-558,1332-1369):
+ * columns of a wave's output patch (rows follow: 32 / columns), channel groups of 8 per LDS stage (a power of two) and
+ * waves of a workgroup that share a tile's K (1, 2, 4 or 8). 0 leaves a choice to the built-in planner; all three 0
+ * removes the entry. `shared_frame`: the layer receives one analog frame for all timesteps. A choice that the kernel
+ * cannot run on the shape (a stage that does not fit a wave's LDS region, more waves than stages) is ignored at launch.
+ * The table is process wide and thread safe; results do not depend on it beyond the order of fp32 additions.
+ */
+int snnf_conv_blocked_tune(int T, int N, int Cin, int H, int W, int Cout, int KH, int KW, int stride_h, int stride_w,
+                           int pad_h, int pad_w, int shared_frame, int patch_cols, int stage_groups, int k_waves);
+
 /* Describes what the most recent snnf_conv_lif / snnf_conv_bias call on this thread selected: kernel family, timesteps per launch, tile
  * and wave decomposition, LDS bytes, grid ("key=value" pairs, empty before the first call). Plays the role of the
  * reference's get_autotune_best_config (kernels/benchmark_conv_lif_temporal_general.py:1332-1369), whose result the

@@ -209,6 +209,40 @@ def test_blocked_conv_without_neuron(B, Cin, Cout, H, W, k, s, p, T, N, resl, ou
     assert torch.allclose(got, want, rtol=2 ** -8, atol=1e-3), (got - want).abs().max()
 
 
+@pytest.mark.parametrize("patch_cols,stage_groups,k_waves,tile,waves,chunks", [
+    (16, 2, 2, "1x2x16", "8x1x2", 2), (4, 4, 1, "1x8x4", "8x1x1", 4), (2, 0, 4, "1x16x2", "8x1x4", 4),
+    (16, 8, 8, "1x2x16", None, None)])      # 8 groups / 8 waves do not fit this layer: the patch is applied, the rest is the planner's
+def test_registered_launch_choices_are_applied_and_keep_parity(B, patch_cols, stage_groups, k_waves, tile, waves, chunks):
+    Cin, Cout, H, W, k, T, N = 128, 64, 16, 16, 3, 4, 2
+    xs, w, b = _case(3300, T, N, Cin, Cout, H, W, k, BF16)
+    lif = (1.0, 0.0, 2.0)
+    ref = O.temporal_conv_lif([xs[t] for t in range(T)], w, b, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), 1, *lif)
+    x = _to_layout(B, xs, "bits", BF16)
+    key = B._plan_key(T, N, Cin, H, W, Cout, k, k, 1, 1, 1, 1, False)
+    assert B.get_autotune_best_config(T, N, Cin, H, W, (Cout, Cin, k, k), [1, 1], [1, 1]) == {}      # not a tuned layer
+    B.register_tuned_plan(key, patch_cols, stage_groups, k_waves)
+    try:
+        out, v = B.conv_lif_blocked(x, dev(w, BF16), dev(b, BF16), [1, 1], [1, 1], lif, out_layout=B.BITS, want_v=True)
+        torch.cuda.synchronize()
+        plan = B.last_conv_plan()
+    finally:
+        B.register_tuned_plan(key, 0, 0, 0)
+    assert plan["tile"] == tile and plan["tuned"] & 1
+    if waves is not None:
+        assert plan["waves"] == waves and plan["stage_chunks"] == chunks and plan["tuned"] == 3
+    check(B.to_dense(out), v, ref, what=f"tuned plan {patch_cols}/{stage_groups}/{k_waves}")
+    B.conv_lif_blocked(x, dev(w, BF16), dev(b, BF16), [1, 1], [1, 1], lif, out_layout=B.BITS)
+    assert B.last_conv_plan()["tuned"] == 0
+
+
+def test_the_committed_table_is_registered_and_reported(B):
+    table = B.load_tuned_plans()
+    for key, entry in table.items():
+        got = B.get_autotune_best_config(entry["T"], entry["N"], entry["Cin"], entry["H"], entry["W"],
+                                         (entry["Cout"], entry["Cin"], *entry["kernel"]), entry["stride"], entry["padding"], entry["shared_frame"])
+        assert got["patch_cols"] == entry["patch_cols"] and got["us"] <= got["planner_us"]
+
+
 def test_blocked_conv_rejects_what_it_does_not_take(B):
     x = B.from_dense(torch.zeros(4, 2, 64, 8, 8, device=DEV, dtype=BF16), B.BITS)
     w = torch.zeros(64, 64, 3, 3, device=DEV, dtype=BF16)

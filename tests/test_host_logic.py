@@ -297,3 +297,20 @@ def test_eager_and_meta_functions_agree_on_the_membrane_dtype():
     s_a, v_a = S.fused_temporal_conv_lif_state(x[:1], w, b, v0, *geo, *lif)
     s_b, v_b = S.fused_temporal_conv_lif_state(x[1:], w, b, v_a, *geo, *lif)
     assert torch.equal(torch.cat([s_a, s_b]), s_all) and torch.equal(v_b, v_all) and v_all.dtype == torch.float32
+
+
+def test_tuned_plan_table_is_well_formed():
+    """The measured launch choices shipped with the package: every entry names a layer shape completely and a choice the
+    registration call accepts."""
+    import json
+    from pathlib import Path
+    path = Path(__file__).resolve().parents[1] / "triton-snn-fusion_amd" / "runtime" / "tuned_blocked_plans.json"
+    table = json.loads(path.read_text())
+    assert table["dtype"] == "bf16" and isinstance(table["layers"], list)
+    seen = set()
+    for e in table["layers"]:
+        key = (e["T"], e["N"], e["Cin"], e["H"], e["W"], e["Cout"], *e["kernel"], *e["stride"], *e["padding"], bool(e["shared_frame"]))
+        assert len(key) == 13 and key not in seen
+        seen.add(key)
+        assert 0 <= e["patch_cols"] <= 32 and e["stage_groups"] in (0, 2, 4, 8) and e["k_waves"] in (0, 1, 2, 4, 8)
+        assert e["us"] < e["planner_us"]

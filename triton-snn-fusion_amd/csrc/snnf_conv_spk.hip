@@ -1,7 +1,10 @@
 // Host side of the convolution + LIF operator on the internal activation layouts (channel-blocked C8, bit-packed BITS):
 // argument validation, patch planning and launch of conv_spk_kernel.
 #include <algorithm>
+#include <array>
 #include <cstdio>
+#include <map>
+#include <mutex>
 
 #include "snnf_conv_spk_kernel.h"
 
@@ -18,9 +21,10 @@ struct SpkPlan {
 // Patch of a wave (PR x PC output pixels of one image, or PI whole planes when a plane has at most 32 pixels) and the
 // channel groups per LDS stage G: the patch with the most useful matrix lanes and the smallest halo whose stage fits the
 // wave's LDS region and its staging slots; the largest such G (fewer, longer stages).
-bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best) {
+bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best, int only_pc = 0, int only_g = 0) {
     best.score = -1.0;
     for (int pc = 1; pc <= 32 && pc <= g0.Wo; ++pc) {
+        if (only_pc > 0 && pc != only_pc) continue;
         const int pr = std::min(32 / pc, g0.Ho);
         const bool whole = pr == g0.Ho && pc == g0.Wo;
         const int pi = whole ? std::max(1, std::min(g0.N, 32 / (pr * pc))) : 1;
@@ -33,6 +37,7 @@ bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best) {
             if (region <= 64 * kSpkSlots && tt * region * 16 <= kWaveLds) G = 1;
         } else {
             for (int cand = g0.gpc; cand >= 2; cand >>= 1) {
+                if (only_g > 0 && cand > only_g) continue;
                 if (cand * region <= 64 * kSpkSlots && tt * cand * region * 16 <= kWaveLds) {
                     G = cand;
                     break;
@@ -54,6 +59,16 @@ bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best) {
     return best.score > 0.0;
 }
 
+// Measured choices for particular layers, registered by the host program (snnf_conv_blocked_tune): patch columns, channel
+// groups per stage and waves sharing a tile's K, by layer shape. A choice the kernel cannot run is ignored.
+using TunedKey = std::array<int, 13>;
+struct TunedPlan { int patch_cols, stage_groups, k_waves; };
+std::mutex tuned_mutex;
+std::map<TunedKey, TunedPlan>& tuned_plans() {
+    static std::map<TunedKey, TunedPlan> plans;
+    return plans;
+}
+
 bool valid_layout(int layout) { return layout == SNNF_LAYOUT_NCHW || layout == SNNF_LAYOUT_C8 || layout == SNNF_LAYOUT_BITS; }
 
 }  // namespace
@@ -61,6 +76,19 @@ bool valid_layout(int layout) { return layout == SNNF_LAYOUT_NCHW || layout == S
 char* conv_plan_buffer();   // the thread's plan text (snnf_conv_igemm.hip), shared with snnf_conv_last_plan()
 
 }  // namespace snnf
+
+extern "C" int snnf_conv_blocked_tune(int T, int N, int Cin, int H, int W, int Cout, int KH, int KW, int stride_h, int stride_w,
+                                      int pad_h, int pad_w, int shared_frame, int patch_cols, int stage_groups, int k_waves) {
+    using namespace snnf;
+    if (patch_cols < 0 || patch_cols > 32 || stage_groups < 0 || k_waves < 0 || k_waves > kSpkWaves || (k_waves & (k_waves - 1)) != 0)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_conv_blocked_tune: patch_cols=%d stage_groups=%d k_waves=%d out of range", patch_cols,
+                    stage_groups, k_waves);
+    const TunedKey key = {T, N, Cin, H, W, Cout, KH, KW, stride_h, stride_w, pad_h, pad_w, shared_frame ? 1 : 0};
+    std::lock_guard<std::mutex> lock(tuned_mutex);
+    if (patch_cols == 0 && stage_groups == 0 && k_waves == 0) tuned_plans().erase(key);
+    else tuned_plans()[key] = TunedPlan{patch_cols, stage_groups, k_waves};
+    return SNNF_OK;
+}
 
 extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
                                      int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
@@ -134,9 +162,17 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
 
     // Timesteps side by side: 4 (2 for T == 2, 1 for a single step or a shared frame), fewer when the halo does not fit.
     int tt = shared || T == 1 ? 1 : (T == 2 ? 2 : 4);
+    TunedPlan tuned = {0, 0, 0};
+    {
+        const TunedKey key = {T, N, Cin, H, W, Cout, KH, KW, stride_h, stride_w, pad_h, pad_w, shared ? 1 : 0};
+        std::lock_guard<std::mutex> lock(tuned_mutex);
+        const auto it = tuned_plans().find(key);
+        if (it != tuned_plans().end()) tuned = it->second;
+    }
     SpkPlan pl = {};
-    bool planned = false;
-    for (; tt >= 1; tt >>= 1) {
+    bool planned = (tuned.patch_cols > 0 || tuned.stage_groups > 0) && plan_spk(g, tt, pl, tuned.patch_cols, tuned.stage_groups);
+    const bool tuned_patch = planned;
+    for (; !planned && tt >= 1; tt >>= 1) {
         planned = plan_spk(g, tt, pl);
         if (planned) break;
     }
@@ -162,6 +198,15 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     const int cus = compute_units();
     int wk_log2 = 0;
     while (wk_log2 < 3 && static_cast<int64_t>(g.n_items) << wk_log2 < static_cast<int64_t>(cus) * 6 && g.nstages >= (2 << wk_log2)) ++wk_log2;
+    bool tuned_split = false;
+    if (tuned.k_waves > 0) {
+        int want = 0;
+        while ((1 << want) < tuned.k_waves) ++want;
+        if (g.nstages >= (1 << want)) {
+            wk_log2 = want;
+            tuned_split = true;
+        }
+    }
     g.wk_log2 = wk_log2;
     const int tiles_per_block = kSpkWaves >> wk_log2;
     // Workgroups that are resident together: one per compute unit, or two where a wave needs at most a quarter of a SIMD's
@@ -217,9 +262,9 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
                           L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset && v_init == nullptr && windows == 1 && Cout % 8 == 0;
     snprintf(snnf::conv_plan_buffer(), 256,
              "kernel=blocked variant=%d window=%d launches=1 tile=%dx%dx%d halo=%dx%d waves=8x1x%d oc_tiles=%d px_tiles=%d "
-             "stage_chunks=%d run=0 lds=%zu grid=%d",
+             "stage_chunks=%d run=0 lds=%zu grid=%d tuned=%d",
              (wk_log2 > 0 ? 50 : 40) + tt + (fast_epi ? 20 : 0), shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
-             L.lds_bytes, grid);
+             L.lds_bytes, grid, (tuned_patch ? 1 : 0) + (tuned_split ? 2 : 0));
     L.fast_epilogue = fast_epi;
     if (x_layout == SNNF_LAYOUT_BITS) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_bits(L, tt) : launch_conv_spk_f16_bits(L, tt);
     return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_c8(L, tt) : launch_conv_spk_f16_c8(L, tt);

@@ -13,8 +13,10 @@ Everything here raises when libsnnf.so is missing or a call is outside what the 
 """
 from __future__ import annotations
 
+import json
 from dataclasses import dataclass
-from typing import Optional, Sequence, Tuple
+from pathlib import Path
+from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
@@ -121,6 +123,49 @@ def pool_blocked(x: Blocked, is_max: bool, kernel: int, stride: int, padding: in
     return out
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# Measured launch choices (the role of the reference's autotune table, kernels/benchmark_conv_lif_temporal_general.py:
+# 524-558,1332-1369): tuned_blocked_plans.json next to this module holds, per layer shape, the patch width, channel
+# groups per LDS stage and K-sharing waves that measured fastest on an MI355X (written by tune_blocked.py); shapes
+# that are not in it run on the library's planner. The table is handed to the library once per process.
+# ---------------------------------------------------------------------------------------------------------------
+TUNED_PLANS_PATH = Path(__file__).resolve().parent / "tuned_blocked_plans.json"
+_TUNED: Optional[Dict[tuple, Dict]] = None
+
+
+def _plan_key(T, N, Cin, H, W, Cout, kh, kw, sh, sw, ph, pw, shared) -> tuple:
+    return (int(T), int(N), int(Cin), int(H), int(W), int(Cout), int(kh), int(kw), int(sh), int(sw), int(ph), int(pw), 1 if shared else 0)
+
+
+def register_tuned_plan(key: tuple, patch_cols: int, stage_groups: int, k_waves: int) -> None:
+    """Registers (all three 0: removes) a launch choice for one layer shape with the library."""
+    _lib.check("snnf_conv_blocked_tune", _lib.lib().snnf_conv_blocked_tune(*key, int(patch_cols), int(stage_groups), int(k_waves)))
+
+
+def load_tuned_plans(path: Optional[Path] = None) -> Dict[tuple, Dict]:
+    """Reads the table and registers every entry; returns it keyed by layer shape. Called on the first convolution."""
+    global _TUNED
+    table: Dict[tuple, Dict] = {}
+    source = TUNED_PLANS_PATH if path is None else Path(path)
+    if source.exists():
+        for entry in json.loads(source.read_text()).get("layers", []):
+            key = _plan_key(entry["T"], entry["N"], entry["Cin"], entry["H"], entry["W"], entry["Cout"], *entry["kernel"],
+                            *entry["stride"], *entry["padding"], entry["shared_frame"])
+            register_tuned_plan(key, entry["patch_cols"], entry["stage_groups"], entry["k_waves"])
+            table[key] = entry
+    _TUNED = table
+    return table
+
+
+def get_autotune_best_config(T, N, Cin, H, W, weight_shape, stride, padding, shared_frame: bool = False) -> Dict:
+    """The measured launch choice of a layer ({} when the layer is not in the table and runs on the planner)."""
+    if _TUNED is None:
+        load_tuned_plans()
+    cout, _, kh, kw = (int(d) for d in weight_shape)
+    key = _plan_key(T, N, Cin, H, W, cout, kh, kw, *_as_pair(stride), *_as_pair(padding), shared_frame)
+    return dict(_TUNED.get(key, {}))
+
+
 def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding,
                      lif: Optional[Sequence[float]], residual: Optional[Blocked] = None, out_layout: int = BITS,
                      v_init: Optional[torch.Tensor] = None, want_v: bool = False):
@@ -140,6 +185,8 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
     dev = x.data.device
     if bias is None:
         bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    if _TUNED is None:
+        load_tuned_plans()
     packed = _packed_weight(weight, bias, x.dtype)
     out = empty_blocked(out_layout, x.T, x.N, cout, ho, wo, x.dtype, dev)
     neuron = lif is not None

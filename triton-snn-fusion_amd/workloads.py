@@ -132,3 +132,26 @@ def algorithmic_conv_bytes(T: int, n: int, cin: int, h: int, w: int, cout: int, 
 
 def conv_flops(T: int, n: int, cin: int, cout: int, ho: int, wo: int, kh: int, kw: int, groups: int) -> int:
     return 2 * T * n * ho * wo * cout * (cin // groups) * kh * kw
+
+
+# The distinct conv(+residual)+LIF layers of the two network configurations (T = 4; ResNet-18 at batch 16 on 224 x 224
+# frames, VGG-11 at batch 64 on 32 x 32 frames), as timed layer by layer and as tuned.
+# (name, Cin, Cout, input size, kernel, stride, padding, residual added before the LIF, one analog frame for all T, count)
+RESNET18_LAYERS = [
+    ("stem 7x7/2 3->64", 3, 64, 224, 7, 2, 3, False, True, 1),
+    ("3x3 64->64 @56", 64, 64, 56, 3, 1, 1, False, False, 2), ("3x3 64->64 @56 +res", 64, 64, 56, 3, 1, 1, True, False, 2),
+    ("3x3/2 64->128 @56", 64, 128, 56, 3, 2, 1, False, False, 1), ("1x1/2 64->128 @56", 64, 128, 56, 1, 2, 0, False, False, 1),
+    ("3x3 128->128 @28", 128, 128, 28, 3, 1, 1, False, False, 1), ("3x3 128->128 @28 +res", 128, 128, 28, 3, 1, 1, True, False, 2),
+    ("3x3/2 128->256 @28", 128, 256, 28, 3, 2, 1, False, False, 1), ("1x1/2 128->256 @28", 128, 256, 28, 1, 2, 0, False, False, 1),
+    ("3x3 256->256 @14", 256, 256, 14, 3, 1, 1, False, False, 1), ("3x3 256->256 @14 +res", 256, 256, 14, 3, 1, 1, True, False, 2),
+    ("3x3/2 256->512 @14", 256, 512, 14, 3, 2, 1, False, False, 1), ("1x1/2 256->512 @14", 256, 512, 14, 1, 2, 0, False, False, 1),
+    ("3x3 512->512 @7", 512, 512, 7, 3, 1, 1, False, False, 1), ("3x3 512->512 @7 +res", 512, 512, 7, 3, 1, 1, True, False, 2),
+]
+VGG11_LAYERS = [
+    ("3x3 3->64 @32", 3, 64, 32, 3, 1, 1, False, True, 1), ("3x3 64->128 @16", 64, 128, 16, 3, 1, 1, False, False, 1),
+    ("3x3 128->256 @8", 128, 256, 8, 3, 1, 1, False, False, 1), ("3x3 256->256 @8", 256, 256, 8, 3, 1, 1, False, False, 1),
+    ("3x3 256->512 @4", 256, 512, 4, 3, 1, 1, False, False, 1), ("3x3 512->512 @4", 512, 512, 4, 3, 1, 1, False, False, 1),
+    ("3x3 512->512 @2", 512, 512, 2, 3, 1, 1, False, False, 2),
+]
+RESNET18_BATCH = 16
+VGG11_BATCH = 64
