@@ -593,6 +593,21 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     }
                 }
             };
+            // The same for exactly four steps 0..3 (the usual window), without a condition per step: the lower half stores
+            // steps 0 and 2, the upper half steps 1 and 3.
+            auto quad_store_bits4 = [&](int j8, uint32_t nibw) __attribute__((always_inline)) {
+                const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(nibw), 32));
+                const uint32_t lo = half ? other : nibw;
+                const uint32_t hi = half ? nibw : other;
+                if (j8 < g.C8out && px_ok) {
+                    unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
+                    const uint32_t first = lane_bits + (half ? static_cast<uint32_t>(g.out_step_stride) : 0u);
+                    const uint32_t sh = 4u * static_cast<uint32_t>(half);
+                    ob[first] = static_cast<unsigned char>(((lo >> sh) & 15u) | (((hi >> sh) & 15u) << 4));
+                    ob[first + 2u * static_cast<uint32_t>(g.out_step_stride)] =
+                        static_cast<unsigned char>(((lo >> (sh + 8u)) & 15u) | (((hi >> (sh + 8u)) & 15u) << 4));
+                }
+            };
             auto quad_end = [&](int j8, const float (&v)[4], uint32_t chm) __attribute__((always_inline)) {
                 if (v_out != nullptr && !g.analog_out && px_ok) {
                     float* __restrict__ vp = v_out + static_cast<int64_t>(j8) * 8 * po;
@@ -629,27 +644,48 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             auto fast_quad = [&](int j8, const float (&xq)[TT][4], const uint32_t (&rb)[TT], bool with_res) __attribute__((always_inline)) {
                 float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                 if constexpr (TT == 1) {
-                    for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
-                        const int cnt = min(8, t_count - ta0);
+                    if (t_count == 4 && !with_res) {
+                        // The usual stem: one frame, four steps, no residual. Straight-line.
                         uint32_t nibw = 0;
-                        for (int i = 0; i < cnt; ++i) {
-                            const uint32_t r = with_res ? fast_res(ta0 + i, j8) >> (4 * half) : 0u;
-                            nibw |= fast_lif4(xq[0], r, with_res, v) << (4 * i);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) nibw |= fast_lif4(xq[0], 0u, false, v) << (4 * i);
+                        quad_store_bits4(j8, nibw);
+                    } else {
+                        for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
+                            const int cnt = min(8, t_count - ta0);
+                            uint32_t nibw = 0;
+                            for (int i = 0; i < cnt; ++i) {
+                                const uint32_t r = with_res ? fast_res(ta0 + i, j8) >> (4 * half) : 0u;
+                                nibw |= fast_lif4(xq[0], r, with_res, v) << (4 * i);
+                            }
+                            quad_store_bits(ta0, cnt, j8, nibw);
                         }
-                        quad_store_bits(ta0, cnt, j8, nibw);
                     }
                 } else {
                     uint32_t nibw = 0;
-                    if (with_res) {
+                    if (t_count == TT) {
+                        // Every step of the window is real (the usual case): no condition per step.
+                        if (with_res) {
 #pragma unroll
-                        for (int tw = 0; tw < TT; ++tw)
-                            if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
+                            for (int tw = 0; tw < TT; ++tw) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
+                        } else {
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                        }
+                        if constexpr (TT == 4) quad_store_bits4(j8, nibw);
+                        else quad_store_bits(0, TT, j8, nibw);
                     } else {
+                        if (with_res) {
 #pragma unroll
-                        for (int tw = 0; tw < TT; ++tw)
-                            if (tw < t_count) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                            for (int tw = 0; tw < TT; ++tw)
+                                if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
+                        } else {
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw)
+                                if (tw < t_count) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                        }
+                        quad_store_bits(0, t_count, j8, nibw);
                     }
-                    quad_store_bits(0, t_count, j8, nibw);
                 }
                 if (v_out != nullptr && px_ok && j8 < g.C8out) {
                     float* __restrict__ vp = v_out + static_cast<int64_t>(j8) * 8 * po;
