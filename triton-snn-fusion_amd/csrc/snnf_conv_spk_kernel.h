@@ -107,6 +107,14 @@ __device__ __forceinline__ const void* sk_kernarg_ptr(int table_offset_bytes, in
 }
 
 // Eight spike bits -> eight 16-bit ones or zeros (ONE = the dtype's 1.0), channel j in element j.
+// fast_div without a branch: the multiply-high runs for a divisor of 1 as well (its multiplier is 0, the quotient then
+// comes from the mask). The staging decode divides three times per item; a uniform branch around each of them costs more
+// than the multiply and keeps the compiler from overlapping the items.
+__device__ __forceinline__ int sk_div(int n, const FastDiv& f) {
+    const uint32_t keep = f.d == 1u ? 0xffffffffu : 0u;
+    return static_cast<int>((__umulhi(static_cast<uint32_t>(n), f.mul) >> f.shift) | (static_cast<uint32_t>(n) & keep));
+}
+
 template <uint32_t ONE>
 __device__ __forceinline__ sk_u32x4 sk_expand_bits(uint32_t byte) {
     const uint32_t m = __umul24(byte, 0x8001u);   // bit i of the byte at bits i and 15 + i
@@ -153,9 +161,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 
     // ---- this lane's output pixel inside the patch, and where its top-left input sits in the staged halo.
     const int ppx = g.PR * g.PC;
-    const int pi = fast_div(l32, g.d_ppx);
+    const int pi = sk_div(l32, g.d_ppx);
     const int prem = l32 - pi * ppx;
-    const int prow = fast_div(prem, g.d_PC);
+    const int prow = sk_div(prem, g.d_PC);
     const int pcol = prem - prow * g.PC;
     const bool lane_in_patch = pi < g.PI;
     const uint32_t lane_b = lane_in_patch ? static_cast<uint32_t>(((pi * g.RR + prow * g.sh) * g.RC + pcol * g.sw) * 16) : 0u;
@@ -206,11 +214,11 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         const int item = (it * tiles_per_block + tile_in_block) * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
         const bool have = item < g.n_items;
         const int item_c = have ? item : 0;
-        const int oc_tile = fast_div(item_c, g.d_n_patches);
+        const int oc_tile = sk_div(item_c, g.d_n_patches);
         const int patch = item_c - oc_tile * g.n_patches;
-        const int imgg = fast_div(patch, g.d_patches_img);
+        const int imgg = sk_div(patch, g.d_patches_img);
         const int prem_i = patch - imgg * g.patches_img;
-        const int py = fast_div(prem_i, g.d_patches_x);
+        const int py = sk_div(prem_i, g.d_patches_x);
         const int n0 = imgg * g.PI;
         const int oh0 = py * g.PR;
         const int ow0 = (prem_i - py * g.patches_x) * g.PC;
@@ -265,11 +273,11 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int e = (jb + j) * 64 + lane_s;
-                    const int gq = fast_div(e, g.d_region);
+                    const int gq = sk_div(e, g.d_region);
                     const int rem = e - gq * g.region;
-                    const int ii = fast_div(rem, g.d_rrrc);
+                    const int ii = sk_div(rem, g.d_rrrc);
                     const int rem2 = rem - ii * (g.RR * g.RC);
-                    const int r = fast_div(rem2, g.d_RC);
+                    const int r = sk_div(rem2, g.d_RC);
                     const int c = rem2 - r * g.RC;
                     const int ih = ih_lo + r, iw = iw_lo + c;
                     const bool exists = e < g.IT;
