@@ -368,6 +368,12 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             if constexpr (PRE) {
                 if (have && s_first < g.nstages) stage_req(s_first);
             }
+            // The epilogue's view of the tile's channel block, opaque from here on: the scalar arithmetic that depends on it
+            // (per-quad base addresses and store predicates, several hundred scalar instructions that the compiler computes
+            // ahead of time) then runs after the tile's first loads have been requested, under their latency, instead of in
+            // front of them.
+            int oc_e = oc_tile;
+            asm volatile("" : "+s"(oc_e));
 #pragma unroll
             for (int f = 0; f < 2; ++f)
 #pragma unroll
@@ -748,10 +754,10 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         const unsigned char* res_ptr[TT];
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw)
-                            res_ptr[tw] = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, min(tw, t_count - 1))) + static_cast<int64_t>(oc_tile) * 8 * po;
+                            res_ptr[tw] = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, min(tw, t_count - 1))) + static_cast<int64_t>(oc_e) * 8 * po;
                         auto req_res = [&](auto fq_tag) __attribute__((always_inline)) {
                             constexpr int fq = decltype(fq_tag)::value;
-                            const uint32_t off = lane_bits + static_cast<uint32_t>(min(fq, g.C8out - 1 - oc_tile * 8) * po);
+                            const uint32_t off = lane_bits + static_cast<uint32_t>(min(fq, g.C8out - 1 - oc_e * 8) * po);
 #pragma unroll
                             for (int tw = 0; tw < TT; ++tw) rb[fq][tw] = res_ptr[tw][off];
                         };
@@ -772,7 +778,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         for (int tw = 0; tw < TT; ++tw)
 #pragma unroll
                             for (int k = 0; k < 4; ++k) xq[tw][k] = acc[tw][fq >> 2][4 * (fq & 3) + k];
-                        fast_quad(oc_tile * 8 + fq, xq, rb[fq], with_res);
+                        fast_quad(oc_e * 8 + fq, xq, rb[fq], with_res);
                     };
                     do_quad(std::integral_constant<int, 0>{});
                     do_quad(std::integral_constant<int, 1>{});
@@ -801,7 +807,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                             default: SNNF_SPK_COPY_QUAD(1, 3); break;
                         }
 #undef SNNF_SPK_COPY_QUAD
-                        general_quad(oc_tile * 8 + fq, xq);
+                        general_quad(oc_e * 8 + fq, xq);
                     }
                 }
             } else {
@@ -830,12 +836,12 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     if constexpr (FAST) {
                         if (e_first < 4 && g.res_layout >= 0 && TT > 1) {
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), oc_tile * 8 + 4 * r + e_first);
+                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), oc_e * 8 + 4 * r + e_first);
                         }
                     }
                     __syncthreads();
                     for (int e_own = e_first; e_own < 4; e_own += WK) {
-                        const int j8 = oc_tile * 8 + 4 * r + e_own;
+                        const int j8 = oc_e * 8 + 4 * r + e_own;
                         float xq[TT][4];
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw) {
