@@ -108,6 +108,34 @@ __global__ __launch_bounds__(kThreads) void pool_blocked_kernel(const void* __re
     }
 }
 
+// Maximum pooling of bit-packed spikes, four neighbouring output pixels of one channel group per thread, for rows whose
+// bytes can be taken eight at a time (W % 8 == 0, Wo == W / 2, a 16-byte aligned tensor is not needed: planes are multiples
+// of 8 bytes from an 8-byte aligned base). The OR of a window's bytes lands in the even bytes of the row word; K == 3 has
+// one column of padding on the left, which is the byte in front of the word (absent at the row's start).
+template <int K>
+__global__ __launch_bounds__(kThreads) void pool_bits_rows_kernel(const unsigned char* __restrict__ x, uint32_t* __restrict__ y, int64_t planes,
+                                                                  int H, int W, int Ho, int Wq) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int64_t per_plane = static_cast<int64_t>(Ho) * Wq;
+    if (item >= planes * per_plane) return;
+    const int64_t plane = item / per_plane;
+    const int rem = static_cast<int>(item - plane * per_plane);
+    const int oy = rem / Wq, m = rem - oy * Wq;
+    const unsigned char* src = x + plane * (static_cast<int64_t>(H) * W) + m * 8;
+    constexpr int PAD = K == 3 ? 1 : 0;
+    uint64_t acc = 0;
+#pragma unroll
+    for (int ky = 0; ky < K; ++ky) {
+        const int iy = oy * 2 - PAD + ky;
+        if (iy < 0 || iy >= H) continue;
+        const unsigned char* row = src + static_cast<int64_t>(iy) * W;
+        const uint64_t q = *reinterpret_cast<const uint64_t*>(row);
+        acc |= q | (q >> 8);
+        if constexpr (K == 3) acc |= (q << 8) | (m > 0 ? static_cast<uint64_t>(row[-1]) : 0ull);
+    }
+    y[item] = __builtin_amdgcn_perm(static_cast<uint32_t>(acc >> 32), static_cast<uint32_t>(acc), 0x06040200u);
+}
+
 template <typename XT>
 int convert_typed(const void* src, int sl, void* dst, int dl, int64_t frames, int C, int C8, int64_t HW, unsigned blocks, hipStream_t hs) {
 #define SNNF_CONVERT(S, D)                                                                                                   \
@@ -201,6 +229,16 @@ extern "C" int snnf_pool2d_blocked(const void* x, int x_layout, void* y, int y_l
     const int64_t items = frames * C8 * Ho * Wo;
     const unsigned blocks = static_cast<unsigned>((items + kThreads - 1) / kThreads);
     hipStream_t hs = as_stream(stream);
+    if (x_layout == SNNF_LAYOUT_BITS && y_layout == SNNF_LAYOUT_BITS && is_max != 0 && W % 8 == 0 && Wo * 2 == W && pad == (kernel == 3 ? 1 : 0) &&
+        aligned_to(x, 8) && aligned_to(y, 4)) {
+        const int64_t rows = frames * C8 * Ho * (Wo / 4);
+        const unsigned row_blocks = static_cast<unsigned>((rows + kThreads - 1) / kThreads);
+        if (kernel == 3)
+            pool_bits_rows_kernel<3><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<uint32_t*>(y), frames * C8, H, W, Ho, Wo / 4);
+        else
+            pool_bits_rows_kernel<2><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<uint32_t*>(y), frames * C8, H, W, Ho, Wo / 4);
+        return check_launch("snnf_pool2d_blocked");
+    }
     return x_dtype == SNNF_BF16 ? pool_typed<bf16_t>(x, x_layout, y, y_layout, frames, C, C8, H, W, Ho, Wo, kernel, pad, is_max != 0, blocks, hs)
                                 : pool_typed<f16_t>(x, x_layout, y, y_layout, frames, C, C8, H, W, Ho, Wo, kernel, pad, is_max != 0, blocks, hs);
 }
