@@ -11,8 +11,12 @@
  *     base + t * step_stride. Timesteps may alias (the same analog frame repeated T times is detected and computed once).
  *   - Layouts are the reference's: activations contiguous NCHW per timestep, conv weight OIHW, linear weight [Fout, Fin].
  *   - dtype codes: SNNF_F32 / SNNF_BF16 / SNNF_F16. Spikes are written as 0/1 in the activation dtype `x_dtype`.
- *     The membrane potential is held in fp32 on chip for the whole time loop; `v_dtype` is only its dtype in memory
- *     (v_init / v_out).
+ *     The membrane potential is held in fp32 on chip for the whole time loop of a launch; `v_dtype` is only its dtype
+ *     in memory (v_init / v_out). A call with more timesteps than one launch takes (16 for the scan, depthwise, linear,
+ *     pointwise and time-outer kernels; 1 to 4 for the matrix kernels, reported as `window` / `launches` by
+ *     snnf_conv_last_plan) hands the membrane from launch to launch through `v_out`, so a 16-bit `v_dtype` is rounded at
+ *     each hand-over: callers that want one rounding after the last step, as the reference's kernels do, pass an fp32
+ *     membrane for such calls and round it themselves (the operator layer above this ABI does).
  *   - `v_init == NULL` means a zero initial membrane (the reference's 0-dim v_init). `v_out` may alias `v_init`.
  *   - LIF update per step (runtime/snn_custom_ops.py:384-409):
  *         h = v + x            if tau <= 1        else   h = v + (x - v) / tau

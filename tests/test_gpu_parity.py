@@ -693,3 +693,64 @@ def test_single_step_lif_runs_the_scan_kernel_on_the_gpu(hip_ops):
             got.append(s)
         check(torch.stack(got), v, ref, v_dtype=vdtype, what=f"single-step lif {shape} {dtype}")
         assert torch.equal(torch.stack(got).float().cpu(), ref[0])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# 16-bit membranes over calls that take several launches: rounded once, after the last step
+# ---------------------------------------------------------------------------------------------------------------
+SEVERAL_LAUNCH_CASES = [  # Cin, Cout, H, W, k, s, p, T, N, lif, host placeholder v_init
+    (4, 8, 24, 23, 3, 1, 1, 8, 7, (0.5, 0.0, 1.0), True),          # IF neuron: nothing decays, every hand-over counts
+    (32, 512, 23, 13, 3, 1, 1, 17, 2, (1.0, -1.0, 2.0), True),      # 17 steps, soft reset
+    (16, 32, 20, 20, 3, 2, 1, 6, 4, (1.0, 0.0, 2.0), False),        # stride 2, membrane continued from a bf16 tensor
+    (512, 32, 20, 20, 1, 1, 0, 17, 8, (0.75, 0.25, 4.0), False),    # pointwise kernel, 16 + 1 steps
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p,T,N,lif,placeholder", SEVERAL_LAUNCH_CASES)
+def test_bf16_membrane_over_several_launches_is_rounded_once(hip_ops, Cin, Cout, H, W, k, s, p, T, N, lif, placeholder):
+    """bf16 activations with the rewriter's host-side 0-dim `v_init` (or a bf16 state) give a bf16 membrane, as in the
+    reference, whose kernel keeps it in fp32 registers over all T and rounds at the final store. A call that this
+    library runs as several launches must not round at the hand-overs: same gate as a single launch. Called twice: the
+    second call knows the layer's number of launches from the first."""
+    from triton_snn_fusion_amd.runtime import hip_convlif_backend as CB
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(8100 + Cin + T, T, N, Cin, Cout, H, W, k, BF16, p=0.25)
+    Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    g = gen(8101)
+    v0 = torch.tensor(0.0) if placeholder else q(torch.randn(N, Cout, Ho, Wo, generator=g) * 0.3, BF16)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (s, s), (p, p), (1, 1), 1, *lif)
+    dv = v0 if placeholder else dev(v0, BF16)                     # the placeholder stays on the host, as the rewriter emits it
+    dx, dw, db = [dev(x, BF16) for x in xs], dev(w_dev, BF16), dev(b_dev, BF16)
+    for call in range(2):
+        sp, v = S.fused_temporal_conv_lif_state(dx, dw, db, dv, [s, s], [p, p], [1, 1], 1, *lif, False)
+        assert v.dtype == BF16 and CB.last_conv_plan()["launches"] > 1
+        check(sp, v, ref, v_threshold=lif[0], v_dtype=BF16, what=f"bf16 membrane, {T} steps, call {call}")
+    _no_fallback(hip_ops, 2)
+
+
+def test_bf16_membrane_beyond_sixteen_steps_in_the_other_operators(hip_ops):
+    """Depthwise, linear and the standalone scan run more than 16 steps as windows of 16; same requirement."""
+    g = gen(8200)
+    T, N, C, H, W = 20, 3, 16, 14, 14
+    xs = [spikes((N, C, H, W), 0.3, g) for _ in range(T)]
+    w = q(torch.randn(C, 1, 3, 3, generator=g) * 0.5, BF16)
+    b = q(torch.randn(C, generator=g) * 0.1, BF16)
+    soft = (1.0, -1.0, 2.0)
+    ref = O.temporal_conv_lif(xs, w, b, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), C, *soft)
+    s, v = S.fused_temporal_depthwise_conv_lif_state([dev(x, BF16) for x in xs], dev(w, BF16), dev(b, BF16), torch.tensor(0.0),
+                                                     [1, 1], [1, 1], [1, 1], C, *soft, False)
+    assert v.dtype == BF16
+    check(s, v, ref, v_dtype=BF16, what="depthwise, 20 steps, bf16 membrane")
+
+    x, w_dev, b_dev, w_ref, b_ref = _linear_case(8201, 20, 48, 256, 192, BF16, True)
+    ref = O.temporal_linear_lif(x, w_ref, b_ref, torch.tensor(0.0), *soft)
+    s, v = S.fused_temporal_linear_lif_state_packed(dev(x, BF16), dev(w_dev, BF16), dev(b_dev, BF16), torch.tensor(0.0), *soft, False)
+    assert v.dtype == BF16
+    check(s, v, ref, v_dtype=BF16, what="linear, 20 steps, bf16 membrane")
+
+    x = q(torch.randn(40, 4, 16, 9, 9, generator=g) * 0.8, BF16)
+    v0 = q(torch.randn(4, 16, 9, 9, generator=g) * 0.3, BF16)
+    ref = O.temporal_lif(x, v0.float(), *soft)
+    s, v = S.fused_temporal_lif_state(dev(x, BF16), dev(v0, BF16), *soft, False)
+    assert v.dtype == BF16
+    check(s, v, ref, v_dtype=BF16, what="scan, 40 steps, bf16 membrane")
+    _no_fallback(hip_ops, 3)

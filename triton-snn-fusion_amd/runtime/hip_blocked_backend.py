@@ -166,6 +166,9 @@ def get_autotune_best_config(T, N, Cin, H, W, weight_shape, stride, padding, sha
     return dict(_TUNED.get(key, {}))
 
 
+_NEEDS_MEMBRANE_BUFFER: set = set()
+
+
 def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding,
                      lif: Optional[Sequence[float]], residual: Optional[Blocked] = None, out_layout: int = BITS,
                      v_init: Optional[torch.Tensor] = None, want_v: bool = False):
@@ -190,7 +193,11 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
     packed = _packed_weight(weight, bias, x.dtype)
     out = empty_blocked(out_layout, x.T, x.N, cout, ho, wo, x.dtype, dev)
     neuron = lif is not None
-    windows = 1 if (x.shared or x.T <= 4) else (x.T + 3) // 4
+    # The kernel needs `v_out` to carry the membrane when it runs the steps as several windows. More than 4 steps always
+    # do; whether a shorter call does (windows of 2 for layers whose accumulators would not fit otherwise) is the planner's
+    # answer, learnt from its refusal the first time such a layer is called without a membrane buffer.
+    layer = (x.layout, x.shared, x.T, x.N, x.C, x.H, x.W, cout, kh, kw, sh, sw, ph, pw, x.dtype)
+    windows = 1 if (x.shared or x.T <= 4) and layer not in _NEEDS_MEMBRANE_BUFFER else 2
     v_out = torch.empty((x.N, cout, ho, wo), dtype=torch.float32, device=dev) if neuron and (want_v or windows > 1) else None
     if residual is not None and (residual.shape != (x.T, x.N, cout, ho, wo) or residual.dtype != x.dtype or residual.shared):
         raise RuntimeError(f"unsupported_residual_shape: residual {residual.shape} does not match the output {(x.T, x.N, cout, ho, wo)}")
@@ -200,9 +207,16 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
             raise RuntimeError("unsupported_membrane_state: v_init must be a float32 [N, Cout, Ho, Wo] tensor on the activations' device")
         vi = v_init if v_init.is_contiguous() else v_init.contiguous()
     v_th, v_reset, tau = (float(lif[0]), float(lif[1]), float(lif[2])) if neuron else (1.0, 0.0, 2.0)
-    _lib.check("snnf_conv_lif_blocked", _lib.lib().snnf_conv_lif_blocked(
-        x.step_pointers(), x.layout, residual.step_pointers() if residual is not None else None,
-        residual.layout if residual is not None else 0, x.T, x.N, x.C, x.H, x.W, _lib.dtype_code(x.dtype),
-        packed.data_ptr(), cout, kh, kw, sh, sw, ph, pw, _lib.ptr(vi), out.data.data_ptr(), out_layout, out.step_stride_bytes(),
-        _lib.ptr(v_out), 1 if neuron else 0, v_th, v_reset, tau, _lib.current_stream(dev)))
+    def launch(v_buffer):
+        return _lib.lib().snnf_conv_lif_blocked(
+            x.step_pointers(), x.layout, residual.step_pointers() if residual is not None else None,
+            residual.layout if residual is not None else 0, x.T, x.N, x.C, x.H, x.W, _lib.dtype_code(x.dtype),
+            packed.data_ptr(), cout, kh, kw, sh, sw, ph, pw, _lib.ptr(vi), out.data.data_ptr(), out_layout, out.step_stride_bytes(),
+            _lib.ptr(v_buffer), 1 if neuron else 0, v_th, v_reset, tau, _lib.current_stream(dev))
+
+    status = launch(v_out)
+    if status != 0 and neuron and v_out is None and b"v_out is required" in _lib.lib().snnf_last_error():
+        _NEEDS_MEMBRANE_BUFFER.add(layer)            # refused before anything was enqueued
+        status = launch(torch.empty((x.N, cout, ho, wo), dtype=torch.float32, device=dev))
+    _lib.check("snnf_conv_lif_blocked", status)
     return out, v_out

@@ -455,19 +455,37 @@ def _run_temporal(kind: str, xs, residuals, weight, bias, v_init, stride, paddin
         spikes, v_next = spike_out, v_out
     steps = _contiguous_steps(xs)
     res = _contiguous_steps(residuals) if residuals is not None else None
-    _launch(kernel_key, steps, res, weight, bias, v_init, stride, padding, v_threshold, v_reset, tau, spikes, v_next)
+    memo = (kernel_key, residuals is not None, T, first.shape, weight.shape, tuple(_as_pair(stride)), tuple(_as_pair(padding)),
+            first.dtype, v_dtype, isinstance(v_init, torch.Tensor) and v_init.dim() > 0)
+    # A call of more timesteps than one launch takes hands the membrane from launch to launch through `v_out`. A 16-bit
+    # membrane would be rounded at every hand-over, where the reference's kernel rounds once after the last step
+    # (kernels/benchmark_conv_lif_temporal_general.py:707-716). Such a call computes with a float32 membrane and rounds
+    # the result; how many launches a layer takes is the planner's answer, known after the layer's first call.
+    wide = v_dtype != torch.float32 and T > 1 and _takes_several_launches(kernel_key, T, memo)
+    v_work = torch.empty(out_shape, dtype=torch.float32, device=first.device) if wide else v_next
+    if wide and isinstance(v_init, torch.Tensor) and v_init.dim() > 0:
+        v_init = v_init.float()
+    _launch(kernel_key, steps, res, weight, bias, v_init, stride, padding, v_threshold, v_reset, tau, spikes, v_work)
+    if wide:
+        v_next.copy_(v_work)
     diagnostics = kernel_dtype_diagnostics(first.dtype)
     if residuals is not None:
         diagnostics["residual_add"] = True
         diagnostics["kernel_kind"] = "temporal_residual"
     return TritonConvLIFResult(
         spikes, v_next, True, kernel_key=kernel_key,
-        kernel_temporal_config=_planned_temporal_config(
-            kernel_key, residuals is not None, T,
-            (kernel_key, residuals is not None, T, first.shape, weight.shape, tuple(_as_pair(stride)), tuple(_as_pair(padding)),
-             first.dtype, v_dtype, isinstance(v_init, torch.Tensor) and v_init.dim() > 0)),
+        kernel_temporal_config=_planned_temporal_config(kernel_key, residuals is not None, T, memo),
         kernel_diagnostics=diagnostics,
     )
+
+
+def _takes_several_launches(kernel_key: str, T: int, memo: tuple) -> bool:
+    if kernel_key.startswith("depthwise_"):
+        return T > _lib.SNNF_MAX_T_PER_LAUNCH     # the depthwise kernel holds up to 16 steps per launch
+    known = _TEMPORAL_CONFIGS.get(memo)
+    if known is None or "plan" not in known:
+        return True                               # not planned yet: assume the worst
+    return int(known["plan"].get("launches", 2)) > 1
 
 
 def _check_output_buffers(spike_out, v_out, spike_shape, v_shape, like: torch.Tensor, v_dtype) -> None:

@@ -93,10 +93,18 @@ def run_triton_fused_temporal_lif_state(x_seq, v_init, v_threshold: float, v_res
         vi = v_init if v_init.is_contiguous() else v_init.contiguous()
     spikes = torch.empty_like(x)
     v_next = torch.empty(x.shape[1:], dtype=v_dtype, device=x.device)
+    # More than 16 steps run as windows that hand the membrane over through `v_out`; a 16-bit membrane would be rounded
+    # at every hand-over, so such a call keeps it in float32 and rounds once at the end.
+    wide = v_dtype != torch.float32 and T > _lib.SNNF_MAX_T_PER_LAUNCH
+    v_work = torch.empty(x.shape[1:], dtype=torch.float32, device=x.device) if wide else v_next
+    if wide and vi is not None:
+        vi = vi.float()
     _lib.check("snnf_lif_scan", lib.snnf_lif_scan(
-        _lib.packed_step_pointers(x), T, numel, _lib.dtype_code(x.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype),
-        spikes.data_ptr(), numel, v_next.data_ptr(), float(v_threshold), float(v_reset), float(tau),
+        _lib.packed_step_pointers(x), T, numel, _lib.dtype_code(x.dtype), _lib.ptr(vi), _lib.dtype_code(v_work.dtype),
+        spikes.data_ptr(), numel, v_work.data_ptr(), float(v_threshold), float(v_reset), float(tau),
         _lib.current_stream(x.device)))
+    if wide:
+        v_next.copy_(v_work)
     config = get_temporal_lif_best_config(T=T, total_elements=numel, dtype=x.dtype)
     diagnostics = {
         "kernel_kind": "standalone_temporal_lif",

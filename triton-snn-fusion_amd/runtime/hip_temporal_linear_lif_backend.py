@@ -134,11 +134,20 @@ def _run_steps(steps: List[torch.Tensor], weight, bias, v_init, v_threshold, v_r
             raise RuntimeError("spike_out and v_out must be contiguous")
         spikes, v_next = spike_out, v_out
     workspace = _split_workspace(lib, first.device, T, M, Fin, Fout)
+    # The library runs more than 16 timesteps as windows that hand the membrane over through `v_out`. A 16-bit membrane
+    # would be rounded at every hand-over; the reference's kernel rounds once, after the last step. So such a call
+    # computes with a float32 membrane and rounds the result.
+    wide = v_dtype != torch.float32 and T > _lib.SNNF_MAX_T_PER_LAUNCH
+    v_work = torch.empty((M, Fout), dtype=torch.float32, device=first.device) if wide else v_next
+    if wide and vi is not None:
+        vi = vi.float()
     _lib.check("snnf_linear_lif_ws", lib.snnf_linear_lif_ws(
         _lib.step_pointers(fixed), T, M, Fin, row_stride, _lib.dtype_code(first.dtype), w.data_ptr(), _lib.ptr(b), Fout,
-        _lib.dtype_code(w.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype), spikes.data_ptr(), M * Fout,
-        v_next.data_ptr(), float(v_threshold), float(v_reset), float(tau), _lib.ptr(workspace),
+        _lib.dtype_code(w.dtype), _lib.ptr(vi), _lib.dtype_code(v_work.dtype), spikes.data_ptr(), M * Fout,
+        v_work.data_ptr(), float(v_threshold), float(v_reset), float(tau), _lib.ptr(workspace),
         0 if workspace is None else workspace.numel(), _lib.current_stream(first.device)))
+    if wide:
+        v_next.copy_(v_work)
     diagnostics = {
         "kernel_kind": "temporal_linear_lif",
         "compute_dtype": "float16" if first.dtype == torch.float16 else "float32",
