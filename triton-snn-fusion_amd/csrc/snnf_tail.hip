@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
             Pack<VT, kVec> pv;
 #pragma unroll
             for (int j = 0; j < kVec; ++j) pv.v[j] = from_float<VT>(v[j]);
-            *reinterpret_cast<Pack<VT, kVec>*>(v_out + base + i0) = pv;
+            store_streaming(v_out + base + i0, pv);
         } else {
 #pragma unroll
             for (int j = 0; j < kVec; ++j)
