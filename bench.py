@@ -29,8 +29,8 @@ METRIC = "fused ConvBN-LIF ms/layer @T=4 + end-to-end img/s; % of HBM/MFMA peak"
 def _parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="mobilenet_block",
                     choices=["mobilenet_block", "conv3x3_block", "linear_block"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])

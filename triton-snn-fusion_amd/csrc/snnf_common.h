@@ -108,12 +108,17 @@ template <typename T, int N> struct alignas(sizeof(T) * N > 16 ? 16 : sizeof(T) 
 
 // Store of results that this kernel does not read again (spikes, final membranes): marked non-temporal, so that the
 // lines stream through L2 instead of displacing the operands that are re-read (on the MobileNet pointwise layer the
-// same stores without the mark cost 17 % of the kernel's time). `dst` is aligned like the pack.
+// same stores without the mark cost 17 % of the kernel's time). Used for launches whose outputs exceed what the caches
+// hold; smaller outputs are stored normally and stay cached for the kernel that reads them. `dst` is aligned like the pack.
+constexpr int64_t kStreamOutBytes = 64ll << 20;   // outputs of a launch from which on they are stored non-temporally (twice the L2s)
 typedef uint32_t snnf_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t snnf_u32x2 __attribute__((ext_vector_type(2)));
 template <typename T, int N>
 __device__ __forceinline__ void store_streaming(T* dst, const Pack<T, N>& value) {
     constexpr int kBytes = static_cast<int>(sizeof(T)) * N;
+    // The empty statements keep these stores apart from an ordinary store of the same value on the other side of a
+    // branch: merged, the two would become one store without the mark.
+    asm volatile("" ::: "memory");
     if constexpr (kBytes % 16 == 0) {
 #pragma unroll
         for (int i = 0; i < kBytes / 16; ++i)
@@ -125,6 +130,7 @@ __device__ __forceinline__ void store_streaming(T* dst, const Pack<T, N>& value)
     } else {
         *reinterpret_cast<Pack<T, N>*>(dst) = value;
     }
+    asm volatile("" ::: "memory");
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -463,6 +463,10 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
             Part& f = parts[nparts++];
             f.g = g; f.tt = -2;
             f.g.tiles_x = full_tiles; f.g.px_base = 0;
+            // Outputs that the caches cannot hold anyway are streamed past L2, which then keeps the activation tiles for
+            // their second pass (the other output-channel tile). Smaller outputs stay cached for the layer that reads them.
+            const int64_t out_bytes = static_cast<int64_t>(N) * Cout * P * (static_cast<int64_t>(window) * dtype_size(x_dtype) + 4);
+            f.g.stream_out = out_bytes >= kStreamOutBytes ? 1 : 0;
             f.g.d_tiles_x = make_fast_div(full_tiles);
             f.lds = pw_config(true, f.g);
         }

@@ -347,7 +347,10 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
             if (fast) {
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi)
-                    if (row_ok[gi]) store_streaming(reinterpret_cast<XT*>(out + lane_off[gi]), pend[gi]);
+                    if (row_ok[gi]) {
+                        if (g.stream_out) store_streaming(reinterpret_cast<XT*>(out + lane_off[gi]), pend[gi]);
+                        else *reinterpret_cast<Pack<XT, 8>*>(out + lane_off[gi]) = pend[gi];
+                    }
             } else {
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi) {
@@ -537,8 +540,13 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                     Pack<float, 4> lo, hi;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) { lo.v[k] = v[gi][k]; hi.v[k] = v[gi][4 + k]; }
-                    store_streaming(dst, lo);
-                    store_streaming(dst + 4, hi);
+                    if (g.stream_out) {
+                        store_streaming(dst, lo);
+                        store_streaming(dst + 4, hi);
+                    } else {
+                        *reinterpret_cast<Pack<float, 4>*>(dst) = lo;
+                        *reinterpret_cast<Pack<float, 4>*>(dst + 4) = hi;
+                    }
                 }
             }
         } else {

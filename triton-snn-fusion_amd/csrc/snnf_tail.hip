@@ -81,7 +81,7 @@ constexpr int kVec = 8;
 template <typename XT, typename VT, int TC>
 __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int T, int planes, int HW, int planes_per_block,
                                                                 const VT* __restrict__ v_init, VT* __restrict__ v_out,
-                                                                int* __restrict__ counts, LifParams lif) {
+                                                                int* __restrict__ counts, LifParams lif, int stream_out) {
     __shared__ int plane_count[kMaxPlanes];
     const int plane0 = blockIdx.x * planes_per_block;
     const int planes_here = min(planes_per_block, planes - plane0);
@@ -150,7 +150,8 @@ __global__ __launch_bounds__(kThreads) void lif_pool_vec_kernel(StepPtrs xs, int
             Pack<VT, kVec> pv;
 #pragma unroll
             for (int j = 0; j < kVec; ++j) pv.v[j] = from_float<VT>(v[j]);
-            store_streaming(v_out + base + i0, pv);
+            if (stream_out) store_streaming(v_out + base + i0, pv);
+            else *reinterpret_cast<Pack<VT, kVec>*>(v_out + base + i0) = pv;
         } else {
 #pragma unroll
             for (int j = 0; j < kVec; ++j)
@@ -323,9 +324,10 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
         const int blocks = (planes + vpb - 1) / vpb;
         const VT* vi = static_cast<const VT*>(v_init);
         VT* vo = static_cast<VT*>(v_out);
-        if (T == 4) lif_pool_vec_kernel<XT, VT, 4><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
-        else if (T == 8) lif_pool_vec_kernel<XT, VT, 8><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
-        else lif_pool_vec_kernel<XT, VT, 0><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif);
+        const int stream_out = static_cast<int64_t>(planes) * HW * static_cast<int64_t>(sizeof(VT)) >= kStreamOutBytes ? 1 : 0;   // see store_streaming
+        if (T == 4) lif_pool_vec_kernel<XT, VT, 4><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif, stream_out);
+        else if (T == 8) lif_pool_vec_kernel<XT, VT, 8><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif, stream_out);
+        else lif_pool_vec_kernel<XT, VT, 0><<<dim3(blocks), kThreads, 0, stream>>>(xs, T, planes, HW, vpb, vi, vo, counts, lif, stream_out);
         return check_launch("snnf_lif_pool_linear(pool)");
     }
     int ppb = (kThreads * kItems) / HW;
