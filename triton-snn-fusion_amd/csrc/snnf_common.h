@@ -118,7 +118,7 @@ __device__ __forceinline__ void store_streaming(T* dst, const Pack<T, N>& value)
     constexpr int kBytes = static_cast<int>(sizeof(T)) * N;
     // The empty statements keep these stores apart from an ordinary store of the same value on the other side of a
     // branch: merged, the two would become one store without the mark.
-    asm volatile("" ::: "memory");
+    asm volatile("");
     if constexpr (kBytes % 16 == 0) {
 #pragma unroll
         for (int i = 0; i < kBytes / 16; ++i)
@@ -130,7 +130,7 @@ __device__ __forceinline__ void store_streaming(T* dst, const Pack<T, N>& value)
     } else {
         *reinterpret_cast<Pack<T, N>*>(dst) = value;
     }
-    asm volatile("" ::: "memory");
+    asm volatile("");
 }
 
 // ---------------------------------------------------------------------------------------------------------------
