@@ -209,9 +209,15 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     }
     const sk_u32x4* __restrict__ table = reinterpret_cast<const sk_u32x4*>(lds);
 
+    // Workgroups are handed to the eight XCDs in turn (workgroup b runs on XCD b % 8) and every XCD has an L2 of its own.
+    // Items are ordered output-channel tile first, so the workgroups of one XCD take a contiguous range of them: an XCD then
+    // reads the weights of few output-channel tiles (one, for a 512-channel layer) instead of the whole tensor.
+    const int nb = static_cast<int>(gridDim.x);
+    const int xcd = static_cast<int>(blockIdx.x) & 7;
+    const int block_l = xcd * (nb >> 3) + min(xcd, nb & 7) + (static_cast<int>(blockIdx.x) >> 3);
     for (int it = 0; it < g.iters; ++it) {
-        // Consecutive items go to consecutive workgroups, so that a layer with fewer items than wave slots still uses every compute unit.
-        const int item = (it * tiles_per_block + tile_in_block) * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
+        // Consecutive items go to different workgroups, so that a layer with fewer items than wave slots still uses every compute unit.
+        const int item = (it * tiles_per_block + tile_in_block) * nb + block_l;
         const bool have = item < g.n_items;
         const int item_c = have ? item : 0;
         const int oc_tile = sk_div(item_c, g.d_n_patches);
