@@ -63,7 +63,8 @@ def test_layout_conversions_are_exact(B, shape, dtype):
 
 @pytest.mark.parametrize("kind,k,p,shape", [("max", 3, 1, (4, 2, 64, 16, 16)), ("max", 3, 1, (2, 1, 20, 9, 11)), ("max", 2, 0, (1, 3, 8, 6, 10)),
                                             ("max", 2, 0, (2, 2, 24, 8, 16)), ("max", 3, 1, (1, 2, 16, 10, 24)),
-                                            ("avg", 2, 0, (4, 2, 64, 8, 8)), ("avg", 2, 0, (2, 2, 12, 7, 9))])
+                                            ("avg", 2, 0, (4, 2, 64, 8, 8)), ("avg", 2, 0, (2, 2, 12, 7, 9)),
+                                            ("avg", 2, 0, (2, 3, 20, 6, 24)), ("avg", 2, 0, (1, 2, 8, 5, 16))])
 def test_pooling_on_the_internal_layouts_is_exact(B, kind, k, p, shape):
     g = gen(3100 + shape[2] + k)
     s = spikes(shape, 0.3, g)

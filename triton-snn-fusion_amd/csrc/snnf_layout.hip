@@ -136,6 +136,32 @@ __global__ __launch_bounds__(kThreads) void pool_bits_rows_kernel(const unsigned
     y[item] = __builtin_amdgcn_perm(static_cast<uint32_t>(acc >> 32), static_cast<uint32_t>(acc), 0x06040200u);
 }
 
+// Average pooling (2 x 2) of bit-packed spikes into channel-blocked quarters, four neighbouring output pixels of one channel
+// group per thread: two 8-byte row words in, 64 contiguous bytes out. A channel's value is a quarter of the number of its
+// bits among the window's four bytes; padded channels hold zero bits and come out as zeros.
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void pool_bits_avg_rows_kernel(const unsigned char* __restrict__ x, XT* __restrict__ y, int64_t planes,
+                                                                      int H, int W, int Ho, int Wq) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int64_t per_plane = static_cast<int64_t>(Ho) * Wq;
+    if (item >= planes * per_plane) return;
+    const int64_t plane = item / per_plane;
+    const int rem = static_cast<int>(item - plane * per_plane);
+    const int oy = rem / Wq, m = rem - oy * Wq;
+    const unsigned char* src = x + plane * (static_cast<int64_t>(H) * W) + static_cast<int64_t>(2 * oy) * W + m * 8;
+    const uint64_t q0 = *reinterpret_cast<const uint64_t*>(src);
+    const uint64_t q1 = *reinterpret_cast<const uint64_t*>(src + W);
+    XT* __restrict__ dst = y + (item * 4) * 8;           // output pixel (plane, oy, 4 m) of [planes][Ho][4 Wq][8]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t window = static_cast<uint32_t>((q0 >> (16 * j)) & 0xffffu) | (static_cast<uint32_t>((q1 >> (16 * j)) & 0xffffu) << 16);
+        Pack<XT, 8> out;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) out.v[c] = from_float<XT>(0.25f * static_cast<float>(__builtin_popcount(window & (0x01010101u << c))));
+        *reinterpret_cast<Pack<XT, 8>*>(dst + j * 8) = out;
+    }
+}
+
 template <typename XT>
 int convert_typed(const void* src, int sl, void* dst, int dl, int64_t frames, int C, int C8, int64_t HW, unsigned blocks, hipStream_t hs) {
 #define SNNF_CONVERT(S, D)                                                                                                   \
@@ -237,6 +263,16 @@ extern "C" int snnf_pool2d_blocked(const void* x, int x_layout, void* y, int y_l
             pool_bits_rows_kernel<3><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<uint32_t*>(y), frames * C8, H, W, Ho, Wo / 4);
         else
             pool_bits_rows_kernel<2><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<uint32_t*>(y), frames * C8, H, W, Ho, Wo / 4);
+        return check_launch("snnf_pool2d_blocked");
+    }
+    if (x_layout == SNNF_LAYOUT_BITS && y_layout == SNNF_LAYOUT_C8 && is_max == 0 && kernel == 2 && pad == 0 && W % 8 == 0 && Wo * 2 == W &&
+        aligned_to(x, 8)) {
+        const int64_t rows = frames * C8 * Ho * (Wo / 4);
+        const unsigned row_blocks = static_cast<unsigned>((rows + kThreads - 1) / kThreads);
+        if (x_dtype == SNNF_BF16)
+            pool_bits_avg_rows_kernel<bf16_t><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<bf16_t*>(y), frames * C8, H, W, Ho, Wo / 4);
+        else
+            pool_bits_avg_rows_kernel<f16_t><<<dim3(row_blocks), kThreads, 0, hs>>>(static_cast<const unsigned char*>(x), static_cast<f16_t*>(y), frames * C8, H, W, Ho, Wo / 4);
         return check_launch("snnf_pool2d_blocked");
     }
     return x_dtype == SNNF_BF16 ? pool_typed<bf16_t>(x, x_layout, y, y_layout, frames, C, C8, H, W, Ho, Wo, kernel, pad, is_max != 0, blocks, hs)
