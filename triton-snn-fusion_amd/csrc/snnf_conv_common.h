@@ -115,6 +115,8 @@ struct ConvGeom {
     int w_lds;                // time-outer kernels: weight fragments streamed from L2 (0), kept in LDS (1) or in registers (2)
     int x_bufs;               // pointwise kernel: activation stages held in LDS (2 = double buffered)
     int px_base;              // pointwise kernel: pixel of each image at which this launch's tile 0 starts
+    int oc_major;             // matrix kernel: an XCD takes the output-channel tiles congruent to it (all pixel tiles) instead of the pixel
+                              // tiles congruent to it (all output-channel tiles); d_oc_tiles then divides by oc_tiles / 8
     int stream_out;           // pointwise kernel: spikes and membrane are stored non-temporally (the launch writes more than the caches hold)
     int tiles_img;            // matrix kernel: tiles per image (tiles_x * tiles_y, tiles never straddle images)
     int run8;                 // matrix kernel: runs of 8 tile pixels are contiguous in memory and aligned for 16-byte

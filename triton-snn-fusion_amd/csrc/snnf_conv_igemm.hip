@@ -416,6 +416,14 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     g.d_TW = make_fast_div(g.TW); g.d_Ho = make_fast_div(g.Ho); g.d_H = make_fast_div(g.H);
     g.d_WTP = make_fast_div(g.WT / 2); g.d_stage_rows = make_fast_div(g.NR * (g.WT / 2));
     g.d_tiles_x = make_fast_div(g.tiles_x); g.d_oc_tiles = make_fast_div(g.oc_tiles);
+    {   // Matrix kernel: which operand an XCD's L2 should keep (see the kernel's tile walk).
+        const int64_t weight_bytes = static_cast<int64_t>(Cout) * Cin * KH * KW * 2;
+        const int64_t act_bytes = static_cast<int64_t>(all_shared ? 1 : window) * N * Cin * H * W * dtype_size(x_dtype);
+        if (mm_kernel && g.oc_tiles % 8 == 0 && weight_bytes > act_bytes) {
+            g.oc_major = 1;
+            g.d_oc_tiles = make_fast_div(g.oc_tiles / 8);
+        }
+    }
     g.tiles_img = g.tiles_x * g.tiles_y; g.d_tiles_img = make_fast_div(g.tiles_img); g.d_KW = make_fast_div(g.KW);
     g.run8 = mm_kernel ? mp.run : 0;
     g.wk_log2 = mm_kernel ? mp.wk_log2 : 0;
@@ -442,7 +450,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     const int cu_per_xcd = (compute_units() + 7) / 8;
     auto grid_for = [&](const ConvGeom& gg, int per_cu) {
         const int px_tiles = mm_kernel ? gg.img_groups * gg.tiles_img : gg.tiles_x * gg.tiles_y;
-        const int work_per_xcd = ((px_tiles + 7) / 8) * gg.oc_tiles;
+        const int work_per_xcd = gg.oc_major ? px_tiles * (gg.oc_tiles / 8) : ((px_tiles + 7) / 8) * gg.oc_tiles;
         int slots = cu_per_xcd * per_cu;
         if (slots > work_per_xcd) slots = work_per_xcd;
         return slots * 8;

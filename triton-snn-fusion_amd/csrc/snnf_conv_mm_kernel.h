@@ -224,19 +224,23 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         }
     };
 
-    // ---- tile walk: pixel tiles congruent to this workgroup's XCD; consecutive work items = output-channel tiles.
+    // ---- tile walk: pixel tiles congruent to this workgroup's XCD; consecutive work items = output-channel tiles (an XCD's
+    // L2 then serves every activation tile to all of its output-channel tiles). Layers whose weights outweigh their
+    // activations turn this around (oc_major): an XCD takes the output-channel tiles congruent to it for all pixel tiles, so
+    // that its L2 holds an eighth of the weights instead of all of them.
     const int xcd = blockIdx.x & 7;
     const int slots_per_xcd = gridDim.x >> 3;
     const int n_px_tiles = g.img_groups * g.tiles_img;       // a tile spans TI images (TI > 1: whole output planes)
-    const int work_per_xcd = ((n_px_tiles + 7) >> 3) * g.oc_tiles;
+    const int oc_per_xcd = g.oc_major ? (g.oc_tiles >> 3) : g.oc_tiles;
+    const int work_per_xcd = (g.oc_major ? n_px_tiles : ((n_px_tiles + 7) >> 3)) * oc_per_xcd;
     int work = blockIdx.x >> 3;
     int oc_tile = 0, img = 0, oh0 = 0, ow0 = 0;
     auto decode = [&](int w, int& oc_t, int& n, int& r0, int& c0) __attribute__((always_inline)) -> bool {
         if (w >= work_per_xcd) return false;
         const int pt = fast_div(w, g.d_oc_tiles);
-        const int px_tile = pt * 8 + xcd;
+        const int px_tile = g.oc_major ? pt : pt * 8 + xcd;
         if (px_tile >= n_px_tiles) return false;
-        oc_t = w - pt * g.oc_tiles;
+        oc_t = g.oc_major ? (w - pt * oc_per_xcd) * 8 + xcd : w - pt * g.oc_tiles;
         const int group = fast_div(px_tile, g.d_tiles_img);
         const int in_img = px_tile - group * g.tiles_img;
         n = group * g.TI;
