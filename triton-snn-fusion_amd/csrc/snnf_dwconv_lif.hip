@@ -287,10 +287,260 @@ int launch(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g
     return check_launch("snnf_dwconv3x3_lif");
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Stride 1, strips of 8 pixels, 16-bit activations: the LDS tile keeps the activations in their 16-bit form (a prefetched
+// vector goes in with one 16-byte write and no conversion) and the taps run on the packed dot-product instruction
+// (two 16-bit products added to an fp32 accumulator): the products are exact in fp32, as with an fp32 multiply-add, and an
+// output takes two instructions per kernel row instead of three. This kernel is bound by its vector and LDS instructions
+// (with a third of the taps it runs at 6.5 TB/s), so the count is what matters.
+// Row layout: input column c at element kDotColOffset + c; the elements before and after the row are the zero halo. For
+// the strip at elements e0 .. e0 + 7 (e0 a multiple of 8) a row costs one 16-byte read and the two dwords around it.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kDotColOffset = 8;
+typedef uint32_t dw_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 dw_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 dw_f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename XT>
+__device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
+    if constexpr (dtype_of<XT>::value == SNNF_BF16)
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(dw_bf16x2, a), __builtin_bit_cast(dw_bf16x2, b), c, false);
+    else
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_f16x2, a), __builtin_bit_cast(dw_f16x2, b), c, false);
+}
+
+template <typename XT, typename VT, bool STD>
+__global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs, StepPtrs residuals, int has_residual,
+                                                                     int T, DwGeom g, const XT* __restrict__ weight,
+                                                                     const XT* __restrict__ bias,
+                                                                     const VT* __restrict__ v_init,
+                                                                     XT* __restrict__ spikes, int64_t spike_step_stride,
+                                                                     VT* __restrict__ v_out, LifParams lif) {
+    extern __shared__ __align__(16) unsigned char dot_tile_bytes[];
+    uint16_t* __restrict__ tile = reinterpret_cast<uint16_t*>(dot_tile_bytes);
+    constexpr int PX = 8;
+    constexpr int KL = kLoadSlots<1>();
+    constexpr uint32_t ES = 2;
+    static_assert(sizeof(XT) == 2, "16-bit activations only");
+
+    const int tid = threadIdx.x;
+    const int band = blockIdx.x % g.bands;
+    const int plane0 = (blockIdx.x / g.bands) * g.PB;
+    const int planes_here = min(g.PB, g.planes - plane0);
+    const int row0 = band * g.TH;
+    const int rows_here = min(g.TH, g.Ho - row0);
+    const int in_row0 = row0 - 1;                      // input row held in LDS row 0
+    const int plane_elems = g.RIN * g.pitch;           // pitch: 16-bit elements per LDS row, a multiple of 8
+    const int buf_elems = g.PB * plane_elems;
+
+    // Zero both tiles once: halo columns and out-of-image rows stay zero for every timestep.
+    for (int i = tid; i < buf_elems; i += kThreads) reinterpret_cast<uint32_t*>(tile)[i] = 0u;   // 2 tiles x buf_elems / 2 dwords
+
+    // ---- fixed ownership of input vectors (8 elements of one input row) for the whole time loop.
+    const int load_vectors = planes_here * g.RIN * g.WV;
+    uint32_t ld_src[KL];     // byte offset from the first plane of this workgroup; 0 for an idle slot
+    int ld_dst[KL];          // element offset into a tile; -1 for an idle slot
+#pragma unroll
+    for (int k = 0; k < KL; ++k) {
+        const int i = tid + k * kThreads;
+        ld_src[k] = 0;
+        ld_dst[k] = -1;
+        if (i < load_vectors) {
+            const int p = i / (g.RIN * g.WV);
+            const int rem = i - p * (g.RIN * g.WV);
+            const int r = rem / g.WV;
+            const int cv = rem - r * g.WV;
+            const int ih = in_row0 + r;
+            if (ih >= 0 && ih < g.H) {
+                ld_src[k] = static_cast<uint32_t>((p * g.H + ih) * g.W + cv * PX) * ES;
+                ld_dst[k] = p * plane_elems + r * g.pitch + kDotColOffset + cv * PX;
+            }
+        }
+    }
+    const int64_t in_base = static_cast<int64_t>(plane0) * g.H * g.W;    // elements
+
+    // ---- fixed ownership of output strips; the weights of a strip's channel as the four operand pairs of a kernel row:
+    // (w1, w2) and (0, w0) serve the even outputs, (w0, w1) and (w2, 0) the odd ones.
+    const int strips_per_plane = rows_here * g.SW;
+    const int strips = planes_here * strips_per_plane;
+    int item_src[kItems];          // element offset of the strip's first input pixel inside a tile (a multiple of 8)
+    uint32_t item_out[kItems];     // element offset of the strip from the first output plane of this workgroup
+    bool item_live[kItems];
+    float v[kItems][PX];
+    uint32_t wp[kItems][3][4];
+    float b[kItems];
+    const int64_t out_base = (static_cast<int64_t>(plane0) * g.Ho + row0) * g.Wo;   // elements
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        const int i = tid + k * kThreads;
+        item_live[k] = i < strips;
+        const int ii = item_live[k] ? i : 0;
+        const int ip = ii / strips_per_plane;
+        const int rem = ii - ip * strips_per_plane;
+        const int ir = rem / g.SW;
+        const int ic = (rem - ir * g.SW) * PX;
+        item_src[k] = ip * plane_elems + ir * g.pitch + kDotColOffset + ic;
+        item_out[k] = static_cast<uint32_t>((ip * g.Ho + ir) * g.Wo + ic);
+        const int c = (plane0 + ip) % g.C;
+        const uint16_t* __restrict__ wbits = reinterpret_cast<const uint16_t*>(weight) + c * 9;
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+            const uint32_t w0 = wbits[kh * 3], w1 = wbits[kh * 3 + 1], w2 = wbits[kh * 3 + 2];
+            wp[k][kh][0] = w1 | (w2 << 16);
+            wp[k][kh][1] = w0 << 16;
+            wp[k][kh][2] = w0 | (w1 << 16);
+            wp[k][kh][3] = w2;
+        }
+        b[k] = to_float(bias[c]);
+        if (item_live[k] && v_init != nullptr) {
+            load_strip_as_float<VT, PX>(v_init + out_base + item_out[k], v[k]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < PX; ++j) v[k][j] = 0.0f;
+        }
+    }
+
+    // ---- prefetch registers and the spikes waiting to be stored.
+    dw_u32x4 pre[KL];
+    auto issue_loads = [&](int t) __attribute__((always_inline)) {
+        const char* __restrict__ x = reinterpret_cast<const char*>(static_cast<const XT*>(dw_table_entry(0, t)) + in_base);
+#pragma unroll
+        for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const dw_u32x4*>(x + ld_src[k]);
+    };
+    Pack<XT, PX> pend[kItems];
+    int pend_t = -1;
+    auto flush = [&]() __attribute__((always_inline)) {
+        XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k)
+            if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+        pend_t = -1;
+    };
+
+    issue_loads(0);
+    __syncthreads();   // zero fill complete
+    int buf = 0;
+    for (int t = 0; t < T; ++t) {
+        uint16_t* __restrict__ cur = tile + buf * buf_elems;
+#pragma unroll
+        for (int k = 0; k < KL; ++k)
+            if (ld_dst[k] >= 0) *reinterpret_cast<dw_u32x4*>(cur + ld_dst[k]) = pre[k];
+        __syncthreads();   // tile of step t complete; every wave is past its reads of the other tile
+        if (pend_t >= 0) flush();
+        if (t + 1 < T) issue_loads(t + 1);
+
+        const XT* __restrict__ res = has_residual ? static_cast<const XT*>(dw_table_entry(sizeof(StepPtrs), t)) + out_base : nullptr;
+#pragma unroll
+        for (int k = 0; k < kItems; ++k) {
+            const uint16_t* __restrict__ src = cur + item_src[k];
+            float acc[PX];
+#pragma unroll
+            for (int j = 0; j < PX; ++j) acc[j] = b[k];
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh) {
+                const uint16_t* __restrict__ row = src + kh * g.pitch;
+                const dw_u32x4 d = *reinterpret_cast<const dw_u32x4*>(row);
+                const uint32_t left = *reinterpret_cast<const uint32_t*>(row - 2);     // (x[-2], x[-1])
+                const uint32_t right = *reinterpret_cast<const uint32_t*>(row + 8);    // (x[8], x[9])
+                const uint32_t A = wp[k][kh][0], B = wp[k][kh][1], C = wp[k][kh][2], D = wp[k][kh][3];
+                acc[0] = dot2_acc<XT>(d[0], A, dot2_acc<XT>(left, B, acc[0]));
+                acc[1] = dot2_acc<XT>(d[0], C, dot2_acc<XT>(d[1], D, acc[1]));
+                acc[2] = dot2_acc<XT>(d[1], A, dot2_acc<XT>(d[0], B, acc[2]));
+                acc[3] = dot2_acc<XT>(d[1], C, dot2_acc<XT>(d[2], D, acc[3]));
+                acc[4] = dot2_acc<XT>(d[2], A, dot2_acc<XT>(d[1], B, acc[4]));
+                acc[5] = dot2_acc<XT>(d[2], C, dot2_acc<XT>(d[3], D, acc[5]));
+                acc[6] = dot2_acc<XT>(d[3], A, dot2_acc<XT>(d[2], B, acc[6]));
+                acc[7] = dot2_acc<XT>(d[3], C, dot2_acc<XT>(right, D, acc[7]));
+            }
+            if (res != nullptr && item_live[k]) {
+                float r8[PX];
+                load_strip_as_float<XT, PX>(res + item_out[k], r8);
+#pragma unroll
+                for (int j = 0; j < PX; ++j) acc[j] += r8[j];
+            }
+#pragma unroll
+            for (int j = 0; j < PX; ++j) {
+                if constexpr (STD) {
+                    const float h = v[k][j] + (acc[j] - v[k][j]) * lif.inv_tau;
+                    const bool fired = h >= lif.v_threshold;
+                    v[k][j] = fired ? lif.v_reset : h;
+                    pend[k].v[j] = spike_value<XT>(fired);
+                } else {
+                    pend[k].v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
+                }
+            }
+        }
+        pend_t = t;
+        buf ^= 1;
+    }
+    if (pend_t >= 0) flush();
+
+#pragma unroll
+    for (int k = 0; k < kItems; ++k) {
+        if (!item_live[k]) continue;
+        Pack<VT, PX> vo;
+#pragma unroll
+        for (int j = 0; j < PX; ++j) vo.v[j] = from_float<VT>(v[k][j]);
+        *reinterpret_cast<Pack<VT, PX>*>(v_out + out_base + item_out[k]) = vo;
+    }
+}
+
+// Launcher of the packed dot-product kernel: the planning of `launch` with 16-bit rows.
+template <typename XT, typename VT>
+int launch_dot(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g, const void* weight, const void* bias,
+               const void* v_init, void* spikes, int64_t spike_step_stride, void* v_out, const LifParams& lif,
+               hipStream_t stream) {
+    constexpr int PX = 8;
+    g.SW = g.Wo / PX;
+    g.WV = g.W / PX;
+    const int max_strips = kThreads * kItems;
+    const int per_plane = g.Ho * g.SW;
+    if (per_plane >= max_strips) {
+        g.PB = 1;
+        g.TH = max_strips / g.SW;
+        if (g.TH < 1) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: output row of %d pixels is too wide", g.Wo);
+    } else {
+        g.TH = g.Ho;
+        g.PB = max_strips / per_plane;
+        if (g.PB > g.planes) g.PB = g.planes;
+    }
+    // Row pitch in 16-bit elements: the row, its offset and two halo elements behind it, rounded to 16 bytes; not a multiple
+    // of 128 bytes, so that the 16-byte reads of lanes that sit in consecutive rows fall into different banks.
+    g.pitch = (g.W + kDotColOffset + 2 + 7) / 8 * 8;
+    if (g.pitch % 64 == 0) g.pitch += 8;
+    const int max_vectors = kThreads * kLoadSlots<1>();
+    auto fits = [&]() {
+        g.bands = (g.Ho + g.TH - 1) / g.TH;
+        g.RIN = g.TH + 2;
+        const size_t bytes = static_cast<size_t>(2) * g.PB * g.RIN * g.pitch * sizeof(uint16_t);
+        return bytes <= kDwMaxLds && g.PB * g.RIN * g.WV <= max_vectors;
+    };
+    while (!fits() && g.PB > 1) g.PB = (g.PB + 1) / 2;
+    while (!fits() && g.TH > 1) g.TH = (g.TH + 1) / 2;
+    if (!fits()) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: input row of %d pixels does not fit LDS", g.W);
+    const size_t lds = static_cast<size_t>(2) * g.PB * g.RIN * g.pitch * sizeof(uint16_t);
+    const int64_t blocks = static_cast<int64_t>((g.planes + g.PB - 1) / g.PB) * g.bands;
+    if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: too many planes");
+    if (lif.charge_mode == CHARGE_SCALE && !lif.soft_reset) {
+        dwconv3x3_lif_dot_kernel<XT, VT, true><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+            xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
+            static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    } else {
+        dwconv3x3_lif_dot_kernel<XT, VT, false><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+            xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
+            static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
+    }
+    return check_launch("snnf_dwconv3x3_lif");
+}
+
+
 template <typename XT, typename VT, int STRIDE>
 int dispatch_px(int px, const StepPtrs& xs, const StepPtrs& res, int has_res, int T, const DwGeom& g,
                 const void* weight, const void* bias, const void* v_init, void* spikes, int64_t sss, void* v_out,
                 const LifParams& lif, hipStream_t stream) {
+    if constexpr (STRIDE == 1 && sizeof(XT) == 2) {
+        if (px == 8) return launch_dot<XT, VT>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
+    }
     if (px == 8) return launch<XT, VT, STRIDE, 8>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
     if (px == 4) return launch<XT, VT, STRIDE, 4>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
     return launch<XT, VT, STRIDE, 1>(xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
