@@ -181,6 +181,7 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
         const XT* __restrict__ res = has_residual ? static_cast<const XT*>(dw_table_entry(sizeof(StepPtrs), t)) + out_base : nullptr;
 #pragma unroll
         for (int k = 0; k < kItems; ++k) {
+            if (__builtin_amdgcn_ballot_w64(item_live[k]) == 0) continue;   // a wave none of whose lanes owns a strip in this round
             const float* __restrict__ src = cur + item_src[k];
             float acc[PX];
 #pragma unroll
@@ -432,6 +433,7 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
         const XT* __restrict__ res = has_residual ? static_cast<const XT*>(dw_table_entry(sizeof(StepPtrs), t)) + out_base : nullptr;
 #pragma unroll
         for (int k = 0; k < kItems; ++k) {
+            if (__builtin_amdgcn_ballot_w64(item_live[k]) == 0) continue;   // a wave none of whose lanes owns a strip in this round
             const uint16_t* __restrict__ src = cur + item_src[k];
             float acc[PX];
 #pragma unroll
