@@ -314,3 +314,20 @@ def test_tuned_plan_table_is_well_formed():
         seen.add(key)
         assert 0 <= e["patch_cols"] <= 32 and e["stage_groups"] in (0, 2, 4, 8) and e["k_waves"] in (0, 1, 2, 4, 8)
         assert e["us"] < e["planner_us"]
+
+
+def test_a_16_bit_membrane_is_kept_wide_until_the_layer_is_known_to_take_one_launch():
+    """Which calls run with a float32 membrane and round once at the end: depthwise above 16 timesteps; any other conv until
+    the planner has reported a single launch for the layer."""
+    memo = ("k3_s1_p1", False, 4, (2, 8, 8, 8), (8, 8, 3, 3), (1, 1), (1, 1), torch.bfloat16, torch.bfloat16, False)
+    CB._TEMPORAL_CONFIGS.pop(memo, None)
+    assert not CB._takes_several_launches("depthwise_k3_s1_p1", 16, memo)
+    assert CB._takes_several_launches("depthwise_k3_s1_p1", 17, memo)
+    assert CB._takes_several_launches("k3_s1_p1", 4, memo)                      # not planned yet: assume the worst
+    try:
+        CB._TEMPORAL_CONFIGS[memo] = {"plan": {"launches": 1}}
+        assert not CB._takes_several_launches("k3_s1_p1", 4, memo)
+        CB._TEMPORAL_CONFIGS[memo] = {"plan": {"launches": 2}}
+        assert CB._takes_several_launches("k3_s1_p1", 4, memo)
+    finally:
+        CB._TEMPORAL_CONFIGS.pop(memo, None)
