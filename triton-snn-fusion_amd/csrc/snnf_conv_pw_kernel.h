@@ -51,7 +51,11 @@ __device__ __forceinline__ const void* kernarg_table_entry(int table_offset_byte
 }
 
 // The two pointer tables MUST be the first two kernel parameters (offsets 0 and sizeof(StepPtrs)).
-template <typename XT, int LM, bool STD, int WM, bool FAST>
+// DIRECT (with FAST and STD, no residual): the LIF step runs on the accumulators where the matrix instruction leaves them
+// (a lane holds 2 adjacent pixels x 16 channels of the wave's 32 x 64 outputs) and spikes and the membrane go to memory
+// from there: the two adjacent pixels of a channel are one 4-byte (spikes) or 8-byte (membrane) store, 32 lanes of a
+// half-wave cover a whole 128- or 256-byte line of one channel row. No trip through LDS, and the LIF step does not wait for one.
+template <typename XT, int LM, bool STD, int WM, bool FAST, bool DIRECT = false>
 __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pw_lif_kernel(const StepPtrs xs, const StepPtrs residuals,
                                                                       const int has_residual, const ConvGeom g,
                                                                       const uint16_t* __restrict__ wpacked,
@@ -310,7 +314,27 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[gi][k] = 0.0f;
         }
-        if (v_init != nullptr) {
+        // DIRECT: membrane of the lane's 2 pixels x 16 channels, register r = channel ocf * 32 + 8 (r / 4) + 4 half + r % 4.
+        float vd[kNPF][16];
+        const uint32_t lane_off_d = static_cast<uint32_t>((ocf * 32 + 4 * half) * P + 2 * l32);   // elements into [Cout, P]
+        auto row_off_d = [&](int r) __attribute__((always_inline)) { return static_cast<uint32_t>((8 * (r >> 2) + (r & 3)) * P); };
+        if constexpr (DIRECT) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                vd[0][r] = 0.0f;
+                vd[1][r] = 0.0f;
+            }
+            if (v_init != nullptr && wave_has_work) {
+                const float* __restrict__ vsrc = static_cast<const float*>(v_init) + tile_off + lane_off_d;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const Pack<float, 2> two = *reinterpret_cast<const Pack<float, 2>*>(vsrc + row_off_d(r));
+                    vd[0][r] = two.v[0];
+                    vd[1][r] = two.v[1];
+                }
+            }
+        }
+        if (!DIRECT && v_init != nullptr) {
             if (fast && vf32) {
                 const char* vbase = reinterpret_cast<const char*>(static_cast<const float*>(v_init) + tile_off);
 #pragma unroll
@@ -341,10 +365,20 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 
         // Spikes of a timestep wait here until the next stage has left its load registers.
         Pack<XT, 8> pend[NG];
+        uint32_t pend_d[16];     // DIRECT: the spikes of 2 adjacent pixels of channel register r
         int pend_step = -1;
         auto flush_spikes = [&]() __attribute__((always_inline)) {
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
-            if (fast) {
+            if constexpr (DIRECT) {
+                XT* __restrict__ dst = reinterpret_cast<XT*>(out) + lane_off_d;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    Pack<XT, 2> two;
+                    *reinterpret_cast<uint32_t*>(&two) = pend_d[r];
+                    if (g.stream_out) store_streaming(dst + row_off_d(r), two);
+                    else *reinterpret_cast<Pack<XT, 2>*>(dst + row_off_d(r)) = two;
+                }
+            } else if (fast) {
 #pragma unroll
                 for (int gi = 0; gi < NG; ++gi)
                     if (row_ok[gi]) {
@@ -485,8 +519,23 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                 if (pend_step >= 0) flush_spikes();   // only when a timestep had no stage of its own (shared frame)
                 const char* __restrict__ res_t =
                     has_residual ? reinterpret_cast<const char*>(static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), step)) + tile_off) : nullptr;
+                if constexpr (DIRECT) {
+                    const uint32_t one16 = F16 ? 0x3C00u : 0x3F80u;
 #pragma unroll
-                for (int gi = 0; gi < NG; ++gi) {
+                    for (int r = 0; r < 16; ++r) {
+                        uint32_t pair = 0u;
+#pragma unroll
+                        for (int pf = 0; pf < kNPF; ++pf) {
+                            const float h = vd[pf][r] + (acc[pf][r] - vd[pf][r]) * lif.inv_tau;
+                            const bool fired = h >= lif.v_threshold;
+                            vd[pf][r] = fired ? lif.v_reset : h;
+                            pair |= fired ? (one16 << (16 * pf)) : 0u;
+                        }
+                        pend_d[r] = pair;
+                    }
+                }
+#pragma unroll
+                for (int gi = 0; gi < (DIRECT ? 0 : NG); ++gi) {
                     __builtin_amdgcn_wave_barrier();
 #pragma unroll
                     for (int rr = 0; rr < 4; ++rr) {
@@ -531,7 +580,17 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 
         // ---- last timestep's spikes and the final membrane.
         if (pend_step >= 0) flush_spikes();
-        if (fast && vf32) {
+        if constexpr (DIRECT) {
+            if (wave_has_work) {
+                float* __restrict__ vdst = static_cast<float*>(v_out) + tile_off + lane_off_d;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
+                    if (g.stream_out) store_streaming(vdst + row_off_d(r), two);
+                    else *reinterpret_cast<Pack<float, 2>*>(vdst + row_off_d(r)) = two;
+                }
+            }
+        } else if (fast && vf32) {
             char* vbase = reinterpret_cast<char*>(static_cast<float*>(v_out) + tile_off);
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi) {
@@ -584,6 +643,7 @@ int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     auto pick = [&](auto lm) -> int {
         constexpr int LMV = decltype(lm)::value;
         if (fast) {
+            if (L.g.w_lds == PW_WEIGHTS_REGS && !L.has_residual) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true, true>);
             if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true>);
             if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_LDS, true>);
             return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_STREAM, true>);
