@@ -371,12 +371,16 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
             if constexpr (DIRECT) {
                 XT* __restrict__ dst = reinterpret_cast<XT*>(out) + lane_off_d;
+                if (g.stream_out) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    Pack<XT, 2> two;
-                    *reinterpret_cast<uint32_t*>(&two) = pend_d[r];
-                    if (g.stream_out) store_streaming(dst + row_off_d(r), two);
-                    else *reinterpret_cast<Pack<XT, 2>*>(dst + row_off_d(r)) = two;
+                    for (int r = 0; r < 16; ++r) {
+                        Pack<XT, 2> two;
+                        *reinterpret_cast<uint32_t*>(&two) = pend_d[r];
+                        store_streaming(dst + row_off_d(r), two);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) *reinterpret_cast<uint32_t*>(dst + row_off_d(r)) = pend_d[r];
                 }
             } else if (fast) {
 #pragma unroll
@@ -583,11 +587,18 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         if constexpr (DIRECT) {
             if (wave_has_work) {
                 float* __restrict__ vdst = static_cast<float*>(v_out) + tile_off + lane_off_d;
+                if (g.stream_out) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
-                    if (g.stream_out) store_streaming(vdst + row_off_d(r), two);
-                    else *reinterpret_cast<Pack<float, 2>*>(vdst + row_off_d(r)) = two;
+                    for (int r = 0; r < 16; ++r) {
+                        const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
+                        store_streaming(vdst + row_off_d(r), two);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
+                        *reinterpret_cast<Pack<float, 2>*>(vdst + row_off_d(r)) = two;
+                    }
                 }
             }
         } else if (fast && vf32) {
