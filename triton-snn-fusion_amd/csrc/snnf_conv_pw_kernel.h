@@ -370,17 +370,18 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         auto flush_spikes = [&]() __attribute__((always_inline)) {
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
             if constexpr (DIRECT) {
-                XT* __restrict__ dst = reinterpret_cast<XT*>(out) + lane_off_d;
+                // Uniform row base + 32-bit lane offset: the stores take the scalar-base addressing form.
+                const uint32_t lane_b = lane_off_d * ES;
                 if (g.stream_out) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         Pack<XT, 2> two;
                         *reinterpret_cast<uint32_t*>(&two) = pend_d[r];
-                        store_streaming(dst + row_off_d(r), two);
+                        store_streaming(reinterpret_cast<XT*>(out + static_cast<size_t>(row_off_d(r)) * ES + lane_b), two);
                     }
                 } else {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) *reinterpret_cast<uint32_t*>(dst + row_off_d(r)) = pend_d[r];
+                    for (int r = 0; r < 16; ++r) *reinterpret_cast<uint32_t*>(out + static_cast<size_t>(row_off_d(r)) * ES + lane_b) = pend_d[r];
                 }
             } else if (fast) {
 #pragma unroll
@@ -586,18 +587,19 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         if (pend_step >= 0) flush_spikes();
         if constexpr (DIRECT) {
             if (wave_has_work) {
-                float* __restrict__ vdst = static_cast<float*>(v_out) + tile_off + lane_off_d;
+                char* __restrict__ vbase = reinterpret_cast<char*>(static_cast<float*>(v_out) + tile_off);   // uniform
+                const uint32_t lane_vb = lane_off_d * 4u;
                 if (g.stream_out) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
-                        store_streaming(vdst + row_off_d(r), two);
+                        store_streaming(reinterpret_cast<float*>(vbase + static_cast<size_t>(row_off_d(r)) * 4u + lane_vb), two);
                     }
                 } else {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const Pack<float, 2> two = {{vd[0][r], vd[1][r]}};
-                        *reinterpret_cast<Pack<float, 2>*>(vdst + row_off_d(r)) = two;
+                        *reinterpret_cast<Pack<float, 2>*>(vbase + static_cast<size_t>(row_off_d(r)) * 4u + lane_vb) = two;
                     }
                 }
             }
