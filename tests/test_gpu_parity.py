@@ -330,6 +330,8 @@ POINTWISE_CASES = [  # Cin, Cout, H, W, dtype, vdtype, lif, T, residual, tensor 
     (128, 64, 16, 16, BF16, F32, (1.0, -1.0, 2.0), 4, False, False),   # soft reset: general variant
     (128, 64, 16, 16, BF16, F32, (0.5, 0.0, 1.0), 5, False, True),     # IF neuron
     (128, 64, 8, 8, F32, F32, (1.0, 0.0, 2.0), 4, True, False),        # fp32 activations (rounded to bf16 on the way in)
+    (128, 64, 8, 8, F32, F32, (1.0, 0.0, 2.0), 4, False, True),        # fp32, no residual: the fast variant with fp32 spike stores
+    (256, 64, 16, 8, F16, F32, (1.0, 0.0, 2.0), 4, False, True),       # f16, weights in LDS, no residual: LIF on the accumulators
     (128, 96, 8, 16, F16, F16, (1.0, 0.0, 2.0), 4, False, True),       # f16 with an f16 membrane
     (192, 64, 16, 8, F16, F32, (1.0, 0.0, 2.0), 17, False, False),     # channel tail in the second chunk, two launch windows
     (128, 64, 16, 16, BF16, F32, (1.0, 0.0, 1.5), 4, False, True),     # tau not a power of two: true division
@@ -409,8 +411,10 @@ FALLBACK_KERNEL_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif
     (44, 256, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "t_in_m"),      # high intensity, Cin % 8 != 0
     (44, 256, 9, 9, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 3, True, True, "t_in_m"),          # + odd plane, residual, v_init
     (52, 320, 10, 10, 3, 1, 1, F16, F32, (1.0, 0.0, 4.0), 6, 2, False, True, "t_in_m"),        # two launch windows, f16
-    (512, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "t_in_m"),     # deep pointwise layer (AI 205)
-    (1024, 1024, 7, 7, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True, "t_in_m"),       # deep pointwise layer (AI 410)
+    (512, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "matrix"),     # deep pointwise layer (AI 205): an image is one row of pixels to the matrix kernel
+    (1024, 1024, 7, 7, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True, "matrix"),       # deep pointwise layer (AI 410), residual, v_init
+    (520, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "matrix"),     # ... and so is a channel count of whole groups that is no multiple of the chunk
+    (516, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, False, "t_in_m"),      # deep pointwise layer whose channels are not whole groups of 8
     (12, 32, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 3.0), 4, 2, False, True, "time_outer"),     # tau not a power of two
     (44, 256, 12, 12, 3, 1, 1, BF16, F32, (0.75, 0.0, 1.5), 4, 2, False, True, "t_in_m"),      # tau not a power of two
 ]
@@ -419,8 +423,9 @@ FALLBACK_KERNEL_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif
 @pytest.mark.parametrize("Cin,Cout,H,W,k,stride,pad,dtype,vdtype,lif,T,N,residual,tensor_v,family", FALLBACK_KERNEL_CASES)
 def test_dense_conv_lif_shapes_outside_the_matrix_and_pointwise_kernels(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N,
                                                                         residual, tensor_v, family):
-    """Layers the 8-wave matrix kernel and the pointwise kernel do not take (input channels that are not whole groups of 8,
-    plain 1x1 layers of high arithmetic intensity) run the time-outer kernel or the 4-wave T-in-M kernel."""
+    """Layers the 8-wave matrix kernel and the pointwise kernel do not take (input channels that are not whole groups of 8)
+    run the time-outer kernel or the 4-wave T-in-M kernel; plain 1x1 layers of high arithmetic intensity run the matrix
+    kernel on images flattened to one row of pixels."""
     from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
     xs, w_dev, b_dev, w_ref, b_ref = _conv_case(1600 + Cin + Cout + H + k, T, N, Cin, Cout, H, W, k, dtype, p=0.25)
     Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1

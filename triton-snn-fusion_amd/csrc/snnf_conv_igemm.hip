@@ -322,8 +322,9 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
                                                        static_cast<double>(T) * N * Cout * Ho_real * Wo_real) +
                          4.0 * N * Cout * Ho_real * Wo_real;
     // Dense layers whose input channels fill whole groups of 8 (or fit a single group) go to the 8-wave matrix kernel
-    // whatever their intensity (its per-tile cost is the lower one); pointwise layers stay with the pointwise kernel.
-    const bool matrix_candidate = !pointwise && (Cin % 8 == 0 || Cin < 8);
+    // whatever their intensity (its per-tile cost is the lower one); pointwise layers stay with the pointwise kernel unless
+    // they are compute bound (deep 512 -> 512 layers: an image is then one row of H * W pixels to the matrix kernel).
+    const bool matrix_candidate = (!pointwise || flops / bytes >= 200.0) && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
     Plan pl = {};
     bool planned = false;

@@ -64,6 +64,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                                                                       XT* __restrict__ spikes, void* __restrict__ v_out,
                                                                       const LifParams lif) {
     extern __shared__ __align__(16) unsigned char lds[];
+    static_assert(!DIRECT || (FAST && STD && sizeof(XT) == 2), "the accumulator-layout LIF step is for the fast variant on 16-bit activations");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
     constexpr int SS = kPwSlots;
@@ -655,8 +656,14 @@ int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     // neuron through the generic update and keep their weights in LDS or stream them.
     auto pick = [&](auto lm) -> int {
         constexpr int LMV = decltype(lm)::value;
+        if constexpr (sizeof(XT) == 2) {
+            if (fast && !L.has_residual) {      // LIF on the accumulators (16-bit spikes: two pixels are one 4-byte store)
+                if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true, true>);
+                if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_LDS, true, true>);
+                return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_STREAM, true, true>);
+            }
+        }
         if (fast) {
-            if (L.g.w_lds == PW_WEIGHTS_REGS && !L.has_residual) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true, true>);
             if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_REGS, true>);
             if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_LDS, true>);
             return run(conv_pw_lif_kernel<XT, LMV, true, PW_WEIGHTS_STREAM, true>);
