@@ -357,6 +357,45 @@ def test_pointwise_conv_lif_variants(hip_ops, Cin, Cout, H, W, dtype, vdtype, li
     _no_fallback(hip_ops, 1)
 
 
+LARGE_POINTWISE_CASES = [  # Cin, Cout, H, W, dtype, lif, T, N, residual, tensor v_init
+    (256, 128, 7, 7, BF16, (1.0, 0.0, 2.0), 4, 1280, True, False),     # weights in LDS, several chunks, odd plane, residual
+    (256, 64, 16, 8, F16, (1.0, 0.0, 2.0), 4, 640, False, True),       # f16, several chunks, LIF on the accumulators
+    (192, 64, 16, 8, F16, (1.0, 0.0, 2.0), 17, 192, False, False),     # channel tail in the last chunk, two launch windows
+    (1024, 64, 56, 56, BF16, (1.0, 0.0, 2.0), 4, 8, False, False),     # weights streamed from L2
+    (1024, 64, 5, 5, BF16, (1.0, 0.0, 2.0), 4, 1000, False, True),     # streamed + odd plane
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,dtype,lif,T,N,residual,tensor_v", LARGE_POINTWISE_CASES)
+def test_pointwise_layers_of_several_chunks(hip_ops, Cin, Cout, H, W, dtype, lif, T, N, residual, tensor_v):
+    """Plain 1x1 layers of more than 128 input channels stay with the pointwise kernel from 200 MB of traffic on (smaller
+    ones run the matrix kernel): its variants for several channel chunks are reached by large layers only."""
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(950 + Cin + Cout + H, T, N, Cin, Cout, H, W, 1, dtype, p=0.25)
+    g = gen(951 + Cin)
+    rs = [q(torch.randn(N, Cout, H, W, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = q(torch.randn(N, Cout, H, W, generator=g) * 0.3, F32) if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, v0, (1, 1), (0, 0), (1, 1), 1, *lif, residuals=rs)
+    dx, dw, db = [dev(x, dtype) for x in xs], dev(w_dev, dtype), dev(b_dev, dtype)
+    dv = dev(v0, F32) if tensor_v else zero_v(F32)
+    if residual:
+        sp, v = S.fused_temporal_conv_add_lif_state(dx, [dev(r, dtype) for r in rs], dw, db, dv, [1, 1], [0, 0], [1, 1], 1, *lif, False)
+    else:
+        sp, v = S.fused_temporal_pointwise_conv_lif_state(dx, dw, db, dv, [1, 1], [0, 0], [1, 1], 1, *lif, False)
+    assert last_conv_plan()["kernel"] == "pointwise", last_conv_plan()
+    check(sp, v, ref, v_threshold=lif[0], v_dtype=F32, what=f"large pointwise {Cin}->{Cout} {H}x{W} x{N}")
+    # the same layer on a batch small enough for the matrix kernel
+    n = 3
+    sp_s, v_s = (S.fused_temporal_conv_add_lif_state([x[:n].contiguous() for x in dx], [dev(r[:n], dtype) for r in rs], dw, db,
+                                                     dv[:n].contiguous() if tensor_v else dv, [1, 1], [0, 0], [1, 1], 1, *lif, False)
+                 if residual else
+                 S.fused_temporal_pointwise_conv_lif_state([x[:n].contiguous() for x in dx], dw, db,
+                                                           dv[:n].contiguous() if tensor_v else dv, [1, 1], [0, 0], [1, 1], 1, *lif, False))
+    assert last_conv_plan()["kernel"] == "matrix", last_conv_plan()
+    check(sp_s, v_s, (ref[0][:, :n], ref[1][:n], ref[2][:, :n]), v_threshold=lif[0], v_dtype=F32, what=f"small pointwise {Cin}->{Cout} {H}x{W} on the matrix kernel")
+    _no_fallback(hip_ops, 2)
+
+
 DENSE_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif, T, N, residual, tensor v_init
     (64, 64, 16, 16, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False),    # whole tiles, 16-byte runs
     (128, 128, 14, 14, 3, 1, 1, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, True),    # K split across waves, 8-byte runs

@@ -324,7 +324,12 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     // Dense layers whose input channels fill whole groups of 8 (or fit a single group) go to the 8-wave matrix kernel
     // whatever their intensity (its per-tile cost is the lower one); pointwise layers stay with the pointwise kernel unless
     // they are compute bound (deep 512 -> 512 layers: an image is then one row of H * W pixels to the matrix kernel).
-    const bool matrix_candidate = (!pointwise || flops / bytes >= 200.0) && (Cin % 8 == 0 || Cin < 8);
+    // Measured on 1x1 layers of more than one channel chunk (T = 4, us on the pointwise / the matrix kernel): 256 -> 256 at 28^2
+    // x 32 images (128 MB) 79 / 55, 256 -> 512 at 28^2 x 16 (103 MB) 78 / 51, 192 -> 64 at 28^2 x 32 (58 MB) 57 / 32, 384 -> 96 at
+    // 14^2 x 32 (26 MB) 42 / 36, 1024 -> 64 at 8^2 x 8 56 / 54, but 256 -> 128 at 56^2 x 32 (360 MB) 90 / 139: the pointwise
+    // kernel keeps the layers that are mostly memory traffic.
+    const bool pointwise_to_matrix = pointwise && (flops / bytes >= 200.0 || (Cin > 128 && bytes < 200.0e6));
+    const bool matrix_candidate = (!pointwise || pointwise_to_matrix) && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
     Plan pl = {};
     bool planned = false;
