@@ -145,6 +145,26 @@ def test_lif_avgpool_linear(hip_ops, dtype, T, N, C, H, W, K, bias):
     _no_fallback(hip_ops, 1)
 
 
+@pytest.mark.parametrize("dtype", [BF16, F16])
+@pytest.mark.parametrize("T,N,C,H,W,K", [(4, 21, 64, 12, 12, 70), (16, 9, 96, 8, 8, 100), (4, 64, 512, 14, 14, 1000), (8, 8, 160, 9, 9, 64)])
+def test_lif_avgpool_linear_on_batches_with_large_counts(hip_ops, dtype, T, N, C, H, W, K):
+    """Batches of 8 samples or more with 64 classes or more and C % 32 == 0 take the matrix-core GEMV, which splits a spike
+    count into count & 255 and count >> 8: strong inputs make most planes count beyond 255 (ragged class and sample tiles,
+    fewer channel steps than waves, a last round of steps that not every wave has)."""
+    g = gen(360 + C)
+    x = q(torch.randn(T, N, C, H, W, generator=g) * 0.5 + 2.0, dtype)
+    w = q(torch.randn(K, C, generator=g) * 0.05, dtype)
+    b = q(torch.randn(K, generator=g) * 0.05, dtype)
+    ref_out, ref_v, _, ref_spikes = O.temporal_lif_avgpool_linear(x, torch.tensor(0.0), w, b, *LIF)
+    assert ref_spikes.sum(dim=(0, 3, 4)).median() > 255
+    out, v = S.fused_temporal_lif_avgpool_linear(dev(x, dtype), zero_v(F32), dev(w, dtype), dev(b, dtype), *LIF, False)
+    assert torch.equal(v.cpu(), ref_v)
+    tol = 8e-3 if dtype == BF16 else 2e-3
+    assert torch.allclose(out.float().cpu(), ref_out, rtol=tol, atol=tol), (out.float().cpu() - ref_out).abs().max()
+    assert ref_out.abs().max() > 0.5      # the sums are far from zero: a dropped high part would show
+    _no_fallback(hip_ops, 1)
+
+
 @pytest.mark.parametrize("N,C,H,W", [(6, 64, 7, 7), (3, 5, 3, 3), (40, 128, 1, 1)])
 def test_lif_avgpool_linear_tensor_v_init(hip_ops, N, C, H, W):
     """A membrane tensor as initial state (vector and element-wise paths of the pooling kernel)."""

@@ -5,7 +5,7 @@
 // where count[n, c] is the number of spikes of plane (n, c) over all T steps: the pooled activations are never
 // materialised per step. Launch 1 streams x once (HBM-bound, 16-byte accesses where the operands allow), keeps the membrane
 // in registers, counts spikes per plane in LDS and writes the integer counts to the workspace; launch 2 is a small GEMV
-// over the counts with wave-shuffle reductions.
+// over the counts: wave-shuffle reductions for a few samples or classes, the matrix cores for batches.
 #include <algorithm>
 #include <mutex>
 #include <type_traits>
@@ -293,6 +293,88 @@ __global__ __launch_bounds__(kThreads) void count_linear_vec_kernel(const int* _
     }
 }
 
+// Matrix-core variant for batches of samples (16-bit weights, C a multiple of 32, counts below 65536): a workgroup owns 16
+// classes x 16 samples; its 4 waves deal the steps of 32 channels among themselves and meet in LDS, summed in wave order.
+// A count is exact in neither 16-bit format, so it enters as two exact operands, count & 255 and count >> 8, against the
+// same weight fragment: out = (W . low + 256 * (W . high)) / HW + T * b with fp32 accumulation.
+typedef __bf16 tail_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 tail_f16x8 __attribute__((ext_vector_type(8)));
+typedef float tail_f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kMmTile = 16;
+constexpr int kMmMaxCount = 65535;
+constexpr int kMmMinSamples = 8;   // below 8 samples or 64 classes the tile is mostly padding: the shuffle kernel is quicker
+constexpr int kMmMinClasses = 64;
+
+template <typename XT>
+__device__ __forceinline__ tail_f32x4 tail_mfma(snnf_u32x4 a, snnf_u32x4 b, tail_f32x4 c) {
+    if constexpr (dtype_of<XT>::value == SNNF_F16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(tail_f16x8, a), __builtin_bit_cast(tail_f16x8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tail_bf16x8, a), __builtin_bit_cast(tail_bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+// Two integers below 256 as a pair of 16-bit floats (exact in both formats).
+template <typename XT>
+__device__ __forceinline__ uint32_t small_pair(int a, int b) {
+    if constexpr (dtype_of<XT>::value == SNNF_F16) {
+        return float_to_f16_bits(static_cast<float>(a)) | (float_to_f16_bits(static_cast<float>(b)) << 16);
+    } else {
+        return (__float_as_uint(static_cast<float>(a)) >> 16) | (__float_as_uint(static_cast<float>(b)) & 0xffff0000u);
+    }
+}
+
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void count_linear_mm_kernel(const int* __restrict__ counts, int N, int C, int K,
+                                                                   const XT* __restrict__ W, const XT* __restrict__ bias,
+                                                                   XT* __restrict__ out, float inv_hw, float steps) {
+    static_assert(sizeof(XT) == 2, "16-bit weights");
+    __shared__ float part[kThreads / 64][64 * 4];
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int k0 = blockIdx.x * kMmTile;
+    const int n0 = blockIdx.y * kMmTile;
+    // Operand order of v_mfma_f32_16x16x32: lane l holds 8 consecutive channels, 8 * (l / 16) on, of row l % 16.
+    const int row = lane & 15;
+    const int sub = (lane >> 4) * 8;
+    const XT* __restrict__ w_row = W + static_cast<int64_t>(min(k0 + row, K - 1)) * C + sub;         // rows beyond K: re-read, not stored
+    const int* __restrict__ c_row = counts + static_cast<int64_t>(min(n0 + row, N - 1)) * C + sub;   // samples beyond N likewise
+    tail_f32x4 acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
+    tail_f32x4 acc_hi = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int ksteps = C >> 5;
+#pragma unroll 4
+    for (int ks = wave; ks < ksteps; ks += kThreads / 64) {
+        const snnf_u32x4 wf = *reinterpret_cast<const snnf_u32x4*>(w_row + ks * 32);
+        const Pack<int, 4> c0 = *reinterpret_cast<const Pack<int, 4>*>(c_row + ks * 32);
+        const Pack<int, 4> c1 = *reinterpret_cast<const Pack<int, 4>*>(c_row + ks * 32 + 4);
+        snnf_u32x4 lo, hi;
+        lo[0] = small_pair<XT>(c0.v[0] & 255, c0.v[1] & 255);
+        lo[1] = small_pair<XT>(c0.v[2] & 255, c0.v[3] & 255);
+        lo[2] = small_pair<XT>(c1.v[0] & 255, c1.v[1] & 255);
+        lo[3] = small_pair<XT>(c1.v[2] & 255, c1.v[3] & 255);
+        hi[0] = small_pair<XT>(c0.v[0] >> 8, c0.v[1] >> 8);
+        hi[1] = small_pair<XT>(c0.v[2] >> 8, c0.v[3] >> 8);
+        hi[2] = small_pair<XT>(c1.v[0] >> 8, c1.v[1] >> 8);
+        hi[3] = small_pair<XT>(c1.v[2] >> 8, c1.v[3] >> 8);
+        acc_lo = tail_mfma<XT>(wf, lo, acc_lo);
+        acc_hi = tail_mfma<XT>(wf, hi, acc_hi);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part[wave][lane * 4 + j] = fmaf(256.0f, acc_hi[j], acc_lo[j]);
+    __syncthreads();
+    // Thread t finishes output t of the tile: class 4 * (l / 16) + j of sample l % 16, with l = t / 4 and j = t % 4.
+    float sum = part[0][threadIdx.x];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) sum += part[w][threadIdx.x];
+    const int l = threadIdx.x >> 2;
+    const int k = k0 + 4 * (l >> 4) + (threadIdx.x & 3);
+    const int n = n0 + (l & 15);
+    if (k < K && n < N) {
+        const float bv = bias != nullptr ? steps * to_float(bias[k]) : 0.0f;
+        out[static_cast<int64_t>(n) * K + k] = from_float<XT>(sum * inv_hw + bv);
+    }
+}
+
 template <typename XT, typename VT>
 int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void* v_out, int* counts,
         const LifParams& lif, hipStream_t stream) {
@@ -340,8 +422,17 @@ int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void*
 }
 
 template <typename XT>
-void run_linear(bool vec, dim3 grid, size_t lds, hipStream_t hs, const int* counts, int C, int K, const void* W, const void* bias,
-                void* out, float inv_hw, float steps) {
+void run_linear(bool vec, bool matrix, dim3 grid, size_t lds, hipStream_t hs, const int* counts, int C, int K, const void* W,
+                const void* bias, void* out, float inv_hw, float steps) {
+    if constexpr (sizeof(XT) == 2) {
+        if (matrix) {
+            const int N = static_cast<int>(grid.y);
+            const dim3 mgrid((K + kMmTile - 1) / kMmTile, (N + kMmTile - 1) / kMmTile);
+            count_linear_mm_kernel<XT><<<mgrid, kThreads, 0, hs>>>(counts, N, C, K, static_cast<const XT*>(W),
+                                                                  static_cast<const XT*>(bias), static_cast<XT*>(out), inv_hw, steps);
+            return;
+        }
+    }
     if (vec) {
         const int N = static_cast<int>(grid.y);
         const dim3 vgrid(grid.x, (N + kSamplesPerWave - 1) / kSamplesPerWave);
@@ -411,9 +502,10 @@ int lif_pool_linear_impl(const char* who, const void* const* xs, int T, int N, i
     const float inv_hw = 1.0f / static_cast<float>(HW);
     const float steps = static_cast<float>(T);
     const bool vec = C % kVec == 0 && aligned_to(fc_weight, 16);
-    if (x_dtype == SNNF_F32) run_linear<float>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
-    else if (x_dtype == SNNF_BF16) run_linear<bf16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
-    else run_linear<f16_t>(vec, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
+    const bool matrix = vec && x_dtype != SNNF_F32 && C % 32 == 0 && N >= kMmMinSamples && K >= kMmMinClasses && static_cast<int64_t>(T) * HW <= kMmMaxCount;
+    if (x_dtype == SNNF_F32) run_linear<float>(vec, false, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
+    else if (x_dtype == SNNF_BF16) run_linear<bf16_t>(vec, matrix, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
+    else run_linear<f16_t>(vec, matrix, grid, lds, hs, counts, C, K, fc_weight, fc_bias, out_sum, inv_hw, steps);
     return check_launch(who);
 }
 
