@@ -224,21 +224,24 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
         }
     };
 
-    // ---- tile walk: pixel tiles congruent to this workgroup's XCD; consecutive work items = output-channel tiles (an XCD's
-    // L2 then serves every activation tile to all of its output-channel tiles). Layers whose weights outweigh their
+    // ---- tile walk: an XCD takes a contiguous range of the pixel tiles (neighbouring tiles share halo pixels and, where a
+    // tile row is shorter than a cache line, the lines they store to: both then meet in one L2); consecutive work items =
+    // output-channel tiles (an XCD's L2 serves every activation tile to all of its output-channel tiles). Layers whose weights outweigh their
     // activations turn this around (oc_major): an XCD takes the output-channel tiles congruent to it for all pixel tiles, so
     // that its L2 holds an eighth of the weights instead of all of them.
     const int xcd = blockIdx.x & 7;
     const int slots_per_xcd = gridDim.x >> 3;
     const int n_px_tiles = g.img_groups * g.tiles_img;       // a tile spans TI images (TI > 1: whole output planes)
     const int oc_per_xcd = g.oc_major ? (g.oc_tiles >> 3) : g.oc_tiles;
-    const int work_per_xcd = (g.oc_major ? n_px_tiles : ((n_px_tiles + 7) >> 3)) * oc_per_xcd;
+    const int px_base = n_px_tiles >> 3, px_rem = n_px_tiles & 7;
+    const int px_start = g.oc_major ? 0 : xcd * px_base + min(xcd, px_rem);
+    const int work_per_xcd = (g.oc_major ? n_px_tiles : px_base + (xcd < px_rem ? 1 : 0)) * oc_per_xcd;
     int work = blockIdx.x >> 3;
     int oc_tile = 0, img = 0, oh0 = 0, ow0 = 0;
     auto decode = [&](int w, int& oc_t, int& n, int& r0, int& c0) __attribute__((always_inline)) -> bool {
         if (w >= work_per_xcd) return false;
         const int pt = fast_div(w, g.d_oc_tiles);
-        const int px_tile = g.oc_major ? pt : pt * 8 + xcd;
+        const int px_tile = px_start + pt;
         if (px_tile >= n_px_tiles) return false;
         oc_t = g.oc_major ? (w - pt * oc_per_xcd) * 8 + xcd : w - pt * g.oc_tiles;
         const int group = fast_div(px_tile, g.d_tiles_img);
