@@ -134,7 +134,14 @@ def packed_step_pointers(x_seq: torch.Tensor):
     return arr
 
 
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(device: torch.device) -> ctypes.c_void_p:
+    """The stream PyTorch would launch on for `device` right now, as a raw hipStream_t."""
+    if _raw_current_stream is not None:     # the handle without a Stream object around it: a few microseconds per operator call
+        index = device.index
+        return ctypes.c_void_p(_raw_current_stream(torch.cuda.current_device() if index is None else index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
