@@ -167,8 +167,9 @@ def test_random_linear_scan_and_tail_cases(hip_ops, seed, cases):
             check(sp, v, ref, v_threshold=lif[0], v_dtype=vdtype, what=what, max_rate=2e-4)
         else:
             T, N, C = rnd.choice([1, 2, 3, 4, 4, 8, 16]), rnd.randint(1, 20), rnd.choice([3, 8, 32, 50, 64, 128, 512])
-            H, W, K = rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 3, 10, 17, 100, 1000])
-            x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + 0.15, dtype)
+            H, W, K = rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 3, 10, 17, 64, 70, 100, 1000])
+            mean = rnd.choice([0.15, 0.15, 2.0])     # strong inputs: spike counts beyond 255 (the matrix-core GEMV splits them)
+            x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + mean, dtype)
             w, b = q(torch.randn(K, C, generator=g) * 0.05, dtype), q(torch.randn(K, generator=g) * 0.05, dtype)
             v_ref, v_dev = _membrane(rnd, g, (N, C, H, W), F32)
             what = f"case {case}: tail T={T} N={N} C={C} {H}x{W} K={K} {dtype} lif={lif}"
