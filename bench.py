@@ -560,6 +560,20 @@ def main() -> int:
                 "mfma": None if groups > 1 else _roofline("mfma", flops, ms, traffic),
             }
         dominant = max(kernels.items(), key=lambda kv: kv[1]["ms"])
+        # The depthwise layer with a bit-packed spike output (one byte = 8 pixels of a row): same kernel, another store.
+        # Reported beside the operator's own figure; the block step above keeps the dense operators.
+        for i, xs in enumerate(inputs):
+            _, w, b, stride, _, groups = prep.layers[i]
+            if groups > 1 and stride == [1, 1] and xs[0].dtype != torch.float32 and int(xs[0].shape[3]) % 8 == 0:
+                from triton_snn_fusion_amd.runtime import hip_blocked_backend as blocked
+                ms, how = _time_kernel(lambda xs=xs, w=w, b=b: blocked.depthwise_conv_lif_rowbits(xs, w, b, prep.lif), args.steps,
+                                       max(3, args.warmup // 2))
+                n, c, h, wd = (int(d) for d in xs[0].shape)
+                nbytes = len(xs) * n * c * h * wd * prep.esize + len(xs) * n * c * h * wd // 8 + n * c * h * wd * 4 + c * 10 * prep.esize
+                kernels[f"layer{i}_depthwise3x3_packed_spikes"] = {
+                    "ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "flops": kernels[f"layer{i}_depthwise3x3"]["flops"],
+                    "hbm": _roofline("hbm", nbytes, ms, None), "mfma": None,
+                    "spike_bytes": {"dense": len(xs) * n * c * h * wd * prep.esize, "packed": len(xs) * n * c * h * wd // 8}}
         ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
         bound = "mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS and dominant[1]["mfma"] is not None else "hbm"
         result["roofline"] = dict(dominant[1][bound], kernel=dominant[0], traffic_measured_in=TRAFFIC_PROFILE)

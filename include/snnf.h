@@ -99,6 +99,23 @@ int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int 
                        float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * The same operator (stride 1, bf16 / fp16 activations, W % 8 == 0, fp32 membrane) with a bit-packed spike output: one
+ * byte holds the spikes of 8 consecutive pixels of a row (bit j = pixel 8 x + j), 16 times fewer bytes than the dense
+ * 0 / 1 elements the reference's kernel stores (kernels/benchmark_conv_lif_temporal_general.py:707-708, depthwise
+ * emitter :713-817). Activations, residuals and membranes must be 16-byte aligned.
+ *   spike_bits : [T, N, C, H, W / 8] bytes, `bits_step_stride` BYTES between timesteps
+ *   v_init     : [N, C, H, W] fp32 or NULL (zeros);  v_out : the same or NULL (final membrane not stored; needs
+ *                T <= SNNF_MAX_T_PER_LAUNCH)
+ * snnf_rowbits_unpack turns `bytes` such bytes into 8 * bytes dense 0 / 1 elements of x_dtype (16-byte aligned).
+ */
+int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T,
+                               int N, int C, int H, int W, int x_dtype,
+                               const void* weight, const void* bias, const void* v_init,
+                               void* spike_bits, int64_t bits_step_stride, void* v_out,
+                               float v_threshold, float v_reset, float tau, void* stream);
+int snnf_rowbits_unpack(const void* bits, void* dense, int64_t bytes, int x_dtype, void* stream);
+
+/*
  * LIF -> global average pool -> Linear, summed over T.
  *   out_sum[n, k] = sum_t ( fc_weight[k, :] . mean_hw(s_t[n, :, :, :]) + fc_bias[k] )
  * Replaces run_fused_temporal_lif_avgpool_linear_kernel (kernels/generated_temporal_lif_avgpool_linear_kernel.py:120-209)

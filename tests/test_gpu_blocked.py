@@ -256,3 +256,66 @@ def test_blocked_conv_rejects_what_it_does_not_take(B):
         B.conv_lif_blocked(x, torch.zeros(64, 1, 3, 3, device=DEV, dtype=BF16), None, [1, 1], [1, 1], LIF)
     with pytest.raises(RuntimeError, match="unsupported_padding"):
         B.conv_lif_blocked(x, w, None, [1, 1], [2, 2], LIF)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Depthwise 3x3 + LIF with row-packed spikes (one byte = 8 consecutive pixels of a row)
+# ---------------------------------------------------------------------------------------------------------------
+def _ref_rowbits(s):
+    """Dense 0/1 [..., W] -> [..., W / 8] uint8, bit j = pixel 8 x + j."""
+    shape = tuple(s.shape[:-1]) + (s.shape[-1] // 8, 8)
+    weights = 2 ** torch.arange(8, dtype=torch.int32)
+    return ((s != 0).to(torch.int32).reshape(shape) * weights).sum(-1).to(torch.uint8)
+
+
+ROWBITS_CASES = [  # dtype, N, C, H, W, T, lif, residual, tensor v_init, want_v
+    (BF16, 2, 16, 28, 56, 4, (1.0, 0.0, 2.0), False, False, True),     # several planes per workgroup
+    (BF16, 1, 8, 56, 56, 4, (1.0, 0.0, 2.0), False, False, False),     # the headline plane, no membrane output
+    (F16, 2, 5, 9, 16, 3, (1.0, -1.0, 2.0), True, True, True),         # soft reset (general neuron), residual, v_init
+    (BF16, 3, 7, 8, 8, 17, (0.5, 0.0, 1.0), False, True, True),        # two launch windows (16 + 1), IF neuron
+    (F16, 1, 3, 96, 160, 2, (1.0, 0.0, 3.0), True, False, True),       # planes cut into row bands, tau not a power of two
+    (BF16, 2, 4, 7, 24, 1, (1.0, 0.0, 2.0), False, False, True),       # a single step
+]
+
+
+@pytest.mark.parametrize("dtype,N,C,H,W,T,lif,residual,tensor_v,want_v", ROWBITS_CASES)
+def test_depthwise_with_row_packed_spikes_against_the_oracle(B, dtype, N, C, H, W, T, lif, residual, tensor_v, want_v):
+    g = gen(4100 + C + H + T)
+    xs = [spikes((N, C, H, W), 0.3, g) for _ in range(T)]
+    w = q(torch.randn(C, 1, 3, 3, generator=g) * 0.5, dtype)
+    b = q(torch.randn(C, generator=g) * 0.1, dtype)
+    rs = [q(torch.randn(N, C, H, W, generator=g) * 0.3, dtype) for _ in range(T)] if residual else None
+    v0 = torch.randn(N, C, H, W, generator=g) * 0.3 if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif(xs, w, b, v0, (1, 1), (1, 1), (1, 1), C, *lif, residuals=rs)
+    dx = [dev(x, dtype) for x in xs]
+    dr = [dev(r, dtype) for r in rs] if residual else None
+    bits, v = B.depthwise_conv_lif_rowbits(dx, dev(w, dtype), dev(b, dtype), lif, residuals=dr,
+                                           v_init=dev(v0, F32) if tensor_v else None, want_v=want_v)
+    assert bits.dtype == torch.uint8 and tuple(bits.shape) == (T, N, C, H, W // 8)
+    assert (v is None) == (not want_v)
+    dense = B.unpack_rowbits(bits, dtype)
+    assert tuple(dense.shape) == (T, N, C, H, W) and dense.dtype == dtype
+    assert torch.equal(_ref_rowbits(dense.float().cpu()), bits.cpu())                 # the unpacker is exact
+    v_chk = v if want_v else dev(ref[1], F32)                                          # no membrane output: spikes only
+    check(dense, v_chk, ref, v_threshold=lif[0], what=f"depthwise row bits {C}x{H}x{W} T={T}")
+    # bit for bit the dense operator's spikes and membrane (same kernel, another store)
+    import triton_snn_fusion_amd.runtime.snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=True)
+    S = torch.ops.snn_custom
+    dv = dev(v0, F32) if tensor_v else torch.zeros((), device=DEV, dtype=F32)
+    if residual:
+        s_d, v_d = S.fused_temporal_conv_add_lif_state_depthwise(dx, dr, dev(w, dtype), dev(b, dtype), dv, [1, 1], [1, 1], [1, 1], C, *lif, False)
+    else:
+        s_d, v_d = S.fused_temporal_depthwise_conv_lif_state(dx, dev(w, dtype), dev(b, dtype), dv, [1, 1], [1, 1], [1, 1], C, *lif, False)
+    assert torch.equal(s_d, dense)
+    if want_v:
+        assert torch.equal(v_d, v)
+
+
+def test_depthwise_row_packed_spikes_reject_what_they_do_not_take(B):
+    g = gen(4200)
+    w, b = dev(torch.randn(4, 1, 3, 3, generator=g), BF16), dev(torch.randn(4, generator=g), BF16)
+    with pytest.raises(RuntimeError, match="unsupported_shape"):
+        B.depthwise_conv_lif_rowbits([dev(spikes((1, 4, 8, 12), 0.3, g), BF16)], w, b, LIF)
+    with pytest.raises(RuntimeError, match="unsupported_dtype"):
+        B.depthwise_conv_lif_rowbits([dev(spikes((1, 4, 8, 16), 0.3, g), F32)], w.float(), b.float(), LIF)

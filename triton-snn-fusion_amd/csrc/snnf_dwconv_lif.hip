@@ -62,6 +62,7 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
                                                                  XT* __restrict__ spikes, int64_t spike_step_stride,
                                                                  VT* __restrict__ v_out, LifParams lif) {
     extern __shared__ __align__(16) float tile[];
+    constexpr bool BITS = false;                       // dense 0 / 1 spikes only (the packed output is the dot-product kernel's)
     constexpr int IN_COLS = (PX - 1) * STRIDE + 3;
     constexpr int KL = kLoadSlots<STRIDE>();           // input vectors a thread prefetches per timestep
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
@@ -142,13 +143,21 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
 #pragma unroll
         for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const Pack<XT, PX>*>(x + ld_src[k]);
     };
-    Pack<XT, PX> pend[kItems];
+    Pack<XT, PX> pend[BITS ? 1 : kItems];
+    uint32_t pend_bits[BITS ? kItems : 1];
     int pend_t = -1;
     auto flush = [&]() __attribute__((always_inline)) {
-        XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+        if constexpr (BITS) {
+            unsigned char* __restrict__ out = reinterpret_cast<unsigned char*>(spikes) + pend_t * spike_step_stride + (out_base >> 3);
 #pragma unroll
-        for (int k = 0; k < kItems; ++k)
-            if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+            for (int k = 0; k < kItems; ++k)
+                if (item_live[k]) out[item_out[k] >> 3] = static_cast<unsigned char>(pend_bits[k]);
+        } else {
+            XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+#pragma unroll
+            for (int k = 0; k < kItems; ++k)
+                if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+        }
         pend_t = -1;
     };
 
@@ -214,23 +223,28 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_kernel(StepPtrs xs, St
 #pragma unroll
                 for (int j = 0; j < PX; ++j) acc[j] += r8[j];
             }
+            uint32_t byte = 0;
 #pragma unroll
             for (int j = 0; j < PX; ++j) {
+                bool fired;
                 if constexpr (STD) {
                     const float h = v[k][j] + (acc[j] - v[k][j]) * lif.inv_tau;
-                    const bool fired = h >= lif.v_threshold;
+                    fired = h >= lif.v_threshold;
                     v[k][j] = fired ? lif.v_reset : h;
-                    pend[k].v[j] = spike_value<XT>(fired);
                 } else {
-                    pend[k].v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
+                    fired = lif_step(acc[j], v[k][j], lif);
                 }
+                if constexpr (BITS) byte |= fired ? (1u << j) : 0u;
+                else pend[k].v[j] = spike_value<XT>(fired);
             }
+            if constexpr (BITS) pend_bits[k] = byte;
         }
         pend_t = t;
         buf ^= 1;
     }
     if (pend_t >= 0) flush();
 
+    if (BITS && v_out == nullptr) return;
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (!item_live[k]) continue;
@@ -310,7 +324,9 @@ __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(dw_f16x2, a), __builtin_bit_cast(dw_f16x2, b), c, false);
 }
 
-template <typename XT, typename VT, bool STD>
+// BITS: the spikes of a strip and timestep leave as one byte (bit j = pixel 8 x + j of the row) instead of eight 16-bit
+// values: [T][N][C][Ho][Wo / 8] bytes, `spike_step_stride` then counts bytes; the final membrane is optional.
+template <typename XT, typename VT, bool STD, bool BITS = false>
 __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs, StepPtrs residuals, int has_residual,
                                                                      int T, DwGeom g, const XT* __restrict__ weight,
                                                                      const XT* __restrict__ bias,
@@ -408,13 +424,21 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
 #pragma unroll
         for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const dw_u32x4*>(x + ld_src[k]);
     };
-    Pack<XT, PX> pend[kItems];
+    Pack<XT, PX> pend[BITS ? 1 : kItems];
+    uint32_t pend_bits[BITS ? kItems : 1];
     int pend_t = -1;
     auto flush = [&]() __attribute__((always_inline)) {
-        XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+        if constexpr (BITS) {
+            unsigned char* __restrict__ out = reinterpret_cast<unsigned char*>(spikes) + pend_t * spike_step_stride + (out_base >> 3);
 #pragma unroll
-        for (int k = 0; k < kItems; ++k)
-            if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+            for (int k = 0; k < kItems; ++k)
+                if (item_live[k]) out[item_out[k] >> 3] = static_cast<unsigned char>(pend_bits[k]);
+        } else {
+            XT* __restrict__ out = spikes + pend_t * spike_step_stride + out_base;
+#pragma unroll
+            for (int k = 0; k < kItems; ++k)
+                if (item_live[k]) *reinterpret_cast<Pack<XT, PX>*>(out + item_out[k]) = pend[k];
+        }
         pend_t = -1;
     };
 
@@ -460,23 +484,28 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
 #pragma unroll
                 for (int j = 0; j < PX; ++j) acc[j] += r8[j];
             }
+            uint32_t byte = 0;
 #pragma unroll
             for (int j = 0; j < PX; ++j) {
+                bool fired;
                 if constexpr (STD) {
                     const float h = v[k][j] + (acc[j] - v[k][j]) * lif.inv_tau;
-                    const bool fired = h >= lif.v_threshold;
+                    fired = h >= lif.v_threshold;
                     v[k][j] = fired ? lif.v_reset : h;
-                    pend[k].v[j] = spike_value<XT>(fired);
                 } else {
-                    pend[k].v[j] = spike_value<XT>(lif_step(acc[j], v[k][j], lif));
+                    fired = lif_step(acc[j], v[k][j], lif);
                 }
+                if constexpr (BITS) byte |= fired ? (1u << j) : 0u;
+                else pend[k].v[j] = spike_value<XT>(fired);
             }
+            if constexpr (BITS) pend_bits[k] = byte;
         }
         pend_t = t;
         buf ^= 1;
     }
     if (pend_t >= 0) flush();
 
+    if (BITS && v_out == nullptr) return;
 #pragma unroll
     for (int k = 0; k < kItems; ++k) {
         if (!item_live[k]) continue;
@@ -488,7 +517,7 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
 }
 
 // Launcher of the packed dot-product kernel: the planning of `launch` with 16-bit rows.
-template <typename XT, typename VT>
+template <typename XT, typename VT, bool BITS = false>
 int launch_dot(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g, const void* weight, const void* bias,
                const void* v_init, void* spikes, int64_t spike_step_stride, void* v_out, const LifParams& lif,
                hipStream_t stream) {
@@ -524,11 +553,11 @@ int launch_dot(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGe
     const int64_t blocks = static_cast<int64_t>((g.planes + g.PB - 1) / g.PB) * g.bands;
     if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: too many planes");
     if (lif.charge_mode == CHARGE_SCALE && !lif.soft_reset) {
-        dwconv3x3_lif_dot_kernel<XT, VT, true><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+        dwconv3x3_lif_dot_kernel<XT, VT, true, BITS><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
             xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
             static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
     } else {
-        dwconv3x3_lif_dot_kernel<XT, VT, false><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+        dwconv3x3_lif_dot_kernel<XT, VT, false, BITS><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
             xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
             static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
     }
@@ -556,8 +585,92 @@ int dispatch_stride(int stride, int px, const StepPtrs& xs, const StepPtrs& res,
     return dispatch_px<XT, VT, 2>(px, xs, res, has_res, T, g, weight, bias, v_init, spikes, sss, v_out, lif, stream);
 }
 
+// One byte of row-packed spikes -> eight 0 / 1 elements (16 bytes).
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void rowbits_unpack_kernel(const unsigned char* __restrict__ bits, XT* __restrict__ dense, int64_t bytes) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= bytes) return;
+    const uint32_t b = bits[i];
+    Pack<XT, 8> out;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out.v[j] = spike_value<XT>(((b >> j) & 1u) != 0u);
+    *reinterpret_cast<Pack<XT, 8>*>(dense + i * 8) = out;
+}
+
 }  // namespace
 }  // namespace snnf
+
+extern "C" int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T, int N, int C, int H, int W,
+                                          int x_dtype, const void* weight, const void* bias, const void* v_init,
+                                          void* spike_bits, int64_t bits_step_stride, void* v_out,
+                                          float v_threshold, float v_reset, float tau, void* stream) {
+    using namespace snnf;
+    const char* who = "snnf_dwconv3x3_lif_rowbits";
+    if (xs == nullptr || weight == nullptr || bias == nullptr || spike_bits == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs, weight, bias and spike_bits must be non-null", who);
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: T=%d N=%d C=%d H=%d W=%d", who, T, N, C, H, W);
+    if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: activations must be bf16 or fp16", who);
+    if (W % 8 != 0) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: W=%d is not a multiple of 8", who, W);
+    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_tau: tau must be nonzero", who);
+    if (static_cast<int64_t>(N) * C > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "%s: N*C too large", who);
+    if (v_out == nullptr && T > SNNF_MAX_T_PER_LAUNCH)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: v_out is required beyond %d timesteps (the membrane passes from launch to launch)", who,
+                    SNNF_MAX_T_PER_LAUNCH);
+    const int64_t frame_bytes = static_cast<int64_t>(N) * C * H * (W / 8);
+    if (bits_step_stride < frame_bytes) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: bits_step_stride=%lld is less than one timestep (%lld bytes)", who,
+                                                    (long long)bits_step_stride, (long long)frame_bytes);
+    bool aligned = (v_init == nullptr || aligned_to(v_init, 16)) && (v_out == nullptr || aligned_to(v_out, 16));
+    for (int t = 0; t < T; ++t) {
+        if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs[%d] is null", who, t);
+        if (residuals != nullptr && residuals[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: residuals[%d] is null", who, t);
+        aligned = aligned && aligned_to(xs[t], 16) && (residuals == nullptr || aligned_to(residuals[t], 16));
+    }
+    if (!aligned) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_alignment: activations, residuals and membranes must be 16-byte aligned", who);
+
+    DwGeom g = {};
+    g.planes = N * C;
+    g.C = C;
+    g.H = H;
+    g.W = W;
+    g.Ho = H;
+    g.Wo = W;
+    const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
+    hipStream_t hs = as_stream(stream);
+    for (int t0 = 0; t0 < T; t0 += SNNF_MAX_T_PER_LAUNCH) {
+        const int tw = (T - t0) < SNNF_MAX_T_PER_LAUNCH ? (T - t0) : SNNF_MAX_T_PER_LAUNCH;
+        StepPtrs xp = {}, rp = {};
+        for (int t = 0; t < tw; ++t) {
+            xp.p[t] = xs[t0 + t];
+            if (residuals != nullptr) rp.p[t] = residuals[t0 + t];
+        }
+        const void* vi = t0 == 0 ? v_init : v_out;
+        void* sp = static_cast<char*>(spike_bits) + static_cast<int64_t>(t0) * bits_step_stride;
+        const int has_res = residuals != nullptr ? 1 : 0;
+        const int rc = x_dtype == SNNF_BF16
+                           ? launch_dot<bf16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs)
+                           : launch_dot<f16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs);
+        if (rc != SNNF_OK) return rc;
+    }
+    return SNNF_OK;
+}
+
+extern "C" int snnf_rowbits_unpack(const void* bits, void* dense, int64_t bytes, int x_dtype, void* stream) {
+    using namespace snnf;
+    if (bits == nullptr || dense == nullptr || bytes < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_rowbits_unpack: bits and dense must be non-null, bytes >= 1");
+    if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_rowbits_unpack: unsupported_dtype: bf16 or fp16");
+    if (!aligned_to(dense, 16)) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_rowbits_unpack: dense must be 16-byte aligned");
+    const int64_t blocks = (bytes + kThreads - 1) / kThreads;
+    if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_rowbits_unpack: too many bytes");
+    hipStream_t hs = as_stream(stream);
+    if (x_dtype == SNNF_BF16)
+        rowbits_unpack_kernel<bf16_t><<<dim3(static_cast<unsigned>(blocks)), kThreads, 0, hs>>>(static_cast<const unsigned char*>(bits), static_cast<bf16_t*>(dense), bytes);
+    else
+        rowbits_unpack_kernel<f16_t><<<dim3(static_cast<unsigned>(blocks)), kThreads, 0, hs>>>(static_cast<const unsigned char*>(bits), static_cast<f16_t*>(dense), bytes);
+    return check_launch("snnf_rowbits_unpack");
+}
 
 extern "C" int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int T, int N, int C, int H, int W,
                                   int stride, int x_dtype, const void* weight, const void* bias, int w_dtype,

@@ -220,3 +220,50 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
         status = launch(torch.empty((x.N, cout, ho, wo), dtype=torch.float32, device=dev))
     _lib.check("snnf_conv_lif_blocked", status)
     return out, v_out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Depthwise 3x3 + LIF with row-packed spikes: one byte = the spikes of 8 consecutive pixels of a row (bit j = pixel 8 x + j).
+# A depthwise lane owns such a strip, so its spikes of a timestep leave as one byte instead of eight 16-bit elements.
+# ---------------------------------------------------------------------------------------------------------------
+def depthwise_conv_lif_rowbits(xs: Sequence[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor, lif: Sequence[float],
+                               residuals: Optional[Sequence[torch.Tensor]] = None, v_init: Optional[torch.Tensor] = None,
+                               want_v: bool = True):
+    """Depthwise 3x3 (stride 1, padding 1) + bias (+ residual) + LIF over the dense steps `xs` ([N, C, H, W] each, bf16 or
+    fp16, W % 8 == 0). Returns (spike bits [T, N, C, H, W / 8] uint8, final membrane [N, C, H, W] fp32 or None)."""
+    first = xs[0]
+    _check_dtype(first.dtype)
+    T = len(xs)
+    n, c, h, w = (int(d) for d in first.shape)
+    if tuple(weight.shape) != (c, 1, 3, 3) or weight.dtype != first.dtype or bias.dtype != first.dtype:
+        raise RuntimeError(f"unsupported_weight: depthwise weight [C, 1, 3, 3] and bias in the activation dtype expected, got {tuple(weight.shape)}")
+    if w % 8 != 0:
+        raise RuntimeError(f"unsupported_shape: rows of {w} pixels do not pack into whole bytes")
+    dev = first.device
+    steps = [x if x.is_contiguous() else x.contiguous() for x in xs]
+    res = [r if r.is_contiguous() else r.contiguous() for r in residuals] if residuals is not None else None
+    vi = None
+    if v_init is not None and isinstance(v_init, torch.Tensor) and v_init.dim() != 0:
+        if tuple(v_init.shape) != (n, c, h, w) or v_init.dtype != torch.float32 or v_init.device != dev:
+            raise RuntimeError("unsupported_membrane_state: v_init must be a float32 [N, C, H, W] tensor on the activations' device")
+        vi = v_init if v_init.is_contiguous() else v_init.contiguous()
+    bits = torch.empty((T, n, c, h, w // 8), dtype=torch.uint8, device=dev)
+    v_out = torch.empty((n, c, h, w), dtype=torch.float32, device=dev) if (want_v or T > _lib.SNNF_MAX_T_PER_LAUNCH) else None
+    wc = weight if weight.is_contiguous() else weight.contiguous()
+    bc = bias if bias.is_contiguous() else bias.contiguous()
+    _lib.check("snnf_dwconv3x3_lif_rowbits", _lib.lib().snnf_dwconv3x3_lif_rowbits(
+        _lib.step_pointers(steps), _lib.step_pointers(res) if res is not None else None, T, n, c, h, w, _lib.dtype_code(first.dtype),
+        wc.data_ptr(), bc.data_ptr(), _lib.ptr(vi), bits.data_ptr(), int(bits.stride(0)), _lib.ptr(v_out),
+        float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
+    return bits, (v_out if want_v else None)
+
+
+def unpack_rowbits(bits: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Row-packed spikes [..., W / 8] uint8 -> dense 0 / 1 elements [..., W] of `dtype` (bf16 or fp16)."""
+    _check_dtype(dtype)
+    if bits.dtype != torch.uint8 or not bits.is_contiguous():
+        raise RuntimeError("unsupported_layout: contiguous uint8 tensor of row-packed spikes expected")
+    dense = torch.empty(tuple(bits.shape[:-1]) + (int(bits.shape[-1]) * 8,), dtype=dtype, device=bits.device)
+    _lib.check("snnf_rowbits_unpack", _lib.lib().snnf_rowbits_unpack(bits.data_ptr(), dense.data_ptr(), bits.numel(), _lib.dtype_code(dtype),
+                                                                   _lib.current_stream(bits.device)))
+    return dense
