@@ -574,6 +574,33 @@ def main() -> int:
                     "ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "flops": kernels[f"layer{i}_depthwise3x3"]["flops"],
                     "hbm": _roofline("hbm", nbytes, ms, None), "mfma": None,
                     "spike_bytes": {"dense": len(xs) * n * c * h * wd * prep.esize, "packed": len(xs) * n * c * h * wd // 8}}
+                # ... and the pointwise layer behind it reading those bytes: the block with its intermediate spikes at one bit each.
+                if i + 1 < len(prep.layers) and prep.layers[i + 1][5] == 1 and tuple(prep.layers[i + 1][1].shape[2:]) == (1, 1) \
+                        and (h * wd) % 64 == 0 and prep.lif[1] == 0.0:
+                    _, w2, b2, _, _, _ = prep.layers[i + 1]
+                    cout = int(w2.shape[0])
+                    bits, _ = blocked.depthwise_conv_lif_rowbits(xs, w, b, prep.lif)
+                    try:
+                        ms2, how2 = _time_kernel(lambda: blocked.pointwise_conv_lif_from_rowbits(bits, w2, b2, prep.lif), args.steps,
+                                                 max(3, args.warmup // 2))
+                    except RuntimeError:      # a neuron or shape outside the fast variant
+                        continue
+                    T_ = len(xs)
+                    nbytes2 = T_ * n * c * h * wd // 8 + T_ * n * cout * h * wd * prep.esize + n * cout * h * wd * 4 + cout * (c + 1) * prep.esize
+                    flops2 = kernels[f"layer{i + 1}_pointwise1x1"]["flops"]
+                    kernels[f"layer{i + 1}_pointwise1x1_from_packed_spikes"] = {
+                        "ms": round(ms2, 4), "timed": how2, "algorithmic_bytes": nbytes2, "flops": flops2,
+                        "hbm": _roofline("hbm", nbytes2, ms2, None), "mfma": _roofline("mfma", flops2, ms2, None)}
+
+                    def packed_block(xs=xs, w=w, b=b, w2=w2, b2=b2):
+                        packed, _ = blocked.depthwise_conv_lif_rowbits(xs, w, b, prep.lif)
+                        return blocked.pointwise_conv_lif_from_rowbits(packed, w2, b2, prep.lif)
+                    ms3 = _time_graph(packed_block, args.steps, max(3, args.warmup // 2))
+                    result["block_with_packed_intermediate_spikes"] = {
+                        "ms_per_step": round(ms3, 4), "images_T_per_s": round(n * T_ / (ms3 * 1e-3), 1), "timed": "graph",
+                        "algorithmic_bytes": nbytes + nbytes2,
+                        "note": "depthwise -> pointwise with the intermediate spikes at one bit each (library entry points, not the "
+                                "operator boundary); inputs, outputs and both membranes as in the block step above"}
         ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
         bound = "mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS and dominant[1]["mfma"] is not None else "hbm"
         result["roofline"] = dict(dominant[1][bound], kernel=dominant[0], traffic_measured_in=TRAFFIC_PROFILE)

@@ -116,6 +116,21 @@ int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residua
 int snnf_rowbits_unpack(const void* bits, void* dense, int64_t bytes, int x_dtype, void* stream);
 
 /*
+ * Pointwise (1x1, stride 1) convolution + bias + LIF over T steps whose input spikes are row-packed as above: the
+ * consumer of snnf_dwconv3x3_lif_rowbits in a depthwise-separable block (the reference hands the depthwise layer's
+ * dense 0 / 1 tensor to run_fused_temporal_general with kernel key k1_s1_p0,
+ * kernels/benchmark_conv_lif_temporal_general.py:971-1323 as called from runtime/triton_convlif_backend.py:513-598).
+ * Same packed weight, arithmetic and outputs as snnf_conv_lif on the unpacked tensor.
+ *   xs_bits[t] : [N, Cin, H, W / 8] bytes;  spikes : [T, N, Cout, H, W] x_dtype (bf16 / fp16);  v_init (or NULL), v_out : fp32
+ * Takes what the pointwise kernel's fast variant takes: the common neuron (power-of-two tau, hard reset), Cin % 8 == 0,
+ * Cout % 32 == 0, H * W % 64 == 0, 16-byte aligned outputs and membranes; SNNF_ERR_UNSUPPORTED otherwise.
+ */
+int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, int H, int W, int x_dtype,
+                            const void* packed_weight, int Cout, const void* v_init,
+                            void* spikes, int64_t spike_step_stride, void* v_out,
+                            float v_threshold, float v_reset, float tau, void* stream);
+
+/*
  * LIF -> global average pool -> Linear, summed over T.
  *   out_sum[n, k] = sum_t ( fc_weight[k, :] . mean_hw(s_t[n, :, :, :]) + fc_bias[k] )
  * Replaces run_fused_temporal_lif_avgpool_linear_kernel (kernels/generated_temporal_lif_avgpool_linear_kernel.py:120-209)

@@ -319,3 +319,71 @@ def test_depthwise_row_packed_spikes_reject_what_they_do_not_take(B):
         B.depthwise_conv_lif_rowbits([dev(spikes((1, 4, 8, 12), 0.3, g), BF16)], w, b, LIF)
     with pytest.raises(RuntimeError, match="unsupported_dtype"):
         B.depthwise_conv_lif_rowbits([dev(spikes((1, 4, 8, 16), 0.3, g), F32)], w.float(), b.float(), LIF)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Pointwise conv + LIF reading row-packed spikes (the consumer of the depthwise layer above)
+# ---------------------------------------------------------------------------------------------------------------
+PW_ROWBITS_CASES = [  # dtype, N, Cin, Cout, H, W, T, tau, tensor v_init
+    (BF16, 2, 128, 256, 8, 16, 4, 2.0, False),     # weights in registers, two output-channel tiles
+    (BF16, 3, 64, 96, 8, 8, 3, 4.0, True),         # weights in LDS, one chunk; Cout % 128 != 0
+    (F16, 2, 256, 64, 16, 8, 4, 2.0, True),        # several chunks, f16
+    (BF16, 1, 24, 32, 8, 24, 2, 2.0, False),       # channel tail inside a chunk
+    (BF16, 2, 1024, 64, 8, 8, 2, 2.0, False),      # weights streamed from L2
+    (F16, 1, 128, 128, 16, 16, 17, 2.0, True),     # two launch windows
+]
+
+
+@pytest.mark.parametrize("dtype,N,Cin,Cout,H,W,T,tau,tensor_v", PW_ROWBITS_CASES)
+def test_pointwise_from_row_packed_spikes_against_the_oracle(B, dtype, N, Cin, Cout, H, W, T, tau, tensor_v):
+    g = gen(4300 + Cin + Cout + T)
+    lif = (1.0, 0.0, tau)
+    xs = [spikes((N, Cin, H, W), 0.25, g) for _ in range(T)]
+    w = q(torch.randn(Cout, Cin, 1, 1, generator=g) * (2.0 / Cin) ** 0.5 * 2.0, dtype)
+    b = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    v0 = torch.randn(N, Cout, H, W, generator=g) * 0.3 if tensor_v else torch.tensor(0.0)
+    ref = O.temporal_conv_lif(xs, w, b, v0, (1, 1), (0, 0), (1, 1), 1, *lif)
+    bits = dev(_ref_rowbits(torch.stack(xs)), torch.uint8)
+    sp, v = B.pointwise_conv_lif_from_rowbits(bits, dev(w, dtype), dev(b, dtype), lif, v_init=dev(v0, F32) if tensor_v else None)
+    assert sp.dtype == dtype and tuple(sp.shape) == (T, N, Cout, H, W) and v.dtype == F32
+    check(sp, v, ref, what=f"pointwise from row bits {Cin}->{Cout} {H}x{W} T={T}")
+    # bit for bit the dense operator on the unpacked spikes (same kernel, another fetch)
+    import triton_snn_fusion_amd.runtime.snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=True)
+    dv = dev(v0, F32) if tensor_v else torch.zeros((), device=DEV, dtype=F32)
+    s_d, v_d = torch.ops.snn_custom.fused_temporal_pointwise_conv_lif_state([dev(x, dtype) for x in xs], dev(w, dtype), dev(b, dtype), dv,
+                                                                            [1, 1], [0, 0], [1, 1], 1, *lif, False)
+    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    if last_conv_plan()["kernel"] == "pointwise":       # small deep layers run the matrix kernel through the operator
+        assert torch.equal(s_d, sp) and torch.equal(v_d, v)
+
+
+def test_depthwise_then_pointwise_through_row_packed_spikes(B):
+    """A depthwise-separable block whose intermediate spikes travel one bit each == the two dense operators."""
+    dtype, T, N, C, Cout, H, W = BF16, 4, 2, 128, 256, 16, 16
+    g = gen(4400)
+    xs = [spikes((N, C, H, W), 0.3, g) for _ in range(T)]
+    wd, bd = q(torch.randn(C, 1, 3, 3, generator=g) * 0.5, dtype), q(torch.randn(C, generator=g) * 0.1, dtype)
+    wp, bp = q(torch.randn(Cout, C, 1, 1, generator=g) * (2.0 / C) ** 0.5 * 2.0, dtype), q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    ref_d = O.temporal_conv_lif(xs, wd, bd, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), C, *LIF)
+    ref_p = O.temporal_conv_lif([ref_d[0][t] for t in range(T)], wp, bp, torch.tensor(0.0), (1, 1), (0, 0), (1, 1), 1, *LIF)
+    bits, _ = B.depthwise_conv_lif_rowbits([dev(x, dtype) for x in xs], dev(wd, dtype), dev(bd, dtype), LIF, want_v=False)
+    sp, v = B.pointwise_conv_lif_from_rowbits(bits, dev(wp, dtype), dev(bp, dtype), LIF)
+    # Teacher forcing as for the network tests: the pointwise layer is gated on the oracle's depthwise spikes only where the
+    # library's depthwise spikes equal them (they do, away from the threshold band the depthwise gate allows).
+    dense = B.unpack_rowbits(bits, dtype)
+    if torch.equal(dense.float().cpu(), ref_d[0]):
+        check(sp, v, ref_p, what="depthwise -> pointwise through row bits")
+    ref_own = O.temporal_conv_lif([dense[t].float().cpu() for t in range(T)], wp, bp, torch.tensor(0.0), (1, 1), (0, 0), (1, 1), 1, *LIF)
+    check(sp, v, ref_own, what="pointwise on the library's own depthwise spikes")
+
+
+def test_pointwise_from_row_packed_spikes_rejects_what_it_does_not_take(B):
+    g = gen(4500)
+    w, b = dev(torch.randn(32, 16, 1, 1, generator=g), BF16), dev(torch.randn(32, generator=g), BF16)
+    bits = torch.zeros(2, 1, 16, 4, 1, dtype=torch.uint8, device=DEV)            # 4 x 8 = 32 pixels: not whole tiles of 64
+    with pytest.raises(RuntimeError, match="unsupported_shape"):
+        B.pointwise_conv_lif_from_rowbits(bits, w, b, LIF)
+    bits = torch.zeros(2, 1, 16, 8, 1, dtype=torch.uint8, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported_shape"):
+        B.pointwise_conv_lif_from_rowbits(bits, w, b, (1.0, -1.0, 2.0))            # soft reset: not the common neuron

@@ -63,7 +63,9 @@ __host__ __device__ inline size_t packed_weight_elems(const PackGeom& p) {
 enum LoadMode : int {
     LOAD_PAIR32 = 0,   // 16-bit activations, pixel pairs 4-byte aligned: one dword load
     LOAD_2X16 = 1,     // 16-bit activations, unaligned: two halfword loads
-    LOAD_2XF32 = 2     // fp32 activations: two dword loads, rounded to bf16 on the way into LDS
+    LOAD_2XF32 = 2,    // fp32 activations: two dword loads, rounded to bf16 on the way into LDS
+    LOAD_ROWBITS = 3   // row-packed spikes (one byte = 8 consecutive pixels of a channel): one byte load, the pair's two bits
+                       // become two 16-bit ones or zeros on the way into LDS (pointwise kernel only)
 };
 
 // Staging items a thread may hold in flight per chunk: modes that need two registers per fetch get half as many.

@@ -246,7 +246,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
                   int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
                   int pad_h, int pad_w, const void* v_init, int v_dtype, void* spikes,
                   int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
-                  void* stream, bool analog_out) {
+                  void* stream, bool analog_out, bool x_rowbits = false) {
     if (xs == nullptr || packed_weight == nullptr || spikes == nullptr || v_out == nullptr)
         return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_conv_lif: xs, packed_weight, spikes and v_out must be non-null");
     if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 ||
@@ -328,7 +328,17 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     // x 32 images (128 MB) 79 / 55, 256 -> 512 at 28^2 x 16 (103 MB) 78 / 51, 192 -> 64 at 28^2 x 32 (58 MB) 57 / 32, 384 -> 96 at
     // 14^2 x 32 (26 MB) 42 / 36, 1024 -> 64 at 8^2 x 8 56 / 54, but 256 -> 128 at 56^2 x 32 (360 MB) 90 / 139: the pointwise
     // kernel keeps the layers that are mostly memory traffic.
-    const bool pointwise_to_matrix = pointwise && (flops / bytes >= 200.0 || (Cin > 128 && bytes < 200.0e6));
+    // Row-packed spikes in (`x_rowbits`): xs[t] are [N][Cin][H * W / 8] bytes; only the pointwise kernel's fast variant reads them.
+    if (x_rowbits) {
+        const bool fast_neuron = lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+        if (!pointwise || residuals != nullptr || xsize != 2 || v_dtype != SNNF_F32 || !fast_neuron || Cin % 8 != 0 || Cout % 32 != 0 ||
+            g.Wo % 64 != 0 || !vec_ok || static_cast<int64_t>(Cout) * g.Wo >= (1LL << 30))
+            return fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_shape: needs a 1x1 stride-1 layer without residual, 16-bit "
+                        "operands, an fp32 membrane, the common neuron (power-of-two tau, hard reset), Cin %% 8 == 0, Cout %% 32 == 0, "
+                        "H * W %% 64 == 0 and 16-byte aligned outputs");
+        all_shared = false;
+    }
+    const bool pointwise_to_matrix = !x_rowbits && pointwise && (flops / bytes >= 200.0 || (Cin > 128 && bytes < 200.0e6));
     const bool matrix_candidate = (!pointwise || pointwise_to_matrix) && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
     Plan pl = {};
@@ -369,7 +379,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_bias: unsupported_shape: only layers the 8-wave matrix kernel takes "
                     "(Cin %% 8 == 0 or Cin < 8, not a plain 1x1/1 convolution, tiles that fit LDS)");
     // Everything else: the time-outer kernels for a shared frame or a low intensity, the 4-wave T-in-M kernel otherwise.
-    bool time_outer = !mm_kernel && (all_shared || flops / bytes < 200.0);
+    bool time_outer = !mm_kernel && (all_shared || x_rowbits || flops / bytes < 200.0);
     // Pointwise kernel: where the weight fragments live (registers only in the fast variant) and the LDS that takes.
     auto pw_config = [&](bool allow_regs, ConvGeom& gg) -> size_t {
         const size_t xb = static_cast<size_t>(64) * gg.pitch;
@@ -531,7 +541,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         L.stream = hs;
         int rc;
         const int tt = parts[part].tt;
-        const int lm = mm_kernel ? mm_load_mode : load_mode;
+        const int lm = x_rowbits ? static_cast<int>(LOAD_ROWBITS) : (mm_kernel ? mm_load_mode : load_mode);
         if (x_dtype == SNNF_F32) rc = launch_conv_f32(L, tt, lm);
         else if (x_dtype == SNNF_BF16) rc = launch_conv_bf16(L, tt, lm);
         else rc = launch_conv_f16(L, tt, lm);
@@ -550,6 +560,16 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
                              void* stream) {
     return snnf::conv_lif_impl(xs, residuals, T, N, Cin, H, W, x_dtype, packed_weight, Cout, KH, KW, stride_h, stride_w, pad_h,
                                pad_w, v_init, v_dtype, spikes, spike_step_stride, v_out, v_threshold, v_reset, tau, stream, false);
+}
+
+extern "C" int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, int H, int W, int x_dtype,
+                                       const void* packed_weight, int Cout, const void* v_init, void* spikes,
+                                       int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
+                                       void* stream) {
+    if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
+        return snnf::fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_dtype: the matrix operands are bf16 or fp16");
+    return snnf::conv_lif_impl(xs_bits, nullptr, T, N, Cin, H, W, x_dtype, packed_weight, Cout, 1, 1, 1, 1, 0, 0, v_init, SNNF_F32, spikes,
+                               spike_step_stride, v_out, v_threshold, v_reset, tau, stream, false, true);
 }
 
 extern "C" int snnf_conv_bias(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,

@@ -66,7 +66,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
     extern __shared__ __align__(16) unsigned char lds[];
     static_assert(!DIRECT || (FAST && STD && sizeof(XT) == 2), "the accumulator-layout LIF step is for the fast variant on 16-bit activations");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
-    constexpr int RPE = LM == LOAD_PAIR32 ? 1 : 2;
+    constexpr int RPE = (LM == LOAD_PAIR32 || LM == LOAD_ROWBITS) ? 1 : 2;
+    static_assert(LM != LOAD_ROWBITS || (FAST && sizeof(XT) == 2), "row-packed spikes: fast variant, 16-bit matrix operands");
     constexpr int SS = kPwSlots;
     constexpr uint32_t ES = static_cast<uint32_t>(sizeof(XT));
     constexpr int NG = 4;                          // epilogue row groups (8 channel rows each) of the wave's 32 channels
@@ -90,7 +91,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
     const int nocf = (g.Cout + 31) >> 5;
     const int64_t frag_stride_ocf = static_cast<int64_t>(total_pairs) * (kFragBytes / 2);
     const int steps_with_input = g.shared_x ? 1 : g.T;
-    const int64_t row_bytes = static_cast<int64_t>(P) * ES;           // one channel row of an image
+    const int64_t row_bytes = LM == LOAD_ROWBITS ? static_cast<int64_t>(P >> 3)   // row-packed spikes: P / 8 bytes per channel row
+                                                 : static_cast<int64_t>(P) * ES;  // one channel row of an image
 
     // ---- kernel constants of the staging: item e = (channel group of 8, pixel pair) of a 64-pixel x CK-channel stage.
     uint32_t item_src[SS], item_dst[SS];
@@ -100,7 +102,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         const int e = s * kConvThreads + tid;
         const int cg = e >> 5, pp = e & 31;
         item_on[s] = cg < groups;
-        item_src[s] = (static_cast<uint32_t>(cg) * 8u * static_cast<uint32_t>(P) + 2u * pp) * ES;
+        item_src[s] = LM == LOAD_ROWBITS ? static_cast<uint32_t>(cg) * static_cast<uint32_t>(P) + (static_cast<uint32_t>(pp) >> 2)   // the byte that holds the pair
+                                         : (static_cast<uint32_t>(cg) * 8u * static_cast<uint32_t>(P) + 2u * pp) * ES;
         item_dst[s] = static_cast<uint32_t>(pp * g.pitch + cg * 16);   // pixel 2 pp -> row pp, pixel 2 pp + 1 -> row pp + 32
     }
     // The 16 bytes of padding behind a pixel's channels are read as a second channel group when a chunk has only one:
@@ -119,7 +122,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
     // outside are redirected to the tile's first pixels (always valid) and zeroed on their way into LDS.
     auto issue_loads = [&](int step, int chunk, int n, int px0) __attribute__((always_inline)) {
         const char* __restrict__ base = static_cast<const char*>(kernarg_table_entry(0, step)) +
-                                        (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES;
+                                        (LM == LOAD_ROWBITS ? (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) >> 3
+                                                            : (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES);
         const bool whole = (FAST || px0 + kPwTile <= P) && (chunk + 1) * g.CK <= g.Cin;
         uint32_t src[SS], second[SS];
         uint32_t bad = 0;
@@ -149,6 +153,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                     const char* __restrict__ row = base + j * row_bytes;
                     if constexpr (LM == LOAD_PAIR32) {
                         pre[s][j][0] = *reinterpret_cast<const uint32_t*>(row + src[s]);
+                    } else if constexpr (LM == LOAD_ROWBITS) {
+                        pre[s][j][0] = *reinterpret_cast<const unsigned char*>(row + src[s]);
                     } else if constexpr (LM == LOAD_2X16) {
                         pre[s][j][0] = *reinterpret_cast<const uint16_t*>(row + src[s]);
                         pre[s][j][1] = *reinterpret_cast<const uint16_t*>(row + src[s] + second[s]);
@@ -168,7 +174,17 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         for (int s = 0; s < SS; ++s) {
             if (item_on[s]) {
                 cv_u32x4 lo, hi;
-                if constexpr (LM == LOAD_PAIR32) {
+                if constexpr (LM == LOAD_ROWBITS) {
+                    // The pair's two bits of each channel's byte -> (1.0 or 0, 1.0 or 0) in the matrix operand's 16-bit format.
+                    const uint32_t sh = 2u * (static_cast<uint32_t>(tid) & 3u);      // pixel pair pp = tid % 32 sits at bits 2 (pp % 4) of its byte
+                    const uint32_t one = F16 ? 0x3C00u : 0x3F80u;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t m = pre[s][j][0] >> sh;
+                        pre[s][j][0] = ((m & 1u) ? one : 0u) | ((m & 2u) ? (one << 16) : 0u);
+                    }
+                }
+                if constexpr (LM == LOAD_PAIR32 || LM == LOAD_ROWBITS) {
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         lo[k] = __builtin_amdgcn_perm(pre[s][2 * k + 1][0], pre[s][2 * k][0], 0x05040100u);
@@ -674,6 +690,12 @@ int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     if constexpr (sizeof(XT) == 4) {
         return pick(std::integral_constant<int, LOAD_2XF32>{});
     } else {
+        if (load_mode == LOAD_ROWBITS) {    // row-packed spikes in: the fast variants with the LIF step on the accumulators
+            if (!fast || L.has_residual) return fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_shape: only layers the fast variant takes");
+            if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_REGS, true, true>);
+            if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_LDS, true, true>);
+            return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_STREAM, true, true>);
+        }
         if (load_mode == LOAD_PAIR32) return pick(std::integral_constant<int, LOAD_PAIR32>{});
         return pick(std::integral_constant<int, LOAD_2X16>{});
     }

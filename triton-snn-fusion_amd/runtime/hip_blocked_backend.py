@@ -267,3 +267,33 @@ def unpack_rowbits(bits: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     _lib.check("snnf_rowbits_unpack", _lib.lib().snnf_rowbits_unpack(bits.data_ptr(), dense.data_ptr(), bits.numel(), _lib.dtype_code(dtype),
                                                                    _lib.current_stream(bits.device)))
     return dense
+
+
+def pointwise_conv_lif_from_rowbits(bits: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], lif: Sequence[float],
+                                    v_init: Optional[torch.Tensor] = None):
+    """Pointwise (1x1, stride 1) convolution + bias + LIF over T steps of row-packed spikes `bits` [T, N, Cin, H, W / 8]
+    uint8 (what depthwise_conv_lif_rowbits writes). Returns (spikes [T, N, Cout, H, W] in the weight's dtype, final
+    membrane [N, Cout, H, W] fp32): the dense outputs of the operator on the unpacked tensor."""
+    _check_dtype(weight.dtype)
+    if bits.dtype != torch.uint8 or bits.dim() != 5 or not bits[0].is_contiguous():
+        raise RuntimeError("unsupported_layout: row-packed spikes [T, N, Cin, H, W / 8] uint8 expected")
+    T, n, cin, h, w8 = (int(d) for d in bits.shape)
+    w = w8 * 8
+    if weight.dim() != 4 or tuple(weight.shape[1:]) != (cin, 1, 1):
+        raise RuntimeError(f"unsupported_weight: pointwise weight [Cout, {cin}, 1, 1] expected, got {tuple(weight.shape)}")
+    cout = int(weight.shape[0])
+    dev = bits.device
+    if bias is None:
+        bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    packed = _packed_weight(weight, bias, weight.dtype)
+    vi = None
+    if v_init is not None and isinstance(v_init, torch.Tensor) and v_init.dim() != 0:
+        if tuple(v_init.shape) != (n, cout, h, w) or v_init.dtype != torch.float32 or v_init.device != dev:
+            raise RuntimeError("unsupported_membrane_state: v_init must be a float32 [N, Cout, H, W] tensor on the activations' device")
+        vi = v_init if v_init.is_contiguous() else v_init.contiguous()
+    spikes = torch.empty((T, n, cout, h, w), dtype=weight.dtype, device=dev)
+    v_out = torch.empty((n, cout, h, w), dtype=torch.float32, device=dev)
+    _lib.check("snnf_pwconv_lif_rowbits", _lib.lib().snnf_pwconv_lif_rowbits(
+        _lib.packed_step_pointers(bits), T, n, cin, h, w, _lib.dtype_code(weight.dtype), packed.data_ptr(), cout, _lib.ptr(vi),
+        spikes.data_ptr(), int(spikes.stride(0)), v_out.data_ptr(), float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
+    return spikes, v_out
