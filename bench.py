@@ -595,7 +595,25 @@ def main() -> int:
                     def packed_block(xs=xs, w=w, b=b, w2=w2, b2=b2):
                         packed, _ = blocked.depthwise_conv_lif_rowbits(xs, w, b, prep.lif)
                         return blocked.pointwise_conv_lif_from_rowbits(packed, w2, b2, prep.lif)
+                    # The same layer writing its spikes row-packed too (bits in, bits out), with and without the final membrane.
+                    for name, want_v in (("packed_in_and_out", True), ("packed_in_and_out_no_membrane", False)):
+                        ms4, how4 = _time_kernel(lambda want_v=want_v: blocked.pointwise_conv_lif_from_rowbits(
+                            bits, w2, b2, prep.lif, packed_out=True, want_v=want_v), args.steps, max(3, args.warmup // 2))
+                        nbytes4 = T_ * n * c * h * wd // 8 + T_ * n * cout * h * wd // 8 + (n * cout * h * wd * 4 if want_v else 0) + cout * (c + 1) * prep.esize
+                        kernels[f"layer{i + 1}_pointwise1x1_{name}"] = {
+                            "ms": round(ms4, 4), "timed": how4, "algorithmic_bytes": nbytes4, "flops": flops2,
+                            "hbm": _roofline("hbm", nbytes4, ms4, None), "mfma": _roofline("mfma", flops2, ms4, None)}
                     ms3 = _time_graph(packed_block, args.steps, max(3, args.warmup // 2))
+
+                    def packed_chain(xs=xs, w=w, b=b, w2=w2, b2=b2):
+                        packed, _ = blocked.depthwise_conv_lif_rowbits(xs, w, b, prep.lif, want_v=False)
+                        return blocked.pointwise_conv_lif_from_rowbits(packed, w2, b2, prep.lif, packed_out=True, want_v=False)
+                    ms5 = _time_graph(packed_chain, args.steps, max(3, args.warmup // 2))
+                    result["block_inside_a_network_on_packed_spikes"] = {
+                        "ms_per_step": round(ms5, 4), "images_T_per_s": round(n * T_ / (ms5 * 1e-3), 1), "timed": "graph",
+                        "algorithmic_bytes": T_ * n * c * h * wd * prep.esize + T_ * n * c * h * wd // 8 * 2 + T_ * n * cout * h * wd // 8,
+                        "note": "dense block input, row-packed spikes between the layers and out of the block, no membrane outputs: "
+                                "what a network executor that owns both ends would run"}
                     result["block_with_packed_intermediate_spikes"] = {
                         "ms_per_step": round(ms3, 4), "images_T_per_s": round(n * T_ / (ms3 * 1e-3), 1), "timed": "graph",
                         "algorithmic_bytes": nbytes + nbytes2,

@@ -121,13 +121,16 @@ int snnf_rowbits_unpack(const void* bits, void* dense, int64_t bytes, int x_dtyp
  * dense 0 / 1 tensor to run_fused_temporal_general with kernel key k1_s1_p0,
  * kernels/benchmark_conv_lif_temporal_general.py:971-1323 as called from runtime/triton_convlif_backend.py:513-598).
  * Same packed weight, arithmetic and outputs as snnf_conv_lif on the unpacked tensor.
- *   xs_bits[t] : [N, Cin, H, W / 8] bytes;  spikes : [T, N, Cout, H, W] x_dtype (bf16 / fp16);  v_init (or NULL), v_out : fp32
+ *   xs_bits[t] : [N, Cin, H, W / 8] bytes;  v_init (or NULL), v_out : [N, Cout, H, W] fp32
+ *   spikes     : spikes_packed == 0: [T, N, Cout, H, W] x_dtype (bf16 / fp16), `spike_step_stride` elements between timesteps;
+ *                spikes_packed != 0: [T, N, Cout, H, W / 8] bytes, `spike_step_stride` BYTES between timesteps, and v_out may be
+ *                NULL (final membrane not stored; needs T <= SNNF_MAX_T_PER_LAUNCH)
  * Takes what the pointwise kernel's fast variant takes: the common neuron (power-of-two tau, hard reset), Cin % 8 == 0,
  * Cout % 32 == 0, H * W % 64 == 0, 16-byte aligned outputs and membranes; SNNF_ERR_UNSUPPORTED otherwise.
  */
 int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, int H, int W, int x_dtype,
                             const void* packed_weight, int Cout, const void* v_init,
-                            void* spikes, int64_t spike_step_stride, void* v_out,
+                            void* spikes, int spikes_packed, int64_t spike_step_stride, void* v_out,
                             float v_threshold, float v_reset, float tau, void* stream);
 
 /*

@@ -356,6 +356,15 @@ def test_pointwise_from_row_packed_spikes_against_the_oracle(B, dtype, N, Cin, C
     from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
     if last_conv_plan()["kernel"] == "pointwise":       # small deep layers run the matrix kernel through the operator
         assert torch.equal(s_d, sp) and torch.equal(v_d, v)
+    # row-packed spikes out as well: the same spikes and membrane, bit for bit; the membrane is optional within one window
+    pb, pv = B.pointwise_conv_lif_from_rowbits(bits, dev(w, dtype), dev(b, dtype), lif, v_init=dev(v0, F32) if tensor_v else None,
+                                               packed_out=True)
+    assert pb.dtype == torch.uint8 and tuple(pb.shape) == (T, N, Cout, H, W // 8)
+    assert torch.equal(B.unpack_rowbits(pb, dtype), sp) and torch.equal(pv, v)
+    if T <= 16:
+        pb2, none = B.pointwise_conv_lif_from_rowbits(bits, dev(w, dtype), dev(b, dtype), lif, v_init=dev(v0, F32) if tensor_v else None,
+                                                      packed_out=True, want_v=False)
+        assert none is None and torch.equal(pb2, pb)
 
 
 def test_depthwise_then_pointwise_through_row_packed_spikes(B):
@@ -369,6 +378,8 @@ def test_depthwise_then_pointwise_through_row_packed_spikes(B):
     ref_p = O.temporal_conv_lif([ref_d[0][t] for t in range(T)], wp, bp, torch.tensor(0.0), (1, 1), (0, 0), (1, 1), 1, *LIF)
     bits, _ = B.depthwise_conv_lif_rowbits([dev(x, dtype) for x in xs], dev(wd, dtype), dev(bd, dtype), LIF, want_v=False)
     sp, v = B.pointwise_conv_lif_from_rowbits(bits, dev(wp, dtype), dev(bp, dtype), LIF)
+    packed, _ = B.pointwise_conv_lif_from_rowbits(bits, dev(wp, dtype), dev(bp, dtype), LIF, packed_out=True, want_v=False)
+    assert torch.equal(B.unpack_rowbits(packed, dtype), sp)      # bits in, bits out, no membrane: the same spikes
     # Teacher forcing as for the network tests: the pointwise layer is gated on the oracle's depthwise spikes only where the
     # library's depthwise spikes equal them (they do, away from the threshold band the depthwise gate allows).
     dense = B.unpack_rowbits(bits, dtype)

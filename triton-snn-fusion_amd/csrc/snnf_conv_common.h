@@ -120,6 +120,7 @@ struct ConvGeom {
     int oc_major;             // matrix kernel: an XCD takes the output-channel tiles congruent to it (all pixel tiles) instead of the pixel
                               // tiles congruent to it (all output-channel tiles); d_oc_tiles then divides by oc_tiles / 8
     int stream_out;           // pointwise kernel: spikes and membrane are stored non-temporally (the launch writes more than the caches hold)
+    int bits_out;             // pointwise kernel: spikes leave row-packed (bytes), spike_step_stride counts bytes, v_out may be null
     int tiles_img;            // matrix kernel: tiles per image (tiles_x * tiles_y, tiles never straddle images)
     int run8;                 // matrix kernel: runs of 8 tile pixels are contiguous in memory and aligned for 16-byte
                               // (8) or 8-byte (4) spike accesses; 0: neither

@@ -246,8 +246,8 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
                   int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w,
                   int pad_h, int pad_w, const void* v_init, int v_dtype, void* spikes,
                   int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
-                  void* stream, bool analog_out, bool x_rowbits = false) {
-    if (xs == nullptr || packed_weight == nullptr || spikes == nullptr || v_out == nullptr)
+                  void* stream, bool analog_out, bool x_rowbits = false, bool out_rowbits = false) {
+    if (xs == nullptr || packed_weight == nullptr || spikes == nullptr || (v_out == nullptr && !(out_rowbits && T <= SNNF_MAX_T_PER_LAUNCH)))
         return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_conv_lif: xs, packed_weight, spikes and v_out must be non-null");
     if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 ||
         pad_h < 0 || pad_w < 0)
@@ -337,7 +337,10 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
                         "operands, an fp32 membrane, the common neuron (power-of-two tau, hard reset), Cin %% 8 == 0, Cout %% 32 == 0, "
                         "H * W %% 64 == 0 and 16-byte aligned outputs");
         all_shared = false;
+    } else if (out_rowbits) {
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: row-packed output needs row-packed input");
     }
+    g.bits_out = out_rowbits ? 1 : 0;
     const bool pointwise_to_matrix = !x_rowbits && pointwise && (flops / bytes >= 200.0 || (Cin > 128 && bytes < 200.0e6));
     const bool matrix_candidate = (!pointwise || pointwise_to_matrix) && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
@@ -489,7 +492,8 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
             f.g.tiles_x = full_tiles; f.g.px_base = 0;
             // Outputs that the caches cannot hold anyway are streamed past L2, which then keeps the activation tiles for
             // their second pass (the other output-channel tile). Smaller outputs stay cached for the layer that reads them.
-            const int64_t out_bytes = static_cast<int64_t>(N) * Cout * P * (static_cast<int64_t>(window) * dtype_size(x_dtype) + 4);
+            const int64_t out_bytes = out_rowbits ? static_cast<int64_t>(N) * Cout * P * (v_out != nullptr ? 4 : 0)
+                                                  : static_cast<int64_t>(N) * Cout * P * (static_cast<int64_t>(window) * dtype_size(x_dtype) + 4);
             f.g.stream_out = out_bytes >= kStreamOutBytes ? 1 : 0;
             f.g.d_tiles_x = make_fast_div(full_tiles);
             f.lds = pw_config(true, f.g);
@@ -533,7 +537,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         L.wpacked = static_cast<const uint16_t*>(packed_weight);
         L.bias = reinterpret_cast<const float*>(L.wpacked + packed_weight_elems(pg));
         L.v_init = t0 == 0 ? v_init : v_out;
-        L.spikes = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
+        L.spikes = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * (out_rowbits ? 1 : xsize);
         L.v_out = v_out;
         L.lif = lif;
         L.grid = grid_for(L.g, per_cu);
@@ -563,13 +567,13 @@ extern "C" int snnf_conv_lif(const void* const* xs, const void* const* residuals
 }
 
 extern "C" int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, int H, int W, int x_dtype,
-                                       const void* packed_weight, int Cout, const void* v_init, void* spikes,
+                                       const void* packed_weight, int Cout, const void* v_init, void* spikes, int spikes_packed,
                                        int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
                                        void* stream) {
     if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
         return snnf::fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_dtype: the matrix operands are bf16 or fp16");
     return snnf::conv_lif_impl(xs_bits, nullptr, T, N, Cin, H, W, x_dtype, packed_weight, Cout, 1, 1, 1, 1, 0, 0, v_init, SNNF_F32, spikes,
-                               spike_step_stride, v_out, v_threshold, v_reset, tau, stream, false, true);
+                               spike_step_stride, v_out, v_threshold, v_reset, tau, stream, false, true, spikes_packed != 0);
 }
 
 extern "C" int snnf_conv_bias(const void* const* xs, const void* const* residuals, int T, int N, int Cin, int H, int W,

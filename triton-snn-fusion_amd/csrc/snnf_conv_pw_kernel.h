@@ -50,12 +50,32 @@ __device__ __forceinline__ const void* kernarg_table_entry(int table_offset_byte
     return *(ka_entry)(ka + table_offset_bytes + i * 8);
 }
 
+// The four halves of two wave-wide compare masks into lanes LANE (lower half-wave's words) and LANE + 4 (upper half-wave's)
+// of `lo` / `hi`: v_writelane_b32 with immediate lane selects. The masks come fresh from vector compares; the idle cycles in
+// front give the scalar registers time to land (a v_writelane issued right behind the compare read a stale value on gfx950).
+template <int LANE>
+__device__ __forceinline__ void write_mask_lanes(uint32_t& lo, uint32_t& hi, uint64_t m0, uint64_t m1) {
+    asm volatile("s_nop 4\n\t"
+                 "v_writelane_b32 %0, %2, %6\n\t"
+                 "v_writelane_b32 %1, %4, %6\n\t"
+                 "v_writelane_b32 %0, %3, %7\n\t"
+                 "v_writelane_b32 %1, %5, %7"
+                 : "+v"(lo), "+v"(hi)
+                 : "s"(static_cast<uint32_t>(m0)), "s"(static_cast<uint32_t>(m0 >> 32)), "s"(static_cast<uint32_t>(m1)),
+                   "s"(static_cast<uint32_t>(m1 >> 32)), "n"(LANE), "n"(LANE + 4));
+}
+
 // The two pointer tables MUST be the first two kernel parameters (offsets 0 and sizeof(StepPtrs)).
 // DIRECT (with FAST and STD, no residual): the LIF step runs on the accumulators where the matrix instruction leaves them
 // (a lane holds 2 adjacent pixels x 16 channels of the wave's 32 x 64 outputs) and spikes and the membrane go to memory
 // from there: the two adjacent pixels of a channel are one 4-byte (spikes) or 8-byte (membrane) store, 32 lanes of a
 // half-wave cover a whole 128- or 256-byte line of one channel row. No trip through LDS, and the LIF step does not wait for one.
-template <typename XT, int LM, bool STD, int WM, bool FAST, bool DIRECT = false>
+// BITS_OUT (with DIRECT): the spikes leave row-packed, one byte per 8 pixels of a channel row. The tile's pixel p then sits
+// in LDS row p (instead of even pixels in rows 0..31 and odd ones behind them), so that accumulator fragment 0 holds pixels
+// 0..31 and fragment 1 pixels 32..63 of the tile: the LIF step's compare masks of the two fragments ARE the 8 bytes of a
+// channel row, and a lane per channel stores them. `spikes` then points to bytes, g.spike_step_stride counts bytes, and
+// v_out may be null (final membrane not stored).
+template <typename XT, int LM, bool STD, int WM, bool FAST, bool DIRECT = false, bool BITS_OUT = false>
 __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pw_lif_kernel(const StepPtrs xs, const StepPtrs residuals,
                                                                       const int has_residual, const ConvGeom g,
                                                                       const uint16_t* __restrict__ wpacked,
@@ -65,6 +85,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                                                                       const LifParams lif) {
     extern __shared__ __align__(16) unsigned char lds[];
     static_assert(!DIRECT || (FAST && STD && sizeof(XT) == 2), "the accumulator-layout LIF step is for the fast variant on 16-bit activations");
+    static_assert(!BITS_OUT || DIRECT, "row-packed spikes leave from the accumulator-layout LIF step");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr int RPE = (LM == LOAD_PAIR32 || LM == LOAD_ROWBITS) ? 1 : 2;
     static_assert(LM != LOAD_ROWBITS || (FAST && sizeof(XT) == 2), "row-packed spikes: fast variant, 16-bit matrix operands");
@@ -104,7 +125,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         item_on[s] = cg < groups;
         item_src[s] = LM == LOAD_ROWBITS ? static_cast<uint32_t>(cg) * static_cast<uint32_t>(P) + (static_cast<uint32_t>(pp) >> 2)   // the byte that holds the pair
                                          : (static_cast<uint32_t>(cg) * 8u * static_cast<uint32_t>(P) + 2u * pp) * ES;
-        item_dst[s] = static_cast<uint32_t>(pp * g.pitch + cg * 16);   // pixel 2 pp -> row pp, pixel 2 pp + 1 -> row pp + 32
+        item_dst[s] = static_cast<uint32_t>((BITS_OUT ? 2 * pp : pp) * g.pitch + cg * 16);   // pixel 2 pp -> row pp, pixel 2 pp + 1 -> row pp + 32 (BITS_OUT: rows 2 pp and 2 pp + 1)
     }
     // The 16 bytes of padding behind a pixel's channels are read as a second channel group when a chunk has only one:
     // keep them zero (staging never writes there).
@@ -217,7 +238,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                     }
                 }
                 *reinterpret_cast<cv_u32x4*>(xb + item_dst[s]) = lo;
-                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s] + 32 * g.pitch) = hi;
+                *reinterpret_cast<cv_u32x4*>(xb + item_dst[s] + (BITS_OUT ? 1 : 32) * g.pitch) = hi;
             }
         }
     };
@@ -333,7 +354,7 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         }
         // DIRECT: membrane of the lane's 2 pixels x 16 channels, register r = channel ocf * 32 + 8 (r / 4) + 4 half + r % 4.
         float vd[kNPF][16];
-        const uint32_t lane_off_d = static_cast<uint32_t>((ocf * 32 + 4 * half) * P + 2 * l32);   // elements into [Cout, P]
+        const uint32_t lane_off_d = static_cast<uint32_t>((ocf * 32 + 4 * half) * P + (BITS_OUT ? l32 : 2 * l32));   // elements into [Cout, P]
         auto row_off_d = [&](int r) __attribute__((always_inline)) { return static_cast<uint32_t>((8 * (r >> 2) + (r & 3)) * P); };
         if constexpr (DIRECT) {
 #pragma unroll
@@ -345,9 +366,14 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                 const float* __restrict__ vsrc = static_cast<const float*>(v_init) + tile_off + lane_off_d;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const Pack<float, 2> two = *reinterpret_cast<const Pack<float, 2>*>(vsrc + row_off_d(r));
-                    vd[0][r] = two.v[0];
-                    vd[1][r] = two.v[1];
+                    if constexpr (BITS_OUT) {      // the lane's pixels are l32 and l32 + 32 of the tile
+                        vd[0][r] = vsrc[row_off_d(r)];
+                        vd[1][r] = vsrc[row_off_d(r) + 32];
+                    } else {
+                        const Pack<float, 2> two = *reinterpret_cast<const Pack<float, 2>*>(vsrc + row_off_d(r));
+                        vd[0][r] = two.v[0];
+                        vd[1][r] = two.v[1];
+                    }
                 }
             }
         }
@@ -383,10 +409,16 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
         // Spikes of a timestep wait here until the next stage has left its load registers.
         Pack<XT, 8> pend[NG];
         uint32_t pend_d[16];     // DIRECT: the spikes of 2 adjacent pixels of channel register r
+        uint32_t pend_lo = 0u, pend_hi = 0u;   // BITS_OUT: lane c < 32 holds the tile's 64 spike bits of channel ocf * 32 + c
         int pend_step = -1;
         auto flush_spikes = [&]() __attribute__((always_inline)) {
             char* __restrict__ out = reinterpret_cast<char*>(spikes + pend_step * g.spike_step_stride + tile_off);
-            if constexpr (DIRECT) {
+            if constexpr (BITS_OUT) {
+                unsigned char* __restrict__ row = reinterpret_cast<unsigned char*>(spikes) + pend_step * g.spike_step_stride +
+                                                  ((tile_off + static_cast<int64_t>(ocf) * 32 * P) >> 3);
+                const snnf_u32x2 word = {pend_lo, pend_hi};
+                if (lane < 32) *reinterpret_cast<snnf_u32x2*>(row + static_cast<uint32_t>(lane) * static_cast<uint32_t>(P >> 3)) = word;
+            } else if constexpr (DIRECT) {
                 // Uniform row base + 32-bit lane offset: the stores take the scalar-base addressing form.
                 const uint32_t lane_b = lane_off_d * ES;
                 if (g.stream_out) {
@@ -541,7 +573,28 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                 if (pend_step >= 0) flush_spikes();   // only when a timestep had no stage of its own (shared frame)
                 const char* __restrict__ res_t =
                     has_residual ? reinterpret_cast<const char*>(static_cast<const XT*>(kernarg_table_entry(sizeof(StepPtrs), step)) + tile_off) : nullptr;
-                if constexpr (DIRECT) {
+                if constexpr (BITS_OUT) {
+                    // The compare of the LIF step is the ballot: bits 0..31 of a mask are the lower half-wave's channel row
+                    // (8 (r / 4) + r % 4), bits 32..63 the upper one's (4 rows on), for pixels 0..31 (fragment 0) or 32..63.
+                    // (the lane selects of v_writelane are immediates: one macro expansion per register)
+#define SNNF_PW_BITS_ROW(r)                                                                                                  \
+    {                                                                                                                        \
+        const float h0 = vd[0][r] + (acc[0][r] - vd[0][r]) * lif.inv_tau;                                                    \
+        const float h1 = vd[1][r] + (acc[1][r] - vd[1][r]) * lif.inv_tau;                                                    \
+        const bool f0 = h0 >= lif.v_threshold;                                                                               \
+        const bool f1 = h1 >= lif.v_threshold;                                                                               \
+        vd[0][r] = f0 ? lif.v_reset : h0;                                                                                    \
+        vd[1][r] = f1 ? lif.v_reset : h1;                                                                                    \
+        const uint64_t m0 = __builtin_amdgcn_ballot_w64(f0);                                                                 \
+        const uint64_t m1 = __builtin_amdgcn_ballot_w64(f1);                                                                 \
+        write_mask_lanes<8 * ((r) >> 2) + ((r) & 3)>(pend_lo, pend_hi, m0, m1);                                              \
+    }
+                    SNNF_PW_BITS_ROW(0) SNNF_PW_BITS_ROW(1) SNNF_PW_BITS_ROW(2) SNNF_PW_BITS_ROW(3)
+                    SNNF_PW_BITS_ROW(4) SNNF_PW_BITS_ROW(5) SNNF_PW_BITS_ROW(6) SNNF_PW_BITS_ROW(7)
+                    SNNF_PW_BITS_ROW(8) SNNF_PW_BITS_ROW(9) SNNF_PW_BITS_ROW(10) SNNF_PW_BITS_ROW(11)
+                    SNNF_PW_BITS_ROW(12) SNNF_PW_BITS_ROW(13) SNNF_PW_BITS_ROW(14) SNNF_PW_BITS_ROW(15)
+#undef SNNF_PW_BITS_ROW
+                } else if constexpr (DIRECT) {
                     const uint32_t one16 = F16 ? 0x3C00u : 0x3F80u;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
@@ -602,7 +655,16 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 
         // ---- last timestep's spikes and the final membrane.
         if (pend_step >= 0) flush_spikes();
-        if constexpr (DIRECT) {
+        if constexpr (BITS_OUT) {
+            if (wave_has_work && v_out != nullptr) {
+                float* __restrict__ vdst = static_cast<float*>(v_out) + tile_off + lane_off_d;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    vdst[row_off_d(r)] = vd[0][r];
+                    vdst[row_off_d(r) + 32] = vd[1][r];
+                }
+            }
+        } else if constexpr (DIRECT) {
             if (wave_has_work) {
                 char* __restrict__ vbase = reinterpret_cast<char*>(static_cast<float*>(v_out) + tile_off);   // uniform
                 const uint32_t lane_vb = lane_off_d * 4u;
@@ -692,6 +754,11 @@ int launch_conv_pw(const ConvLaunch& L, int load_mode, bool fast) {
     } else {
         if (load_mode == LOAD_ROWBITS) {    // row-packed spikes in: the fast variants with the LIF step on the accumulators
             if (!fast || L.has_residual) return fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_shape: only layers the fast variant takes");
+            if (L.g.bits_out) {
+                if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_REGS, true, true, true>);
+                if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_LDS, true, true, true>);
+                return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_STREAM, true, true, true>);
+            }
             if (L.g.w_lds == PW_WEIGHTS_REGS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_REGS, true, true>);
             if (L.g.w_lds == PW_WEIGHTS_LDS) return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_LDS, true, true>);
             return run(conv_pw_lif_kernel<XT, LOAD_ROWBITS, true, PW_WEIGHTS_STREAM, true, true>);

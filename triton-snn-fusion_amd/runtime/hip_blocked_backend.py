@@ -270,10 +270,11 @@ def unpack_rowbits(bits: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 def pointwise_conv_lif_from_rowbits(bits: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], lif: Sequence[float],
-                                    v_init: Optional[torch.Tensor] = None):
+                                    v_init: Optional[torch.Tensor] = None, packed_out: bool = False, want_v: bool = True):
     """Pointwise (1x1, stride 1) convolution + bias + LIF over T steps of row-packed spikes `bits` [T, N, Cin, H, W / 8]
     uint8 (what depthwise_conv_lif_rowbits writes). Returns (spikes [T, N, Cout, H, W] in the weight's dtype, final
-    membrane [N, Cout, H, W] fp32): the dense outputs of the operator on the unpacked tensor."""
+    membrane [N, Cout, H, W] fp32): the dense outputs of the operator on the unpacked tensor. `packed_out`: the spikes
+    leave row-packed as well ([T, N, Cout, H, W / 8] uint8), and the membrane only when asked for (`want_v`)."""
     _check_dtype(weight.dtype)
     if bits.dtype != torch.uint8 or bits.dim() != 5 or not bits[0].is_contiguous():
         raise RuntimeError("unsupported_layout: row-packed spikes [T, N, Cin, H, W / 8] uint8 expected")
@@ -291,9 +292,14 @@ def pointwise_conv_lif_from_rowbits(bits: torch.Tensor, weight: torch.Tensor, bi
         if tuple(v_init.shape) != (n, cout, h, w) or v_init.dtype != torch.float32 or v_init.device != dev:
             raise RuntimeError("unsupported_membrane_state: v_init must be a float32 [N, Cout, H, W] tensor on the activations' device")
         vi = v_init if v_init.is_contiguous() else v_init.contiguous()
-    spikes = torch.empty((T, n, cout, h, w), dtype=weight.dtype, device=dev)
-    v_out = torch.empty((n, cout, h, w), dtype=torch.float32, device=dev)
+    if packed_out:
+        spikes = torch.empty((T, n, cout, h, w8), dtype=torch.uint8, device=dev)
+    else:
+        spikes = torch.empty((T, n, cout, h, w), dtype=weight.dtype, device=dev)
+    need_v = want_v or not packed_out or T > _lib.SNNF_MAX_T_PER_LAUNCH
+    v_out = torch.empty((n, cout, h, w), dtype=torch.float32, device=dev) if need_v else None
     _lib.check("snnf_pwconv_lif_rowbits", _lib.lib().snnf_pwconv_lif_rowbits(
         _lib.packed_step_pointers(bits), T, n, cin, h, w, _lib.dtype_code(weight.dtype), packed.data_ptr(), cout, _lib.ptr(vi),
-        spikes.data_ptr(), int(spikes.stride(0)), v_out.data_ptr(), float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
-    return spikes, v_out
+        spikes.data_ptr(), 1 if packed_out else 0, int(spikes.stride(0)), _lib.ptr(v_out),
+        float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
+    return spikes, (v_out if (want_v or not packed_out) else None)
