@@ -103,13 +103,15 @@ int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int 
  * byte holds the spikes of 8 consecutive pixels of a row (bit j = pixel 8 x + j), 16 times fewer bytes than the dense
  * 0 / 1 elements the reference's kernel stores (kernels/benchmark_conv_lif_temporal_general.py:707-708, depthwise
  * emitter :713-817). Activations, residuals and membranes must be 16-byte aligned.
+ *   xs[t]      : x_packed == 0: [N, C, H, W] x_dtype; x_packed != 0: [N, C, H, W / 8] bytes packed the same way (the
+ *                output of this entry point or of snnf_pwconv_lif_rowbits; x_dtype then names the weight / operand dtype)
  *   spike_bits : [T, N, C, H, W / 8] bytes, `bits_step_stride` BYTES between timesteps
  *   v_init     : [N, C, H, W] fp32 or NULL (zeros);  v_out : the same or NULL (final membrane not stored; needs
  *                T <= SNNF_MAX_T_PER_LAUNCH)
  * snnf_rowbits_unpack turns `bytes` such bytes into 8 * bytes dense 0 / 1 elements of x_dtype (16-byte aligned).
  */
 int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T,
-                               int N, int C, int H, int W, int x_dtype,
+                               int N, int C, int H, int W, int x_dtype, int x_packed,
                                const void* weight, const void* bias, const void* v_init,
                                void* spike_bits, int64_t bits_step_stride, void* v_out,
                                float v_threshold, float v_reset, float tau, void* stream);

@@ -310,6 +310,11 @@ def test_depthwise_with_row_packed_spikes_against_the_oracle(B, dtype, N, C, H, 
     assert torch.equal(s_d, dense)
     if want_v:
         assert torch.equal(v_d, v)
+    # row-packed spikes in as well: the same bytes and membrane
+    packed_in = dev(_ref_rowbits(torch.stack(xs)), torch.uint8)
+    bits2, v2 = B.depthwise_conv_lif_rowbits(packed_in, dev(w, dtype), dev(b, dtype), lif, residuals=dr,
+                                             v_init=dev(v0, F32) if tensor_v else None, want_v=want_v)
+    assert torch.equal(bits2, bits) and (not want_v or torch.equal(v2, v))
 
 
 def test_depthwise_row_packed_spikes_reject_what_they_do_not_take(B):
@@ -398,3 +403,28 @@ def test_pointwise_from_row_packed_spikes_rejects_what_it_does_not_take(B):
     bits = torch.zeros(2, 1, 16, 8, 1, dtype=torch.uint8, device=DEV)
     with pytest.raises(RuntimeError, match="unsupported_shape"):
         B.pointwise_conv_lif_from_rowbits(bits, w, b, (1.0, -1.0, 2.0))            # soft reset: not the common neuron
+
+
+def test_two_blocks_chained_on_row_packed_spikes(B):
+    """pointwise (bits out) -> depthwise (bits in, bits out) -> pointwise (bits in): the same spikes as the dense operators."""
+    import triton_snn_fusion_amd.runtime.snn_custom_ops as ops
+    ops.configure_fused_op("hip", strict_triton=True)
+    S = torch.ops.snn_custom
+    dtype, T, N, C0, C1, C2, H, W = BF16, 4, 2, 64, 128, 64, 16, 16
+    g = gen(4600)
+    xs = [spikes((N, C0, H, W), 0.3, g) for _ in range(T)]
+    w1, b1 = dev(q(torch.randn(C1, C0, 1, 1, generator=g) * (2.0 / C0) ** 0.5 * 2.0, dtype), dtype), dev(q(torch.randn(C1, generator=g) * 0.1, dtype), dtype)
+    wd, bd = dev(q(torch.randn(C1, 1, 3, 3, generator=g) * 0.5, dtype), dtype), dev(q(torch.randn(C1, generator=g) * 0.1, dtype), dtype)
+    w2, b2 = dev(q(torch.randn(C2, C1, 1, 1, generator=g) * (2.0 / C1) ** 0.5 * 2.0, dtype), dtype), dev(q(torch.randn(C2, generator=g) * 0.1, dtype), dtype)
+    zero = torch.zeros((), device=DEV, dtype=F32)
+    dx = [dev(x, dtype) for x in xs]
+    s1, _ = S.fused_temporal_pointwise_conv_lif_state(dx, w1, b1, zero, [1, 1], [0, 0], [1, 1], 1, *LIF, False)
+    s2, _ = S.fused_temporal_depthwise_conv_lif_state(list(s1.unbind(0)), wd, bd, zero, [1, 1], [1, 1], [1, 1], C1, *LIF, False)
+    s3, v3 = S.fused_temporal_pointwise_conv_lif_state(list(s2.unbind(0)), w2, b2, zero, [1, 1], [0, 0], [1, 1], 1, *LIF, False)
+    p0 = dev(_ref_rowbits(torch.stack(xs)), torch.uint8)
+    p1, _ = B.pointwise_conv_lif_from_rowbits(p0, w1, b1, LIF, packed_out=True, want_v=False)
+    p2, _ = B.depthwise_conv_lif_rowbits(p1, wd, bd, LIF, want_v=False)
+    p3, pv3 = B.pointwise_conv_lif_from_rowbits(p2, w2, b2, LIF, packed_out=True, want_v=True)
+    assert torch.equal(B.unpack_rowbits(p1, dtype), s1)
+    assert torch.equal(B.unpack_rowbits(p2, dtype), s2)
+    assert torch.equal(B.unpack_rowbits(p3, dtype), s3) and torch.equal(pv3, v3)

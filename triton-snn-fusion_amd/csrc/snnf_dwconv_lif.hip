@@ -326,7 +326,9 @@ __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
 
 // BITS: the spikes of a strip and timestep leave as one byte (bit j = pixel 8 x + j of the row) instead of eight 16-bit
 // values: [T][N][C][Ho][Wo / 8] bytes, `spike_step_stride` then counts bytes; the final membrane is optional.
-template <typename XT, typename VT, bool STD, bool BITS = false>
+// BITS_IN: the input spikes arrive row-packed as well ([N][C][H][W / 8] bytes per timestep): a thread fetches one byte where it
+// fetched a 16-byte vector and expands it on its way into LDS.
+template <typename XT, typename VT, bool STD, bool BITS = false, bool BITS_IN = false>
 __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs, StepPtrs residuals, int has_residual,
                                                                      int T, DwGeom g, const XT* __restrict__ weight,
                                                                      const XT* __restrict__ bias,
@@ -369,7 +371,8 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
             const int cv = rem - r * g.WV;
             const int ih = in_row0 + r;
             if (ih >= 0 && ih < g.H) {
-                ld_src[k] = static_cast<uint32_t>((p * g.H + ih) * g.W + cv * PX) * ES;
+                ld_src[k] = BITS_IN ? static_cast<uint32_t>((p * g.H + ih) * g.WV + cv)      // bytes: one per 8 pixels
+                                    : static_cast<uint32_t>((p * g.H + ih) * g.W + cv * PX) * ES;
                 ld_dst[k] = p * plane_elems + r * g.pitch + kDotColOffset + cv * PX;
             }
         }
@@ -418,11 +421,29 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
     }
 
     // ---- prefetch registers and the spikes waiting to be stored.
-    dw_u32x4 pre[KL];
+    dw_u32x4 pre[BITS_IN ? 1 : KL];
+    uint32_t pre_byte[BITS_IN ? KL : 1];
     auto issue_loads = [&](int t) __attribute__((always_inline)) {
-        const char* __restrict__ x = reinterpret_cast<const char*>(static_cast<const XT*>(dw_table_entry(0, t)) + in_base);
+        if constexpr (BITS_IN) {
+            const unsigned char* __restrict__ x = static_cast<const unsigned char*>(dw_table_entry(0, t)) + (in_base >> 3);
 #pragma unroll
-        for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const dw_u32x4*>(x + ld_src[k]);
+            for (int k = 0; k < KL; ++k) pre_byte[k] = x[ld_src[k]];
+        } else {
+            const char* __restrict__ x = reinterpret_cast<const char*>(static_cast<const XT*>(dw_table_entry(0, t)) + in_base);
+#pragma unroll
+            for (int k = 0; k < KL; ++k) pre[k] = *reinterpret_cast<const dw_u32x4*>(x + ld_src[k]);
+        }
+    };
+    // Eight spike bits -> eight 16-bit ones or zeros (pixel j in element j).
+    auto expand = [&](uint32_t byte) __attribute__((always_inline)) -> dw_u32x4 {
+        constexpr uint32_t ONE = dtype_of<XT>::value == SNNF_F16 ? 0x3c00u : 0x3f80u;
+        const uint32_t m = __umul24(byte, 0x8001u);   // bit i of the byte at bits i and 15 + i
+        dw_u32x4 d;
+        d[0] = __umul24(m & 0x10001u, ONE);
+        d[1] = __umul24((m >> 2) & 0x10001u, ONE);
+        d[2] = __umul24((m >> 4) & 0x10001u, ONE);
+        d[3] = __umul24((m >> 6) & 0x10001u, ONE);
+        return d;
     };
     Pack<XT, PX> pend[BITS ? 1 : kItems];
     uint32_t pend_bits[BITS ? kItems : 1];
@@ -448,8 +469,13 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
     for (int t = 0; t < T; ++t) {
         uint16_t* __restrict__ cur = tile + buf * buf_elems;
 #pragma unroll
-        for (int k = 0; k < KL; ++k)
-            if (ld_dst[k] >= 0) *reinterpret_cast<dw_u32x4*>(cur + ld_dst[k]) = pre[k];
+        for (int k = 0; k < KL; ++k) {
+            if constexpr (BITS_IN) {
+                if (ld_dst[k] >= 0) *reinterpret_cast<dw_u32x4*>(cur + ld_dst[k]) = expand(pre_byte[k]);
+            } else {
+                if (ld_dst[k] >= 0) *reinterpret_cast<dw_u32x4*>(cur + ld_dst[k]) = pre[k];
+            }
+        }
         __syncthreads();   // tile of step t complete; every wave is past its reads of the other tile
         if (pend_t >= 0) flush();
         if (t + 1 < T) issue_loads(t + 1);
@@ -517,7 +543,7 @@ __global__ __launch_bounds__(kThreads) void dwconv3x3_lif_dot_kernel(StepPtrs xs
 }
 
 // Launcher of the packed dot-product kernel: the planning of `launch` with 16-bit rows.
-template <typename XT, typename VT, bool BITS = false>
+template <typename XT, typename VT, bool BITS = false, bool BITS_IN = false>
 int launch_dot(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGeom g, const void* weight, const void* bias,
                const void* v_init, void* spikes, int64_t spike_step_stride, void* v_out, const LifParams& lif,
                hipStream_t stream) {
@@ -553,11 +579,11 @@ int launch_dot(const StepPtrs& xs, const StepPtrs& res, int has_res, int T, DwGe
     const int64_t blocks = static_cast<int64_t>((g.planes + g.PB - 1) / g.PB) * g.bands;
     if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_dwconv3x3_lif: too many planes");
     if (lif.charge_mode == CHARGE_SCALE && !lif.soft_reset) {
-        dwconv3x3_lif_dot_kernel<XT, VT, true, BITS><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+        dwconv3x3_lif_dot_kernel<XT, VT, true, BITS, BITS_IN><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
             xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
             static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
     } else {
-        dwconv3x3_lif_dot_kernel<XT, VT, false, BITS><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
+        dwconv3x3_lif_dot_kernel<XT, VT, false, BITS, BITS_IN><<<dim3(static_cast<unsigned>(blocks)), kThreads, lds, stream>>>(
             xs, res, has_res, T, g, static_cast<const XT*>(weight), static_cast<const XT*>(bias),
             static_cast<const VT*>(v_init), static_cast<XT*>(spikes), spike_step_stride, static_cast<VT*>(v_out), lif);
     }
@@ -601,7 +627,7 @@ __global__ __launch_bounds__(kThreads) void rowbits_unpack_kernel(const unsigned
 }  // namespace snnf
 
 extern "C" int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T, int N, int C, int H, int W,
-                                          int x_dtype, const void* weight, const void* bias, const void* v_init,
+                                          int x_dtype, int x_packed, const void* weight, const void* bias, const void* v_init,
                                           void* spike_bits, int64_t bits_step_stride, void* v_out,
                                           float v_threshold, float v_reset, float tau, void* stream) {
     using namespace snnf;
@@ -624,7 +650,7 @@ extern "C" int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* con
     for (int t = 0; t < T; ++t) {
         if (xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs[%d] is null", who, t);
         if (residuals != nullptr && residuals[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: residuals[%d] is null", who, t);
-        aligned = aligned && aligned_to(xs[t], 16) && (residuals == nullptr || aligned_to(residuals[t], 16));
+        aligned = aligned && (x_packed != 0 || aligned_to(xs[t], 16)) && (residuals == nullptr || aligned_to(residuals[t], 16));
     }
     if (!aligned) return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_alignment: activations, residuals and membranes must be 16-byte aligned", who);
 
@@ -647,9 +673,15 @@ extern "C" int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* con
         const void* vi = t0 == 0 ? v_init : v_out;
         void* sp = static_cast<char*>(spike_bits) + static_cast<int64_t>(t0) * bits_step_stride;
         const int has_res = residuals != nullptr ? 1 : 0;
-        const int rc = x_dtype == SNNF_BF16
-                           ? launch_dot<bf16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs)
-                           : launch_dot<f16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs);
+        int rc;
+        if (x_packed != 0)
+            rc = x_dtype == SNNF_BF16
+                     ? launch_dot<bf16_t, float, true, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs)
+                     : launch_dot<f16_t, float, true, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs);
+        else
+            rc = x_dtype == SNNF_BF16
+                     ? launch_dot<bf16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs)
+                     : launch_dot<f16_t, float, true>(xp, rp, has_res, tw, g, weight, bias, vi, sp, bits_step_stride, v_out, lif, hs);
         if (rc != SNNF_OK) return rc;
     }
     return SNNF_OK;

@@ -230,12 +230,22 @@ def depthwise_conv_lif_rowbits(xs: Sequence[torch.Tensor], weight: torch.Tensor,
                                residuals: Optional[Sequence[torch.Tensor]] = None, v_init: Optional[torch.Tensor] = None,
                                want_v: bool = True):
     """Depthwise 3x3 (stride 1, padding 1) + bias (+ residual) + LIF over the dense steps `xs` ([N, C, H, W] each, bf16 or
-    fp16, W % 8 == 0). Returns (spike bits [T, N, C, H, W / 8] uint8, final membrane [N, C, H, W] fp32 or None)."""
+    fp16, W % 8 == 0), or over row-packed spikes (`xs` one uint8 tensor [T, N, C, H, W / 8]: the output of this function or
+    of pointwise_conv_lif_from_rowbits(packed_out=True)). Returns (spike bits [T, N, C, H, W / 8] uint8, final membrane
+    [N, C, H, W] fp32 or None)."""
+    packed_in = isinstance(xs, torch.Tensor)
+    if packed_in:
+        if xs.dtype != torch.uint8 or xs.dim() != 5 or not xs[0].is_contiguous():
+            raise RuntimeError("unsupported_layout: row-packed spikes [T, N, C, H, W / 8] uint8 expected")
+        xs = list(xs.unbind(0))
     first = xs[0]
-    _check_dtype(first.dtype)
+    op_dtype = weight.dtype if packed_in else first.dtype
+    _check_dtype(op_dtype)
     T = len(xs)
     n, c, h, w = (int(d) for d in first.shape)
-    if tuple(weight.shape) != (c, 1, 3, 3) or weight.dtype != first.dtype or bias.dtype != first.dtype:
+    if packed_in:
+        w *= 8
+    if tuple(weight.shape) != (c, 1, 3, 3) or weight.dtype != op_dtype or bias.dtype != op_dtype:
         raise RuntimeError(f"unsupported_weight: depthwise weight [C, 1, 3, 3] and bias in the activation dtype expected, got {tuple(weight.shape)}")
     if w % 8 != 0:
         raise RuntimeError(f"unsupported_shape: rows of {w} pixels do not pack into whole bytes")
@@ -252,8 +262,8 @@ def depthwise_conv_lif_rowbits(xs: Sequence[torch.Tensor], weight: torch.Tensor,
     wc = weight if weight.is_contiguous() else weight.contiguous()
     bc = bias if bias.is_contiguous() else bias.contiguous()
     _lib.check("snnf_dwconv3x3_lif_rowbits", _lib.lib().snnf_dwconv3x3_lif_rowbits(
-        _lib.step_pointers(steps), _lib.step_pointers(res) if res is not None else None, T, n, c, h, w, _lib.dtype_code(first.dtype),
-        wc.data_ptr(), bc.data_ptr(), _lib.ptr(vi), bits.data_ptr(), int(bits.stride(0)), _lib.ptr(v_out),
+        _lib.step_pointers(steps), _lib.step_pointers(res) if res is not None else None, T, n, c, h, w, _lib.dtype_code(op_dtype),
+        1 if packed_in else 0, wc.data_ptr(), bc.data_ptr(), _lib.ptr(vi), bits.data_ptr(), int(bits.stride(0)), _lib.ptr(v_out),
         float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
     return bits, (v_out if want_v else None)
 
