@@ -607,9 +607,7 @@ def main() -> int:
 
                     # The block as a network executor that owns both ends of its tensors would run it: row-packed spikes in,
                     # between the layers and out, no membrane outputs.
-                    stacked = torch.stack(list(xs))
-                    weights8 = (2 ** torch.arange(8, device=stacked.device, dtype=torch.int32))
-                    packed_x = ((stacked.reshape(tuple(stacked.shape[:-1]) + (wd // 8, 8)) != 0).to(torch.int32) * weights8).sum(-1).to(torch.uint8)
+                    packed_x = blocked.pack_rowbits(torch.stack(list(xs)))
 
                     def packed_chain(w=w, b=b, w2=w2, b2=b2):
                         packed, _ = blocked.depthwise_conv_lif_rowbits(packed_x, w, b, prep.lif, want_v=False)

@@ -108,7 +108,8 @@ int snnf_dwconv3x3_lif(const void* const* xs, const void* const* residuals, int 
  *   spike_bits : [T, N, C, H, W / 8] bytes, `bits_step_stride` BYTES between timesteps
  *   v_init     : [N, C, H, W] fp32 or NULL (zeros);  v_out : the same or NULL (final membrane not stored; needs
  *                T <= SNNF_MAX_T_PER_LAUNCH)
- * snnf_rowbits_unpack turns `bytes` such bytes into 8 * bytes dense 0 / 1 elements of x_dtype (16-byte aligned).
+ * snnf_rowbits_unpack turns `bytes` such bytes into 8 * bytes dense 0 / 1 elements of x_dtype (16-byte aligned);
+ * snnf_rowbits_pack is its inverse (bit j = element j != 0), for a network's first packed operator.
  */
 int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T,
                                int N, int C, int H, int W, int x_dtype, int x_packed,
@@ -116,6 +117,7 @@ int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residua
                                void* spike_bits, int64_t bits_step_stride, void* v_out,
                                float v_threshold, float v_reset, float tau, void* stream);
 int snnf_rowbits_unpack(const void* bits, void* dense, int64_t bytes, int x_dtype, void* stream);
+int snnf_rowbits_pack(const void* dense, void* bits, int64_t bytes, int x_dtype, void* stream);
 
 /*
  * Pointwise (1x1, stride 1) convolution + bias + LIF over T steps whose input spikes are row-packed as above: the

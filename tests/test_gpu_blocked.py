@@ -421,7 +421,8 @@ def test_two_blocks_chained_on_row_packed_spikes(B):
     s1, _ = S.fused_temporal_pointwise_conv_lif_state(dx, w1, b1, zero, [1, 1], [0, 0], [1, 1], 1, *LIF, False)
     s2, _ = S.fused_temporal_depthwise_conv_lif_state(list(s1.unbind(0)), wd, bd, zero, [1, 1], [1, 1], [1, 1], C1, *LIF, False)
     s3, v3 = S.fused_temporal_pointwise_conv_lif_state(list(s2.unbind(0)), w2, b2, zero, [1, 1], [0, 0], [1, 1], 1, *LIF, False)
-    p0 = dev(_ref_rowbits(torch.stack(xs)), torch.uint8)
+    p0 = B.pack_rowbits(torch.stack(dx))
+    assert torch.equal(p0.cpu(), _ref_rowbits(torch.stack(xs))) and torch.equal(B.unpack_rowbits(p0, dtype), torch.stack(dx))
     p1, _ = B.pointwise_conv_lif_from_rowbits(p0, w1, b1, LIF, packed_out=True, want_v=False)
     p2, _ = B.depthwise_conv_lif_rowbits(p1, wd, bd, LIF, want_v=False)
     p3, pv3 = B.pointwise_conv_lif_from_rowbits(p2, w2, b2, LIF, packed_out=True, want_v=True)

@@ -38,6 +38,7 @@ SIGNATURES = {
                                 _f, _f, _f, _vp]),
     "snnf_dwconv3x3_lif_rowbits": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i64, _vp, _f, _f, _f, _vp]),
     "snnf_rowbits_unpack": (_i, [_vp, _vp, _i64, _i, _vp]),
+    "snnf_rowbits_pack": (_i, [_vp, _vp, _i64, _i, _vp]),
     "snnf_pwconv_lif_rowbits": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _vp, _f, _f, _f, _vp]),
     "snnf_lif_pool_linear_workspace_bytes": (_sz, [_i, _i]),
     "snnf_lif_pool_linear": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _sz,

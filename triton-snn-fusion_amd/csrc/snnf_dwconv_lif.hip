@@ -623,8 +623,37 @@ __global__ __launch_bounds__(kThreads) void rowbits_unpack_kernel(const unsigned
     *reinterpret_cast<Pack<XT, 8>*>(dense + i * 8) = out;
 }
 
+// Eight dense elements (16 bytes) -> one byte of row-packed spikes (bit j = element j != 0).
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void rowbits_pack_kernel(const XT* __restrict__ dense, unsigned char* __restrict__ bits, int64_t bytes) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= bytes) return;
+    const Pack<XT, 8> in = *reinterpret_cast<const Pack<XT, 8>*>(dense + i * 8);
+    uint32_t b = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) b |= to_float(in.v[j]) != 0.0f ? (1u << j) : 0u;
+    bits[i] = static_cast<unsigned char>(b);
+}
+
 }  // namespace
 }  // namespace snnf
+
+extern "C" int snnf_rowbits_pack(const void* dense, void* bits, int64_t bytes, int x_dtype, void* stream) {
+    using namespace snnf;
+    if (bits == nullptr || dense == nullptr || bytes < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_rowbits_pack: dense and bits must be non-null, bytes >= 1");
+    if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_rowbits_pack: unsupported_dtype: bf16 or fp16");
+    if (!aligned_to(dense, 16)) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_rowbits_pack: dense must be 16-byte aligned");
+    const int64_t blocks = (bytes + kThreads - 1) / kThreads;
+    if (blocks > 0x7fffffffLL) return fail(SNNF_ERR_UNSUPPORTED, "snnf_rowbits_pack: too many bytes");
+    hipStream_t hs = as_stream(stream);
+    if (x_dtype == SNNF_BF16)
+        rowbits_pack_kernel<bf16_t><<<dim3(static_cast<unsigned>(blocks)), kThreads, 0, hs>>>(static_cast<const bf16_t*>(dense), static_cast<unsigned char*>(bits), bytes);
+    else
+        rowbits_pack_kernel<f16_t><<<dim3(static_cast<unsigned>(blocks)), kThreads, 0, hs>>>(static_cast<const f16_t*>(dense), static_cast<unsigned char*>(bits), bytes);
+    return check_launch("snnf_rowbits_pack");
+}
 
 extern "C" int snnf_dwconv3x3_lif_rowbits(const void* const* xs, const void* const* residuals, int T, int N, int C, int H, int W,
                                           int x_dtype, int x_packed, const void* weight, const void* bias, const void* v_init,

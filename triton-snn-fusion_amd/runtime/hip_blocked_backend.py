@@ -313,3 +313,15 @@ def pointwise_conv_lif_from_rowbits(bits: torch.Tensor, weight: torch.Tensor, bi
         spikes.data_ptr(), 1 if packed_out else 0, int(spikes.stride(0)), _lib.ptr(v_out),
         float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
     return spikes, (v_out if (want_v or not packed_out) else None)
+
+
+def pack_rowbits(dense: torch.Tensor) -> torch.Tensor:
+    """Dense spikes [..., W] (bf16 or fp16, W % 8 == 0) -> row-packed [..., W / 8] uint8, bit j = element 8 x + j != 0."""
+    _check_dtype(dense.dtype)
+    if int(dense.shape[-1]) % 8 != 0:
+        raise RuntimeError(f"unsupported_shape: rows of {int(dense.shape[-1])} pixels do not pack into whole bytes")
+    src = dense if dense.is_contiguous() else dense.contiguous()
+    bits = torch.empty(tuple(src.shape[:-1]) + (int(src.shape[-1]) // 8,), dtype=torch.uint8, device=src.device)
+    _lib.check("snnf_rowbits_pack", _lib.lib().snnf_rowbits_pack(src.data_ptr(), bits.data_ptr(), bits.numel(), _lib.dtype_code(src.dtype),
+                                                               _lib.current_stream(src.device)))
+    return bits
