@@ -475,6 +475,7 @@ FALLBACK_KERNEL_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, vdtype, lif
     (520, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, False, False, "matrix"),     # ... and so is a channel count of whole groups that is no multiple of the chunk
     (516, 512, 14, 14, 1, 1, 0, BF16, F32, (1.0, 0.0, 2.0), 4, 2, True, False, "t_in_m"),      # deep pointwise layer whose channels are not whole groups of 8
     (12, 32, 12, 12, 3, 1, 1, BF16, F32, (1.0, 0.0, 3.0), 4, 2, False, True, "time_outer"),     # tau not a power of two
+    (36, 44, 40, 21, 7, 2, 0, BF16, BF16, (1.0, -1.0, 2.0), 4, 3, False, False, "t_in_m"),      # 7x7 at stride 2: no tile of all 64 lanes fits the staging slots
     (44, 256, 12, 12, 3, 1, 1, BF16, F32, (0.75, 0.0, 1.5), 4, 2, False, True, "t_in_m"),      # tau not a power of two
 ]
 

@@ -43,6 +43,10 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
                                            : kConvThreads * (staging_items(load_mode) / tt);
     const int cus = compute_units() * (tt == 0 ? 2 : 1);
     double best = -1.0;
+    // Tiles normally fill the waves' pixel lanes (TH * TW == PT where the layer allows). When no such tile fits the staging
+    // slots or LDS (large kernels at stride 2 on channel counts off the fast paths), tiles of half, a quarter, ... of the
+    // lanes are tried: idle lanes, but the layer runs.
+    for (int shrink = 1; shrink <= 16 && best <= 0.0; shrink *= 2)
     for (int wn_log2 = 0; wn_log2 <= 2; ++wn_log2) {
         const int wm_log2 = 2 - wn_log2;
         const int PT = (1 << wm_log2) * 32 * kNPF;
@@ -50,7 +54,8 @@ bool plan_uncached(const ConvGeom& g0, int t_in, int tt, int load_mode, bool wan
         const int oc_tiles = (g0.Cout + OT - 1) / OT;
         const double oc_eff = static_cast<double>(g0.Cout) / (static_cast<double>(oc_tiles) * OT);
         for (int tw = 1; tw <= g0.Wo && tw <= PT; ++tw) {
-            int th = PT / tw;
+            int th = PT / tw / shrink;
+            if (th < 1) continue;
             if (th > rows) th = rows;
             ConvGeom c = g0;
             c.TW = tw;
