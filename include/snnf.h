@@ -129,7 +129,7 @@ int snnf_rowbits_pack(const void* dense, void* bits, int64_t bytes, int x_dtype,
  *   spikes     : spikes_packed == 0: [T, N, Cout, H, W] x_dtype (bf16 / fp16), `spike_step_stride` elements between timesteps;
  *                spikes_packed != 0: [T, N, Cout, H, W / 8] bytes, `spike_step_stride` BYTES between timesteps, and v_out may be
  *                NULL (final membrane not stored; needs T <= SNNF_MAX_T_PER_LAUNCH)
- * Takes what the pointwise kernel's fast variant takes: the common neuron (power-of-two tau, hard reset), Cin % 8 == 0,
+ * Takes what the pointwise kernel's fast variant takes: the common neuron (tau a power of two above 1, hard reset), Cin % 8 == 0,
  * Cout % 32 == 0, H * W % 64 == 0, 16-byte aligned outputs and membranes; SNNF_ERR_UNSUPPORTED otherwise.
  */
 int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, int H, int W, int x_dtype,

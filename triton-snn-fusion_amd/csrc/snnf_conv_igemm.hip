@@ -339,7 +339,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
         if (!pointwise || residuals != nullptr || xsize != 2 || v_dtype != SNNF_F32 || !fast_neuron || Cin % 8 != 0 || Cout % 32 != 0 ||
             g.Wo % 64 != 0 || !vec_ok || static_cast<int64_t>(Cout) * g.Wo >= (1LL << 30))
             return fail(SNNF_ERR_UNSUPPORTED, "snnf_pwconv_lif_rowbits: unsupported_shape: needs a 1x1 stride-1 layer without residual, 16-bit "
-                        "operands, an fp32 membrane, the common neuron (power-of-two tau, hard reset), Cin %% 8 == 0, Cout %% 32 == 0, "
+                        "operands, an fp32 membrane, the common neuron (tau a power of two above 1, hard reset), Cin %% 8 == 0, Cout %% 32 == 0, "
                         "H * W %% 64 == 0 and 16-byte aligned outputs");
         all_shared = false;
     } else if (out_rowbits) {
