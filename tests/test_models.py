@@ -327,3 +327,31 @@ def test_fx_rewritten_graph_runs_on_the_hip_kernels(hip_ops, name):
     cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
     print(f"{name}: FX graph vs executor, cosine similarity of the logits {cos:.5f}")
     assert cos > 0.8, cos
+
+
+@pytest.mark.gpu
+def test_internal_layouts_fall_back_to_the_dense_operator_for_a_refused_layer(hip_ops, monkeypatch):
+    """A layer the blocked kernel refuses (large kernels on many channels: `unsupported_*`) runs the dense operator on
+    unpacked tensors and re-enters the internal layout; the network's output stays that of the other executors."""
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
+    T = 4
+    _, dense = _fused("resnet18", T)
+    _, internal = _fused("resnet18", T, internal=True)
+    x = _frame("resnet18")
+    want = dense(x).float().cpu()
+    real = B.conv_lif_blocked
+    calls = {"n": 0, "refused": 0}
+
+    def picky(xb, weight, *args, **kwargs):
+        calls["n"] += 1
+        if calls["n"] in (2, 5, 7):          # three layers along the network (with and without a residual)
+            calls["refused"] += 1
+            raise RuntimeError("unsupported_shape: refused for the test")
+        return real(xb, weight, *args, **kwargs)
+
+    monkeypatch.setattr(B, "conv_lif_blocked", picky)
+    got = internal(x).float().cpu()
+    assert calls["refused"] == 3
+    cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
+    assert cos > 0.8, cos
+    assert hip_ops.get_fused_op_call_stats()["fallback"] == 0
