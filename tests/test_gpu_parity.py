@@ -792,6 +792,26 @@ def test_bf16_membrane_over_several_launches_is_rounded_once(hip_ops, Cin, Cout,
     _no_fallback(hip_ops, 2)
 
 
+def test_bf16_membrane_calls_of_one_layer_repeat_bit_for_bit(hip_ops):
+    """A 3x3 layer with Cout % 64 == 0 at T = 4 takes the matrix kernel's one-launch variant with a float32 membrane and
+    windows of 2 with a 16-bit one. Every call of the layer must compute the same way whatever earlier calls have
+    recorded about it: calls 1..3 agree bit for bit, and equal the float32-membrane call with its membrane rounded once."""
+    T, N, Cin, Cout, H, W = 4, 3, 64, 64, 16, 16
+    xs, w_dev, b_dev, w_ref, b_ref = _conv_case(8150, T, N, Cin, Cout, H, W, 3, BF16, p=0.25)
+    dx, dw, db = [dev(x, BF16) for x in xs], dev(w_dev, BF16), dev(b_dev, BF16)
+    geo = ([1, 1], [1, 1], [1, 1], 1)
+    runs = [S.fused_temporal_conv_lif_state(dx, dw, db, torch.tensor(0.0), *geo, *LIF, False) for _ in range(3)]
+    for sp, v in runs:
+        assert v.dtype == BF16
+        assert torch.equal(sp, runs[0][0]) and torch.equal(v, runs[0][1])
+    sp32, v32 = S.fused_temporal_conv_lif_state(dx, dw, db, zero_v(F32), *geo, *LIF, False)
+    assert v32.dtype == F32
+    assert torch.equal(sp32, runs[0][0]) and torch.equal(v32.to(BF16), runs[0][1])
+    ref = O.temporal_conv_lif(xs, w_ref, b_ref, torch.tensor(0.0), (1, 1), (1, 1), (1, 1), 1, *LIF)
+    check(runs[0][0], runs[0][1], ref, v_dtype=BF16, what="bf16 membrane, repeated calls")
+    _no_fallback(hip_ops, 4)
+
+
 def test_bf16_membrane_beyond_sixteen_steps_in_the_other_operators(hip_ops):
     """Depthwise, linear and the standalone scan run more than 16 steps as windows of 16; same requirement."""
     g = gen(8200)

@@ -246,8 +246,15 @@ def test_operator_names_and_schemas_are_the_reference_abi():
     assert set(ops.OPERATORS) == expected
     for name in expected:
         assert str(getattr(torch.ops.snn_custom, name).default) == f"snn_custom.{name}.default"
-    schema = str(torch.ops.snn_custom.fused_temporal_linear_lif_state_packed_out.default._schema)
-    assert "Tensor? bias" in schema and "Tensor(a!) spike_out" in schema and "Tensor(b!) v_out" in schema and schema.endswith("-> ()")
+    # Every schema, argument for argument, against the fixture written from the reference's definitions
+    # (runtime/snn_custom_ops.py:1966-2073).
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "op_schemas.json")) as f:
+        fixture = json.load(f)["schemas"]
+    assert set(fixture) == expected
+    for name, schema in fixture.items():
+        assert str(getattr(torch.ops.snn_custom, name).default._schema) == schema, name
 
 
 def test_workloads_are_seeded_and_bn_fold_is_exact_algebra():
@@ -316,18 +323,11 @@ def test_tuned_plan_table_is_well_formed():
         assert e["us"] < e["planner_us"]
 
 
-def test_a_16_bit_membrane_is_kept_wide_until_the_layer_is_known_to_take_one_launch():
-    """Which calls run with a float32 membrane and round once at the end: depthwise above 16 timesteps; any other conv until
-    the planner has reported a single launch for the layer."""
-    memo = ("k3_s1_p1", False, 4, (2, 8, 8, 8), (8, 8, 3, 3), (1, 1), (1, 1), torch.bfloat16, torch.bfloat16, False)
-    CB._TEMPORAL_CONFIGS.pop(memo, None)
-    assert not CB._takes_several_launches("depthwise_k3_s1_p1", 16, memo)
-    assert CB._takes_several_launches("depthwise_k3_s1_p1", 17, memo)
-    assert CB._takes_several_launches("k3_s1_p1", 4, memo)                      # not planned yet: assume the worst
-    try:
-        CB._TEMPORAL_CONFIGS[memo] = {"plan": {"launches": 1}}
-        assert not CB._takes_several_launches("k3_s1_p1", 4, memo)
-        CB._TEMPORAL_CONFIGS[memo] = {"plan": {"launches": 2}}
-        assert CB._takes_several_launches("k3_s1_p1", 4, memo)
-    finally:
-        CB._TEMPORAL_CONFIGS.pop(memo, None)
+def test_which_16_bit_membrane_calls_run_with_a_float32_working_membrane():
+    """Calls that may take several launches compute with a float32 membrane and round once at the end: depthwise above 16
+    timesteps, and every multi-step call of the other convolution kernels (their launch count depends on the membrane
+    dtype itself, so the rule must not depend on what an earlier call of the layer recorded)."""
+    assert not CB._takes_several_launches("depthwise_k3_s1_p1", 16)
+    assert CB._takes_several_launches("depthwise_k3_s1_p1", 17)
+    assert CB._takes_several_launches("k3_s1_p1", 4)
+    assert CB._takes_several_launches("k1_s1_p0", 2)

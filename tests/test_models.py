@@ -197,17 +197,8 @@ def _fused(name, T=4, gain=5.0, internal=False):
     return model, M.fuse_network(model, T, BF16, DEV, internal_layouts=internal)
 
 
-@pytest.mark.gpu
-@pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
-def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
-    """`internal`: spikes bit-packed and analog activations channel-blocked between the network's own operators; the
-    executor records every operator's operands and results converted back to dense tensors."""
-    T = 4
-    model, fused = _fused(name, T, internal=internal)
-    fused.record = []
-    out = fused(_frame(name))
-    torch.cuda.synchronize()
+def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
+    """Every recorded operator call of one forward against the oracle on that call's own operands (teacher forcing)."""
     kinds = [e["kind"] for e in fused.record]
     assert kinds.count("conv_lif") == (7 if name == "vgg11" else 16) and kinds.count("tail") == 1
     active = 0
@@ -244,6 +235,41 @@ def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, in
         assert stats["fallback"] == 0 and stats["triton"] == 1, stats
     else:
         assert stats["fallback"] == 0 and stats["triton"] == kinds.count("conv_lif") + 1, stats
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
+    """`internal`: spikes bit-packed and analog activations channel-blocked between the network's own operators; the
+    executor records every operator's operands and results converted back to dense tensors."""
+    T = 4
+    model, fused = _fused(name, T, internal=internal)
+    fused.record = []
+    out = fused(_frame(name))
+    torch.cuda.synchronize()
+    _check_recorded_operators(hip_ops, name, fused, out, T, internal)
+
+
+FULL = {"vgg11": dict(size=32, batch=64), "resnet18": dict(size=224, batch=16)}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_full_width_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
+    """The two benchmark configurations at their real size (width 64; VGG-11 T=4 B=64 32x32, ResNet-18 T=4 B=16 224x224):
+    every operator call of one forward, with the launch plans those sizes select, against the oracle on its own operands."""
+    T = 4
+    cfg = FULL[name]
+    model = M.build_network(name, width=64, gain=5.0)
+    fused = M.fuse_network(model, T, BF16, DEV, internal_layouts=internal)
+    x = q(torch.randn(cfg["batch"], 3, cfg["size"], cfg["size"], generator=gen(7)), BF16)
+    fused.record = []
+    print(f"full-width {name} internal={internal}", flush=True)
+    out = fused(x)
+    torch.cuda.synchronize()
+    _check_recorded_operators(hip_ops, name, fused, out, T, internal)
 
 
 @pytest.mark.gpu

@@ -52,20 +52,43 @@ def sources() -> List[Path]:
     return sorted(CSRC_DIR.glob("*.hip"))
 
 
-def _compile_one(hipcc: str, src: Path) -> Path:
+# Compiler warnings that are known and accepted: (file the warning points into, text it contains). Anything else fails
+# the build, so that a new warning (an unroll request the compiler refuses leaves a loop over a register array rolled,
+# an unused variable marks dead code) is seen when it appears and not after the kernels have slowed down.
+ALLOWED_WARNINGS = (
+    # outer epilogue loop of the 4-wave fallback kernel: too large to unroll for its widest tiles; measured as is
+    ("snnf_conv_kernel.h", "loop not unrolled"),
+)
+_NOISE = ("is not a recognized feature for this target", "warning generated", "warnings generated")
+
+
+def _split_warnings(stderr: str):
+    """(allowed, unexpected) warning lines of one compiler run; the host pass's note about the packed-fp32 feature and
+    the summary lines are dropped."""
+    allowed, unexpected = [], []
+    for line in stderr.splitlines():
+        if "warning:" not in line or any(n in line for n in _NOISE):
+            continue
+        if any(name in line and text in line for name, text in ALLOWED_WARNINGS):
+            allowed.append(line)
+        else:
+            unexpected.append(line)
+    return allowed, unexpected
+
+
+def _compile_one(hipcc: str, src: Path):
     obj = OBJ_DIR / (src.stem + ".o")
     cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
-    noise = "is not a recognized feature for this target"
-    warnings = "\n".join(line for line in proc.stderr.splitlines() if line.strip() and noise not in line)
-    if warnings.strip():
-        sys.stderr.write(f"[build] {src.name}:\n{warnings}\n")
-    return obj
+    allowed, unexpected = _split_warnings(proc.stderr)
+    if unexpected:
+        sys.stderr.write(f"[build] {src.name}:\n{proc.stderr}\n")
+    return obj, len(allowed), unexpected
 
 
-def build_library(jobs: int = 4, keep_objects: bool = False, verbose: bool = True) -> Path:
+def build_library(jobs: int = 4, keep_objects: bool = False, verbose: bool = True, allow_new_warnings: bool = False) -> Path:
     """Compiles every csrc/*.hip for gfx950 and links lib/libsnnf.so. Always recompiles."""
     hipcc = _hipcc()
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
@@ -76,7 +99,14 @@ def build_library(jobs: int = 4, keep_objects: bool = False, verbose: bool = Tru
     if verbose:
         print(f"[build] hipcc={hipcc} arch={OFFLOAD_ARCH} sources={[s.name for s in srcs]}", flush=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
-        objs = list(pool.map(lambda s: _compile_one(hipcc, s), srcs))
+        results = list(pool.map(lambda s: _compile_one(hipcc, s), srcs))
+    objs = [r[0] for r in results]
+    n_allowed = sum(r[1] for r in results)
+    unexpected = [line for r in results for line in r[2]]
+    if verbose:
+        print(f"[build] compiler warnings: {n_allowed + len(unexpected)} ({n_allowed} known, {len(unexpected)} new)", flush=True)
+    if unexpected and not allow_new_warnings:
+        raise RuntimeError("new compiler warnings (fix them or list them in ALLOWED_WARNINGS):\n" + "\n".join(unexpected))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -94,8 +124,9 @@ def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--jobs", type=int, default=4)
     ap.add_argument("--keep-objects", action="store_true")
+    ap.add_argument("--allow-new-warnings", action="store_true", help="do not fail on compiler warnings outside ALLOWED_WARNINGS")
     args = ap.parse_args()
-    build_library(jobs=args.jobs, keep_objects=args.keep_objects)
+    build_library(jobs=args.jobs, keep_objects=args.keep_objects, allow_new_warnings=args.allow_new_warnings)
 
 
 if __name__ == "__main__":

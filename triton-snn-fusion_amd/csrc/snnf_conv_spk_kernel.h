@@ -137,12 +137,17 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     // for memory in turn.
     {
         auto ka = __builtin_amdgcn_kernarg_segment_ptr();
-        uint32_t d0, d1, d2, d3, d4, d5, d6, d7, d8, d9, d10;
+        // The explicit arguments are two step tables, the geometry, five pointers and the neuron: the last dword that is
+        // touched must lie inside them (what follows is the hidden-argument area, which the compiler may leave out).
+        constexpr size_t kExplicitArgBytes = 2 * sizeof(StepPtrs) + sizeof(SpkGeom) + 5 * sizeof(void*) + sizeof(LifParams);
+        static_assert(0x280 + 4 <= kExplicitArgBytes, "argument prefetch reads past the explicit kernel arguments");
+        static_assert(kExplicitArgBytes <= 0x2c0, "argument prefetch does not cover the last cache line of the arguments");
+        uint32_t d0, d1, d2, d3, d4, d5, d6, d7, d8, d9;
         asm volatile(
-            "s_load_dword %0, %11, 0x40\n\ts_load_dword %1, %11, 0x80\n\ts_load_dword %2, %11, 0xc0\n\ts_load_dword %3, %11, 0x100\n\t"
-            "s_load_dword %4, %11, 0x140\n\ts_load_dword %5, %11, 0x180\n\ts_load_dword %6, %11, 0x1c0\n\ts_load_dword %7, %11, 0x200\n\t"
-            "s_load_dword %8, %11, 0x240\n\ts_load_dword %9, %11, 0x280\n\ts_load_dword %10, %11, 0x2c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(d0), "=&s"(d1), "=&s"(d2), "=&s"(d3), "=&s"(d4), "=&s"(d5), "=&s"(d6), "=&s"(d7), "=&s"(d8), "=&s"(d9), "=&s"(d10)
+            "s_load_dword %0, %10, 0x40\n\ts_load_dword %1, %10, 0x80\n\ts_load_dword %2, %10, 0xc0\n\ts_load_dword %3, %10, 0x100\n\t"
+            "s_load_dword %4, %10, 0x140\n\ts_load_dword %5, %10, 0x180\n\ts_load_dword %6, %10, 0x1c0\n\ts_load_dword %7, %10, 0x200\n\t"
+            "s_load_dword %8, %10, 0x240\n\ts_load_dword %9, %10, 0x280\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(d0), "=&s"(d1), "=&s"(d2), "=&s"(d3), "=&s"(d4), "=&s"(d5), "=&s"(d6), "=&s"(d7), "=&s"(d8), "=&s"(d9)
             : "s"(ka));
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -174,7 +179,6 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const int tiles_per_block = SK ? (kSpkWaves >> g.wk_log2) : kSpkWaves;
     const int po = g.Ho * g.Wo;
     const int nsteps_t = g.shared_x ? 1 : g.T;          // timesteps with a convolution of their own
-    const uint16_t* __restrict__ wlane = wpacked + lane * 8;
     const int hg = g.tap_pairs ? 1 : (g.G >> 1);        // k-slot pairs per tap and stage
     const int nst = g.tap_pairs ? g.npairs : g.taps * hg;   // matrix steps per stage
     const bool common_lif = lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;

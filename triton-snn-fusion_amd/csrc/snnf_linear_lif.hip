@@ -206,12 +206,13 @@ __global__ __launch_bounds__(LinWaves<TT>::value * 64) void linear_lif_kernel(St
         float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
-            if (t >= g.T) break;
-            float sum = 0.0f;
+            if (t < g.T) {      // a guard, not a break: a second loop exit keeps the compiler from unrolling over t
+                float sum = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW; w += 2) sum += partial[(w * TT + t) * SLAB + slot] + partial[((w + 1) * TT + t) * SLAB + slot];
-            const float cur = sum + bv;
-            spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+                for (int w = 0; w < NW; w += 2) sum += partial[(w * TT + t) * SLAB + slot] + partial[((w + 1) * TT + t) * SLAB + slot];
+                const float cur = sum + bv;
+                spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+            }
         }
         v_out[o] = from_float<VT>(v);
     }
@@ -404,8 +405,10 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     // and runs the recurrence. It leaves the counter at zero for the next launch. The sums and the counter travel as
     // device-scope atomic stores, loads and adds (relaxed): those go through to memory, past the L2 caches of the chip's
     // partitions, which do not see each other's lines. A device-scope fence would do too, but it writes back a whole L2
-    // per wave that executes it and costs more than the kernel. Order: a workgroup barrier waits for each thread's stores
-    // to be acknowledged before one thread counts the workgroup in.
+    // per wave that executes it and costs more than the kernel. Order: every thread waits until its own write-through
+    // stores have been acknowledged (an explicit wait on the vector-memory counter: neither a workgroup barrier nor a
+    // workgroup-scope fence implies one for global stores), then the workgroup barrier, then one thread counts the
+    // workgroup in. The last arriver's loads are device-scope atomic loads issued after it has read the counter.
     const int parts = static_cast<int>(gridDim.z);
     const int tile = static_cast<int>(blockIdx.y * gridDim.x + blockIdx.x);
     if (parts > 1) {
@@ -421,6 +424,7 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
                 __hip_atomic_store(mine + t * OUTS + e, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this thread's partial sums have reached memory
         __syncthreads();
         if (tid == 0) {
             const int before = __hip_atomic_fetch_add(ws_count + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -442,16 +446,17 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         const float* __restrict__ all = ws_partial + static_cast<int64_t>(tile) * parts * (TT * OUTS) + e;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
-            if (t >= g.T) break;
-            float sum = 0.0f;
-            if (parts > 1) {
-                for (int z = 0; z < parts; ++z) sum += __hip_atomic_load(all + (static_cast<int64_t>(z) * TT + t) * OUTS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            } else {
+            if (t < g.T) {      // a guard, not a break: a second loop exit keeps the compiler from unrolling over t
+                float sum = 0.0f;
+                if (parts > 1) {
+                    for (int z = 0; z < parts; ++z) sum += __hip_atomic_load(all + (static_cast<int64_t>(z) * TT + t) * OUTS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
 #pragma unroll
-                for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+                    for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
+                }
+                const float cur = sum + bv;
+                spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
             }
-            const float cur = sum + bv;
-            spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
         }
         v_out[o] = from_float<VT>(v);
     }

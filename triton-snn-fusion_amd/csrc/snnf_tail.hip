@@ -342,7 +342,6 @@ __global__ __launch_bounds__(kThreads) void count_linear_mm_kernel(const int* __
     tail_f32x4 acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
     tail_f32x4 acc_hi = {0.0f, 0.0f, 0.0f, 0.0f};
     const int ksteps = C >> 5;
-#pragma unroll 4
     for (int ks = wave; ks < ksteps; ks += kThreads / 64) {
         const snnf_u32x4 wf = *reinterpret_cast<const snnf_u32x4*>(w_row + ks * 32);
         const Pack<int, 4> c0 = *reinterpret_cast<const Pack<int, 4>*>(c_row + ks * 32);

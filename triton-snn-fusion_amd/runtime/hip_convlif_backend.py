@@ -459,9 +459,10 @@ def _run_temporal(kind: str, xs, residuals, weight, bias, v_init, stride, paddin
             first.dtype, v_dtype, isinstance(v_init, torch.Tensor) and v_init.dim() > 0)
     # A call of more timesteps than one launch takes hands the membrane from launch to launch through `v_out`. A 16-bit
     # membrane would be rounded at every hand-over, where the reference's kernel rounds once after the last step
-    # (kernels/benchmark_conv_lif_temporal_general.py:707-716). Such a call computes with a float32 membrane and rounds
-    # the result; how many launches a layer takes is the planner's answer, known after the layer's first call.
-    wide = v_dtype != torch.float32 and T > 1 and _takes_several_launches(kernel_key, T, memo)
+    # (kernels/benchmark_conv_lif_temporal_general.py:707-716). How many launches the matrix kernels take depends on the
+    # membrane dtype itself (their one-launch variant needs a float32 membrane), so every multi-step call with a 16-bit
+    # membrane computes with a float32 working membrane and rounds the result once: the same arithmetic on every call.
+    wide = v_dtype != torch.float32 and T > 1 and _takes_several_launches(kernel_key, T)
     v_work = torch.empty(out_shape, dtype=torch.float32, device=first.device) if wide else v_next
     if wide and isinstance(v_init, torch.Tensor) and v_init.dim() > 0:
         v_init = v_init.float()
@@ -479,13 +480,10 @@ def _run_temporal(kind: str, xs, residuals, weight, bias, v_init, stride, paddin
     )
 
 
-def _takes_several_launches(kernel_key: str, T: int, memo: tuple) -> bool:
+def _takes_several_launches(kernel_key: str, T: int) -> bool:
     if kernel_key.startswith("depthwise_"):
         return T > _lib.SNNF_MAX_T_PER_LAUNCH     # the depthwise kernel holds up to 16 steps per launch
-    known = _TEMPORAL_CONFIGS.get(memo)
-    if known is None or "plan" not in known:
-        return True                               # not planned yet: assume the worst
-    return int(known["plan"].get("launches", 2)) > 1
+    return True                                   # matrix kernels: windows of 2 or 4 steps, chosen per membrane dtype
 
 
 def _check_output_buffers(spike_out, v_out, spike_shape, v_shape, like: torch.Tensor, v_dtype) -> None:

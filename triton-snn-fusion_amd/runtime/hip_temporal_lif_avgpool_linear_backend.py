@@ -35,42 +35,69 @@ def strict_temporal_lif_avgpool_linear_enabled(strict: bool = False) -> bool:
     return bool(strict) or os.environ.get("CHRONOS_STRICT_TEMPORAL_LIF_AVGPOOL_LINEAR_TRITON", "0") == "1"
 
 
+def _same_place_and_dtype(t: torch.Tensor, like: torch.Tensor) -> bool:
+    return t.device == like.device and t.dtype == like.dtype
+
+
+def _input_reasons(x_seq: torch.Tensor) -> List[str]:
+    """What the pooling kernel needs of its input: a [T, N, C, H, W] tensor on the GPU in one of the three dtypes, T within
+    one launch, planes that a workgroup can walk."""
+    found: List[str] = []
+    if x_seq.device.type != "cuda":
+        found.append("unsupported_device: x_seq is not CUDA")
+    if x_seq.dtype not in SUPPORTED_DTYPES:
+        found.append(f"unsupported_dtype: x_seq dtype must be float32, bfloat16 or float16, got {x_seq.dtype}")
+    if x_seq.dim() != 5:
+        found.append(f"unsupported_rank: x_seq.dim must be 5, got {x_seq.dim()}")
+        return found
+    T, _, _, H, W = (int(d) for d in x_seq.shape)
+    if T < 1 or T > MAX_TIMESTEPS:
+        found.append(f"unsupported_temporal_length: T must be in 1..{MAX_TIMESTEPS}, got {T}")
+    if H * W > MAX_PLANE_ELEMENTS:
+        found.append(f"unsupported_shape: H*W must be at most {MAX_PLANE_ELEMENTS}, got {H * W}")
+    return found
+
+
+def _classifier_reasons(x_seq: torch.Tensor, fc_weight, fc_bias) -> List[str]:
+    """[classes, C] weights (and an optional [classes] bias) stored like the activations."""
+    if not isinstance(fc_weight, torch.Tensor) or fc_weight.dim() != 2:
+        return ["fc_weight must be a 2D tensor"]
+    found: List[str] = []
+    classes, features = (int(d) for d in fc_weight.shape)
+    if x_seq.dim() == 5 and features != int(x_seq.shape[2]):
+        found.append(f"unsupported_linear: fc in_features {features} must match channels {int(x_seq.shape[2])}")
+    if not _same_place_and_dtype(fc_weight, x_seq):
+        found.append("unsupported_dtype: fc_weight device/dtype must match x_seq")
+    if isinstance(fc_bias, torch.Tensor) and fc_bias.numel() > 0:      # None or an empty tensor: no bias
+        if fc_bias.numel() != classes:
+            found.append("unsupported_linear: fc_bias shape does not match out_features")
+        if not _same_place_and_dtype(fc_bias, x_seq):
+            found.append("unsupported_dtype: fc_bias device/dtype must match x_seq")
+    return found
+
+
+def _state_reasons(x_seq: torch.Tensor, v_init) -> List[str]:
+    """A 0-dim `v_init` stands for zeros; a full one must have the neurons' shape, in the activation dtype or float32."""
+    if not isinstance(v_init, torch.Tensor):
+        return ["v_init must be a tensor"]
+    if v_init.dim() == 0:
+        return []
+    found: List[str] = []
+    if x_seq.dim() == 5 and v_init.shape != x_seq.shape[1:]:
+        found.append(f"unsupported_membrane_state: v_init shape {tuple(v_init.shape)} does not match {tuple(x_seq.shape[1:])}")
+    if v_init.device != x_seq.device or v_init.dtype not in (x_seq.dtype, torch.float32):
+        found.append("unsupported_dtype: v_init device/dtype must match x_seq (or be float32)")
+    return found
+
+
 def check_temporal_lif_avgpool_linear_support(x_seq, v_init, fc_weight, fc_bias, tau) -> List[str]:
-    """Counterpart of runtime/triton_temporal_lif_avgpool_linear_backend.py:22-55."""
+    """Counterpart of runtime/triton_temporal_lif_avgpool_linear_backend.py:22-55: the reasons (each with the
+    `unsupported_*:` prefix the operator layer turns into a statistics key) why a call cannot run on the HIP tail kernels;
+    empty when it can. Wider than the reference's: bfloat16, any T up to one launch window, float32 membranes next to
+    16-bit activations."""
     if not isinstance(x_seq, torch.Tensor):
         return ["x_seq must be a tensor"]
-    reasons: List[str] = []
-    if not x_seq.is_cuda:
-        reasons.append("unsupported_device: x_seq is not CUDA")
-    if x_seq.dim() != 5:
-        reasons.append(f"unsupported_rank: x_seq.dim must be 5, got {x_seq.dim()}")
-    if x_seq.dtype not in SUPPORTED_DTYPES:
-        reasons.append(f"unsupported_dtype: x_seq dtype must be float32, bfloat16 or float16, got {x_seq.dtype}")
-    if x_seq.dim() == 5:
-        if not 1 <= int(x_seq.shape[0]) <= MAX_TIMESTEPS:
-            reasons.append(f"unsupported_temporal_length: T must be in 1..{MAX_TIMESTEPS}, got {int(x_seq.shape[0])}")
-        if int(x_seq.shape[3]) * int(x_seq.shape[4]) > MAX_PLANE_ELEMENTS:
-            reasons.append(f"unsupported_shape: H*W must be at most {MAX_PLANE_ELEMENTS}, got {int(x_seq.shape[3]) * int(x_seq.shape[4])}")
-    if not isinstance(v_init, torch.Tensor):
-        reasons.append("v_init must be a tensor")
-    elif v_init.dim() != 0:
-        if x_seq.dim() == 5 and tuple(v_init.shape) != tuple(x_seq.shape[1:]):
-            reasons.append(
-                f"unsupported_membrane_state: v_init shape {tuple(v_init.shape)} does not match {tuple(x_seq.shape[1:])}")
-        if v_init.device != x_seq.device or v_init.dtype not in (x_seq.dtype, torch.float32):
-            reasons.append("unsupported_dtype: v_init device/dtype must match x_seq (or be float32)")
-    if not isinstance(fc_weight, torch.Tensor) or fc_weight.dim() != 2:
-        reasons.append("fc_weight must be a 2D tensor")
-    elif x_seq.dim() == 5:
-        if int(fc_weight.shape[1]) != int(x_seq.shape[2]):
-            reasons.append(f"unsupported_linear: fc in_features {fc_weight.shape[1]} must match channels {x_seq.shape[2]}")
-        if fc_weight.device != x_seq.device or fc_weight.dtype != x_seq.dtype:
-            reasons.append("unsupported_dtype: fc_weight device/dtype must match x_seq")
-    if isinstance(fc_bias, torch.Tensor) and fc_bias.numel() > 0:
-        if isinstance(fc_weight, torch.Tensor) and fc_weight.dim() == 2 and fc_bias.numel() != fc_weight.shape[0]:
-            reasons.append("unsupported_linear: fc_bias shape does not match out_features")
-        if fc_bias.device != x_seq.device or fc_bias.dtype != x_seq.dtype:
-            reasons.append("unsupported_dtype: fc_bias device/dtype must match x_seq")
+    reasons = _input_reasons(x_seq) + _state_reasons(x_seq, v_init) + _classifier_reasons(x_seq, fc_weight, fc_bias)
     if float(tau) == 0.0:
         reasons.append("unsupported_tau: tau must be nonzero")
     return reasons
@@ -110,14 +137,13 @@ def run_triton_fused_temporal_lif_avgpool_linear(x_seq, v_init, fc_weight, fc_bi
         w.data_ptr(), _lib.ptr(b), K, _lib.dtype_code(w.dtype), out_sum.data_ptr(), v_next.data_ptr(),
         workspace.data_ptr(), ws_bytes, float(v_threshold), float(v_reset), float(tau), _lib.current_stream(x.device)))
     diagnostics = {
-        "kernel_kind": "standalone_temporal_lif_avgpool_linear",
-        "fuse_organization": "two_stage_fused_pipeline",
-        "stage_0": "lif_recurrence_plus_spike_count_per_plane",
-        "stage_1": "linear_over_time_summed_counts",
-        "intermediate_materialization": "counts[N,C] int32",
-        "compute_dtype": "float16" if x.dtype == torch.float16 else "float32",
-        "T": T,
-        "shape": tuple(x.shape),
+        "kernel_kind": "temporal_lif_avgpool_linear",
+        "launches": ["lif_scan_with_spike_counts_per_plane", "classifier_on_summed_counts"],
+        "workspace": f"int32 spike counts [{N}, {C}]",
+        "membrane_dtype": str(v_dtype),
+        "accumulator_dtype": "float32",
+        "timesteps": T,
+        "plane": (H, W),
         "classes": K,
     }
     return TritonTemporalLIFAvgPoolLinearResult(out_sum, v_next, True, kernel_diagnostics=diagnostics)

@@ -172,7 +172,10 @@ def _run_steps(steps: List[torch.Tensor], weight, bias, v_init, v_threshold, v_r
 # leaves its counters zero). A call under stream capture cannot allocate, and its stream exists only for the capture, so
 # captured calls share one workspace per device that the eager calls before the capture (the warm-up every capture
 # needs anyway) have prepared; without one they run unsplit. Graphs that share it must not replay concurrently.
+# A captured graph holds the raw address of the workspace it was captured with, so a workspace that a larger layer
+# outgrows is never handed back to the allocator: it moves to `_RETIRED_WORKSPACES` and lives as long as the process.
 _WORKSPACES: Dict = {}
+_RETIRED_WORKSPACES: list = []
 
 
 def _split_workspace(lib, device, T: int, M: int, Fin: int, Fout: int):
@@ -188,6 +191,8 @@ def _split_workspace(lib, device, T: int, M: int, Fin: int, Fout: int):
         if have is None or have.numel() < need:
             if capturing:
                 return None
+            if have is not None:
+                _RETIRED_WORKSPACES.append(have)     # an earlier capture may still replay on it
             _WORKSPACES[k] = torch.zeros(need, dtype=torch.uint8, device=device)
     return _WORKSPACES[key]
 
