@@ -189,6 +189,69 @@ def test_fx_rewrite_leaves_a_layer_alone_when_its_state_chain_is_broken():
         assert torch.allclose(gm(x), want)
 
 
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_layout_propagation_graph_invariants(name):
+    """compile_temporal(internal_layouts=True): every fused convolution, LIF-free convolution and pool of the rewritten graph
+    calls an internal-layout entry point on `Blocked` values; dense tensors exist at the input (one conversion of the
+    shared frame) and in front of the tail operator (one conversion, of a tensor the last convolution wrote dense)."""
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
+    T = 4
+    model = M.build_network(name, width=16, gain=5.0)
+    gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, internal_layouts=True)
+    S = torch.ops.snn_custom
+    calls = [n for n in gm.graph.nodes if n.op == "call_function"]
+    targets = [n.target for n in calls]
+    n_conv, n_pool = (8, 4) if name == "vgg11" else (20, 1)
+    assert targets.count(R.blocked_conv_lif) == n_conv and targets.count(R.blocked_pool) == n_pool
+    assert stats.internal_layout_nodes == n_conv + n_pool and not stats.skipped
+    assert targets.count(R.blocked_input) == 1 and targets.count(R.blocked_to_dense) == 1 and targets.count(R.blocked_residual) == 0
+    assert targets.count(S.fused_temporal_lif_avgpool_linear) == 1
+    dense_ops = (S.fused_temporal_conv_lif_state, S.fused_temporal_conv_add_lif_state, R.pooled_frames, R.conv_bias_frames)
+    assert not any(t in dense_ops for t in targets) and not any(n.op == "call_module" for n in gm.graph.nodes)
+    first = next(n for n in calls if n.target is R.blocked_input)
+    assert first.args[0].op == "placeholder" and first.args[1:] == (T, True)          # one shared analog frame
+    convs = [n for n in calls if n.target is R.blocked_conv_lif]
+    # layouts: spikes leave bit-packed, LIF-free shortcut sums channel-blocked, the tensor the tail reads dense
+    assert [n.args[7] for n in convs if n.args[5] is not None] == [B.BITS] * sum(n.args[5] is not None for n in convs)
+    plain = [n for n in convs if n.args[5] is None]
+    assert [n.args[7] for n in plain] == ([B.NCHW] if name == "vgg11" else [B.C8, B.C8, B.C8, B.NCHW])
+    assert convs[-1] is plain[-1] and next(iter(convs[-1].users)).target is R.blocked_to_dense
+    if name == "resnet18":
+        # residuals: the block input itself (bits) for plain blocks, the shortcut convolution's output for down-sampling ones
+        with_res = [n for n in convs if n.args[6] is not None]
+        assert len(with_res) == 8 and all(n.args[6].target in (R.blocked_conv_lif, R.blocked_pool) for n in with_res)
+        assert sum(n.args[6] in plain for n in with_res) == 3
+        assert plain[-1].args[6] is not None                                            # the pre-tail sum is the convolution's residual
+    # every operand of a converted node is another converted node (or the input conversion): no dense hop in between
+    for n in convs + [c for c in calls if c.target is R.blocked_pool]:
+        assert n.args[0].target in (R.blocked_conv_lif, R.blocked_pool, R.blocked_input)
+
+
+def test_fx_layout_propagation_keeps_dense_tensors_around_nodes_it_does_not_know():
+    """A stateless layer the pass has no kernel for (here a Hardtanh between two fused layers) reads a dense tensor and hands
+    one on: the graph converts once on either side of it."""
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = M.ConvBNNeuron(3, 16, 3, 1, 1)
+            self.clip = torch.nn.Hardtanh(0.0, 0.5)
+            self.b = M.ConvBNNeuron(16, 16, 3, 1, 1)
+            self.c = M.ConvBNNeuron(16, 16, 3, 1, 1)
+
+        def forward(self, x):
+            return self.c(self.b(self.clip(self.a(x)))).mean((2, 3))
+
+    net = M.init_synthetic_(Net(), gain=5.0)
+    gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(net, 4), internal_layouts=True)
+    targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+    assert targets.count(R.blocked_conv_lif) == 3 and stats.internal_layout_nodes == 3
+    assert targets.count(R.blocked_input) == 2 and targets.count(R.blocked_to_dense) == 2
+    convs = [n for n in gm.graph.nodes if n.op == "call_function" and n.target is R.blocked_conv_lif]
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
+    assert [n.args[7] for n in convs] == [B.NCHW, B.BITS, B.NCHW]       # only the b -> c hand-over stays inside the layouts
+    assert convs[2].args[0] is convs[1]
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # Fused form (GPU)
 # ---------------------------------------------------------------------------------------------------------------
@@ -353,6 +416,68 @@ def test_fx_rewritten_graph_runs_on_the_hip_kernels(hip_ops, name):
     cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
     print(f"{name}: FX graph vs executor, cosine similarity of the logits {cos:.5f}")
     assert cos > 0.8, cos
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_graph_on_the_internal_layouts_equals_the_hand_lowered_executor(hip_ops, name):
+    """The layout-propagated graph launches the same kernels on the same operands as `fuse_network(internal_layouts=True)`:
+    bit-identical logits, eagerly and under HIP graph replay, with only the tail going through the dense operator layer."""
+    T = 4
+    model, internal = _fused(name, T, internal=True)
+    gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16, internal_layouts=True)
+    assert not stats.skipped and stats.internal_layout_nodes == (12 if name == "vgg11" else 21)
+    frames = [_frame(name, seed=30 + i).to(DEV, BF16) for i in range(3)]
+    hip_ops.reset_fused_op_call_stats()
+    with torch.no_grad():
+        got = gm(frames[0])
+    stats_ops = hip_ops.get_fused_op_call_stats()
+    assert stats_ops["fallback"] == 0 and stats_ops["triton"] == 1, stats_ops
+    assert torch.equal(got, internal(frames[0]))
+    # whole-graph capture and replay, eager work in between
+    static_in = frames[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        gm(static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        static_out = gm(static_in)
+    for f in frames + [frames[0]]:
+        want = internal(f).clone()
+        torch.cuda.synchronize()
+        static_in.copy_(f)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, want)
+
+
+@pytest.mark.gpu
+def test_fx_graph_with_an_unknown_layer_between_fused_layers_on_the_gpu(hip_ops):
+    """Dense hand-overs around a node the layout pass does not know: same logits as the dense rewritten graph up to
+    near-threshold flips (both graphs run the same arithmetic on different kernels)."""
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = M.ConvBNNeuron(3, 16, 3, 1, 1)
+            self.clip = torch.nn.Hardtanh(0.0, 0.5)
+            self.b = M.ConvBNNeuron(16, 32, 3, 1, 1)
+            self.c = M.ConvBNNeuron(32, 16, 3, 1, 1)
+
+        def forward(self, x):
+            return self.c(self.b(self.clip(self.a(x)))).mean((2, 3))
+
+    net = M.init_synthetic_(Net(), gain=5.0)
+    x = q(torch.randn(2, 3, 16, 16, generator=gen(41)), BF16).to(DEV, BF16)
+    dense, _ = R.compile_temporal(M.SingleStepModeLoopWrapper(net, 4), device=DEV, dtype=BF16)
+    blocked, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(net, 4), device=DEV, dtype=BF16, internal_layouts=True)
+    assert stats.internal_layout_nodes == 3
+    with torch.no_grad():
+        want, got = dense(x).float(), blocked(x).float()
+    assert float((want - got).abs().max()) <= 0.05 and float(want.abs().max()) > 0.05, (want, got)
+    assert hip_ops.get_fused_op_call_stats()["fallback"] == 0
 
 
 @pytest.mark.gpu

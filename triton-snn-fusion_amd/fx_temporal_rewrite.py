@@ -289,6 +289,7 @@ class RewriteStats:
     temporal_lif_avgpool_linear_groups: int = 0
     replaced_patterns: int = 0
     batched_timestep_calls: int = 0
+    internal_layout_nodes: int = 0
     skipped: List[str] = field(default_factory=list)
 
 
@@ -545,6 +546,224 @@ def batch_timestep_calls(gm: fx.GraphModule) -> int:
     return removed
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# Internal layouts between the fused operators of one graph
+# ---------------------------------------------------------------------------------------------------------------
+# The reference's executor recognises fused convolution nodes of the rewritten graph and runs them on a faster entry point
+# of the same backend, with pooled caller-owned buffers (runtime/fx_standalone_executor.py:900-952), and its rewrite is what
+# hands it those nodes (compiler/fx_lif_temporal_rewrite.py:2037-2113, 2214-2333). The counterpart here is a pass over the
+# rewritten graph: wherever a fused operator's [T, N, C, H, W] output is consumed by other operators the internal-layout
+# kernels serve (fused convolutions, LIF-free convolutions, pools), the tensor between them travels bit-packed (spikes) or
+# channel-blocked (analog values) as a `Blocked` value and the nodes call the internal-layout entry points
+# (runtime/hip_blocked_backend.py); dense tensors remain at the graph's inputs and outputs and in front of every node the
+# pass does not know. The graph functions below are the targets of the new nodes.
+def blocked_input(frames, T: int, shared: bool):
+    """Graph input side: one analog frame [N, C, H, W] shared by all T steps, or a dense [T, N, C, H, W] tensor (or the
+    list of its T steps), into the channel-blocked layout."""
+    from .runtime import hip_blocked_backend as B
+    if shared:
+        x = B.from_dense(frames.contiguous(), B.C8, shared=True)
+        x.T = int(T)
+        return x
+    if isinstance(frames, (list, tuple)):
+        frames = torch.stack(list(frames))
+    return B.from_dense(frames, B.C8)
+
+
+def blocked_residual(frames):
+    """A dense [T, N, C, H, W] tensor (or the list of its steps) as a residual operand: no conversion, the kernel reads
+    dense residuals as they are."""
+    from .runtime import hip_blocked_backend as B
+    if isinstance(frames, (list, tuple)):
+        frames = torch.stack(list(frames))
+    return B.from_dense(frames, B.NCHW)
+
+
+def blocked_conv_lif(x, weight, bias, stride, padding, lif, residual, out_layout: int):
+    """Conv + folded BN (+ residual) + LIF over the T steps of a `Blocked` value, or without a neuron when `lif` is None."""
+    from .runtime import hip_blocked_backend as B
+    out, _ = B.conv_lif_blocked_or_dense(x, weight, bias, stride, padding, lif, residual=residual, out_layout=out_layout)
+    return out
+
+
+def blocked_pool(x, is_max: bool, kernel: int, stride: int, padding: int):
+    from .runtime import hip_blocked_backend as B
+    try:
+        return B.pool_blocked(x, is_max, kernel, stride, padding)
+    except RuntimeError as exc:
+        if "unsupported" not in str(exc):
+            raise
+    y = pooled_frames(B.to_dense(x), is_max, kernel, stride, padding)
+    return B.from_dense(y.contiguous(), x.layout if is_max else B.C8)
+
+
+def blocked_to_dense(x):
+    from .runtime import hip_blocked_backend as B
+    return B.to_dense(x)
+
+
+def _scalar_zero_node(gm: fx.GraphModule, node) -> bool:
+    return _is_scalar_zero(gm, node)
+
+
+def _sequence_source(arg, T_hint: Optional[int] = None):
+    """What a list of per-timestep operands is made of: ("shared", frame node, T) for one node repeated, ("stack", node, T)
+    for stack[0], ..., stack[T-1] in order, ("list", [nodes], T) otherwise; a single node stands for a whole stack."""
+    if isinstance(arg, fx.Node):
+        return ("stack", arg, T_hint)
+    parts = list(arg)
+    T = len(parts)
+    if T > 1 and all(p is parts[0] for p in parts):
+        return ("shared", parts[0], T)
+    if (all(isinstance(p, fx.Node) and p.op == "call_function" and p.target is operator.getitem for p in parts)
+            and len({p.args[0] for p in parts}) == 1 and [p.args[1] for p in parts] == list(range(T))):
+        return ("stack", parts[0].args[0], T)
+    return ("list", parts, T)
+
+
+def propagate_internal_layouts(gm: fx.GraphModule) -> int:
+    """Moves every chain fused operator -> (pool | LIF-free convolution) -> fused operator of a rewritten graph onto the
+    internal layouts. Returns the number of nodes that now call an internal-layout entry point. A node is converted when
+    it is a fused (residual) convolution from the scalar-zero membrane with nobody reading its final membrane, a
+    `conv_bias_frames` / `pooled_frames` call, or the sum of a LIF-free convolution and a stack (folded into that
+    convolution as its residual); everything else keeps reading dense tensors, converted once where needed."""
+    from .runtime import hip_blocked_backend as B
+    S = torch.ops.snn_custom
+    conv_ops = {S.fused_temporal_conv_lif_state: False, S.fused_temporal_conv_lif_state.default: False,
+                S.fused_temporal_conv_add_lif_state: True, S.fused_temporal_conv_add_lif_state.default: True}
+    graph = gm.graph
+
+    def fused_conv(node: fx.Node):
+        """(has_residual, spike stack node) of a convertible fused convolution node, else None."""
+        if node.op != "call_function" or node.target not in conv_ops or node.kwargs:
+            return None
+        res = conv_ops[node.target]
+        a = node.args
+        base = 2 if res else 1
+        if len(a) != base + 11:
+            return None
+        w, b, v0, stride, padding, dilation, groups = a[base:base + 7]
+        if not _scalar_zero_node(gm, v0) or list(dilation) != [1, 1] or int(groups) != 1:
+            return None
+        items = find_tuple_getitems(node)
+        if len(node.users) != 1 or 0 not in items:
+            return None                       # somebody reads the final membrane (or the tuple itself)
+        return res, items[0]
+
+    def pool_ok(node: fx.Node) -> bool:
+        if node.op != "call_function" or node.target is not pooled_frames or node.kwargs or len(node.args) != 5:
+            return False
+        _, is_max, k, s, p = node.args
+        return (bool(is_max) and k in (2, 3) and s == 2) or (not is_max and k == 2 and s == 2 and p == 0)
+
+    def plain_conv_ok(node: fx.Node) -> bool:
+        return node.op == "call_function" and node.target is conv_bias_frames and not node.kwargs and len(node.args) == 5
+
+    def pretail_sum(node: fx.Node):
+        """(conv_bias_frames node, other operand) when `node` adds a LIF-free convolution that nobody else reads to a stack."""
+        if not _is_add_node(node) or len(node.args) != 2 or node.kwargs:
+            return None
+        for conv, other in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
+            if isinstance(conv, fx.Node) and plain_conv_ok(conv) and len(conv.users) == 1 and isinstance(other, fx.Node):
+                return conv, other
+        return None
+
+    # Phase 1: which nodes will read their operands as Blocked values (a node's own output layout depends on them).
+    convertible = set()
+    absorbed = set()        # LIF-free convolutions folded into the sum that follows them
+    for node in graph.nodes:
+        pair = pretail_sum(node)
+        if pair is not None:
+            convertible.add(node)
+            absorbed.add(pair[0])
+        elif fused_conv(node) is not None or pool_ok(node) or plain_conv_ok(node):
+            convertible.add(node)
+    convertible -= absorbed
+
+    def reads_blocked(stack: fx.Node) -> Tuple[bool, bool]:
+        """(some user reads the stack as a Blocked value, some user needs it dense)."""
+        blocked = dense = False
+        for user in stack.users:
+            if user in absorbed:
+                user = next(iter(user.users))
+            if user.op == "call_function" and user.target is operator.getitem and isinstance(user.args[1], int):
+                for leaf in user.users:
+                    if leaf in convertible and fused_conv(leaf) is not None:
+                        blocked = True
+                    else:
+                        dense = True
+            elif user in convertible:
+                blocked = True
+            else:
+                dense = True
+        return blocked, dense
+
+    blocked_of: Dict[fx.Node, fx.Node] = {}      # stack-level node -> node holding its Blocked value
+    layout_of: Dict[fx.Node, int] = {}
+    inputs: Dict[Tuple, fx.Node] = {}
+    converted = 0
+
+    def as_blocked(arg, residual: bool, T_hint=None) -> fx.Node:
+        kind, src, T = _sequence_source(arg, T_hint)
+        if kind == "stack" and src in blocked_of:
+            return blocked_of[src]
+        key = (kind, src if kind != "list" else tuple(src), residual)
+        if key not in inputs:
+            if residual:
+                inputs[key] = graph.call_function(blocked_residual, (src if kind != "list" else list(src),))
+            else:
+                inputs[key] = graph.call_function(blocked_input, (src if kind != "list" else list(src), T, kind == "shared"))
+        return inputs[key]
+
+    for node in list(graph.nodes):
+        if node not in convertible:
+            continue
+        with graph.inserting_before(node):
+            conv = fused_conv(node)
+            pair = pretail_sum(node)
+            if conv is not None:
+                res, stack = conv
+                base = 2 if res else 1
+                w, b, _, stride, padding = node.args[base:base + 5]
+                lif = tuple(node.args[base + 7:base + 10])
+                wants_blocked, wants_dense = reads_blocked(stack)
+                out_layout = B.BITS if wants_blocked or not wants_dense else B.NCHW
+                xb = as_blocked(node.args[0], residual=False)
+                rb = as_blocked(node.args[1], residual=True) if res else None
+                new = graph.call_function(blocked_conv_lif, (xb, w, b, list(stride), list(padding), lif, rb, out_layout))
+            elif pair is not None:
+                stack = node
+                plain, other = pair
+                x_arg, w, b, stride, padding = plain.args
+                wants_blocked, wants_dense = reads_blocked(stack)
+                out_layout = B.C8 if wants_blocked else B.NCHW
+                xb = as_blocked(x_arg, residual=False)
+                rb = as_blocked(other, residual=True)
+                new = graph.call_function(blocked_conv_lif, (xb, w, b, list(stride), list(padding), None, rb, out_layout))
+            elif plain_conv_ok(node):
+                stack = node
+                x_arg, w, b, stride, padding = node.args
+                wants_blocked, wants_dense = reads_blocked(stack)
+                out_layout = B.C8 if wants_blocked or not wants_dense else B.NCHW
+                new = graph.call_function(blocked_conv_lif, (as_blocked(x_arg, residual=False), w, b, list(stride), list(padding), None, None, out_layout))
+            else:
+                stack = node
+                if node.args[0] not in blocked_of:
+                    continue                      # a pool of a dense tensor stays on the dense pooling kernel
+                new = graph.call_function(blocked_pool, (blocked_of[node.args[0]], *node.args[1:]))
+            blocked_of[stack] = new
+            converted += 1
+    # Phase 2: whoever still reads a converted stack as a tensor gets it converted back (a no-op for dense outputs).
+    for stack, new in blocked_of.items():
+        with graph.inserting_after(new):
+            dense = graph.call_function(blocked_to_dense, (new,))
+        stack.replace_all_uses_with(dense)
+    _emit_in_dependency_order(gm)
+    gm.graph.lint()
+    gm.recompile()
+    return converted
+
+
 def _emit_in_dependency_order(gm: fx.GraphModule) -> None:
     """Rebuilds the graph from its output backwards: dead nodes (the replaced per-timestep chains) disappear and every
     node lands after its operands, whatever position it was inserted at."""
@@ -578,18 +797,25 @@ def _emit_in_dependency_order(gm: fx.GraphModule) -> None:
 
 
 def compile_temporal(wrapper: nn.Module, tail_first: bool = False, device=None, dtype: Optional[torch.dtype] = None,
-                     batch_time: bool = True) -> Tuple[fx.GraphModule, RewriteStats]:
+                     batch_time: bool = True, internal_layouts: bool = False) -> Tuple[fx.GraphModule, RewriteStats]:
     """Traces `wrapper` (a module that runs a single-step spiking network T times on the same input and averages) and
     rewrites it to fused temporal operators. BatchNorm is folded with the parameters as they are at call time (fold in
     fp32, before any cast); `device` / `dtype` then move and cast the rewritten module (weights and activations in
     `dtype`, the membranes stay fp32). `tail_first`: give the neuron in front of the classifier to the
     LIF -> AvgPool -> Linear operator (its convolution then stays a plain layer); by default the convolution patterns
     claim it, as in the reference, whose tail rewrite only sees the neurons the convolution rewrites left over.
-    `batch_time`: also merge the per-timestep calls of stateless layers into one call over T*N frames."""
+    `batch_time`: also merge the per-timestep calls of stateless layers into one call over T*N frames.
+    `internal_layouts` (needs `batch_time`; the compiled module then runs on the GPU with bfloat16 / float16 tensors only):
+    tensors between the graph's own fused operators, pools and LIF-free convolutions travel bit-packed / channel-blocked
+    and those nodes call the internal-layout kernels (`propagate_internal_layouts`)."""
     gm = trace_single_step_loop(wrapper)
     stats = rewrite_temporal_to_fused(gm, tail_first=tail_first)
     if batch_time:
         stats.batched_timestep_calls = batch_timestep_calls(gm)
+    if internal_layouts:
+        if not batch_time:
+            raise ValueError("internal_layouts needs batch_time: the pass works on whole [T, N, C, H, W] stacks")
+        stats.internal_layout_nodes = propagate_internal_layouts(gm)
     if device is not None or dtype is not None:
         gm.to(device=device, dtype=dtype)
         for name, buf in list(gm.named_buffers()):

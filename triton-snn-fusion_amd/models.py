@@ -334,41 +334,16 @@ class _FusedNetwork(nn.Module):
         self._log(kind="pool", name=name, x=x_seq, pool=pool, y=y, native=config is not None)
         return y
 
-    def _conv_lif_b_dense(self, x, layer: _FusedLayer, residual, out_layout):
-        from .runtime import hip_blocked_backend as B
-        dense = B.to_dense(x)
-        xs = [dense[0]] * x.T if x.shared else list(dense.unbind(0))
-        rs = None if residual is None else list(B.to_dense(residual).unbind(0))
-        S = torch.ops.snn_custom
-        if layer.lif is not None:
-            if rs is None:
-                y, v = S.fused_temporal_conv_lif_state(xs, layer.weight, layer.bias, self.zero_v, *layer.geometry, *layer.lif, False)
-            else:
-                y, v = S.fused_temporal_conv_add_lif_state(xs, rs, layer.weight, layer.bias, self.zero_v, *layer.geometry, *layer.lif, False)
-        else:
-            saved, self.record = self.record, None       # the caller logs the layer itself
-            try:
-                y = self.plain_conv("", torch.stack(xs), layer, None if rs is None else torch.stack(rs))
-            finally:
-                self.record = saved
-            v = None
-        return B.from_dense(y.contiguous(), out_layout), v
-
     # -- the same operators on the internal layouts ----------------------------------------------------------------
     def conv_lif_b(self, name: str, x, layer: _FusedLayer, residual=None, out_layout=None):
         """Conv + folded BN (+ residual) + LIF (`layer.lif`), or without a neuron when the layer has none, on Blocked tensors."""
         from .runtime import hip_blocked_backend as B
         if out_layout is None:
             out_layout = B.BITS if layer.lif is not None else B.C8
-        try:
-            out, v = B.conv_lif_blocked(x, layer.weight, layer.bias, layer.stride, layer.padding, layer.lif, residual=residual,
-                                        out_layout=out_layout, want_v=self.keep_membranes or self.record is not None)
-        except RuntimeError as exc:
-            if "unsupported" not in str(exc):
-                raise
-            # A layer the blocked kernel does not take (large kernels on many channels): the dense operators on unpacked
-            # tensors, and the result back into the layout the next operator expects.
-            out, v = self._conv_lif_b_dense(x, layer, residual, out_layout)
+        # A layer the blocked kernel does not take (large kernels on many channels) runs the dense entry points on
+        # unpacked tensors, and its result goes back into the layout the next operator expects.
+        out, v = B.conv_lif_blocked_or_dense(x, layer.weight, layer.bias, layer.stride, layer.padding, layer.lif, residual=residual,
+                                             out_layout=out_layout, want_v=self.keep_membranes or self.record is not None)
         if self.record is not None:
             T = x.T
             xs = list(B.to_dense(x).unbind(0)) if not x.shared else [B.to_dense(x)[0]] * T

@@ -222,6 +222,48 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
     return out, v_out
 
 
+def conv_lif_dense_on_blocked(x: Blocked, weight: torch.Tensor, bias: torch.Tensor, stride, padding, lif: Optional[Sequence[float]],
+                              residual: Optional[Blocked] = None, out_layout: int = BITS):
+    """The same layer through the dense entry points on unpacked tensors, for a layer the internal-layout kernel refuses
+    (large kernels on many channels): unpack, `snnf_conv_lif` / `snnf_conv_bias` through the operator layer, and the result
+    back into `out_layout`. Returns (Blocked output, final membrane or None)."""
+    from .hip_convlif_backend import run_hip_temporal_conv_bias
+    dense = to_dense(x)
+    xs = [dense[0]] * x.T if x.shared else list(dense.unbind(0))
+    rs = None if residual is None else list(to_dense(residual).unbind(0))
+    geometry = ([int(s) for s in _as_pair(stride)], [int(p) for p in _as_pair(padding)], [1, 1], 1)
+    if lif is not None:
+        zero_v = torch.zeros((), dtype=torch.float32, device=dense.device)
+        S = torch.ops.snn_custom
+        if rs is None:
+            y, v = S.fused_temporal_conv_lif_state(xs, weight, bias, zero_v, *geometry, *lif, False)
+        else:
+            y, v = S.fused_temporal_conv_add_lif_state(xs, rs, weight, bias, zero_v, *geometry, *lif, False)
+    else:
+        v = None
+        try:
+            y = run_hip_temporal_conv_bias(xs, weight, bias, geometry[0], geometry[1], rs)
+        except RuntimeError as exc:
+            if "unsupported" not in str(exc):
+                raise
+            y = torch.nn.functional.conv2d(torch.stack(xs).flatten(0, 1), weight, bias, geometry[0], geometry[1])
+            y = y.view(x.T, x.N, *y.shape[1:])
+            if rs is not None:
+                y = y + torch.stack(rs)
+    return from_dense(y.contiguous(), out_layout), v
+
+
+def conv_lif_blocked_or_dense(x: Blocked, weight: torch.Tensor, bias: torch.Tensor, stride, padding, lif: Optional[Sequence[float]],
+                              residual: Optional[Blocked] = None, out_layout: int = BITS, want_v: bool = False):
+    """conv_lif_blocked, and for a layer it refuses (`unsupported_*`) the dense entry points on unpacked tensors."""
+    try:
+        return conv_lif_blocked(x, weight, bias, stride, padding, lif, residual=residual, out_layout=out_layout, want_v=want_v)
+    except RuntimeError as exc:
+        if "unsupported" not in str(exc):
+            raise
+    return conv_lif_dense_on_blocked(x, weight, bias, stride, padding, lif, residual=residual, out_layout=out_layout)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # Depthwise 3x3 + LIF with row-packed spikes: one byte = the spikes of 8 consecutive pixels of a row (bit j = pixel 8 x + j).
 # A depthwise lane owns such a strip, so its spikes of a timestep leave as one byte instead of eight 16-bit elements.
