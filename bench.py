@@ -96,23 +96,30 @@ def _time_graph(fn, steps: int, warmup: int):
     return start.elapsed_time(stop) / steps
 
 
-def _time_kernel(fn, steps: int, warmup: int, reps: int = 10):
+def _time_kernel(fn, steps: int, warmup: int, reps: int = 10, rotate=None):
     """Average milliseconds per launch of the operator `fn`: `reps` launches captured into one HIP graph and replayed,
     HIP events on the replay stream, so that the figure is the kernel's own duration and not the Python call around it.
+    `rotate`: a list of callables that run the same operator on distinct input buffers; the launches of the graph then
+    cycle through them and every launch keeps its own output buffers, so that no launch finds its operands in the
+    last-level cache from the launch before (a cold figure; with one `fn` the launches re-read one input: warm).
     Falls back to timing eager launches when capture is not possible."""
     import torch
+    calls = list(rotate) if rotate else [fn]
     try:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            for _ in range(3):
-                fn()
+            for i in range(max(3, len(calls))):
+                calls[i % len(calls)]()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
+        keep = []
         with torch.cuda.graph(graph):
-            for _ in range(reps):
-                fn()
+            for i in range(reps):
+                out = calls[i % len(calls)]()
+                if rotate:
+                    keep.append(out)
         replays = max(1, steps // reps)
         for _ in range(max(1, warmup // reps)):
             graph.replay()
@@ -125,11 +132,16 @@ def _time_kernel(fn, steps: int, warmup: int, reps: int = 10):
         stop.record()
         torch.cuda.synchronize()
         ms = start.elapsed_time(stop) / (replays * reps)
-        del graph
+        del graph, keep
         return ms, "graph"
     except Exception:
         torch.cuda.synchronize()
-        return _time_gpu(fn, steps, warmup)[0], "eager"
+        return _time_gpu(lambda: [c() for c in calls], steps, warmup)[0] / len(calls), "eager"
+
+
+# Distinct operand sets a cold per-kernel figure rotates over: with 4 sets a launch's input was last read three launches
+# (more than a gigabyte of traffic at the headline shape) ago, far beyond the 256 MB last-level cache.
+COLD_SETS = 4
 
 
 # `roofline.traffic` (HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE) is not measured inside this script: a
@@ -433,33 +445,31 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
 
 
 def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
-    """Eager fp32 PyTorch-CPU path (the oracle's restatement of the reference's eager ops) on a bounded sample."""
+    """Eager fp32 PyTorch-CPU path (the oracle's restatement of the reference's eager ops), all host cores, at the
+    configuration's own batch; the single-thread figure beside it runs on a smaller batch so that the whole baseline stays
+    within `seconds_budget`."""
     import torch
     from oracle import snn_oracle as O
     from triton_snn_fusion_amd import workloads as W
-    if wl_name == "mobilenet_block":
-        sample_batch = 4
-        wl = W.mobilenet_block(batch=sample_batch)
-    elif wl_name == "conv3x3_block":
-        sample_batch = 8
-        wl = W.conv3x3_block(batch=sample_batch)
-    else:
-        sample_batch = 64
-        wl = W.linear_block(batch=sample_batch)
+    make = getattr(W, wl_name)
+    full_batch = {"mobilenet_block": 32, "conv3x3_block": 8, "linear_block": 64}[wl_name]      # BASELINE.json's batches
+    small_batch = {"mobilenet_block": 4, "conv3x3_block": 8, "linear_block": 64}[wl_name]
     v0 = torch.tensor(0.0)
 
-    def run():
-        if wl.linear_weight is not None:
-            return O.temporal_linear_lif(wl.x_seq, wl.linear_weight, wl.linear_bias, v0, *wl.lif)
-        xs = [wl.x_seq[t] for t in range(wl.T)]
-        out = None
-        for layer in wl.conv_layers:
-            out = O.temporal_conv_lif(xs, layer.weight, layer.bias, v0, layer.stride, layer.padding, (1, 1),
-                                      layer.groups, *wl.lif)
-            xs = [out[0][t] for t in range(wl.T)]
-        return out
+    def runner(wl):
+        def run():
+            if wl.linear_weight is not None:
+                return O.temporal_linear_lif(wl.x_seq, wl.linear_weight, wl.linear_bias, v0, *wl.lif)
+            xs = [wl.x_seq[t] for t in range(wl.T)]
+            out = None
+            for layer in wl.conv_layers:
+                out = O.temporal_conv_lif(xs, layer.weight, layer.bias, v0, layer.stride, layer.padding, (1, 1),
+                                          layer.groups, *wl.lif)
+                xs = [out[0][t] for t in range(wl.T)]
+            return out
+        return run
 
-    def median_ms(budget):
+    def median_s(run, budget):
         run()  # warm-up
         times = []
         t_begin = time.perf_counter()
@@ -470,22 +480,24 @@ def _cpu_baseline(wl_name: str, seconds_budget: float = 20.0):
         times.sort()
         return times[len(times) // 2], len(times)
 
-    median, count = median_ms(seconds_budget * 0.6)
+    wl = make(batch=full_batch)
+    median, count = median_s(runner(wl), seconds_budget * 0.6)
     threads = int(torch.get_num_threads())
+    wl_small = wl if small_batch == full_batch else make(batch=small_batch)
     torch.set_num_threads(1)
     try:
-        median_1, count_1 = median_ms(seconds_budget * 0.4)
+        median_1, count_1 = median_s(runner(wl_small), seconds_budget * 0.4)
     finally:
         torch.set_num_threads(threads)
-    times = [0.0] * count
     return {
-        "single_thread": {"value": round(sample_batch * wl.T / median_1, 2), "cores": 1, "ms_per_step": round(median_1 * 1e3, 3), "runs": count_1},
-        "value": round(sample_batch * wl.T / median, 2),
+        "single_thread": {"value": round(small_batch * wl.T / median_1, 2), "cores": 1, "ms_per_step": round(median_1 * 1e3, 3),
+                          "runs": count_1, "sample": f"batch {small_batch}"},
+        "value": round(full_batch * wl.T / median, 2),
         "unit": "images*T/s",
-        "cores": int(torch.get_num_threads()),
+        "cores": threads,
         "kind": "port",
-        "sample": f"{wl_name} at batch {sample_batch} (of the GPU run's batch), fp32 eager PyTorch-CPU ops, "
-                  f"median of {len(times)} runs, {median * 1e3:.1f} ms per step",
+        "sample": f"{wl_name} at batch {full_batch} (the configuration's own batch), fp32 eager PyTorch-CPU ops, "
+                  f"median of {count} runs, {median * 1e3:.1f} ms per step",
         "ms_per_step": round(median * 1e3, 3),
         "host_cpus": os.cpu_count(),
     }
@@ -575,14 +587,22 @@ def main() -> int:
         inputs = prep.layer_inputs()
         torch.cuda.synchronize()
         for i, xs in enumerate(inputs):
-            ms, how = _time_kernel(lambda i=i, xs=xs: prep.run_layer(i, xs), args.steps, max(3, args.warmup // 2))
+            # Warm: ten launches on one input. Cold: the launches rotate over COLD_SETS copies of the input and keep their
+            # outputs apart; "ms" and the roofline fractions are the cold ones.
+            ms_warm, how = _time_kernel(lambda i=i, xs=xs: prep.run_layer(i, xs), args.steps, max(3, args.warmup // 2))
+            copies = [[x.clone() for x in xs] for _ in range(COLD_SETS)]
+            ms, how = _time_kernel(None, args.steps, max(3, args.warmup // 2),
+                                   rotate=[lambda i=i, c=c: prep.run_layer(i, c) for c in copies])
+            del copies
             nbytes, flops = prep.layer_work(i, xs)
             groups = prep.layers[i][5]
             kind = "depthwise3x3" if groups > 1 else ("pointwise1x1" if tuple(prep.layers[i][1].shape[2:]) == (1, 1) else "conv")
             traffic = None
+            hbm = _roofline("hbm", nbytes, ms, traffic)
+            hbm["frac_warm"] = _roofline("hbm", nbytes, ms_warm)["frac"]
             kernels[f"layer{i}_{kind}"] = {
-                "ms": round(ms, 4), "timed": how, "algorithmic_bytes": nbytes, "flops": flops,
-                "hbm": _roofline("hbm", nbytes, ms, traffic),
+                "ms": round(ms, 4), "ms_warm": round(ms_warm, 4), "timed": how, "cold_input_sets": COLD_SETS,
+                "algorithmic_bytes": nbytes, "flops": flops, "hbm": hbm,
                 "mfma": None if groups > 1 else _roofline("mfma", flops, ms, traffic),
             }
         dominant = max(kernels.items(), key=lambda kv: kv[1]["ms"])
