@@ -189,6 +189,81 @@ def test_fx_rewrite_leaves_a_layer_alone_when_its_state_chain_is_broken():
         assert torch.allclose(gm(x), want)
 
 
+class _EncoderMlp(torch.nn.Module):
+    """A neuron on the analog frame (no layer in front), one Conv+BN+neuron, then two Linear+neuron layers and a Linear
+    readout: the Linear -> LIF and standalone LIF pattern families next to the convolution one."""
+
+    def __init__(self):
+        super().__init__()
+        self.enc = M.CustomStatefulIFNode(v_threshold=0.5)
+        self.conv = M.ConvBNNeuron(3, 8, 3, 2, 1)
+        self.fc1, self.sn1 = torch.nn.Linear(8 * 4 * 4, 32), M.CustomStatefulIFNode()
+        self.fc2, self.sn2 = torch.nn.Linear(32, 16, bias=False), M.CustomStatefulIFNode(v_reset=-1.0)
+        self.head = torch.nn.Linear(16, 5)
+
+    def forward(self, x):
+        y = torch.flatten(self.conv(self.enc(x)), 1)
+        return self.head(self.sn2(self.fc2(self.sn1(self.fc1(y)))))
+
+
+@pytest.mark.parametrize("window", [None, 2])
+def test_fx_rewrite_linear_lif_and_standalone_lif_pattern_families(window):
+    T = 4
+    net = M.init_synthetic_(_EncoderMlp(), gain=4.0)
+    wrapper = M.SingleStepModeLoopWrapper(net, T)
+    x = torch.randn(3, 3, 8, 8, generator=gen(11))
+    with torch.no_grad():
+        want = wrapper(x)
+    gm, stats = R.compile_temporal(wrapper, window=window)
+    S = torch.ops.snn_custom
+    targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+    per_layer = 1 if window is None else T // window
+    assert targets.count(S.fused_temporal_lif_state) == per_layer and stats.temporal_lif_groups == 1
+    assert targets.count(S.fused_temporal_linear_lif_state) == 2 * per_layer and stats.temporal_linear_lif_groups == 2
+    assert targets.count(S.fused_temporal_conv_lif_state) == per_layer and stats.temporal_conv_bn_lif_groups == 1
+    assert stats.temporal_windows == 4 * per_layer and stats.replaced_patterns == 4 * T and not stats.skipped
+    assert not any(R.is_custom_lif_state_node(n) for n in gm.graph.nodes)
+    # the encoder reads one frame T times: its stack is built from the placeholder; the Linear layers take lists of T nodes
+    for n in gm.graph.nodes:
+        if n.op == "call_function" and n.target is S.fused_temporal_linear_lif_state:
+            assert isinstance(n.args[0], (list, tuple)) and len(n.args[0]) == (T if window is None else window)
+            assert n.args[2] is None or n.args[2].op == "get_attr"                   # the bias-free layer passes None
+    # windows chain through the final membrane: every window after a layer's first starts from the previous one's second output
+    fused = [n for n in gm.graph.nodes if n.op == "call_function" and n.target in
+             (S.fused_temporal_lif_state, S.fused_temporal_linear_lif_state, S.fused_temporal_conv_lif_state)]
+    from_zero = [n for n in fused if any(isinstance(a, torch.fx.Node) and a.op == "get_attr" and "zero_membrane" in a.target for a in n.args)]
+    assert len(from_zero) == 4 and len(fused) - len(from_zero) == 4 * (per_layer - 1)
+    with torch.no_grad():
+        got = gm(x)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5), float((got - want).abs().max())
+    assert float(want.abs().max()) > 0.01
+
+
+@pytest.mark.parametrize("T,window,allow_tail,fused_per_layer,single_steps", [(4, 2, True, 2, 0), (5, 3, True, 2, 0), (5, 3, False, 1, 2),
+                                                                           (5, 2, True, 2, 1), (4, 4, True, 1, 0)])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_rewrite_temporal_windows_shorter_than_T(name, T, window, allow_tail, fused_per_layer, single_steps):
+    """Windows of `window` steps: every window is one fused node, the next window (or a step that stayed a single-step
+    neuron call) continues from its final membrane; the result equals the eager T-step loop."""
+    model = M.build_network(name, width=8, gain=5.0)
+    wrapper = M.SingleStepModeLoopWrapper(model, T)
+    size = 32
+    x = torch.randn(2, 3, size, size, generator=gen(12))
+    with torch.no_grad():
+        want = wrapper(x)
+    gm, stats = R.compile_temporal(wrapper, tail_first=True, window=window, allow_tail=allow_tail)
+    S = torch.ops.snn_custom
+    targets = [n.target for n in gm.graph.nodes if n.op == "call_function"]
+    layers = 8 if name == "vgg11" else 17
+    n_fused = sum(t in (S.fused_temporal_conv_lif_state, S.fused_temporal_conv_add_lif_state, S.fused_temporal_lif_avgpool_linear) for t in targets)
+    assert n_fused == layers * fused_per_layer == stats.temporal_windows and not stats.skipped
+    left = sum(R.is_custom_lif_state_node(n) for n in gm.graph.nodes)
+    assert left == layers * single_steps
+    with torch.no_grad():
+        got = gm(x)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5), float((got - want).abs().max())
+
+
 @pytest.mark.parametrize("name", ["vgg11", "resnet18"])
 def test_fx_layout_propagation_graph_invariants(name):
     """compile_temporal(internal_layouts=True): every fused convolution, LIF-free convolution and pool of the rewritten graph
@@ -478,6 +553,59 @@ def test_fx_graph_with_an_unknown_layer_between_fused_layers_on_the_gpu(hip_ops)
         want, got = dense(x).float(), blocked(x).float()
     assert float((want - got).abs().max()) <= 0.05 and float(want.abs().max()) > 0.05, (want, got)
     assert hip_ops.get_fused_op_call_stats()["fallback"] == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [None, 2])
+def test_fx_graph_reaches_the_linear_and_scan_kernels(hip_ops, window):
+    """Linear -> LIF and standalone LIF layers of a compiled graph run on `snnf_linear_lif` / `snnf_lif_scan` (no eager
+    fallback), window by window when asked; the logits follow the eager CPU loop on the same bf16-rounded parameters."""
+    T = 4
+    net = M.init_synthetic_(_EncoderMlp(), gain=4.0)
+    with torch.no_grad():
+        for prm in net.parameters():
+            prm.copy_(q(prm, BF16))
+    x = q(torch.randn(3, 3, 8, 8, generator=gen(13)), BF16)
+    wrapper = M.SingleStepModeLoopWrapper(net, T)
+    with torch.no_grad():
+        M.reset_lif_modules(net)
+        want = wrapper(x)
+    gm, stats = R.compile_temporal(wrapper, device=DEV, dtype=BF16, window=window)
+    assert not stats.skipped and stats.temporal_linear_lif_groups == 2 and stats.temporal_lif_groups == 1
+    hip_ops.reset_fused_op_call_stats()
+    with torch.no_grad():
+        got = gm(x.to(DEV, BF16)).float().cpu()
+    s = hip_ops.get_fused_op_call_stats()
+    per_layer = 1 if window is None else T // window
+    assert s["fallback"] == 0 and s["triton"] == 4 * per_layer, s
+    by_kind = s.get("by_op_kind", {})
+    print("native calls by operator:", by_kind)
+    assert float((got - want).abs().max()) <= 0.08 * max(1.0, float(want.abs().max())), (got, want)
+    assert float(want.abs().max()) > 0.01
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_fx_graph_with_windows_of_two_steps_on_the_gpu(hip_ops, name):
+    """T = 4 as two chained windows of 2: twice the fused nodes, every later window continuing from a float32 membrane;
+    the logits stay those of the one-window graph up to near-threshold flips."""
+    T = 4
+    model, _ = _fused(name, T)
+    x = _frame(name).to(DEV, BF16)
+    whole, _ = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16)
+    halves, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16, window=2)
+    layers = 8 if name == "vgg11" else 17
+    assert stats.temporal_windows == 2 * layers and not stats.skipped
+    hip_ops.reset_fused_op_call_stats()
+    with torch.no_grad():
+        got = halves(x).float().cpu()
+    s = hip_ops.get_fused_op_call_stats()
+    assert s["fallback"] == 0 and s["triton"] == 2 * layers, s
+    with torch.no_grad():
+        want = whole(x).float().cpu()
+    cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
+    print(f"{name}: windows of 2 vs one window, cosine similarity of the logits {cos:.5f}")
+    assert cos > 0.8, cos      # same bar as the other executor comparisons: flips near the threshold cascade with random weights
 
 
 @pytest.mark.gpu

@@ -2,20 +2,25 @@
 
 Counterpart of the reference's rewrite pipeline for the patterns the fused operators serve
 (compiler/fx_lif_temporal_rewrite.py: `collect_conv_bn_lif_state_patterns` :337, `collect_conv_bn_add_lif_state_patterns`
-:423, `collect_temporal_lif_avgpool_linear_patterns` :791, `group_temporal_patterns` :884, `check_temporal_state_chain`
-:929, `rewrite_temporal_conv_bn_lif_state_to_fused` :2037, residual :2214, tail :2745; BatchNorm folding
-compiler/fx_lif_rewrite.py:340-353). The reference obtains its graph from torch.compile and works on function-level
+:423, `collect_standalone_lif_state_patterns` :534, `collect_temporal_linear_lif_state_patterns` :694,
+`collect_temporal_lif_avgpool_linear_patterns` :791, `group_temporal_patterns` :884, `check_temporal_state_chain` :929,
+`make_temporal_windows` :955-1094, `rewrite_temporal_conv_bn_lif_state_to_fused` :2037, residual :2214, standalone LIF
+:2408, Linear + LIF :2548, tail :2745; BatchNorm folding compiler/fx_lif_rewrite.py:340-353). The reference obtains its graph from torch.compile and works on function-level
 nodes; this one traces a `SingleStepModeLoopWrapper`-style module with `torch.fx.symbolic_trace`, so convolutions,
 BatchNorms, pools and the classifier are `call_module` nodes and each neuron call is a
 `torch.ops.snn_custom.lif_forward_state` node whose membrane operand is the previous call's second output.
 
 Pipeline (`compile_temporal`):
   1. `trace_single_step_loop`  - unrolls the T iterations; a neuron's first membrane is the scalar-zero constant.
-  2. collect                   - Conv2d -> BatchNorm2d -> LIF, Conv2d -> BatchNorm2d -> add(residual) -> LIF, and the tail
-                                 LIF -> AdaptiveAvgPool2d(1) -> flatten -> Linear -> running sum; one pattern per timestep.
-  3. group + check             - patterns of one layer (same conv and BN module) ordered by timestep; the state chain must be
-                                 v_getitem[t-1] -> v_prev[t] with a scalar-zero start, otherwise the layer is left alone.
-  4. rewrite                   - one fused operator node per layer over the list of its T inputs (operator chosen by
+  2. collect                   - Conv2d -> BatchNorm2d -> LIF, Conv2d -> BatchNorm2d -> add(residual) -> LIF, Linear -> LIF, the
+                                 tail LIF -> AdaptiveAvgPool2d(1) -> flatten -> Linear -> running sum, and LIF calls on their
+                                 own; one pattern per timestep.
+  3. group + check             - patterns of one layer (same conv and BN module, same Linear, same neuron) ordered by
+                                 timestep; the state chain must be v_getitem[t-1] -> v_prev[t] with a scalar-zero start,
+                                 otherwise the layer is left alone.
+  4. windows                   - a layer's T patterns are cut into windows of `window` consecutive timesteps (all T by
+                                 default); the final membrane of one window is the initial membrane of the next.
+  5. rewrite                   - one fused operator node per window over the list of its inputs (operator chosen by
                                  convolution kind: regular / pointwise / depthwise, as compiler/fx_lif_temporal_rewrite.py
                                  :1625-1662), folded weights as graph attributes, per-timestep spikes as `spike_stack[t]`.
 The graph is then re-emitted in dependency order, which turns the time-major trace into layer-major execution.
@@ -242,6 +247,117 @@ def collect_temporal_lif_avgpool_linear_patterns(gm: fx.GraphModule, excluded_li
     return patterns
 
 
+@dataclass
+class TemporalLinearLifPattern:
+    layer_id: str
+    timestep_index: int
+    linear_node: fx.Node
+    linear_input: fx.Node
+    lif_node: fx.Node
+    spike_getitem: Optional[fx.Node]
+    v_getitem: Optional[fx.Node]
+    v_prev_node: object
+    lif_params: Tuple
+
+
+@dataclass
+class TemporalLifPattern:
+    layer_id: str
+    timestep_index: int
+    lif_node: fx.Node
+    input_node: fx.Node
+    spike_getitem: Optional[fx.Node]
+    v_getitem: Optional[fx.Node]
+    v_prev_node: object
+    lif_params: Tuple
+
+
+def collect_temporal_linear_lif_state_patterns(gm: fx.GraphModule, excluded_lif_nodes=None) -> List[TemporalLinearLifPattern]:
+    """LIF(Linear(x)) with the Linear feeding only its neuron (compiler/fx_lif_temporal_rewrite.py:694-770)."""
+    excluded = set(excluded_lif_nodes or [])
+    counts: Dict[str, int] = {}
+    patterns: List[TemporalLinearLifPattern] = []
+    for node in gm.graph.nodes:
+        if node in excluded or not is_custom_lif_state_node(node) or not _lif_state_is_usable(node)[0]:
+            continue
+        linear = node.args[0]
+        if not isinstance(linear, fx.Node) or _module_of(gm, linear, nn.Linear) is None or len(linear.users) != 1:
+            continue
+        if not isinstance(linear.args[0], fx.Node):
+            continue
+        layer_id = f"linear_lif|fc={linear.target}|params={tuple(node.args[2:6])!r}"
+        getitems = find_tuple_getitems(node)
+        t = counts.get(layer_id, 0)
+        counts[layer_id] = t + 1
+        patterns.append(TemporalLinearLifPattern(layer_id, t, linear, linear.args[0], node, getitems.get(0), getitems.get(1),
+                                                 node.args[1], tuple(node.args[2:6])))
+    return patterns
+
+
+def _produces_rank_two(gm: fx.GraphModule, node) -> bool:
+    """Linear outputs and flattened tensors are [N, F]; the temporal LIF operator takes [T, N, C, H, W] only
+    (runtime/snn_custom_ops.py:529; the same exclusion as compiler/fx_lif_temporal_rewrite.py:563-568)."""
+    if not isinstance(node, fx.Node):
+        return True
+    if _module_of(gm, node, (nn.Linear, nn.Flatten)) is not None:
+        return True
+    if node.op == "call_function" and node.target is torch.flatten:
+        return True
+    if node.op == "call_method" and node.target in ("flatten", "view", "reshape"):
+        return True
+    rank = node.meta.get("chronos_rank")
+    return rank is not None and rank != 4
+
+
+def collect_standalone_lif_state_patterns(gm: fx.GraphModule, excluded_lif_nodes=None) -> List[TemporalLifPattern]:
+    """LIF calls that no other pattern has claimed, on [N, C, H, W] inputs (compiler/fx_lif_temporal_rewrite.py:534-598).
+    The reference keys a layer by the call's occurrence inside a timestep and its shape; here a layer is one neuron's state
+    chain: it starts at a call on the scalar-zero membrane and continues through v_getitem -> v_prev."""
+    excluded = set(excluded_lif_nodes or [])
+    patterns: List[TemporalLifPattern] = []
+    chain_of: Dict[fx.Node, Tuple[str, int]] = {}
+    chains = 0
+    for node in gm.graph.nodes:
+        if not is_custom_lif_state_node(node):
+            continue
+        v_prev = node.args[1]
+        if isinstance(v_prev, fx.Node) and v_prev.op == "call_function" and v_prev.target is operator.getitem and v_prev.args[0] in chain_of:
+            layer_id, t = chain_of[v_prev.args[0]]
+            chain_of[node] = (layer_id, t + 1)
+        else:
+            chain_of[node] = (f"standalone_lif|chain={chains}|params={tuple(node.args[2:6])!r}", 0)
+            chains += 1
+        if node in excluded or not _lif_state_is_usable(node)[0] or _produces_rank_two(gm, node.args[0]):
+            continue
+        layer_id, t = chain_of[node]
+        getitems = find_tuple_getitems(node)
+        patterns.append(TemporalLifPattern(layer_id, t, node, node.args[0], getitems.get(0), getitems.get(1), node.args[1],
+                                           tuple(node.args[2:6])))
+    return patterns
+
+
+def make_temporal_windows(groups: List["TemporalGroup"], window_size: Optional[int], allow_tail: bool = True) -> List["TemporalGroup"]:
+    """Cuts every group's timestep-ordered patterns into windows of `window_size` consecutive timesteps (None: one window of
+    all of them). A shorter last window is kept when `allow_tail`; windows of a single timestep are left to the single-step
+    nodes already in the graph (compiler/fx_lif_temporal_rewrite.py:955-974). Patterns of a window must be consecutive."""
+    windows: List[TemporalGroup] = []
+    for group in groups:
+        steps = [p.timestep_index for p in group.patterns]
+        if steps != list(range(steps[0], steps[0] + len(steps))):
+            continue        # a claimed or unusable call interrupts the layer: leave it alone
+        size = len(group.patterns) if window_size is None else int(window_size)
+        if size < 1:
+            continue
+        for start in range(0, len(group.patterns), size):
+            chunk = group.patterns[start:start + size]
+            if len(chunk) < size and not allow_tail:
+                continue
+            if len(chunk) <= 1 and window_size is not None:
+                continue
+            windows.append(TemporalGroup(group.layer_id, chunk))
+    return windows
+
+
 def group_temporal_patterns(patterns) -> List[TemporalGroup]:
     grouped: Dict[str, List] = {}
     for p in patterns:
@@ -252,7 +368,7 @@ def group_temporal_patterns(patterns) -> List[TemporalGroup]:
 def check_temporal_state_chain(gm: fx.GraphModule, patterns) -> Tuple[bool, str]:
     """The membrane of step t must be exactly the second output of step t-1, the first one the scalar zero, and nothing
     else may read the intermediate membranes."""
-    if not _is_scalar_zero(gm, patterns[0].v_prev_node):
+    if patterns[0].timestep_index == 0 and not _is_scalar_zero(gm, patterns[0].v_prev_node):
         return False, f"{patterns[0].lif_node.name} does not start from the scalar-zero membrane"
     for prev, nxt in zip(patterns, patterns[1:]):
         if prev.v_getitem is None or nxt.v_prev_node is not prev.v_getitem:
@@ -287,6 +403,9 @@ class RewriteStats:
     temporal_conv_bn_lif_groups: int = 0
     temporal_conv_bn_add_lif_groups: int = 0
     temporal_lif_avgpool_linear_groups: int = 0
+    temporal_linear_lif_groups: int = 0
+    temporal_lif_groups: int = 0
+    temporal_windows: int = 0
     replaced_patterns: int = 0
     batched_timestep_calls: int = 0
     internal_layout_nodes: int = 0
@@ -321,8 +440,11 @@ def _folded_params(gm: fx.GraphModule, group: TemporalGroup, index: int) -> Tupl
     return _register(gm, f"fused_weight_{index}", w), _register(gm, f"fused_bias_{index}", b), conv
 
 
-def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] = None, tail_first: bool = False) -> RewriteStats:
-    """Replaces every layer whose T patterns pass the state-chain check by one fused temporal operator node."""
+def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] = None, tail_first: bool = False,
+                              window_size: Optional[int] = None, allow_tail: bool = True) -> RewriteStats:
+    """Replaces every layer whose patterns pass the state-chain check by fused temporal operator nodes: one per window of
+    `window_size` consecutive timesteps (None: one node over all T). The final membrane of a window is the initial membrane
+    of the layer's next step, fused or not (compiler/fx_lif_temporal_rewrite.py:955-974, 2085, 2144-2145)."""
     stats = stats or RewriteStats()
     S = torch.ops.snn_custom
     graph = gm.graph
@@ -331,6 +453,35 @@ def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] 
     zero_name = _register(gm, "chronos_zero_membrane", torch.zeros((), dtype=torch.float32, device=device))
     index = 0
     claimed = set()
+    in_a_family = set()      # neuron calls behind a convolution, a Linear or in front of the classifier: never "standalone"
+
+    def windows_of(group: TemporalGroup, check) -> List[TemporalGroup]:
+        ok, reason = check(gm, group.patterns)
+        if not ok:
+            stats.skipped.append(f"{group.layer_id}: {reason}")
+            return []
+        return make_temporal_windows([group], window_size, allow_tail)
+
+    def initial_membrane(first) -> fx.Node:
+        """Scalar zero for a layer's first step; otherwise whatever feeds that step now: the previous window's final
+        membrane, or the second output of a single step that was left alone."""
+        if first.timestep_index == 0:
+            return graph.get_attr(zero_name)
+        return first.lif_node.args[1]
+
+    def finish_window(window: TemporalGroup, fused: fx.Node) -> None:
+        """Per-timestep spikes become `spike_stack[i]`; a later step that continues from the window reads `fused[1]`."""
+        spike_stack = graph.call_function(operator.getitem, (fused, 0))
+        for i, p in enumerate(window.patterns):
+            if p.spike_getitem is not None:
+                p.spike_getitem.replace_all_uses_with(graph.call_function(operator.getitem, (spike_stack, i)))
+            claimed.add(p.lif_node)
+        last = window.patterns[-1].v_getitem
+        if last is not None and len(last.users) > 0:
+            last.replace_all_uses_with(graph.call_function(operator.getitem, (fused, 1)))
+        stats.replaced_patterns += len(window.patterns)
+        stats.temporal_windows += 1
+
     tail_groups = []
     if tail_first:
         # The neuron in front of the classifier belongs to the tail operator; its convolution stays a plain layer.
@@ -342,67 +493,104 @@ def rewrite_temporal_to_fused(gm: fx.GraphModule, stats: Optional[RewriteStats] 
     conv_groups = [(g, False) for g in group_temporal_patterns(collect_conv_bn_lif_state_patterns(gm))]
     conv_groups += [(g, True) for g in group_temporal_patterns(collect_conv_bn_add_lif_state_patterns(gm))]
     for group, residual in conv_groups:
+        in_a_family.update(p.lif_node for p in group.patterns)
         if any(p.lif_node in claimed for p in group.patterns):
             continue
-        ok, reason = check_temporal_state_chain(gm, group.patterns)
-        if not ok:
-            stats.skipped.append(f"{group.layer_id}: {reason}")
+        windows = windows_of(group, check_temporal_state_chain)
+        if not windows:
             continue
         w_name, b_name, conv = _folded_params(gm, group, index)
         index += 1
         kind = classify_conv_kind(conv)
-        # Operands are read from the nodes now: an earlier rewrite may have redirected them to its spike_stack[t].
-        xs = [p.conv_node.args[0] for p in group.patterns]
-        residuals = [next(a for a in p.add_node.args if a is not p.bn_node) for p in group.patterns] if residual else None
-        # New nodes go in front of the output; the graph is re-emitted in dependency order at the end.
-        with graph.inserting_before(output_node):
-            w_node = graph.get_attr(w_name)
-            b_node = graph.get_attr(b_name)
-            v0 = graph.get_attr(zero_name)
         geometry = (list(conv.stride), list(conv.padding), list(conv.dilation), int(conv.groups))
         lif = tuple(group.patterns[0].lif_params)
-        if residual:
-            op = S.fused_temporal_conv_add_lif_state_depthwise if kind == "depthwise" else S.fused_temporal_conv_add_lif_state
-            args = (xs, residuals, w_node, b_node, v0, *geometry, *lif)
-        else:
-            op = {"regular": S.fused_temporal_conv_lif_state, "pointwise": S.fused_temporal_pointwise_conv_lif_state,
-                  "depthwise": S.fused_temporal_depthwise_conv_lif_state}[kind]
-            args = (xs, w_node, b_node, v0, *geometry, *lif)
-        with graph.inserting_before(output_node):
-            fused = graph.call_function(op, args)
-            spike_stack = graph.call_function(operator.getitem, (fused, 0))
-            for p in group.patterns:
-                if p.spike_getitem is not None:
-                    spike_t = graph.call_function(operator.getitem, (spike_stack, p.timestep_index))
-                    p.spike_getitem.replace_all_uses_with(spike_t)
-                claimed.add(p.lif_node)
+        for window in windows:
+            # Operands are read from the nodes now: an earlier rewrite may have redirected them to its spike_stack[t].
+            xs = [p.conv_node.args[0] for p in window.patterns]
+            residuals = [next(a for a in p.add_node.args if a is not p.bn_node) for p in window.patterns] if residual else None
+            # New nodes go in front of the output; the graph is re-emitted in dependency order at the end.
+            with graph.inserting_before(output_node):
+                w_node = graph.get_attr(w_name)
+                b_node = graph.get_attr(b_name)
+                v0 = initial_membrane(window.patterns[0])
+                if residual:
+                    op = S.fused_temporal_conv_add_lif_state_depthwise if kind == "depthwise" else S.fused_temporal_conv_add_lif_state
+                    args = (xs, residuals, w_node, b_node, v0, *geometry, *lif)
+                else:
+                    op = {"regular": S.fused_temporal_conv_lif_state, "pointwise": S.fused_temporal_pointwise_conv_lif_state,
+                          "depthwise": S.fused_temporal_depthwise_conv_lif_state}[kind]
+                    args = (xs, w_node, b_node, v0, *geometry, *lif)
+                finish_window(window, graph.call_function(op, args))
         if residual:
             stats.temporal_conv_bn_add_lif_groups += 1
         else:
             stats.temporal_conv_bn_lif_groups += 1
-        stats.replaced_patterns += len(group.patterns)
+
+    # Linear -> LIF: the list form of the operator reads the T inputs where they are (no stack).
+    for group in group_temporal_patterns(collect_temporal_linear_lif_state_patterns(gm, excluded_lif_nodes=claimed)):
+        in_a_family.update(p.lif_node for p in group.patterns)
+        windows = windows_of(group, check_temporal_state_chain)
+        if not windows:
+            continue
+        fc = gm.get_submodule(group.patterns[0].linear_node.target)
+        w_name = _register(gm, f"fused_linear_weight_{index}", fc.weight.detach().contiguous())
+        b_name = None if fc.bias is None else _register(gm, f"fused_linear_bias_{index}", fc.bias.detach().contiguous())
+        index += 1
+        for window in windows:
+            xs = [p.linear_node.args[0] for p in window.patterns]
+            with graph.inserting_before(output_node):
+                w_node = graph.get_attr(w_name)
+                b_node = None if b_name is None else graph.get_attr(b_name)
+                v0 = initial_membrane(window.patterns[0])
+                finish_window(window, graph.call_function(S.fused_temporal_linear_lif_state, (xs, w_node, b_node, v0, *group.patterns[0].lif_params)))
+        stats.temporal_linear_lif_groups += 1
 
     if not tail_first:
         tail_groups = group_temporal_patterns(collect_temporal_lif_avgpool_linear_patterns(gm, excluded_lif_nodes=claimed))
     for group in tail_groups:
-        ok, reason = check_temporal_lif_avgpool_linear_state_and_acc_chain(gm, group.patterns)
-        if not ok:
-            stats.skipped.append(f"{group.layer_id}: {reason}")
+        in_a_family.update(p.lif_node for p in group.patterns)
+        windows = windows_of(group, check_temporal_lif_avgpool_linear_state_and_acc_chain)
+        if not windows:
             continue
         fc = gm.get_submodule(group.patterns[0].linear_node.target)
         w_name = _register(gm, "fused_fc_weight", fc.weight.detach().contiguous())
         b_name = _register(gm, "fused_fc_bias", fc.bias.detach().contiguous() if fc.bias is not None else torch.empty(0, dtype=fc.weight.dtype, device=fc.weight.device))
-        xs = [p.lif_node.args[0] for p in group.patterns]
-        with graph.inserting_before(output_node):
-            x_seq = graph.call_function(torch.stack, (xs,))
-            w_node = graph.get_attr(w_name)
-            b_node = graph.get_attr(b_name)
-            v0 = graph.get_attr(zero_name)
-            fused = graph.call_function(S.fused_temporal_lif_avgpool_linear, (x_seq, v0, w_node, b_node, *group.patterns[0].lif_params))
-            out_sum = graph.call_function(operator.getitem, (fused, 0))
-        group.patterns[-1].acc_node.replace_all_uses_with(out_sum)
+        for window in windows:
+            xs = [p.lif_node.args[0] for p in window.patterns]
+            first, last = window.patterns[0], window.patterns[-1]
+            # The running sum in front of the window, as the graph holds it now (0 for the first step).
+            acc_before = next(a for a in first.acc_node.args if a is not first.linear_node)
+            with graph.inserting_before(output_node):
+                x_seq = graph.call_function(torch.stack, (xs,))
+                w_node = graph.get_attr(w_name)
+                b_node = graph.get_attr(b_name)
+                v0 = initial_membrane(first)
+                fused = graph.call_function(S.fused_temporal_lif_avgpool_linear, (x_seq, v0, w_node, b_node, *first.lif_params))
+                out_sum = graph.call_function(operator.getitem, (fused, 0))
+                if isinstance(acc_before, fx.Node) or acc_before != 0:
+                    out_sum = graph.call_function(operator.add, (acc_before, out_sum))
+                if last.v_getitem is not None and len(last.v_getitem.users) > 0:
+                    last.v_getitem.replace_all_uses_with(graph.call_function(operator.getitem, (fused, 1)))
+            last.acc_node.replace_all_uses_with(out_sum)
+            claimed.update(p.lif_node for p in window.patterns)
+            stats.replaced_patterns += len(window.patterns)
+            stats.temporal_windows += 1
         stats.temporal_lif_avgpool_linear_groups += 1
-        stats.replaced_patterns += len(group.patterns)
+
+    # Neurons on their own (no convolution or Linear in front that a pattern above has taken): one scan over the stacked inputs.
+    for group in group_temporal_patterns(collect_standalone_lif_state_patterns(gm, excluded_lif_nodes=claimed | in_a_family)):
+        if any(p.lif_node in claimed for p in group.patterns):
+            continue
+        windows = windows_of(group, check_temporal_state_chain)
+        if not windows:
+            continue
+        for window in windows:
+            xs = [p.lif_node.args[0] for p in window.patterns]
+            with graph.inserting_before(output_node):
+                x_seq = graph.call_function(torch.stack, (xs,))
+                v0 = initial_membrane(window.patterns[0])
+                finish_window(window, graph.call_function(S.fused_temporal_lif_state, (x_seq, v0, *group.patterns[0].lif_params)))
+        stats.temporal_lif_groups += 1
 
     _emit_in_dependency_order(gm)
     gm.graph.lint()
@@ -797,19 +985,22 @@ def _emit_in_dependency_order(gm: fx.GraphModule) -> None:
 
 
 def compile_temporal(wrapper: nn.Module, tail_first: bool = False, device=None, dtype: Optional[torch.dtype] = None,
-                     batch_time: bool = True, internal_layouts: bool = False) -> Tuple[fx.GraphModule, RewriteStats]:
+                     batch_time: bool = True, internal_layouts: bool = False, window: Optional[int] = None,
+                     allow_tail: bool = True) -> Tuple[fx.GraphModule, RewriteStats]:
     """Traces `wrapper` (a module that runs a single-step spiking network T times on the same input and averages) and
     rewrites it to fused temporal operators. BatchNorm is folded with the parameters as they are at call time (fold in
     fp32, before any cast); `device` / `dtype` then move and cast the rewritten module (weights and activations in
     `dtype`, the membranes stay fp32). `tail_first`: give the neuron in front of the classifier to the
     LIF -> AvgPool -> Linear operator (its convolution then stays a plain layer); by default the convolution patterns
     claim it, as in the reference, whose tail rewrite only sees the neurons the convolution rewrites left over.
+    `window` / `allow_tail`: fuse windows of that many consecutive timesteps instead of all T (the reference's
+    `--temporal-fuse-window`); a window hands its final membrane to the layer's next step.
     `batch_time`: also merge the per-timestep calls of stateless layers into one call over T*N frames.
     `internal_layouts` (needs `batch_time`; the compiled module then runs on the GPU with bfloat16 / float16 tensors only):
     tensors between the graph's own fused operators, pools and LIF-free convolutions travel bit-packed / channel-blocked
     and those nodes call the internal-layout kernels (`propagate_internal_layouts`)."""
     gm = trace_single_step_loop(wrapper)
-    stats = rewrite_temporal_to_fused(gm, tail_first=tail_first)
+    stats = rewrite_temporal_to_fused(gm, tail_first=tail_first, window_size=window, allow_tail=allow_tail)
     if batch_time:
         stats.batched_timestep_calls = batch_timestep_calls(gm)
     if internal_layouts:
