@@ -237,7 +237,8 @@ int snnf_conv_lif(const void* const* xs, const void* const* residuals, int T,
  * reference corresponds to it: its rewrite leaves LIF-free Conv+BN nodes (the 1x1 downsample shortcuts of a ResNet,
  * whose output is the `residuals` operand of fused_temporal_conv_add_lif_state, runtime/snn_custom_ops.py:491-518) to
  * the framework's convolution; this entry point keeps such a layer on the NCHW tensors the fused operators exchange.
- * Supported: Cin % 8 == 0 or Cin < 8, anything but a plain 1x1 stride-1 convolution; SNNF_ERR_UNSUPPORTED otherwise.
+ * Supported: Cin % 8 == 0 or Cin < 8 (a plain 1x1 stride-1 layer runs with each image as one row of pixels);
+ * SNNF_ERR_UNSUPPORTED otherwise.
  *   out : [T, N, Cout, Ho, Wo] x_dtype (frame stride `out_step_stride` elements) */
 int snnf_conv_bias(const void* const* xs, const void* const* residuals /* nullable */, int T,
                    int N, int Cin, int H, int W, int x_dtype,

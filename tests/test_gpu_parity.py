@@ -578,6 +578,8 @@ CONV_BIAS_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, T, N, residual, a
     (32, 64, 16, 16, 3, 2, 1, F16, 4, 2, False, True),        # fp16
     (64, 64, 8, 8, 3, 1, 1, F32, 1, 4, False, False),         # fp32 in and out (bf16 matrix operands)
     (256, 64, 6, 6, 3, 1, 1, BF16, 4, 2, True, False),        # deep: K split across waves
+    (64, 128, 8, 8, 1, 1, 0, BF16, 4, 3, False, False),       # plain 1x1 / stride 1: an image is one row of pixels
+    (128, 256, 7, 9, 1, 1, 0, F16, 3, 2, True, False),        # the same with a residual, odd plane
 ]
 
 
@@ -602,11 +604,7 @@ def test_conv_bias_without_neuron(hip_ops, Cin, Cout, H, W, k, stride, pad, dtyp
 
 
 def test_conv_bias_rejects_what_the_matrix_kernel_does_not_take(hip_ops):
-    x = [torch.zeros(2, 64, 8, 8, device=DEV, dtype=BF16)]
-    w = torch.zeros(64, 64, 1, 1, device=DEV, dtype=BF16)
     from triton_snn_fusion_amd.runtime.hip_convlif_backend import run_hip_temporal_conv_bias
-    with pytest.raises(RuntimeError, match="unsupported_shape"):
-        run_hip_temporal_conv_bias(x, w, None, [1, 1], [0, 0])      # plain 1x1 / stride 1
     w12 = torch.zeros(64, 12, 3, 3, device=DEV, dtype=BF16)
     with pytest.raises(RuntimeError, match="unsupported_shape"):
         run_hip_temporal_conv_bias([torch.zeros(2, 12, 8, 8, device=DEV, dtype=BF16)], w12, None, [1, 1], [1, 1])   # Cin % 8 != 0

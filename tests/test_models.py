@@ -15,7 +15,8 @@ from triton_snn_fusion_amd import fx_temporal_rewrite as R
 from triton_snn_fusion_amd import models as M
 
 BF16, F32 = torch.bfloat16, torch.float32
-SMALL = {"vgg11": dict(width=16, size=32, batch=3), "resnet18": dict(width=16, size=64, batch=2)}
+SMALL = {"vgg11": dict(width=16, size=32, batch=3), "resnet18": dict(width=16, size=64, batch=2), "mobilenet": dict(width=32, size=64, batch=2)}
+NEURONS = {"vgg11": 8, "resnet18": 17, "mobilenet": 9}          # neuron modules = fused layers incl. the tail
 
 
 def _frame(name, seed=5):
@@ -26,7 +27,7 @@ def _frame(name, seed=5):
 # ---------------------------------------------------------------------------------------------------------------
 # Eager form (CPU)
 # ---------------------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_single_step_loop_wrapper_and_state_reset(name):
     model = M.build_network(name, width=8, gain=5.0)
     x = torch.randn(2, 3, 32, 32, generator=gen(1))
@@ -43,20 +44,20 @@ def test_single_step_loop_wrapper_and_state_reset(name):
     assert not torch.equal(per_step[0], per_step[1])
     assert torch.equal(y, y_again) and not torch.equal(y, y_stale)
     neurons = [m for m in model.modules() if isinstance(m, M.CustomStatefulIFNode)]
-    assert len(neurons) == (8 if name == "vgg11" else 17)
+    assert len(neurons) == NEURONS[name]
     assert all(n.v.dim() == 4 for n in neurons)
     M.reset_lif_modules(model)
     assert all(n.v.dim() == 0 for n in neurons)
 
 
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_batchnorm_folding_keeps_the_network_function(name):
     model = M.build_network(name, width=8, gain=5.0)
     folded = M.fold_batchnorm(model)
     assert not any(isinstance(m, torch.nn.BatchNorm2d) for m in folded.modules())
     x = torch.randn(2, 3, 32, 32, generator=gen(2))
     with torch.no_grad():
-        block, fblock = (model.features[0], folded.features[0]) if name == "vgg11" else (model.stem, folded.stem)
+        block, fblock = (model.stem, folded.stem) if name == "resnet18" else (model.features[0], folded.features[0])
         pre = block.bn(block.conv(x))
         assert torch.allclose(fblock.conv(x), pre, rtol=1e-5, atol=1e-5)
         M.reset_lif_modules(model)
@@ -65,7 +66,7 @@ def test_batchnorm_folding_keeps_the_network_function(name):
     assert torch.allclose(y, y_f, rtol=1e-3, atol=1e-3)
 
 
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_fused_operator_sequence_is_the_eager_network_exactly_on_cpu(name):
     """Wiring: on CPU tensors the snn_custom operators evaluate the eager formulas, so the layer-major fused form and the
     time-major single-step form run the same fp32 arithmetic in a different order of calls and must agree exactly."""
@@ -82,6 +83,9 @@ def test_fused_operator_sequence_is_the_eager_network_exactly_on_cpu(name):
     if name == "vgg11":
         assert kinds == ["conv_lif", "pool", "conv_lif", "pool", "conv_lif", "conv_lif", "pool", "conv_lif", "conv_lif", "pool",
                          "conv_lif", "plain_conv", "tail"]
+    elif name == "mobilenet":
+        assert kinds == ["conv_lif"] * 8 + ["plain_conv", "tail"]
+        assert [e["layer"].groups > 1 for e in fused.record[:8]] == [False, True, False, True, False, True, False, True]
     else:
         assert kinds.count("conv_lif") == 16 and kinds.count("plain_conv") == 4 and kinds[-2:] == ["plain_conv", "tail"]
         assert sum(e["kind"] == "conv_lif" and e["residuals"] is not None for e in fused.record) == 7
@@ -338,7 +342,7 @@ def _fused(name, T=4, gain=5.0, internal=False):
 def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
     """Every recorded operator call of one forward against the oracle on that call's own operands (teacher forcing)."""
     kinds = [e["kind"] for e in fused.record]
-    assert kinds.count("conv_lif") == (7 if name == "vgg11" else 16) and kinds.count("tail") == 1
+    assert kinds.count("conv_lif") == NEURONS[name] - 1 and kinds.count("tail") == 1
     active = 0
     for e in fused.record:
         if e["kind"] == "conv_lif":
@@ -346,7 +350,7 @@ def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
             xs = [x.float().cpu() for x in e["xs"]]
             rs = None if e["residuals"] is None else [r.float().cpu() for r in e["residuals"]]
             ref = O.temporal_conv_lif(xs, L.weight.float().cpu(), L.bias.float().cpu(), torch.tensor(0.0), tuple(L.stride),
-                                      tuple(L.padding), (1, 1), 1, *L.lif, residuals=rs)
+                                      tuple(L.padding), (1, 1), L.groups, *L.lif, residuals=rs)
             check(e["spikes"], e["v"], ref, what=f"{name} {e['name']}")
             active += int(ref[0].mean() > 0.01)
         elif e["kind"] == "plain_conv":
@@ -368,7 +372,13 @@ def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
             assert torch.allclose(out.float().cpu(), ref_out / T, rtol=8e-3, atol=8e-3)
     assert active >= 5, "the test network is nearly silent"
     stats = hip_ops.get_fused_op_call_stats()
-    if internal:      # only the tail goes through the dense operator layer
+    if internal and name == "mobilenet":
+        # row-packed spikes between the stride-1 depthwise and the pointwise layers; the stem (analog frame), the two stride-2
+        # depthwise layers and the tail go through the dense operator layer, the LIF-free last convolution through snnf_conv_bias
+        packed = [e["name"] for e in fused.record if e.get("blocked")]
+        assert packed == ["features.1", "features.2", "features.4", "features.5", "features.6"], packed
+        assert stats["fallback"] == 0 and stats["triton"] == 4, stats
+    elif internal:      # only the tail goes through the dense operator layer
         assert all(e.get("blocked") for e in fused.record if e["kind"] != "tail")
         assert stats["fallback"] == 0 and stats["triton"] == 1, stats
     else:
@@ -377,7 +387,7 @@ def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
     """`internal`: spikes bit-packed and analog activations channel-blocked between the network's own operators; the
     executor records every operator's operands and results converted back to dense tensors."""
@@ -389,14 +399,15 @@ def test_fused_network_operator_by_operator_against_the_oracle(hip_ops, name, in
     _check_recorded_operators(hip_ops, name, fused, out, T, internal)
 
 
-FULL = {"vgg11": dict(size=32, batch=64), "resnet18": dict(size=224, batch=16)}
+FULL = {"vgg11": dict(size=32, batch=64), "resnet18": dict(size=224, batch=16), "mobilenet": dict(size=64, batch=32)}
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_full_width_network_operator_by_operator_against_the_oracle(hip_ops, name, internal):
-    """The two benchmark configurations at their real size (width 64; VGG-11 T=4 B=64 32x32, ResNet-18 T=4 B=16 224x224):
+    """The benchmark configurations at their real size (width 64; VGG-11 T=4 B=64 32x32, ResNet-18 T=4 B=16 224x224, and the
+    MobileNet-style network T=4 B=32 64x64):
     every operator call of one forward, with the launch plans those sizes select, against the oracle on its own operands."""
     T = 4
     cfg = FULL[name]
@@ -437,7 +448,7 @@ def test_fused_network_tracks_the_eager_network(hip_ops, name):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_internal_layouts_track_the_dense_executor(hip_ops, name):
     """Same network, same operands: the two executors differ in summation order only, so the first layer agrees up to
     near-threshold flips and the logits point the same way."""
@@ -452,11 +463,13 @@ def test_internal_layouts_track_the_dense_executor(hip_ops, name):
     cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
     print(f"{name}: internal layouts vs dense executor, cosine similarity of the logits {cos:.5f}")
     assert cos > 0.8, cos
+    if name == "mobilenet":     # the row-packed entry points are the dense kernels with another fetch / store: the same bits
+        assert torch.equal(got, want)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("internal", [False, True], ids=["dense", "internal_layouts"])
-@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18", "mobilenet"])
 def test_fused_network_graph_replay_matches_eager_launches(hip_ops, name, internal):
     T = 4
     _, fused = _fused(name, T, internal=internal)

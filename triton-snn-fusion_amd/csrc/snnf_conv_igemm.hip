@@ -347,7 +347,8 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     }
     g.bits_out = out_rowbits ? 1 : 0;
     const bool pointwise_to_matrix = !x_rowbits && pointwise && (flops / bytes >= 200.0 || (Cin > 128 && bytes < 200.0e6));
-    const bool matrix_candidate = (!pointwise || pointwise_to_matrix) && (Cin % 8 == 0 || Cin < 8);
+    // A neuron-free pointwise layer (snnf_conv_bias) has no other kernel to go to: the pointwise kernel always runs a neuron.
+    const bool matrix_candidate = (!pointwise || pointwise_to_matrix || (analog_out && !x_rowbits)) && (Cin % 8 == 0 || Cin < 8);
     int window = 0;
     Plan pl = {};
     bool planned = false;
@@ -385,7 +386,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     }
     if (analog_out && !mm_kernel)
         return fail(SNNF_ERR_UNSUPPORTED, "snnf_conv_bias: unsupported_shape: only layers the 8-wave matrix kernel takes "
-                    "(Cin %% 8 == 0 or Cin < 8, not a plain 1x1/1 convolution, tiles that fit LDS)");
+                    "(Cin %% 8 == 0 or Cin < 8, tiles that fit LDS)");
     // Everything else: the time-outer kernels for a shared frame or a low intensity, the 4-wave T-in-M kernel otherwise.
     bool time_outer = !mm_kernel && (all_shared || x_rowbits || flops / bytes < 200.0);
     // Pointwise kernel: where the weight fragments live (registers only in the fast variant) and the LDS that takes.

@@ -104,9 +104,9 @@ def _neuron() -> CustomStatefulIFNode:
 class ConvBNNeuron(nn.Module):
     """Conv2d (no bias) -> BatchNorm2d -> neuron; `sn` is None for a LIF-free convolution (shortcut, pre-tail)."""
 
-    def __init__(self, cin: int, cout: int, kernel: int, stride: int, padding: int, neuron: bool = True):
+    def __init__(self, cin: int, cout: int, kernel: int, stride: int, padding: int, neuron: bool = True, groups: int = 1):
         super().__init__()
-        self.conv = nn.Conv2d(cin, cout, kernel, stride, padding, bias=False)
+        self.conv = nn.Conv2d(cin, cout, kernel, stride, padding, groups=groups, bias=False)
         self.bn = nn.BatchNorm2d(cout, eps=BN_EPS)
         self.sn = _neuron() if neuron else None
 
@@ -188,6 +188,36 @@ class SpikingResNet18(nn.Module):
         return self.fc(torch.flatten(self.avgpool(y), 1))
 
 
+# (output channels, stride of the depthwise layer) of the depthwise-separable blocks behind the 3x3/2 stem of 32 channels.
+MOBILENET_BLOCKS = ((64, 1), (128, 2), (128, 1), (256, 2))
+
+
+class SpikingMobileNet(nn.Module):
+    """MobileNetV1-style network (counterpart of the reference zoo's MobileNet entries, benchmarks/
+    validate_chronos_baselines.py:312-847, in shape only): stem Conv3x3/2 + BN + LIF, then depthwise-separable blocks
+    (depthwise Conv3x3 + BN + LIF, pointwise Conv1x1 + BN + LIF), tail LIF -> global average pool -> Linear. The last
+    pointwise convolution's neuron is the tail's neuron. `width` scales every channel count (32 = the full network)."""
+
+    def __init__(self, num_classes: int = 10, in_channels: int = 3, width: int = 32, blocks: Sequence[Tuple[int, int]] = MOBILENET_BLOCKS):
+        super().__init__()
+        scale = lambda c: max(8, c * width // 32 // 8 * 8)      # multiples of 8: whole channel groups for the matrix kernels
+        cin = scale(32)
+        layers: List[nn.Module] = [ConvBNNeuron(in_channels, cin, 3, 2, 1)]
+        for i, (cout, stride) in enumerate(blocks):
+            cout = scale(cout)
+            layers.append(ConvBNNeuron(cin, cin, 3, stride, 1, groups=cin))
+            layers.append(ConvBNNeuron(cin, cout, 1, 1, 0, neuron=i + 1 < len(blocks)))
+            cin = cout
+        self.features = nn.Sequential(*layers)
+        self.tail_sn = _neuron()
+        self.avgpool = nn.AdaptiveAvgPool2d((1, 1))
+        self.fc = nn.Linear(cin, num_classes)
+
+    def forward(self, x):
+        y = self.tail_sn(self.features(x))
+        return self.fc(torch.flatten(self.avgpool(y), 1))
+
+
 def init_synthetic_(model: nn.Module, seed: int = 0, gain: float = 1.0) -> nn.Module:
     """Kaiming-normal convolution and classifier weights (scaled by `gain`), classifier bias N(0, 0.01^2), BatchNorm
     gamma U(0.8, 1.2), beta N(0, 0.1^2), running mean N(0, 0.1^2), running variance U(0.5, 1.5); CPU generator `seed`."""
@@ -223,7 +253,7 @@ def fold_batchnorm(model: nn.Module, round_to: Optional[torch.dtype] = None) -> 
             if isinstance(m, ConvBNNeuron) and isinstance(m.bn, nn.BatchNorm2d):
                 w, b = fold_bn_into_conv_params(m.conv.weight.float(), m.conv.bias, m.bn.running_mean.float(),
                                                 m.bn.running_var.float(), m.bn.weight.float(), m.bn.bias.float(), m.bn.eps)
-                conv = nn.Conv2d(m.conv.in_channels, m.conv.out_channels, m.conv.kernel_size, m.conv.stride, m.conv.padding, bias=True)
+                conv = nn.Conv2d(m.conv.in_channels, m.conv.out_channels, m.conv.kernel_size, m.conv.stride, m.conv.padding, groups=m.conv.groups, bias=True)
                 conv.weight.copy_(rounded(w))
                 conv.bias.copy_(rounded(b))
                 m.conv, m.bn = conv.to(w.device), nn.Identity()
@@ -252,11 +282,12 @@ class _FusedLayer:
             self.bias = b.to(device=device, dtype=dtype).contiguous()
         self.stride = [int(s) for s in m.conv.stride]
         self.padding = [int(p) for p in m.conv.padding]
+        self.groups = int(m.conv.groups)
         self.lif = m.sn.lif_params if m.sn is not None else None
 
     @property
     def geometry(self):
-        return (self.stride, self.padding, [1, 1], 1)
+        return (self.stride, self.padding, [1, 1], self.groups)
 
 
 class _FusedNetwork(nn.Module):
@@ -292,7 +323,14 @@ class _FusedNetwork(nn.Module):
     def conv_lif(self, name: str, xs: List[torch.Tensor], layer: _FusedLayer, residuals: Optional[List[torch.Tensor]] = None):
         S = torch.ops.snn_custom
         if residuals is None:
-            spikes, v = S.fused_temporal_conv_lif_state(xs, layer.weight, layer.bias, self.zero_v, *layer.geometry, *layer.lif, False)
+            # The operator per convolution kind, as the reference's rewrite selects it (compiler/fx_lif_temporal_rewrite.py:1625-1662).
+            if layer.groups > 1:
+                op = S.fused_temporal_depthwise_conv_lif_state
+            elif tuple(layer.weight.shape[2:]) == (1, 1) and layer.stride == [1, 1] and layer.padding == [0, 0]:
+                op = S.fused_temporal_pointwise_conv_lif_state
+            else:
+                op = S.fused_temporal_conv_lif_state
+            spikes, v = op(xs, layer.weight, layer.bias, self.zero_v, *layer.geometry, *layer.lif, False)
         else:
             spikes, v = S.fused_temporal_conv_add_lif_state(xs, residuals, layer.weight, layer.bias, self.zero_v,
                                                             *layer.geometry, *layer.lif, False)
@@ -497,10 +535,81 @@ class FusedSpikingResNet18(_FusedNetwork):
         return self.tail(B.to_dense(seq), self.tail_lif, self.fc_weight, self.fc_bias)
 
 
+class FusedSpikingMobileNet(_FusedNetwork):
+    """Layer-major execution of `SpikingMobileNet`. Dense form: the depthwise / pointwise / regular `snn_custom` operators.
+    Internal form (`internal_layouts=True`): behind the stem the spikes travel row-packed (one byte = 8 consecutive pixels of
+    a channel's row), which is what a depthwise lane holds after a LIF step: `snnf_dwconv3x3_lif_rowbits` ->
+    `snnf_pwconv_lif_rowbits` -> ... with no dense spike tensor and no membrane written between them. A layer those entry
+    points do not take (a stride-2 depthwise layer, rows that are no multiple of 8 pixels, planes that are no multiple of 64
+    pixels) runs the dense operator on unpacked spikes and its output is packed again."""
+
+    def __init__(self, model: SpikingMobileNet, T: int, dtype: torch.dtype = torch.bfloat16, device="cuda:0", internal_layouts: bool = False):
+        super().__init__(T, dtype, device, internal_layouts=internal_layouts)
+        self.layers = [_FusedLayer(m, dtype, self.device_) for m in model.features]
+        self.tail_lif = model.tail_sn.lif_params
+        self.fc_weight = model.fc.weight.detach().to(device=self.device_, dtype=dtype).contiguous()
+        self.fc_bias = model.fc.bias.detach().to(device=self.device_, dtype=dtype).contiguous()
+
+    def run(self, x):
+        seq: Optional[torch.Tensor] = None
+        for i, layer in enumerate(self.layers):
+            if layer.lif is not None:
+                xs = [x] * self.T if seq is None else list(seq.unbind(0))
+                seq = self.conv_lif(f"features.{i}", xs, layer)
+            else:
+                seq = self.plain_conv(f"features.{i}", seq, layer)
+        return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
+
+    def run_blocked(self, x):
+        from .runtime import hip_blocked_backend as B
+        common = lambda lif: lif is not None and float(lif[1]) == 0.0      # hard reset to zero: what the row-packed variants serve
+        dense = self.conv_lif("features.0", [x] * self.T, self.layers[0])    # the analog frame goes through the dense operator
+        bits = None                                                           # row-packed spikes [T, N, C, H, W / 8], or None
+        for i, layer in enumerate(self.layers[1:], start=1):
+            name = f"features.{i}"
+            if bits is None and dense.shape[-1] % 8 == 0 and layer.lif is not None:
+                bits, dense = B.pack_rowbits(dense), None
+            depthwise = layer.groups > 1
+            took = False
+            if bits is not None and common(layer.lif):
+                h, w = int(bits.shape[3]), int(bits.shape[4]) * 8
+                try:
+                    if depthwise and layer.stride == [1, 1]:
+                        out, v = B.depthwise_conv_lif_rowbits(bits, layer.weight, layer.bias, layer.lif, want_v=self.record is not None)
+                        took = True
+                    elif not depthwise and tuple(layer.weight.shape[2:]) == (1, 1) and layer.stride == [1, 1] and (h * w) % 64 == 0:
+                        out, v = B.pointwise_conv_lif_from_rowbits(bits, layer.weight, layer.bias, layer.lif, packed_out=True,
+                                                                   want_v=self.record is not None)
+                        took = True
+                except RuntimeError as exc:
+                    if "unsupported" not in str(exc):
+                        raise
+            if took:
+                if self.record is not None:
+                    self._log(kind="conv_lif", name=name, xs=list(B.unpack_rowbits(bits, self.dtype).unbind(0)), residuals=None, layer=layer,
+                              spikes=B.unpack_rowbits(out, self.dtype), v=v, blocked=True)
+                bits = out
+                continue
+            # Dense operators on unpacked spikes (stride-2 depthwise layers, the LIF-free last convolution, odd shapes).
+            if dense is None:
+                dense = B.unpack_rowbits(bits, self.dtype)
+                bits = None
+            if layer.lif is not None:
+                dense = self.conv_lif(name, list(dense.unbind(0)), layer)
+            else:
+                dense = self.plain_conv(name, dense, layer)
+        if dense is None:
+            dense = B.unpack_rowbits(bits, self.dtype)
+        return self.tail(dense, self.tail_lif, self.fc_weight, self.fc_bias)
+
+
 def build_network(name: str, width: int = 64, num_classes: Optional[int] = None, seed: int = 0, gain: float = 1.0) -> nn.Module:
-    """`vgg11` (10 classes) or `resnet18` (1000 classes) with the synthetic initialisation."""
+    """`vgg11` (10 classes), `resnet18` (1000 classes) or `mobilenet` (10 classes; `width` 64 is the full network, as for
+    the other two) with the synthetic initialisation."""
     if name == "vgg11":
         model = SpikingVGG11(num_classes=10 if num_classes is None else num_classes, width=width)
+    elif name == "mobilenet":
+        model = SpikingMobileNet(num_classes=10 if num_classes is None else num_classes, width=width // 2)
     elif name == "resnet18":
         model = SpikingResNet18(num_classes=1000 if num_classes is None else num_classes, width=width)
     else:
@@ -516,4 +625,6 @@ def fuse_network(model: nn.Module, T: int, dtype: torch.dtype = torch.bfloat16, 
         return FusedSpikingVGG11(model, T, dtype, device, internal_layouts)
     if isinstance(model, SpikingResNet18):
         return FusedSpikingResNet18(model, T, dtype, device, internal_layouts)
+    if isinstance(model, SpikingMobileNet):
+        return FusedSpikingMobileNet(model, T, dtype, device, internal_layouts)
     raise TypeError(f"no fused executor for {type(model).__name__}")
