@@ -744,7 +744,8 @@ def main() -> int:
                     flops = 2 * T_ * M_ * fin_ * fout_
                 ai = flops / nbytes
                 entry["algorithmic_bytes"], entry["flops"] = nbytes, flops
-                entry["matrix_operand_dtype"] = "f16" if args.dtype == "f16" and name != "conv3x3_block" else "bf16"
+                entry["matrix_operand_dtype"] = ("bf16 hi + lo terms of every fp32 operand (3 matrix products per fp32 product)" if name == "conv3x3_block"
+                                                 else ("f16" if args.dtype == "f16" else "bf16"))
                 entry["roofline"] = _roofline("mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm", flops if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else nbytes, kms)
                 entry["hbm"], entry["mfma"] = _roofline("hbm", nbytes, kms), _roofline("mfma", flops, kms)
             except Exception as exc:

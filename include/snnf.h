@@ -214,8 +214,11 @@ int snnf_linear_lif_ws(const void* const* xs, int T, int M, int Fin, int64_t x_r
  *
  * Two steps: (1) snnf_conv_pack_weight rewrites the OIHW weight (+ bias) into the matrix-core operand order once per
  * weight tensor and activation dtype; (2) snnf_conv_lif consumes the packed weight on every call. The packed buffer is
- * opaque; its size is snnf_conv_packed_weight_bytes(). fp32 activations/weights are rounded to bf16 for the matrix cores (fp32
- * accumulate); fp16 activations use the fp16 matrix path.
+ * opaque; its size is snnf_conv_packed_weight_bytes(). fp32 activations / weights enter the matrix cores as two bf16 terms each
+ * (the value rounded to bf16 and the rounded remainder; three of the four products are accumulated in fp32, the fourth is
+ * below 2^-16 of the result): the reference multiplies fp32 tensors in TF32 (kernels/benchmark_conv_lif_temporal_general.py:
+ * 673-674), this keeps about 16 mantissa bits. The depthwise kernel multiplies fp32 tensors in fp32. fp16 activations use the
+ * fp16 matrix path, bf16 ones the bf16 path.
  *   xs[t]        : [N, Cin, H, W] x_dtype
  *   residuals[t] : [N, Cout, Ho, Wo] x_dtype or residuals == NULL
  *   spikes       : [T, N, Cout, Ho, Wo] x_dtype (timestep stride `spike_step_stride` elements); v_out : [N, Cout, Ho, Wo] v_dtype

@@ -236,16 +236,17 @@ def test_linear_lif_list_out_and_leading_dims_forms_agree(hip_ops):
 # ---------------------------------------------------------------------------------------------------------------
 def _conv_case(seed, T, N, Cin, Cout, H, W, k, dtype, analog=False, p=0.2, gain=2.0):
     g = gen(seed)
+    # fp32 tensors keep their fp32 values: the kernels split them into two bf16 terms each for the matrix cores and the
+    # oracle is held to them unrounded.
     if analog:
-        xs = [q(torch.randn(N, Cin, H, W, generator=g), BF16 if dtype == F32 else dtype) for _ in range(T)]
+        xs = [q(torch.randn(N, Cin, H, W, generator=g), dtype) for _ in range(T)]
     else:
         xs = [spikes((N, Cin, H, W), p, g) for _ in range(T)]
     w = torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * k * k)) ** 0.5 * gain
     b = torch.randn(Cout, generator=g) * 0.1
-    w_ref = q(w, BF16 if dtype == F32 else dtype)
+    w_ref = q(w, dtype)
     b_ref = b if dtype == F32 else q(b, dtype)
-    w_dev = w if dtype == F32 else w_ref
-    return xs, w_dev, b_ref, w_ref, b_ref
+    return xs, w_ref, b_ref, w_ref, b_ref
 
 
 CONV_KEYS = [  # k, stride, pad, Cin, Cout, H, W, analog
@@ -551,7 +552,7 @@ SHARED_FRAME_CASES = [  # Cin, Cout, H, W, k, stride, pad, dtype, lif, T, N, res
 def test_conv_shared_analog_frame_variants(hip_ops, Cin, Cout, H, W, k, stride, pad, dtype, lif, T, N, residual, tensor_v):
     """One analog frame for all T timesteps: convolved once, T LIF steps on the same accumulators."""
     g = gen(1300 + Cin + Cout + H + k)
-    op_dtype = BF16 if dtype == F32 else dtype     # fp32 frames and weights enter the matrix cores as bf16
+    op_dtype = dtype                               # fp32 frames and weights stay fp32 (two bf16 terms each on the matrix cores)
     x = q(torch.randn(N, Cin, H, W, generator=g), op_dtype)
     w = q(torch.randn(Cout, Cin, k, k, generator=g) * (1.5 / (Cin * k * k) ** 0.5), op_dtype)
     b = q(torch.randn(Cout, generator=g) * 0.1, dtype)

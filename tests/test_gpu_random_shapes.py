@@ -48,6 +48,7 @@ def test_random_dense_conv_lif_cases(hip_ops, seed, cases):
         H, W = rnd.randint(max(1, k - 2 * p), 24), rnd.randint(max(1, k - 2 * p), 24)
         T, N = rnd.choice([1, 2, 3, 4, 4, 4, 5, 6, 8, 9, 17]), rnd.randint(1, 9)
         dtype, op_dt, vdtype = _dtypes(rnd)
+        op_dt = dtype       # convolutions: fp32 operands stay unrounded (two bf16 terms each on the matrix cores; fp32 taps when depthwise)
         analog, with_res, lif = rnd.random() < 0.25, rnd.random() < 0.3, rnd.choice(LIFS)
         Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
         groups = Cin if depthwise else 1

@@ -68,6 +68,14 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
     return u >> 16;
 }
 
+// The bf16 term of an fp32 value for part `part` of the split described at kSplitParts (snnf_conv_common.h): the value
+// rounded to bf16 (parts 0 and 1) or what that rounding left over, rounded to bf16 (part 2). x - hi is exact in fp32.
+__device__ __forceinline__ uint32_t split_bf16_bits(float x, bool low_term) {
+    const uint32_t hi = float_to_bf16_bits(x);
+    if (!low_term) return hi;
+    return float_to_bf16_bits(x - __uint_as_float(hi << 16));
+}
+
 __device__ __forceinline__ float f16_bits_to_float(uint32_t bits) {
     union { uint16_t u; _Float16 h; } cvt;
     cvt.u = static_cast<uint16_t>(bits);

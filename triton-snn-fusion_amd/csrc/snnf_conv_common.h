@@ -34,9 +34,17 @@ __host__ __device__ inline int chunk_channels(int Cin, int taps, bool wide_activ
     return 128;
 }
 
+// fp32 tensors keep (nearly) fp32 accuracy on the 16-bit matrix cores by a split of both operands into two bf16 terms,
+// x = x_hi + x_lo and w = w_hi + w_lo (hi = the value rounded to bf16, lo = the remainder rounded to bf16), and three of the
+// four products: w_hi x_hi + w_lo x_hi + w_hi x_lo (the fourth is below 2^-16 of the result). The three products are three
+// "parts" of the channel axis: the packed weight holds the real channel chunks three times over (w_hi, w_lo, w_hi) and the
+// kernels stage the real activation chunks three times (x_hi, x_hi, x_lo). 16-bit tensors have one part.
+constexpr int kSplitParts = 3;
+
 struct PackGeom {
     int Cout, Cin, KH, KW;
     int CK, nchunks, npairs, nocf;
+    int nchunks_r;   // real channel chunks; nchunks = parts * nchunks_r
 };
 
 __host__ __device__ inline PackGeom make_pack_geom(int Cout, int Cin, int KH, int KW, bool wide_activations) {
@@ -46,7 +54,8 @@ __host__ __device__ inline PackGeom make_pack_geom(int Cout, int Cin, int KH, in
     p.KH = KH;
     p.KW = KW;
     p.CK = chunk_channels(Cin, KH * KW, wide_activations);
-    p.nchunks = (Cin + p.CK - 1) / p.CK;
+    p.nchunks_r = (Cin + p.CK - 1) / p.CK;
+    p.nchunks = (wide_activations ? kSplitParts : 1) * p.nchunks_r;
     const int slots = KH * KW * (p.CK / 8);
     p.npairs = (slots + 1) / 2;
     p.nocf = (Cout + 31) / 32;
@@ -67,6 +76,12 @@ enum LoadMode : int {
     LOAD_ROWBITS = 3   // row-packed spikes (one byte = 8 consecutive pixels of a channel): one byte load, the pair's two bits
                        // become two 16-bit ones or zeros on the way into LDS (pointwise kernel only)
 };
+
+// Part (0, 1, 2) and real channel chunk of virtual chunk `vchunk` of an fp32 tensor's three-part channel axis.
+__device__ __forceinline__ void split_chunk(int vchunk, int nchunks_r, int& part, int& chunk) {
+    part = vchunk >= 2 * nchunks_r ? 2 : (vchunk >= nchunks_r ? 1 : 0);
+    chunk = vchunk - part * nchunks_r;
+}
 
 // Staging items a thread may hold in flight per chunk: modes that need two registers per fetch get half as many.
 __host__ __device__ constexpr int staging_items(int load_mode) { return load_mode == LOAD_PAIR32 ? kMaxItems : kMaxItems / 2; }
@@ -105,6 +120,7 @@ struct ConvGeom {
     int wm_log2, wn_log2;     // waves along pixels / along output channels (WM * WN == 4)
     int oc_tiles;             // ceil(Cout / (WN * 64))
     int CK, nchunks, npairs, groups_log2;
+    int nchunks_r;            // real channel chunks of the activations (nchunks counts the three parts of an fp32 tensor)
     int NR, WT;               // LDS tile: input rows x input columns (per timestep)
     int pitch;                // bytes per LDS pixel = CK * 2 + 16
     int T;                    // timesteps stored by this launch (<= TT)

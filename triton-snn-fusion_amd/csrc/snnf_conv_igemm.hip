@@ -146,8 +146,10 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw
                 const int NRT = ti * NR;                           // stacked halo rows
                 const int img_groups = (g0.N + ti - 1) / ti;
                 // An LDS stage holds as many packed channel chunks as fit (fewer barriers and exposed load latencies per tile).
+                // (The three parts of an fp32 tensor's channel axis are staged differently: a stage must lie inside one part.)
+                const bool parts = g0.nchunks != g0.nchunks_r;
                 int sc = 1;
-                while (sc * 2 <= g0.nchunks && sc * 2 * g0.CK <= 256 &&
+                while (sc * 2 <= g0.nchunks_r && (!parts || g0.nchunks_r % (sc * 2) == 0) && sc * 2 * g0.CK <= 256 &&
                        static_cast<size_t>(tt) * NRT * WT * (sc * 2 * g0.CK * 2 + 16) + stage_bytes <= lds_cap &&
                        sc * 2 * groups * NRT * (WT / 2) <= max_items)
                     sc *= 2;
@@ -289,7 +291,7 @@ int conv_lif_impl(const void* const* xs, const void* const* residuals, int T, in
     g.Ho = (g.H + 2 * pad_h - KH) / stride_h + 1;
     g.Wo = (g.W + 2 * pad_w - KW) / stride_w + 1;
     const PackGeom pg = make_pack_geom(Cout, Cin, KH, KW, x_dtype == SNNF_F32);
-    g.CK = pg.CK; g.nchunks = pg.nchunks; g.npairs = pg.npairs;
+    g.CK = pg.CK; g.nchunks = pg.nchunks; g.npairs = pg.npairs; g.nchunks_r = pg.nchunks_r;
     g.groups_log2 = 0;
     while ((8 << g.groups_log2) < pg.CK) ++g.groups_log2;
     g.pitch = pg.CK * 2 + 16;

@@ -127,7 +127,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
         }
     };
 
+    int pre_part = 0;       // fp32 tensors: which of the three parts of the channel axis `pre` holds (2: the low terms)
     auto issue_loads = [&](int chunk) __attribute__((always_inline)) {
+        if constexpr (LM == LOAD_2XF32) split_chunk(chunk, g.nchunks_r, pre_part, chunk);
         const int64_t chunk_bytes = static_cast<int64_t>(chunk) * g.CK * plane * ES;
 #pragma unroll
         for (int u = 0; u < MI; ++u) {
@@ -172,8 +174,8 @@ __global__ __launch_bounds__(kConvThreads) void conv_lif_kernel(const StepPtrs x
                         e0[j] = pre[u][j][0];
                         e1[j] = pre[u][j][1];
                     } else {
-                        e0[j] = float_to_bf16_bits(__uint_as_float(pre[u][j][0]));
-                        e1[j] = float_to_bf16_bits(__uint_as_float(pre[u][j][1]));
+                        e0[j] = split_bf16_bits(__uint_as_float(pre[u][j][0]), pre_part == 2);
+                        e1[j] = split_bf16_bits(__uint_as_float(pre[u][j][1]), pre_part == 2);
                     }
                 }
                 cv_u32x4 lo, hi;

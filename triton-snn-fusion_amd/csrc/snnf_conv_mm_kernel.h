@@ -114,8 +114,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 
     // Loads of stage `stg` (stage_chunks channel chunks) of the tile whose halo starts at input (row ih_lo, column iw_lo)
     // of image n.
+    int pre_part = 0;       // fp32 tensors: which of the three parts of the channel axis `pre` holds (2: the low terms)
     auto issue_loads = [&](int stg, int n, int ih_lo, int iw_lo) __attribute__((always_inline)) {
-        const int chunk = stg * g.stage_chunks;                                                  // first chunk of the stage
+        int chunk = stg * g.stage_chunks;                                                        // first chunk of the stage
+        // fp32 tensors: a stage lies inside one part (the planner picks stage_chunks that divide the real chunk count).
+        if constexpr (LM == LOAD_2XF32) split_chunk(chunk, g.nchunks_r, pre_part, chunk);
         const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
         const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
         uint32_t off0[SS], off1[SS];
@@ -201,8 +204,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                                 e0[j] = pre[s][t][j][0];
                                 e1[j] = pre[s][t][j][1];
                             } else {
-                                e0[j] = float_to_bf16_bits(__uint_as_float(pre[s][t][j][0]));
-                                e1[j] = float_to_bf16_bits(__uint_as_float(pre[s][t][j][1]));
+                                e0[j] = split_bf16_bits(__uint_as_float(pre[s][t][j][0]), pre_part == 2);
+                                e1[j] = split_bf16_bits(__uint_as_float(pre[s][t][j][1]), pre_part == 2);
                             }
                         }
 #pragma unroll

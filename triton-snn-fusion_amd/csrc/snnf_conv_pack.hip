@@ -15,8 +15,11 @@ __global__ void pack_weight_kernel(const WT* __restrict__ w, const WT* __restric
         int64_t frag = idx >> 9;
         const int pair = frag % p.npairs;
         frag /= p.npairs;
-        const int chunk = frag % p.nchunks;
+        const int vchunk = frag % p.nchunks;
         const int ocf = frag / p.nchunks;
+        // fp32 tensors: three parts of the channel axis hold w_hi, w_lo, w_hi (see kSplitParts).
+        const int part = vchunk / p.nchunks_r;
+        const int chunk = vchunk - part * p.nchunks_r;
         const int oc = ocf * 32 + (lane & 31);
         const int slot = pair * 2 + (lane >> 5);
         const int groups = p.CK / 8;
@@ -25,7 +28,7 @@ __global__ void pack_weight_kernel(const WT* __restrict__ w, const WT* __restric
         float v = 0.0f;
         if (oc < p.Cout && ci < p.Cin && tap < p.KH * p.KW)
             v = to_float(w[(static_cast<int64_t>(oc) * p.Cin + ci) * (p.KH * p.KW) + tap]);
-        packed[idx] = TO_F16 ? static_cast<uint16_t>(float_to_f16_bits(v)) : static_cast<uint16_t>(float_to_bf16_bits(v));
+        packed[idx] = TO_F16 ? static_cast<uint16_t>(float_to_f16_bits(v)) : static_cast<uint16_t>(split_bf16_bits(v, part == 1));
     }
     if (idx < p.nocf * 32) bias_out[idx] = (bias != nullptr && idx < p.Cout) ? to_float(bias[idx]) : 0.0f;
 }

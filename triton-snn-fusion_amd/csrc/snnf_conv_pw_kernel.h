@@ -141,7 +141,9 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
 
     // Loads of stage (step, chunk) of the tile at pixel px0 of image n. Every load is unconditional: items that lie
     // outside are redirected to the tile's first pixels (always valid) and zeroed on their way into LDS.
+    int pre_part = 0;       // fp32 tensors: which of the three parts of the channel axis `pre` holds (2: the low terms)
     auto issue_loads = [&](int step, int chunk, int n, int px0) __attribute__((always_inline)) {
+        if constexpr (LM == LOAD_2XF32) split_chunk(chunk, g.nchunks_r, pre_part, chunk);
         const char* __restrict__ base = static_cast<const char*>(kernarg_table_entry(0, step)) +
                                         (LM == LOAD_ROWBITS ? (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) >> 3
                                                             : (static_cast<int64_t>(n * g.Cin + chunk * g.CK) * P + px0) * ES);
@@ -219,8 +221,8 @@ __global__ __launch_bounds__(kConvThreads, 2) __attribute__((amdgpu_waves_per_eu
                             e0[j] = pre[s][j][0];
                             e1[j] = pre[s][j][1];
                         } else {
-                            e0[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][0]));
-                            e1[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][1]));
+                            e0[j] = split_bf16_bits(__uint_as_float(pre[s][j][0]), pre_part == 2);
+                            e1[j] = split_bf16_bits(__uint_as_float(pre[s][j][1]), pre_part == 2);
                         }
                     }
 #pragma unroll

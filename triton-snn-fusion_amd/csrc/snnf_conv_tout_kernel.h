@@ -120,7 +120,9 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
         }
     };
 
+    int pre_part = 0;       // fp32 tensors: which of the three parts of the channel axis `pre` holds (2: the low terms)
     auto issue_loads = [&](int step, int chunk) __attribute__((always_inline)) {
+        if constexpr (LM == LOAD_2XF32) split_chunk(chunk, g.nchunks_r, pre_part, chunk);
         const char* __restrict__ base = static_cast<const char*>(step_pointer(xs, step)) + static_cast<int64_t>(chunk) * g.CK * plane * ES;
 #pragma unroll
         for (int s = 0; s < SS; ++s) {
@@ -166,8 +168,8 @@ __global__ __launch_bounds__(kConvThreads, 2) void conv_lif_tout_kernel(const St
                             e0[j] = pre[s][j][0];
                             e1[j] = pre[s][j][1];
                         } else {
-                            e0[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][0]));
-                            e1[j] = float_to_bf16_bits(__uint_as_float(pre[s][j][1]));
+                            e0[j] = split_bf16_bits(__uint_as_float(pre[s][j][0]), pre_part == 2);
+                            e1[j] = split_bf16_bits(__uint_as_float(pre[s][j][1]), pre_part == 2);
                         }
                     }
 #pragma unroll

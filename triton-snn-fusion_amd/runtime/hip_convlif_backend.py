@@ -214,6 +214,9 @@ def _check_compute_dtype(compute_dtype, dtype: torch.dtype) -> None:
 def kernel_dtype_diagnostics(dtype: torch.dtype) -> Dict:
     """Counterpart of kernels/benchmark_conv_lif_temporal_general.py:264-293 for the HIP kernels."""
     operand = "float16" if dtype == torch.float16 else "bfloat16"
+    if dtype == torch.float32:
+        # fp32 tensors: value = hi + lo with both terms bf16; w_hi x_hi + w_lo x_hi + w_hi x_lo accumulated in fp32
+        operand = "bfloat16 hi + lo terms (3 products per fp32 product)"
     return {
         "compute_dtype": _compute_dtype_name(dtype),
         "matrix_operand_dtype": operand,
