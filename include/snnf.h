@@ -178,7 +178,9 @@ int snnf_lif_pool_linear_static(const void* const* xs, int T, int N, int C, int 
  * called by runtime/triton_temporal_linear_lif_backend.py:185-274.
  *   xs[t] : [M, Fin] x_dtype (row stride `x_row_stride` elements)   weight : [Fout, Fin] w_dtype   bias : [Fout] w_dtype or NULL
  *   spikes : [T, M, Fout] x_dtype (timestep stride `spike_step_stride` elements)   v_out : [M, Fout] v_dtype
- * fp32 operands are rounded to bf16 for the matrix cores (fp32 accumulate); fp16 operands use the fp16 matrix path.
+ * fp32 operands enter the matrix cores as two bf16 terms each (three of the four products, fp32 accumulate: about 16 mantissa
+ * bits; the reference multiplies fp32 tensors in TF32, kernels/generated_temporal_linear_lif_kernel.py:142,155-158); fp16
+ * operands use the fp16 matrix path.
  */
 int snnf_linear_lif(const void* const* xs, int T, int M, int Fin, int64_t x_row_stride, int x_dtype,
                     const void* weight, const void* bias, int Fout, int w_dtype,

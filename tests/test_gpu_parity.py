@@ -189,9 +189,9 @@ def _linear_case(seed, T, M, Fin, Fout, dtype, bias=True, p=0.1):
     x = spikes((T, M, Fin), p, g)
     w = torch.randn(Fout, Fin, generator=g) * (2.0 / Fin) ** 0.5 * 3.0
     b = torch.randn(Fout, generator=g) * 0.01 if bias else None
-    wq = q(w, BF16 if dtype == F32 else dtype)        # fp32 operands are rounded to bf16 by the kernel
+    wq = q(w, dtype)        # fp32 operands stay fp32: the kernel multiplies them as two bf16 terms each
     bq = None if b is None else q(b, dtype)
-    return x, w if dtype == F32 else wq, b if dtype == F32 else bq, wq, bq if b is not None else None
+    return x, wq, bq, wq, bq if b is not None else None
 
 
 @pytest.mark.parametrize("dtype,vdtype", [(BF16, F32), (F32, F32), (F16, F16), (BF16, BF16)])

@@ -146,8 +146,9 @@ def test_random_linear_scan_and_tail_cases(hip_ops, seed, cases):
             Fin = rnd.choice([8, 16, 37, 64, 100, 128, 200, 256, 264, 512, 1000, 2048, 4096, 4104])
             Fout = rnd.choice([1, 8, 16, 37, 48, 64, 100, 130, 256, 1000, 1024])
             bias = rnd.random() < 0.8
-            x = spikes((T, M, Fin), 0.1, g)
-            w = q(torch.randn(Fout, Fin, generator=g) * (2.0 / Fin) ** 0.5 * 3.0, op_dt)
+            analog = rnd.random() < 0.2
+            x = q(torch.randn(T, M, Fin, generator=g) * 0.3, dtype) if analog else spikes((T, M, Fin), 0.1, g)
+            w = q(torch.randn(Fout, Fin, generator=g) * (2.0 / Fin) ** 0.5 * 3.0, dtype)      # fp32 stays fp32: two bf16 terms on the matrix cores
             b = None if not bias else (torch.randn(Fout, generator=g) * 0.01 if dtype == F32 else q(torch.randn(Fout, generator=g) * 0.01, dtype))
             v_ref, v_dev = _membrane(rnd, g, (M, Fout), vdtype)
             what = f"case {case}: linear T={T} M={M} {Fin}->{Fout} bias={bias} {dtype} membrane {vdtype} lif={lif}"

@@ -22,11 +22,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kTileOC = 16;   // output features per workgroup
 constexpr int kTileM = 16;    // rows per workgroup (per timestep)
 
+// fp32 tensors: both operands enter the matrix cores as two bf16 terms (value rounded to bf16, and the rounded remainder),
+// and three of the four products are accumulated: w_hi x_hi + w_lo x_hi + w_hi x_lo (the fourth is below 2^-16 of the
+// result). The three products are three passes over K ("K parts"): part 0 multiplies the high terms, part 1 the weights' low
+// terms with the activations' high terms, part 2 the other way round. 16-bit tensors have one part.
 struct LinGeom {
     int T, M, Fin, Fout;
     int64_t x_row_stride;      // elements
     int64_t spike_step_stride; // elements
     int ksteps;                // ceil(Fin / 32)
+    int kparts;                // 1, or 3 for fp32 tensors
 };
 
 // Eight consecutive K elements of one row as a matrix-core operand (bf16 for fp32/bf16 storage, fp16 for fp16 storage).
@@ -35,15 +40,16 @@ template <> struct Frag<bf16_t> { using type = bf16x8; };
 template <> struct Frag<float> { using type = bf16x8; };
 template <> struct Frag<f16_t> { using type = f16x8; };
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+// Two fp32 values as a pair of bf16 terms: their roundings to bf16, or (low_term) what those roundings left over.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi, bool low_term) {
+    return split_bf16_bits(lo, low_term) | (split_bf16_bits(hi, low_term) << 16);
 }
 
 // Loads k .. k+7 of `row`; elements at or beyond `kmax` read as zero. FAST requires 16-byte aligned rows and kmax % 8 == 0
 // and is branch-free (an octet beyond kmax re-reads the row's first one and is zeroed): a branch around a load would make
 // the compiler wait for every load before it issues the next.
 template <typename XT, bool FAST>
-__device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, int kmax) {
+__device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, int kmax, bool low_term = false) {
     u32x4 out = {0u, 0u, 0u, 0u};
     if constexpr (FAST) {
         const bool inside = k < kmax;
@@ -53,10 +59,10 @@ __device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, i
         } else {
             const f32x4 a = *reinterpret_cast<const f32x4*>(src);
             const f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
-            out[0] = pack_bf16x2(a[0], a[1]);
-            out[1] = pack_bf16x2(a[2], a[3]);
-            out[2] = pack_bf16x2(b[0], b[1]);
-            out[3] = pack_bf16x2(b[2], b[3]);
+            out[0] = pack_bf16x2(a[0], a[1], low_term);
+            out[1] = pack_bf16x2(a[2], a[3], low_term);
+            out[2] = pack_bf16x2(b[0], b[1], low_term);
+            out[3] = pack_bf16x2(b[2], b[3], low_term);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) out[j] = inside ? out[j] : 0u;
@@ -73,7 +79,7 @@ __device__ __forceinline__ u32x4 load_octet(const XT* __restrict__ row, int k, i
         for (int j = 0; j < 4; ++j) {
             const float lo = (k + 2 * j) < kmax ? to_float(row[k + 2 * j]) : 0.0f;
             const float hi = (k + 2 * j + 1) < kmax ? to_float(row[k + 2 * j + 1]) : 0.0f;
-            out[j] = pack_bf16x2(lo, hi);
+            out[j] = pack_bf16x2(lo, hi, low_term);
         }
     }
     return out;
@@ -96,15 +102,15 @@ __device__ __forceinline__ RawOctet<XT> load_raw_octet(const XT* __restrict__ sr
     return r;
 }
 template <typename XT>
-__device__ __forceinline__ u32x4 finish_octet(const RawOctet<XT>& r, bool inside) {
+__device__ __forceinline__ u32x4 finish_octet(const RawOctet<XT>& r, bool inside, bool low_term) {
     u32x4 out;
     if constexpr (sizeof(XT) == 2) {
         out = r.lo;
     } else {
-        out[0] = pack_bf16x2(r.lo[0], r.lo[1]);
-        out[1] = pack_bf16x2(r.lo[2], r.lo[3]);
-        out[2] = pack_bf16x2(r.hi[0], r.hi[1]);
-        out[3] = pack_bf16x2(r.hi[2], r.hi[3]);
+        out[0] = pack_bf16x2(r.lo[0], r.lo[1], low_term);
+        out[1] = pack_bf16x2(r.lo[2], r.lo[3], low_term);
+        out[2] = pack_bf16x2(r.hi[0], r.hi[1], low_term);
+        out[3] = pack_bf16x2(r.hi[2], r.hi[3], low_term);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) out[j] = inside ? out[j] : 0u;
@@ -164,11 +170,16 @@ __global__ __launch_bounds__(LinWaves<TT>::value * 64) void linear_lif_kernel(St
     // matrix instruction; the other wave of the SIMD covers the wait.
     u32x4 a0[OCF], a1[OCF], b0[TT], b1[TT];
     auto fetch = [&](int s, u32x4 (&a)[OCF], u32x4 (&b)[TT]) __attribute__((always_inline)) {
+        int part = 0;        // fp32 tensors: step s of K part `part` (see LinGeom)
+        if constexpr (sizeof(XT) == 4) {
+            part = s >= 2 * g.ksteps ? 2 : (s >= g.ksteps ? 1 : 0);
+            s -= part * g.ksteps;
+        }
         const int k = s * 32 + koff;
 #pragma unroll
-        for (int f = 0; f < OCF; ++f) a[f] = load_octet<XT, FAST>(wrow[f], k, g.Fin);
+        for (int f = 0; f < OCF; ++f) a[f] = load_octet<XT, FAST>(wrow[f], k, g.Fin, part == 1);
 #pragma unroll
-        for (int t = 0; t < TT; ++t) b[t] = load_octet<XT, FAST>(xrow[t], k, g.Fin);
+        for (int t = 0; t < TT; ++t) b[t] = load_octet<XT, FAST>(xrow[t], k, g.Fin, part == 2);
     };
     auto multiply = [&](const u32x4 (&a)[OCF], const u32x4 (&b)[TT]) __attribute__((always_inline)) {
 #pragma unroll
@@ -176,8 +187,9 @@ __global__ __launch_bounds__(LinWaves<TT>::value * 64) void linear_lif_kernel(St
 #pragma unroll
             for (int f = 0; f < OCF; ++f) acc[f][t] = mfma16<XT>(a[f], b[t], acc[f][t]);
     };
-    for (int s = 2 * wave; s < g.ksteps; s += 2 * NW) {
-        const bool second = s + 1 < g.ksteps;
+    const int all_steps = g.kparts * g.ksteps;
+    for (int s = 2 * wave; s < all_steps; s += 2 * NW) {
+        const bool second = s + 1 < all_steps;
         fetch(s, a0, b0);
         if (second) fetch(s + 1, a1, b1);
         multiply(a0, b0);
@@ -293,6 +305,7 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     const XT* item_row[SH::ITEMS];
     uint32_t item_dst[SH::ITEMS];
     bool item_live[SH::ITEMS];
+    bool item_is_w[SH::ITEMS];
 #pragma unroll
     for (int j = 0; j < SH::ITEMS; ++j) {
         const int row = tid / kSlabOctets + j * (NT / kSlabOctets);
@@ -309,6 +322,7 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
             ptr = W + static_cast<int64_t>(min(oc0 + r - TT * kTileM, g.Fout - 1)) * g.Fin;
         }
         item_row[j] = ptr;
+        item_is_w[j] = r >= TT * kTileM;
         item_dst[j] = static_cast<uint32_t>(r * kSlabPitch + octet * 16);
     }
 
@@ -329,13 +343,22 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     constexpr int RING = SH::RING;
     RawOctet<XT> pre[RING][SH::ITEMS];
     bool pre_inside[RING];
-    // K split over workgroups: workgroup z of a tile takes slabs [z * slabs_per_part, ...) (all of them without a split).
+    int pre_part[RING];       // fp32 tensors: the K part a slab belongs to (see LinGeom)
+    // K split over workgroups: workgroup z of a tile takes slabs [z * slabs_per_part, ...) (all of them without a split). The
+    // slabs of an fp32 tensor's three K parts follow each other: slab s is slab s % unit of part s / unit.
     const int slab0 = static_cast<int>(blockIdx.z) * slabs_per_part;
-    const int kend = min(g.Fin, (slab0 + slabs_per_part) * SLABK);      // this part's K range ends here: beyond it, zeros
+    const int unit = (g.Fin + SLABK - 1) / SLABK;                        // slabs of one pass over K
+    const int slab_end = min(g.kparts * unit, slab0 + slabs_per_part);   // this workgroup's slabs end here: beyond it, zeros
     const int rounds = (slabs_per_part + RING - 1) / RING;
     auto fetch = [&](int slab, int r) __attribute__((always_inline)) {
-        const int k = slab * SLABK + octet * 8;
-        pre_inside[r] = k < kend;
+        int part = 0, real = slab;
+        if constexpr (sizeof(XT) == 4) {
+            part = slab >= 2 * unit ? 2 : (slab >= unit ? 1 : 0);
+            real = slab - part * unit;
+        }
+        pre_part[r] = part;
+        const int k = real * SLABK + octet * 8;
+        pre_inside[r] = slab < slab_end && k < g.Fin;
         const int ks = pre_inside[r] ? k : 0;
 #pragma unroll
         for (int j = 0; j < SH::ITEMS; ++j) pre[r][j] = load_raw_octet<XT>(item_row[j] + ks);   // items beyond the rows re-read row 0
@@ -354,7 +377,8 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
             unsigned char* buf = staged_lds + (DB ? (r & 1) * SH::slab_bytes : 0);      // RING is even
 #pragma unroll
             for (int j = 0; j < SH::ITEMS; ++j)
-                if (item_live[j]) *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r]);
+                if (item_live[j])
+                    *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r], pre_part[r] == (item_is_w[j] ? 1 : 2));
             __syncthreads();
             fetch(slab + RING, r);
             // This wave's K steps of the slab (every KSPLIT-th), four at a time: their operand reads go out together.
@@ -504,7 +528,7 @@ int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, 
                   void* v_out, const LifParams& lif, hipStream_t stream) {
     dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
     if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
-    const int unit_slabs = (g.Fin + kSlabK - 1) / kSlabK;
+    const int unit_slabs = g.kparts * ((g.Fin + kSlabK - 1) / kSlabK);        // all K parts of an fp32 tensor
     const int64_t tiles = static_cast<int64_t>(grid.x) * grid.y;
     const size_t part_bytes = static_cast<size_t>(TT) * OCF * kTileOC * kTileM * sizeof(float);
     int parts = ws.base != nullptr ? linear_split_parts(tiles, unit_slabs, part_bytes, ws.bytes) : 1;
@@ -640,6 +664,7 @@ static int linear_lif_impl(const char* who, const void* const* xs, int T, int M,
         g.x_row_stride = x_row_stride;
         g.spike_step_stride = spike_step_stride;
         g.ksteps = (Fin + 31) / 32;
+        g.kparts = x_dtype == SNNF_F32 ? 3 : 1;
         const void* vi = t0 == 0 ? v_init : v_out;
         void* sp = static_cast<char*>(spikes) + static_cast<int64_t>(t0) * spike_step_stride * xsize;
         int rc;
