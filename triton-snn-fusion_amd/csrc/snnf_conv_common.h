@@ -18,7 +18,7 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kEpiPitch = 68;       // floats per channel row of the epilogue stage (64 pixels + padding)
 constexpr size_t kToutStageBytes = 4 * 64 * 12 * sizeof(float);   // time-outer kernel: four waves x 64 pixels x (8 rows + padding)
 constexpr size_t kPwStageBytes = 4 * 8 * 68 * sizeof(float);      // pointwise kernel: four waves x 8 channel rows x (64 pixels + padding)
-constexpr size_t kMmBiasBytes = 512 * sizeof(float);                  // matrix kernel: the workgroup's bias values (at most 8 waves x 64 channels)
+constexpr size_t kMmBiasBytes = 512 * sizeof(float) + 16;             // matrix kernel: the workgroup's bias values (at most 8 waves x 64 channels) + one flag word
 constexpr size_t kMmStageBytesPerWave = 16 * 40 * sizeof(float);  // matrix kernel, per wave: 16 channel rows x (32 pixels + padding)
 constexpr size_t kEpiBytes = 4 * 4 * 8 * kEpiPitch * sizeof(float);  // four waves x (up to 4 steps x 8 channel rows)
 

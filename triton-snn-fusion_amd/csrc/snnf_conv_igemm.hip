@@ -146,14 +146,14 @@ bool plan_mm_uncached(const ConvGeom& g0, int tt, int load_mode, int vec, int nw
                 const int NRT = ti * NR;                           // stacked halo rows
                 const int img_groups = (g0.N + ti - 1) / ti;
                 // An LDS stage holds as many packed channel chunks as fit (fewer barriers and exposed load latencies per tile).
-                // (The three parts of an fp32 tensor's channel axis are staged differently: a stage must lie inside one part.)
-                const bool parts = g0.nchunks != g0.nchunks_r;
+                // fp32 tensors: a stage holds real chunks, each pixel's channels twice (high and low bf16 terms side by side).
+                const int row_mult = g0.nchunks != g0.nchunks_r ? 2 : 1;
                 int sc = 1;
-                while (sc * 2 <= g0.nchunks_r && (!parts || g0.nchunks_r % (sc * 2) == 0) && sc * 2 * g0.CK <= 256 &&
-                       static_cast<size_t>(tt) * NRT * WT * (sc * 2 * g0.CK * 2 + 16) + stage_bytes <= lds_cap &&
+                while (sc * 2 <= g0.nchunks_r && sc * 2 * g0.CK * row_mult <= 256 &&
+                       static_cast<size_t>(tt) * NRT * WT * (sc * 2 * g0.CK * 2 * row_mult + 16) + stage_bytes <= lds_cap &&
                        sc * 2 * groups * NRT * (WT / 2) <= max_items)
                     sc *= 2;
-                const int pitch = sc * g0.CK * 2 + 16;
+                const int pitch = sc * g0.CK * 2 * row_mult + 16;
                 size_t tiles_bytes = static_cast<size_t>(tt) * NRT * WT * pitch;
                 const size_t partial_bytes = static_cast<size_t>(nw) * 8 * 1024;        // the split-K partial sums of one timestep
                 if (wk_log2 > 0 && tiles_bytes < partial_bytes) tiles_bytes = partial_bytes;

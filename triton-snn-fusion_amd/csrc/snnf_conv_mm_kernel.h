@@ -63,7 +63,12 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 
     const int groups = 1 << g.groups_log2;                   // channel groups of 8 per packed chunk
     const int stage_groups = groups * g.stage_chunks;        // ... per LDS stage (a stage holds stage_chunks chunks)
-    const int nstages = (g.nchunks + g.stage_chunks - 1) / g.stage_chunks;
+    // fp32 tensors (see kSplitParts): a stage holds stage_chunks REAL channel chunks, fetched once and written to LDS as their
+    // high and their low bf16 terms side by side ([hi: stage channels][lo: stage channels] per pixel); the matrix steps of a
+    // stage then run the three parts of the packed weight against them (w_hi on hi, w_lo on hi, w_hi on lo).
+    constexpr int PARTS = LM == LOAD_2XF32 ? kSplitParts : 1;
+    const int nstages = (g.nchunks_r + g.stage_chunks - 1) / g.stage_chunks;
+    const int lo_off = g.stage_chunks * g.CK * 2;            // bytes from a pixel's high terms to its low terms
     const int WTP = g.WT >> 1;
     const int rows_all = g.TI * g.NR;                        // halo rows of the TI images of a tile, stacked
     const int tile_px = g.TH * g.TW;                         // output pixels per image and tile
@@ -72,6 +77,9 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
     // The workgroup's bias values (its 64 x WN output channels) are fetched with the first loads of a tile and parked in LDS
     // until the epilogue, which would otherwise wait for them from memory group by group.
     float* __restrict__ bias_lds = reinterpret_cast<float*>(lds + g.mm_stage_off) + NW * kMmStageFloats;
+    // fp32 tensors: set by any thread that stages a non-zero low term (activations that are exact in bf16, spikes above all,
+    // have none: the third part of the matrix steps is then skipped for the stage). One word behind the bias values.
+    volatile int& stage_has_low_terms = *reinterpret_cast<volatile int*>(bias_lds + 512);
     float bias_pre = 0.0f;
     auto fetch_bias = [&](int oc_t) __attribute__((always_inline)) {
         const int oc = (oc_t << g.wn_log2) * 64 + tid;
@@ -114,11 +122,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 
     // Loads of stage `stg` (stage_chunks channel chunks) of the tile whose halo starts at input (row ih_lo, column iw_lo)
     // of image n.
-    int pre_part = 0;       // fp32 tensors: which of the three parts of the channel axis `pre` holds (2: the low terms)
     auto issue_loads = [&](int stg, int n, int ih_lo, int iw_lo) __attribute__((always_inline)) {
-        int chunk = stg * g.stage_chunks;                                                        // first chunk of the stage
-        // fp32 tensors: a stage lies inside one part (the planner picks stage_chunks that divide the real chunk count).
-        if constexpr (LM == LOAD_2XF32) split_chunk(chunk, g.nchunks_r, pre_part, chunk);
+        const int chunk = stg * g.stage_chunks;                                                  // first (real) chunk of the stage
         const int64_t origin = (static_cast<int64_t>(n) * g.Cin + chunk * g.CK) * plane;     // elements, always inside the tensor
         const int tile_rel = ih_lo * g.W + iw_lo;                                               // may be negative
         uint32_t off0[SS], off1[SS];
@@ -187,7 +192,24 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int t = 0; t < TT; ++t) {
                     cv_u32x4 lo, hi;
-                    if constexpr (LM == LOAD_PAIR32) {
+                    if constexpr (LM == LOAD_2XF32) {
+                        // fp32: the high terms to the item's place, the low terms lo_off bytes behind them.
+                        cv_u32x4 lo2, hi2;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const float a0 = __uint_as_float(pre[s][t][2 * k][0]), a1 = __uint_as_float(pre[s][t][2 * k + 1][0]);
+                            const float b0 = __uint_as_float(pre[s][t][2 * k][1]), b1 = __uint_as_float(pre[s][t][2 * k + 1][1]);
+                            lo[k] = split_bf16_bits(a0, false) | (split_bf16_bits(a1, false) << 16);
+                            hi[k] = split_bf16_bits(b0, false) | (split_bf16_bits(b1, false) << 16);
+                            lo2[k] = zero0 ? 0u : (split_bf16_bits(a0, true) | (split_bf16_bits(a1, true) << 16));
+                            hi2[k] = zero1 ? 0u : (split_bf16_bits(b0, true) | (split_bf16_bits(b1, true) << 16));
+                        }
+                        unsigned char* dst2 = lds + t * tile_bytes + item_dst[s] + lo_off;
+                        *reinterpret_cast<cv_u32x4*>(dst2) = lo2;
+                        *reinterpret_cast<cv_u32x4*>(dst2 + g.pitch) = hi2;
+                        // (a low term is +0 or -0 when the value is exact in bf16: the sign bits do not count)
+                        if (((lo2[0] | lo2[1] | lo2[2] | lo2[3] | hi2[0] | hi2[1] | hi2[2] | hi2[3]) & 0x7fff7fffu) != 0u) stage_has_low_terms = 1;
+                    } else if constexpr (LM == LOAD_PAIR32) {
                         // An item whose first column is real and whose second is not is a row's last column: its first
                         // column sits in the upper halves.
                         const uint32_t first = (!zero0 && zero1) ? 0x07060302u : 0x05040100u;
@@ -200,13 +222,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
                         uint32_t e0[8], e1[8];
 #pragma unroll
                         for (int j = 0; j < 8; ++j) {
-                            if constexpr (LM == LOAD_2X16) {
-                                e0[j] = pre[s][t][j][0];
-                                e1[j] = pre[s][t][j][1];
-                            } else {
-                                e0[j] = split_bf16_bits(__uint_as_float(pre[s][t][j][0]), pre_part == 2);
-                                e1[j] = split_bf16_bits(__uint_as_float(pre[s][t][j][1]), pre_part == 2);
-                            }
+                            e0[j] = pre[s][t][j][0];
+                            e1[j] = pre[s][t][j][1];
                         }
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
@@ -322,9 +339,16 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
 
         int next_work = work, next_oc_tile = oc_tile, next_img = img, next_oh0 = oh0, next_ow0 = ow0;
         bool next_tile = false;
+        int stage_now = 0;       // the LDS stage the matrix steps are working on
         // One pair of k-slots: slot 2 * pair + half -> (tap, channel group); both halves' LDS offsets are computed on the
         // scalar unit, a lane picks its half's.
         auto mma_pair = [&](int q, const unsigned char* __restrict__ bp0, const cv_u32x4& a0, const cv_u32x4& a1) __attribute__((always_inline)) {
+            if constexpr (PARTS > 1) {   // q counts the stage's pairs three times over: part 2 reads the low terms
+                const int sp = min(g.stage_chunks, g.nchunks_r - stage_now * g.stage_chunks) * g.npairs;
+                const int part = q >= 2 * sp ? 2 : (q >= sp ? 1 : 0);
+                q -= part * sp;
+                bp0 += part == 2 ? lo_off : 0;
+            }
             const int sub = fast_div(q, g.d_npairs);                 // chunk inside the stage
             const int pair = q - sub * g.npairs;
             const unsigned char* __restrict__ bp = bp0 + sub * (groups * 16);
@@ -343,21 +367,38 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) __attribute__((amdgpu_waves_per_eu
             }
         };
         // Weight fragments stream from L2 two pairs ahead of their use, through three register sets.
+        // `gpair`: first pair of the stage + the pair's index in the stage (fp32: the index runs over the three parts, each
+        // of which lies nchunks_r chunks further in the packed weight).
         auto load_frags = [&](int gpair, cv_u32x4& a0, cv_u32x4& a1) __attribute__((always_inline)) {
+            if constexpr (PARTS > 1) {
+                const int first = stage_now * g.stage_chunks * g.npairs;
+                const int sp = min(g.stage_chunks, g.nchunks_r - stage_now * g.stage_chunks) * g.npairs;
+                const int q = gpair - first;
+                const int part = q >= 2 * sp ? 2 : (q >= sp ? 1 : 0);
+                gpair += part * (g.nchunks_r * g.npairs - sp);
+            }
             const int64_t o = static_cast<int64_t>(min(gpair, total_pairs - 1)) * (kFragBytes / 2);
             a0 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off0 + o);
             a1 = *reinterpret_cast<const cv_u32x4*>(wlane + w_off1 + o);
         };
         cv_u32x4 wa[3][2];
         for (int chunk = 0; chunk < nstages; ++chunk) {        // `chunk` counts LDS stages from here on
+            stage_now = chunk;
             const int gp0 = chunk * g.stage_chunks * g.npairs;
-            const int spairs = min(g.stage_chunks, g.nchunks - chunk * g.stage_chunks) * g.npairs;   // pairs of this stage
+            const int spairs_all = PARTS * min(g.stage_chunks, g.nchunks_r - chunk * g.stage_chunks) * g.npairs;   // pairs of this stage (all parts)
             load_frags(gp0 + wk, wa[0][0], wa[0][1]);  // in flight across the barriers and the LDS writes below
             load_frags(gp0 + wk + WK, wa[1][0], wa[1][1]);
+            if constexpr (PARTS > 1) {
+                if (tid == 0) stage_has_low_terms = 0;     // every wave has read the previous stage's flag before it got here
+            }
             __syncthreads();   // every wave is done reading the previous stage (and with the previous tile's epilogue)
             write_lds();       // waits for the stage's loads
             if (chunk == 0 && tid < (64 << g.wn_log2)) bias_lds[tid] = bias_pre;
             __syncthreads();
+            int spairs = spairs_all;
+            if constexpr (PARTS > 1) {
+                if (__builtin_amdgcn_readfirstlane(static_cast<int>(stage_has_low_terms)) == 0) spairs = (spairs_all / PARTS) * 2;
+            }
             // ---- the stage after this one: next chunk, or the first chunk of the next tile.
             {
                 int nc = chunk + 1, nimg = img, nih = ih_lo, niw = iw_lo;
