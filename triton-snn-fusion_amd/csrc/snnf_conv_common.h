@@ -68,6 +68,10 @@ __host__ __device__ inline size_t packed_weight_elems(const PackGeom& p) {
     return static_cast<size_t>(p.nocf) * p.nchunks * p.npairs * (kFragBytes / 2);
 }
 
+// fp32 bias values behind the packed weight: zero beyond Cout, padded to whole tiles of 64 channels and followed by 64 more
+// zeros (kernels read a tile's bias, or "no bias", without a bounds check).
+__host__ __device__ inline size_t packed_bias_floats(const PackGeom& p) { return static_cast<size_t>((p.nocf + 1) / 2) * 64 + 64; }
+
 // How activations are fetched from global memory while staging: two adjacent pixels of one channel per fetch.
 enum LoadMode : int {
     LOAD_PAIR32 = 0,   // 16-bit activations, pixel pairs 4-byte aligned: one dword load

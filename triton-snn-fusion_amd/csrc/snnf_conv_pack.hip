@@ -1,4 +1,6 @@
 // Repacks an OIHW convolution weight (+ bias) into the fragment order the implicit-GEMM kernel reads.
+#include <algorithm>
+
 #include "snnf_conv_common.h"
 
 namespace snnf {
@@ -30,7 +32,7 @@ __global__ void pack_weight_kernel(const WT* __restrict__ w, const WT* __restric
             v = to_float(w[(static_cast<int64_t>(oc) * p.Cin + ci) * (p.KH * p.KW) + tap]);
         packed[idx] = TO_F16 ? static_cast<uint16_t>(float_to_f16_bits(v)) : static_cast<uint16_t>(split_bf16_bits(v, part == 1));
     }
-    if (idx < p.nocf * 32) bias_out[idx] = (bias != nullptr && idx < p.Cout) ? to_float(bias[idx]) : 0.0f;
+    if (idx < static_cast<int64_t>(packed_bias_floats(p))) bias_out[idx] = (bias != nullptr && idx < p.Cout) ? to_float(bias[idx]) : 0.0f;
 }
 
 }  // namespace
@@ -40,7 +42,7 @@ extern "C" size_t snnf_conv_packed_weight_bytes(int Cout, int Cin, int KH, int K
     using namespace snnf;
     if (Cout < 1 || Cin < 1 || KH < 1 || KW < 1 || !valid_dtype(x_dtype)) return 0;
     const PackGeom p = make_pack_geom(Cout, Cin, KH, KW, x_dtype == SNNF_F32);
-    return packed_weight_elems(p) * 2 + static_cast<size_t>(p.nocf) * 32 * sizeof(float);
+    return packed_weight_elems(p) * 2 + packed_bias_floats(p) * sizeof(float);
 }
 
 extern "C" int snnf_conv_pack_weight(const void* weight, const void* bias, int w_dtype, int Cout, int Cin, int KH, int KW,
@@ -59,7 +61,7 @@ extern "C" int snnf_conv_pack_weight(const void* weight, const void* bias, int w
     const int64_t total = static_cast<int64_t>(packed_weight_elems(p));
     uint16_t* out = static_cast<uint16_t*>(packed);
     float* bias_out = reinterpret_cast<float*>(out + total);
-    const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+    const unsigned blocks = static_cast<unsigned>((std::max<int64_t>(total, static_cast<int64_t>(packed_bias_floats(p))) + 255) / 256);
     hipStream_t hs = as_stream(stream);
     const bool to_f16 = x_dtype == SNNF_F16;
 #define SNNF_PACK(WT)                                                                                                   \

@@ -11,7 +11,7 @@
 namespace snnf {
 namespace {
 
-constexpr int kWaveLds = (static_cast<int>(kMaxLds) - static_cast<int>(kSpkTableBytes)) / kSpkWaves / 16 * 16;   // private staging bytes of a wave
+constexpr int kWaveLds = (static_cast<int>(kMaxLds) - static_cast<int>(kSpkHeaderBytes)) / kSpkWaves / 16 * 16;   // private staging bytes of a wave
 
 struct SpkPlan {
     int PR, PC, PI, RR, RC, region, G, patches_x, patches_y, img_groups;
@@ -34,11 +34,11 @@ bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best, int only_pc = 0, int onl
         const int region = pi * rr * rc;
         int G = 0;
         if (g0.tap_pairs) {
-            if (region <= 64 * kSpkSlots && tt * region * 16 <= kWaveLds) G = 1;
+            if (region <= 64 * kSpkSlots && tt * (region + 1) * 16 <= kWaveLds) G = 1;
         } else {
             for (int cand = g0.gpc; cand >= 2; cand >>= 1) {
                 if (only_g > 0 && cand > only_g) continue;
-                if (cand * region <= 64 * kSpkSlots && tt * cand * region * 16 <= kWaveLds) {
+                if (cand * region <= 64 * kSpkSlots && tt * (cand * region + 1) * 16 <= kWaveLds) {   // + the dummy item of a timestep
                     G = cand;
                     break;
                 }
@@ -190,7 +190,7 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     g.nstages = (g.C8in + g.G - 1) / g.G;
     g.IT = g.G * g.region;
     g.JT = (g.IT + 63) / 64;
-    g.lds_wave_bytes = tt * g.IT * 16;
+    g.lds_wave_bytes = tt * (g.IT + 1) * 16;
     const int oc_tiles = (Cout + 63) / 64;
     g.n_items = g.n_patches * oc_tiles;
     // Split K over waves of a workgroup while the layer has fewer items than the machine has SIMDs (one wave each) and
@@ -212,7 +212,7 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     // Workgroups that are resident together: one per compute unit, or two where a wave needs at most a quarter of a SIMD's
     // registers (one timestep's accumulators) and two staging areas fit the LDS. The tiles are dealt evenly over as many
     // rounds as that takes.
-    const size_t lds_bytes = std::max(kSpkTableBytes + static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes, wk_log2 > 0 ? kSpkTableBytes + kSpkPartialBytes : size_t{0});
+    const size_t lds_bytes = std::max(kSpkHeaderBytes + static_cast<size_t>(kSpkWaves) * g.lds_wave_bytes, wk_log2 > 0 ? kSpkHeaderBytes + kSpkPartialBytes : size_t{0});
     const int resident = cus * ((tt == 1 && 2 * (lds_bytes + 1024) <= kMaxLds) ? 2 : 1);
     const int blocks = (g.n_items + tiles_per_block - 1) / tiles_per_block;
     g.iters = (blocks + resident - 1) / resident;

@@ -36,6 +36,9 @@ constexpr int kSpkSlots = SPK_SLOTS;                      // staging items per l
 constexpr size_t kSpkPartialBytes = kSpkWaves * 16 * 64 * 16;  // split-K: every wave parks 4 quads x up to 4 timesteps of partial sums per round
 constexpr int kSpkMaxSteps = 60;                  // matrix steps per stage, at most (the step table holds 4 more)
 constexpr size_t kSpkTableBytes = (kSpkMaxSteps + 4) * 16;      // the workgroup's step table at the start of LDS
+constexpr int kSpkDescs = 64 * kSpkSlots;                       // staging items of one timestep, at most
+constexpr size_t kSpkDescBytes = kSpkDescs * 8;                 // the workgroup's staging descriptors behind the step table
+constexpr size_t kSpkHeaderBytes = kSpkTableBytes + kSpkDescBytes;   // what precedes the waves' staging regions in LDS
 
 struct SpkGeom {
     int N, Cin, H, W, Cout, KH, KW, sh, sw, ph, pw, Ho, Wo;
@@ -160,9 +163,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const int lane = tid & 63;
     const int half = lane >> 5;
     const int l32 = lane & 31;
-    unsigned char* const wlds = lds + kSpkTableBytes + wave * g.lds_wave_bytes;
+    unsigned char* const wlds = lds + kSpkHeaderBytes + wave * g.lds_wave_bytes;
     const int region16 = g.region * 16;        // bytes of one channel group of the halo
-    const int tile_t = g.G * region16;         // bytes of one timestep's stage
+    const int tile_t = g.G * region16 + 16;    // bytes of one timestep's stage: its items and one dummy item that absorbs the writes of idle staging slots
 
     // ---- this lane's output pixel inside the patch, and where its top-left input sits in the staged halo.
     const int ppx = g.PR * g.PC;
@@ -209,8 +212,30 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             e[3] = 0u;
             table[tid] = e;
         }
+        // ---- staging descriptors of the workgroup: item e of a timestep's stage = (channel group gq, image ii, halo row r, halo
+        // column c); its element offset from the stage's first item and the four coordinates, packed. Built once; the staging
+        // of every stage of every tile reads them back instead of dividing (three divisions per item otherwise). Items beyond
+        // the stage carry channel group 255, which no stage has.
+        Pack<uint32_t, 2>* __restrict__ desc_w = reinterpret_cast<Pack<uint32_t, 2>*>(lds + kSpkTableBytes);
+        for (int e = tid; e < kSpkDescs; e += kSpkWaves * 64) {
+            Pack<uint32_t, 2> d;
+            d.v[0] = 0u;
+            d.v[1] = 0xff000000u;
+            if (e < g.IT) {
+                const int gq = sk_div(e, g.d_region);
+                const int rem = e - gq * g.region;
+                const int ii = sk_div(rem, g.d_rrrc);
+                const int rem2 = rem - ii * (g.RR * g.RC);
+                const int r = sk_div(rem2, g.d_RC);
+                const int c = rem2 - r * g.RC;
+                d.v[0] = static_cast<uint32_t>(((ii * g.C8in + gq) * g.H + r) * g.W + c);
+                d.v[1] = static_cast<uint32_t>(r) | (static_cast<uint32_t>(c) << 8) | (static_cast<uint32_t>(ii) << 16) | (static_cast<uint32_t>(gq) << 24);
+            }
+            desc_w[e] = d;
+        }
         __syncthreads();
     }
+    const Pack<uint32_t, 2>* __restrict__ desc = reinterpret_cast<const Pack<uint32_t, 2>*>(lds + kSpkTableBytes);
     const sk_u32x4* __restrict__ table = reinterpret_cast<const sk_u32x4*>(lds);
 
     // Workgroups are handed to the eight XCDs in turn (workgroup b runs on XCD b % 8) and every XCD has an L2 of its own.
@@ -274,27 +299,21 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             constexpr bool PRE = FAST && IN == SNNF_LAYOUT_BITS;
             uint32_t pre_raw[TT][4];
             uint32_t pre_ok = 0;
-            // Decodes the 4 items of batch jb of stage s: their global index (0 when they are padding) and the two flag nibbles
-            // (bit j: real data; bit 4 + j: the item exists and is written).
+            // Decodes the 4 items of batch jb of stage s from the workgroup's descriptors: their global index (0 when they are
+            // padding) and a flag nibble (bit j: real data).
             auto batch_decode = [&](int s, int jb, int lane_s, int (&idx)[4]) __attribute__((always_inline)) -> uint32_t {
                 const int gg0 = s * g.G;
                 const int base_u = ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
                 uint32_t ok_bits = 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int e = (jb + j) * 64 + lane_s;
-                    const int gq = sk_div(e, g.d_region);
-                    const int rem = e - gq * g.region;
-                    const int ii = sk_div(rem, g.d_rrrc);
-                    const int rem2 = rem - ii * (g.RR * g.RC);
-                    const int r = sk_div(rem2, g.d_RC);
-                    const int c = rem2 - r * g.RC;
-                    const int ih = ih_lo + r, iw = iw_lo + c;
-                    const bool exists = e < g.IT;
-                    const bool ok = exists && n0 + ii < g.N && gg0 + gq < g.C8in && static_cast<unsigned>(ih) < static_cast<unsigned>(g.H) &&
-                                    static_cast<unsigned>(iw) < static_cast<unsigned>(g.W);
-                    idx[j] = ok ? base_u + ((ii * g.C8in + gq) * g.H + r) * g.W + c : 0;
-                    ok_bits |= (ok ? (1u << j) : 0u) | (exists ? (16u << j) : 0u);
+                    const Pack<uint32_t, 2> d = desc[(jb + j) * 64 + lane_s];
+                    const int r = static_cast<int>(d.v[1] & 255u), c = static_cast<int>((d.v[1] >> 8) & 255u);
+                    const int ii = static_cast<int>((d.v[1] >> 16) & 255u), gq = static_cast<int>(d.v[1] >> 24);
+                    const bool ok = n0 + ii < g.N && gg0 + gq < g.C8in && static_cast<unsigned>(ih_lo + r) < static_cast<unsigned>(g.H) &&
+                                    static_cast<unsigned>(iw_lo + c) < static_cast<unsigned>(g.W);
+                    idx[j] = ok ? base_u + static_cast<int>(d.v[0]) : 0;
+                    ok_bits |= ok ? (1u << j) : 0u;
                 }
                 return ok_bits;
             };
@@ -313,7 +332,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const sk_u32x4 d = sk_expand_bits<ONE>(((ok_bits >> j) & 1u) ? raw[t][j] : 0u);
-                        if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
+                        // every slot writes: an item beyond the stage goes to the timestep's dummy item
+                        *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + min((jb + j) * 64 + lane_s, g.IT) * 16) = d;
                     }
             };
             // Requests the first batch of stage s (PRE only).
@@ -360,7 +380,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                                     sk_u32x4 d;
 #pragma unroll
                                     for (int k = 0; k < 4; ++k) d[k] = ((ok_bits >> j) & 1u) ? raw[j][k] : 0u;
-                                    if ((ok_bits >> (4 + j)) & 1u) *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + ((jb + j) * 64 + lane_s) * 16) = d;
+                                    *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + min((jb + j) * 64 + lane_s, g.IT) * 16) = d;
                                 }
                             }
                         }
@@ -824,7 +844,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then), four
                 // quads per round for all TT timesteps; quad 4 r + e of round r is finished by wave (4 r + e) mod WK of the tile,
                 // which adds the WK partial sums in a fixed order and then runs that quad's timesteps like the unsplit kernel.
-                float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkTableBytes);      // [wave][e 0..3][tw][lane][4]
+                float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkHeaderBytes);      // [wave][e 0..3][tw][lane][4]
                 for (int r = 0; r < 2; ++r) {
                     __syncthreads();   // the previous round's sums are consumed (first round: every wave is done with its staging region)
 #define SNNF_SPK_PARK_QUAD(E, F)                                                                                                 \
