@@ -259,7 +259,9 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     L.lds_bytes = lds_bytes;
     L.stream = as_stream(stream);
     const bool fast_epi = neuron && out_layout == SNNF_LAYOUT_BITS && (residuals == nullptr || res_layout == SNNF_LAYOUT_BITS) &&
-                          L.lif.charge_mode == CHARGE_SCALE && !L.lif.soft_reset && v_init == nullptr && windows == 1 && Cout % 8 == 0;
+                          L.lif.charge_mode == CHARGE_SCALE && L.lif.inv_tau == 0.5f && L.lif.v_reset == 0.0f &&
+                          L.lif.v_threshold >= 1e-30f && L.lif.v_threshold <= 1e30f &&   // its multiples by 2^t stay normal numbers
+                          v_init == nullptr && windows == 1 && Cout % 8 == 0;
     snprintf(snnf::conv_plan_buffer(), 256,
              "kernel=blocked variant=%d window=%d launches=1 tile=%dx%dx%d halo=%dx%d waves=8x1x%d oc_tiles=%d px_tiles=%d "
              "stage_chunks=%d run=0 lds=%zu grid=%d tuned=%d",

@@ -85,8 +85,8 @@ struct SpkLaunch {
     int grid;
     size_t lds_bytes;
     hipStream_t stream;
-    bool fast_epilogue;   // the straight-line epilogue applies: bit-packed output, no or a bit-packed residual, the common neuron,
-                          // zero initial membrane, one window, whole channel groups
+    bool fast_epilogue;   // the straight-line epilogue applies: bit-packed output, no or a bit-packed residual, the usual neuron
+                          // (tau 2, hard reset to 0), zero initial membrane, one window, whole channel groups
 };
 
 template <bool F16>
@@ -185,6 +185,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const int hg = g.tap_pairs ? 1 : (g.G >> 1);        // k-slot pairs per tap and stage
     const int nst = g.tap_pairs ? g.npairs : g.taps * hg;   // matrix steps per stage
     const bool common_lif = lif.charge_mode == CHARGE_SCALE && !lif.soft_reset;
+    const bool half_tau = lif.inv_tau == 0.5f;
 
     // ---- step table of the workgroup: for step i of a stage, the byte offset of its weight fragments from the stage's
     // first pair and the LDS offset of its activations for the lower / upper half of a wave (tap and channel group of
@@ -588,7 +589,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     if (common_lif) {   // power-of-two tau, hard reset: one test per quad step instead of two per neuron step
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
-                            const float h = v[k] + (x[k] - v[k]) * lif.inv_tau;
+                            // tau = 2: (v + x) / 2, one rounding, the form the straight-line epilogue computes.
+                            const float h = half_tau ? (v[k] + x[k]) * 0.5f : v[k] + (x[k] - v[k]) * lif.inv_tau;
                             const bool fired = h >= lif.v_threshold;
                             v[k] = fired ? lif.v_reset : h;
                             nib |= fired ? (1u << k) : 0u;
@@ -622,9 +624,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // other half of the wave holds the other nibble of every byte (lanes l and l + 32 own the same pixel); even
             // steps are stored by the lower half, odd steps by the upper half.
             auto quad_store_bits = [&](int ta0, int cnt, int j8, uint32_t nibw) __attribute__((always_inline)) {
-                const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(nibw), 32));
-                const uint32_t lo = half ? other : nibw;
-                const uint32_t hi = half ? nibw : other;
+                const auto both = __builtin_amdgcn_permlane32_swap(nibw, nibw, false, false);   // [0]: lanes 0..31's word, [1]: lanes 32..63's
+                const uint32_t lo = both[0];
+                const uint32_t hi = both[1];
                 if (j8 < g.C8out && px_ok) {
                     unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
 #pragma unroll
@@ -637,21 +639,6 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     }
                 }
             };
-            // The same for exactly four steps 0..3 (the usual window), without a condition per step: the lower half stores
-            // steps 0 and 2, the upper half steps 1 and 3.
-            auto quad_store_bits4 = [&](int j8, uint32_t nibw) __attribute__((always_inline)) {
-                const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(nibw), 32));
-                const uint32_t lo = half ? other : nibw;
-                const uint32_t hi = half ? nibw : other;
-                if (j8 < g.C8out && px_ok) {
-                    unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
-                    const uint32_t first = lane_bits + (half ? static_cast<uint32_t>(g.out_step_stride) : 0u);
-                    const uint32_t sh = 4u * static_cast<uint32_t>(half);
-                    ob[first] = static_cast<unsigned char>(((lo >> sh) & 15u) | (((hi >> sh) & 15u) << 4));
-                    ob[first + 2u * static_cast<uint32_t>(g.out_step_stride)] =
-                        static_cast<unsigned char>(((lo >> (sh + 8u)) & 15u) | (((hi >> (sh + 8u)) & 15u) << 4));
-                }
-            };
             auto quad_end = [&](int j8, const float (&v)[4], uint32_t chm) __attribute__((always_inline)) {
                 if (v_out != nullptr && !g.analog_out && px_ok) {
                     float* __restrict__ vp = v_out + static_cast<int64_t>(j8) * 8 * po;
@@ -661,21 +648,32 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 }
             };
 
-            // FAST: the layer as it runs inside a network - bit-packed output, no or a bit-packed residual, the common neuron
-            // (power-of-two tau, hard reset), zero initial membrane, one window, whole channel groups. Straight-line code.
-            // One LIF step of 4 neurons: sums x (+ the residual bits of this half of the byte), returns the spike nibble.
-            auto fast_lif4 = [&](const float (&x)[4], uint32_t res_half, bool with_res, float (&v)[4]) __attribute__((always_inline)) -> uint32_t {
-                uint32_t nib = 0;
+            // FAST: the layer as it runs inside a network - bit-packed output, no or a bit-packed residual, the usual neuron
+            // (tau = 2, hard reset to 0, a threshold whose power-of-two multiples are normal numbers), zero initial membrane,
+            // one window, whole channel groups. Straight-line code.
+            // The membrane is kept scaled, S_t = 2^t v_t: a step is then S += 2^(t-1) x (every scaling is exact, so S_t / 2^t
+            // is bit for bit the (v + x) / 2 of the general path), a comparison against 2^t v_th and a select, and the carry of
+            // the comparison is shifted into the quad's word of quiet (not fired) bits: four instructions per neuron step.
+            // After n steps the word holds step i's nibble at bits [4 (n - 1 - i), +4), bit k of a nibble = neuron k.
+            auto fast_step4 = [&](const float (&x)[4], int t, float (&S)[4], uint32_t& quiet) __attribute__((always_inline)) {
+                const float c = __uint_as_float(static_cast<uint32_t>(127 + t) << 23);                                   // 2^t
+                const float th2 = __uint_as_float(__float_as_uint(lif.v_threshold) + (static_cast<uint32_t>(t + 1) << 23));   // 2^(t+1) v_th
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    float xx = x[k];
-                    if (with_res) xx += __uint_as_float(static_cast<uint32_t>(static_cast<int32_t>(res_half << (31 - k)) >> 31) & 0x3f800000u);
-                    const float h = v[k] + (xx - v[k]) * lif.inv_tau;
-                    const bool fired = h >= lif.v_threshold;
-                    v[k] = fired ? lif.v_reset : h;
-                    nib |= fired ? (1u << k) : 0u;
-                }
-                return nib;
+                for (int k = 3; k >= 0; --k)
+                    asm("v_fmac_f32 %0, %2, %3\n\t"
+                        "v_cmp_nle_f32 vcc, %4, %0\n\t"
+                        "v_cndmask_b32 %0, 0, %0, vcc\n\t"
+                        "v_addc_co_u32 %1, vcc, %1, %1, vcc"
+                        : "+v"(S[k]), "+v"(quiet)
+                        : "s"(c), "v"(x[k]), "s"(th2)
+                        : "vcc");
+            };
+            // x += the residual spikes of this half of the byte (bit k of the nibble -> 0.0 / 1.0 through one byte each).
+            auto fast_add_res = [&](uint32_t res_byte, float (&x)[4]) __attribute__((always_inline)) {
+                const uint32_t nib = (res_byte >> (4 * half)) & 15u;
+                const uint32_t spread = __umul24(nib, 0x00204081u) & 0x01010101u;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) x[k] += static_cast<float>((spread >> (8 * k)) & 0xffu);
             };
             // Residual byte of channel group j8 at timestep ta for this lane's pixel (this half's nibble is picked at the use,
             // so that nothing waits on the load where it is issued). Lanes without a pixel read pixel 0 of image 0 (their
@@ -684,57 +682,101 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const unsigned char* __restrict__ res_t = static_cast<const unsigned char*>(sk_kernarg_ptr(kResTable, ta));
                 return (res_t + static_cast<int64_t>(min(j8, g.C8out - 1)) * po)[lane_bits];
             };
+            // Bit-packed store of the n <= 8 steps [ta0, ta0 + n) of a quad from its word of quiet bits. Lanes l and l + 32 own
+            // the two nibbles of every byte of a pixel and swap their words in registers; even steps are stored by the lower
+            // half of the wave, odd steps by the upper half.
+            auto fast_store = [&](int ta0, int n, int j8, uint32_t quiet) __attribute__((always_inline)) {
+                const uint32_t fired = ~quiet;
+                const auto both = __builtin_amdgcn_permlane32_swap(fired, fired, false, false);   // [0]: lanes 0..31's word, [1]: lanes 32..63's
+                if (j8 < g.C8out && px_ok) {
+                    unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) {
+                        const int i = 2 * m + half;
+                        if (i < n) {
+                            const uint32_t sh = 4u * static_cast<uint32_t>(n - 1 - i);
+                            const uint32_t byte = ((both[0] >> sh) & 15u) | (((both[1] >> sh) & 15u) << 4);
+                            ob[static_cast<uint32_t>(ta0 + i) * static_cast<uint32_t>(g.out_step_stride) + lane_bits] = static_cast<unsigned char>(byte);
+                        }
+                    }
+                }
+            };
+            // The same for exactly the four steps 0..3 (the usual window), without a condition per step: the lower half
+            // stores steps 0 and 2, the upper half steps 1 and 3.
+            auto fast_store4 = [&](int j8, uint32_t quiet) __attribute__((always_inline)) {
+                const uint32_t fired = ~quiet;
+                const auto both = __builtin_amdgcn_permlane32_swap(fired, fired, false, false);
+                if (j8 < g.C8out && px_ok) {
+                    unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
+                    const uint32_t first = lane_bits + (half ? static_cast<uint32_t>(g.out_step_stride) : 0u);
+                    const uint32_t sh = half ? 8u : 12u;
+                    ob[first] = static_cast<unsigned char>(((both[0] >> sh) & 15u) | (((both[1] >> sh) & 15u) << 4));
+                    ob[first + 2u * static_cast<uint32_t>(g.out_step_stride)] =
+                        static_cast<unsigned char>(((both[0] >> (sh - 8u)) & 15u) | (((both[1] >> (sh - 8u)) & 15u) << 4));
+                }
+            };
             // All steps of one quad whose sums are xq[tw][k]: residual, LIF, bit-packed store, optional membrane store.
             auto fast_quad = [&](int j8, const float (&xq)[TT][4], const uint32_t (&rb)[TT], bool with_res) __attribute__((always_inline)) {
-                float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                float S[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                 if constexpr (TT == 1) {
                     if (t_count == 4 && !with_res) {
                         // The usual stem: one frame, four steps, no residual. Straight-line.
-                        uint32_t nibw = 0;
+                        uint32_t quiet = 0;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) nibw |= fast_lif4(xq[0], 0u, false, v) << (4 * i);
-                        quad_store_bits4(j8, nibw);
+                        for (int i = 0; i < 4; ++i) fast_step4(xq[0], i, S, quiet);
+                        fast_store4(j8, quiet);
                     } else {
                         for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
                             const int cnt = min(8, t_count - ta0);
-                            uint32_t nibw = 0;
+                            uint32_t quiet = 0;
                             for (int i = 0; i < cnt; ++i) {
-                                const uint32_t r = with_res ? fast_res(ta0 + i, j8) >> (4 * half) : 0u;
-                                nibw |= fast_lif4(xq[0], r, with_res, v) << (4 * i);
+                                float x[4];
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) x[k] = xq[0][k];
+                                if (with_res) fast_add_res(fast_res(ta0 + i, j8), x);
+                                fast_step4(x, ta0 + i, S, quiet);
                             }
-                            quad_store_bits(ta0, cnt, j8, nibw);
+                            fast_store(ta0, cnt, j8, quiet);
                         }
                     }
                 } else {
-                    uint32_t nibw = 0;
+                    uint32_t quiet = 0;
                     if (t_count == TT) {
                         // Every step of the window is real (the usual case): no condition per step.
                         if (with_res) {
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
+                            for (int tw = 0; tw < TT; ++tw) {
+                                float x[4];
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) x[k] = xq[tw][k];
+                                fast_add_res(rb[tw], x);
+                                fast_step4(x, tw, S, quiet);
+                            }
                         } else {
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                            for (int tw = 0; tw < TT; ++tw) fast_step4(xq[tw], tw, S, quiet);
                         }
-                        if constexpr (TT == 4) quad_store_bits4(j8, nibw);
-                        else quad_store_bits(0, TT, j8, nibw);
+                        if constexpr (TT == 4) fast_store4(j8, quiet);
+                        else fast_store(0, TT, j8, quiet);
                     } else {
-                        if (with_res) {
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw)
-                                if (tw < t_count) nibw |= fast_lif4(xq[tw], rb[tw] >> (4 * half), true, v) << (4 * tw);
-                        } else {
+                        for (int tw = 0; tw < TT; ++tw) {
+                            if (tw < t_count) {
+                                float x[4];
 #pragma unroll
-                            for (int tw = 0; tw < TT; ++tw)
-                                if (tw < t_count) nibw |= fast_lif4(xq[tw], 0u, false, v) << (4 * tw);
+                                for (int k = 0; k < 4; ++k) x[k] = xq[tw][k];
+                                if (with_res) fast_add_res(rb[tw], x);
+                                fast_step4(x, tw, S, quiet);
+                            }
                         }
-                        quad_store_bits(0, t_count, j8, nibw);
+                        fast_store(0, t_count, j8, quiet);
                     }
                 }
                 if (v_out != nullptr && px_ok && j8 < g.C8out) {
                     float* __restrict__ vp = v_out + static_cast<int64_t>(j8) * 8 * po;
+                    const float unscale = __uint_as_float(static_cast<uint32_t>(127 - t_count) << 23);   // 2^-t_count
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) vp[lane_nchw + static_cast<uint32_t>(k * po)] = v[k];
+                    for (int k = 0; k < 4; ++k) vp[lane_nchw + static_cast<uint32_t>(k * po)] = S[k] * unscale;
                 }
             };
             // All steps of one quad, any layouts and neuron (the general path).
