@@ -188,8 +188,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const bool half_tau = lif.inv_tau == 0.5f;
 
     // ---- step table of the workgroup: for step i of a stage, the byte offset of its weight fragments from the stage's
-    // first pair and the LDS offset of its activations for the lower / upper half of a wave (tap and channel group of
-    // the half's k-slot). The matrix loop then needs no index arithmetic. Steps beyond the last repeat it (prefetch only).
+    // first pair and the LDS offset of its activations (tap and channel group of the half's k-slot), once for the lower and
+    // once for the upper half of a wave: a lane reads the 8 bytes of its half. The matrix loop then needs no index
+    // arithmetic. Steps beyond the last repeat it (prefetch only).
     {
         sk_u32x4* __restrict__ table = reinterpret_cast<sk_u32x4*>(lds);
         if (tid < nst + 4) {
@@ -200,7 +201,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const int kh0 = tap0 / g.KW, kh1 = tap1 / g.KW;
                 e[0] = static_cast<uint32_t>(i * kFragBytes);
                 e[1] = static_cast<uint32_t>((kh0 * g.RC + (tap0 - kh0 * g.KW)) * 16);
-                e[2] = static_cast<uint32_t>((kh1 * g.RC + (tap1 - kh1 * g.KW)) * 16);
+                e[3] = static_cast<uint32_t>((kh1 * g.RC + (tap1 - kh1 * g.KW)) * 16);
             } else {
                 const int tap = i >> g.hg_log2;
                 const int gp = i & (hg - 1);
@@ -208,9 +209,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const int tapoff = (kh * g.RC + (tap - kh * g.KW)) * 16;
                 e[0] = static_cast<uint32_t>((tap * g.pair_tap_stride + gp) * kFragBytes);
                 e[1] = static_cast<uint32_t>(tapoff + (2 * gp) * region16);
-                e[2] = static_cast<uint32_t>(tapoff + (2 * gp + 1) * region16);
+                e[3] = static_cast<uint32_t>(tapoff + (2 * gp + 1) * region16);
             }
-            e[3] = 0u;
+            e[2] = e[0];
             table[tid] = e;
         }
         // ---- staging descriptors of the workgroup: item e of a timestep's stage = (channel group gq, image ii, halo row r, halo
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         __syncthreads();
     }
     const Pack<uint32_t, 2>* __restrict__ desc = reinterpret_cast<const Pack<uint32_t, 2>*>(lds + kSpkTableBytes);
-    const sk_u32x4* __restrict__ table = reinterpret_cast<const sk_u32x4*>(lds);
+    const Pack<uint32_t, 2>* __restrict__ table = reinterpret_cast<const Pack<uint32_t, 2>*>(lds + 8 * half);   // entry i of this half: table[2 * i]
 
     // Workgroups are handed to the eight XCDs in turn (workgroup b runs on XCD b % 8) and every XCD has an L2 of its own.
     // Items are ordered output-channel tile first, so the workgroups of one XCD take a contiguous range of them: an XCD then
@@ -432,11 +433,11 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     sk_u32x4 wb[2][TT];
                     uint32_t bo[4];
                     // Requests the weight fragments of the step described by table entry `e` and notes where its activations are.
-                    auto req_a = [&](int slot, const sk_u32x4& e) __attribute__((always_inline)) {
-                        const uint32_t voff = lane16 + e[0];
+                    auto req_a = [&](int slot, const Pack<uint32_t, 2>& e) __attribute__((always_inline)) {
+                        const uint32_t voff = lane16 + e.v[0];
                         wa[slot][0] = *reinterpret_cast<const sk_u32x4*>(pa0 + voff);
                         wa[slot][1] = *reinterpret_cast<const sk_u32x4*>(pa1 + voff);
-                        bo[slot] = half ? e[2] : e[1];
+                        bo[slot] = e.v[1];
                     };
                     auto read_b = [&](int slot, uint32_t boff) __attribute__((always_inline)) {
 #pragma unroll
@@ -450,9 +451,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         }
                     };
                     req_a(0, table[0]);
-                    req_a(1, table[1]);
-                    req_a(2, table[2]);
-                    sk_u32x4 ent = table[3];       // entry of the step whose weights are requested next
+                    req_a(1, table[2]);
+                    req_a(2, table[4]);
+                    Pack<uint32_t, 2> ent = table[6];       // entry of the step whose weights are requested next
                     stage_in(stage);
                     if constexpr (PRE) {
                         if (stage + s_step < g.nstages) stage_req(stage + s_step);
@@ -460,29 +461,58 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     read_b(0, bo[0]);
                     int st = 0;
                     // Four steps per trip, no branch inside: weights three steps ahead (4 register sets), activations one step
-                    // ahead (2 sets). The scheduling fences keep each step's operand requests ahead of the previous step's
-                    // matrix instructions; left alone the compiler sinks them below, where their latency is exposed.
+                    // ahead (2 sets). A wave issues in order and a matrix instruction occupies the matrix pipe for 32 cycles: the
+                    // requests of the coming steps are therefore spread between the matrix instructions of the current one (each
+                    // gap takes a few of them for free) instead of standing in a block in front of them, where the matrix pipe
+                    // would run dry while they issue.
+                    auto step_order = [&]() __attribute__((always_inline)) {
+                        constexpr int kMfma = 0x008, kValu = 0x002, kVmemRead = 0x020, kDsRead = 0x100;
+                        __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kVmemRead, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                        if constexpr (TT >= 2) {
+                            __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                        }
+                        if constexpr (TT >= 4) {
+                            __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kValu, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(kMfma, 2, 0);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    };
                     for (; st + 4 <= nst; st += 4) {
                         req_a(3, ent);
-                        ent = table[st + 4];
+                        ent = table[2 * (st + 4)];
                         read_b(1, bo[1]);
-                        __builtin_amdgcn_sched_barrier(0);
                         mma(0, 0);
+                        step_order();
                         req_a(0, ent);
-                        ent = table[st + 5];
+                        ent = table[2 * (st + 5)];
                         read_b(0, bo[2]);
-                        __builtin_amdgcn_sched_barrier(0);
                         mma(1, 1);
+                        step_order();
                         req_a(1, ent);
-                        ent = table[st + 6];
+                        ent = table[2 * (st + 6)];
                         read_b(1, bo[3]);
-                        __builtin_amdgcn_sched_barrier(0);
                         mma(2, 0);
+                        step_order();
                         req_a(2, ent);
-                        ent = table[st + 7];
+                        ent = table[2 * (st + 7)];
                         read_b(0, bo[0]);
-                        __builtin_amdgcn_sched_barrier(0);
                         mma(3, 1);
+                        step_order();
                     }
                     // The last nst % 4 steps: wa[0..2] hold their weight fragments, wb[0] the first one's activations.
                     if (st < nst) {
@@ -915,13 +945,34 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     for (int e_own = e_first; e_own < 4; e_own += WK) {
                         const int j8 = oc_e * 8 + 4 * r + e_own;
                         float xq[TT][4];
+                        {
+                            // The partial sums of the tile's waves, all timesteps of a wave (of two waves) in flight together (WK is a power
+                            // of two >= 2); added in the order of the waves.
+                            sk_f32x4 sum[TT];
 #pragma unroll
-                        for (int tw = 0; tw < TT; ++tw) {
-                            sk_f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-                            for (int k = 0; k < WK; ++k)
-                                sum += *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 4 + e_own) * TT + tw) * 64 + lane) * 4);
+                            for (int tw = 0; tw < TT; ++tw) sum[tw] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                            if constexpr (FAST) {
+                                for (int k = 0; k < WK; k += 2) {
+                                    sk_f32x4 p0[TT], p1[TT];
 #pragma unroll
-                            for (int k = 0; k < 4; ++k) xq[tw][k] = sum[k];
+                                    for (int tw = 0; tw < TT; ++tw) {
+                                        p0[tw] = *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 4 + e_own) * TT + tw) * 64 + lane) * 4);
+                                        p1[tw] = *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k + 1) * 4 + e_own) * TT + tw) * 64 + lane) * 4);
+                                    }
+#pragma unroll
+                                    for (int tw = 0; tw < TT; ++tw) sum[tw] = (sum[tw] + p0[tw]) + p1[tw];
+                                }
+                            } else {   // the general epilogue has no registers to spare: one wave's sums at a time
+                                for (int k = 0; k < WK; ++k) {
+#pragma unroll
+                                    for (int tw = 0; tw < TT; ++tw)
+                                        sum[tw] += *reinterpret_cast<const sk_f32x4*>(part + ((((tile_in_block * WK + k) * 4 + e_own) * TT + tw) * 64 + lane) * 4);
+                                }
+                            }
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw)
+#pragma unroll
+                                for (int k = 0; k < 4; ++k) xq[tw][k] = sum[tw][k];
                         }
                         if constexpr (FAST) {
                             if (e_own != e_first && g.res_layout >= 0 && TT > 1) {
