@@ -38,7 +38,8 @@ constexpr int kSpkMaxSteps = 60;                  // matrix steps per stage, at 
 constexpr size_t kSpkTableBytes = (kSpkMaxSteps + 4) * 16;      // the workgroup's step table at the start of LDS
 constexpr int kSpkDescs = 64 * kSpkSlots;                       // staging items of one timestep, at most
 constexpr size_t kSpkDescBytes = kSpkDescs * 8;                 // the workgroup's staging descriptors behind the step table
-constexpr size_t kSpkHeaderBytes = kSpkTableBytes + kSpkDescBytes;   // what precedes the waves' staging regions in LDS
+constexpr size_t kSpkPosBytes = 32 * 4;            // where each of the 32 pixels of a tile sits inside the patch
+constexpr size_t kSpkHeaderBytes = kSpkTableBytes + kSpkDescBytes + kSpkPosBytes;   // what precedes the waves' staging regions in LDS
 
 struct SpkGeom {
     int N, Cin, H, W, Cout, KH, KW, sh, sw, ph, pw, Ho, Wo;
@@ -167,15 +168,6 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     const int region16 = g.region * 16;        // bytes of one channel group of the halo
     const int tile_t = g.G * region16 + 16;    // bytes of one timestep's stage: its items and one dummy item that absorbs the writes of idle staging slots
 
-    // ---- this lane's output pixel inside the patch, and where its top-left input sits in the staged halo.
-    const int ppx = g.PR * g.PC;
-    const int pi = sk_div(l32, g.d_ppx);
-    const int prem = l32 - pi * ppx;
-    const int prow = sk_div(prem, g.d_PC);
-    const int pcol = prem - prow * g.PC;
-    const bool lane_in_patch = pi < g.PI;
-    const uint32_t lane_b = lane_in_patch ? static_cast<uint32_t>(((pi * g.RR + prow * g.sh) * g.RC + pcol * g.sw) * 16) : 0u;
-
     const int WK = SK ? (1 << g.wk_log2) : 1;
     const int wk = SK ? (wave & (WK - 1)) : 0;
     const int tile_in_block = SK ? (wave >> g.wk_log2) : wave;
@@ -235,6 +227,17 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             }
             desc_w[e] = d;
         }
+        // ---- where pixel p of a tile sits inside the patch: image, row and column, packed. Every item reads its lane's entry
+        // back: kept in registers these values would live (or be spilled) across the matrix loop of every variant.
+        if (tid < 32) {
+            const int ppx = g.PR * g.PC;
+            const int pi = sk_div(tid, g.d_ppx);
+            const int prem = tid - pi * ppx;
+            const int prow = sk_div(prem, g.d_PC);
+            const int pcol = prem - prow * g.PC;
+            reinterpret_cast<uint32_t*>(lds + kSpkTableBytes + kSpkDescBytes)[tid] =
+                static_cast<uint32_t>(pi) | (static_cast<uint32_t>(prow) << 8) | (static_cast<uint32_t>(pcol) << 16);
+        }
         __syncthreads();
     }
     const Pack<uint32_t, 2>* __restrict__ desc = reinterpret_cast<const Pack<uint32_t, 2>*>(lds + kSpkTableBytes);
@@ -262,9 +265,20 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         const int ih_lo = oh0 * g.sh - g.ph;
         const int iw_lo = ow0 * g.sw - g.pw;
 
+        // ---- this lane's output pixel inside the patch, and where its top-left input sits in the staged halo.
+        const uint32_t lane_pos = reinterpret_cast<const uint32_t*>(lds + kSpkTableBytes + kSpkDescBytes)[l32];
+        const int pi = static_cast<int>(lane_pos & 255u);
+        const int prow = static_cast<int>((lane_pos >> 8) & 255u);
+        const int pcol = static_cast<int>(lane_pos >> 16);
+        const bool lane_in_patch = pi < g.PI;
+        const uint32_t lane_b = lane_in_patch ? static_cast<uint32_t>(((pi * g.RR + prow * g.sh) * g.RC + pcol * g.sw) * 16) : 0u;
+
         const int ocf0 = oc_tile * 2;
-        const int64_t w_off0 = static_cast<int64_t>(min(ocf0, g.nocf - 1)) * g.frag_stride;
-        const int64_t w_off1 = static_cast<int64_t>(min(ocf0 + 1, g.nocf - 1)) * g.frag_stride;
+        // With K split over two waves the second one computes the tile's two 32-channel fragments in swapped places: each wave
+        // then finishes the fragment in its accumulators' first half (fragment wk) and hands over the second half.
+        const int swap_f = (SK && WK == 2) ? wk : 0;
+        const int64_t w_off0 = static_cast<int64_t>(min(ocf0 + swap_f, g.nocf - 1)) * g.frag_stride;
+        const int64_t w_off1 = static_cast<int64_t>(min(ocf0 + 1 - swap_f, g.nocf - 1)) * g.frag_stride;
 
         // ---- this lane's output pixel.
         const int n = n0 + pi;
@@ -537,15 +551,15 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             const int t_count = g.shared_x ? g.T : min(TT, g.T - t0);      // LIF steps of this window
             // (Made opaque here: everything derived from the lane's pixel offset is then computed after the matrix loop instead of
             // before it, where the compiler would otherwise park two dozen store addresses in registers or scratch memory.)
-            int pxo_e = pxo, n_e = n_c;
-            asm volatile("" : "+v"(pxo_e), "+v"(n_e));
-            const uint32_t lane_nchw = static_cast<uint32_t>((n_e * g.Cout + 4 * half) * po + pxo_e);        // elements
-            const uint32_t lane_c8 = static_cast<uint32_t>(((n_e * g.C8out) * po + pxo_e) * 8 + 4 * half);   // elements
+            int pxo_e = pxo, n_e = n_c, half_e = half;
+            asm volatile("" : "+v"(pxo_e), "+v"(n_e), "+v"(half_e));
+            const uint32_t lane_nchw = static_cast<uint32_t>((n_e * g.Cout + 4 * half_e) * po + pxo_e);        // elements
+            const uint32_t lane_c8 = static_cast<uint32_t>(((n_e * g.C8out) * po + pxo_e) * 8 + 4 * half_e);   // elements
             const uint32_t lane_bits = static_cast<uint32_t>((n_e * g.C8out) * po + pxo_e);                  // bytes
 
             // Valid-channel mask and initial membrane of the quad of channel group j8.
             auto quad_begin = [&](int j8, float (&v)[4], uint32_t& chm) __attribute__((always_inline)) {
-                const int ch0 = j8 * 8 + 4 * half;
+                const int ch0 = j8 * 8 + 4 * half_e;
                 chm = 0;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -573,7 +587,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     raw[1] = r2.v[1];
                 } else {
                     const uint16_t* __restrict__ rp = reinterpret_cast<const uint16_t*>(res_t) + static_cast<int64_t>(j8) * 8 * po;
-                    const int ch0 = j8 * 8 + 4 * half;
+                    const int ch0 = j8 * 8 + 4 * half_e;
                     uint32_t e[4];
 #pragma unroll
                     for (int k = 0; k < 4; ++k) e[k] = ch0 + k < g.Cout ? rp[lane_nchw + static_cast<uint32_t>(k * po)] : 0u;
@@ -585,7 +599,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 if (g.res_layout < 0) return;
                 if (g.res_layout == SNNF_LAYOUT_BITS) {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) x[k] += ((raw[0] >> (4 * half + k)) & 1u) ? 1.0f : 0.0f;
+                    for (int k = 0; k < 4; ++k) x[k] += ((raw[0] >> (4 * half_e + k)) & 1u) ? 1.0f : 0.0f;
                 } else {
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
@@ -661,7 +675,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
 #pragma unroll
                     for (int m = 0; m < 4; ++m) {
-                        const int i = 2 * m + half;
+                        const int i = 2 * m + half_e;
                         if (i < cnt) {
                             const uint32_t byte = ((lo >> (4 * i)) & 15u) | (((hi >> (4 * i)) & 15u) << 4);
                             ob[static_cast<uint32_t>(ta0 + i) * static_cast<uint32_t>(g.out_step_stride) + lane_bits] = static_cast<unsigned char>(byte);
@@ -700,7 +714,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             };
             // x += the residual spikes of this half of the byte (bit k of the nibble -> 0.0 / 1.0 through one byte each).
             auto fast_add_res = [&](uint32_t res_byte, float (&x)[4]) __attribute__((always_inline)) {
-                const uint32_t nib = (res_byte >> (4 * half)) & 15u;
+                const uint32_t nib = (res_byte >> (4 * half_e)) & 15u;
                 const uint32_t spread = __umul24(nib, 0x00204081u) & 0x01010101u;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) x[k] += static_cast<float>((spread >> (8 * k)) & 0xffu);
@@ -722,7 +736,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
 #pragma unroll
                     for (int m = 0; m < 4; ++m) {
-                        const int i = 2 * m + half;
+                        const int i = 2 * m + half_e;
                         if (i < n) {
                             const uint32_t sh = 4u * static_cast<uint32_t>(n - 1 - i);
                             const uint32_t byte = ((both[0] >> sh) & 15u) | (((both[1] >> sh) & 15u) << 4);
@@ -738,8 +752,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const auto both = __builtin_amdgcn_permlane32_swap(fired, fired, false, false);
                 if (j8 < g.C8out && px_ok) {
                     unsigned char* __restrict__ ob = out + static_cast<int64_t>(j8) * po;
-                    const uint32_t first = lane_bits + (half ? static_cast<uint32_t>(g.out_step_stride) : 0u);
-                    const uint32_t sh = half ? 8u : 12u;
+                    const uint32_t first = lane_bits + (half_e ? static_cast<uint32_t>(g.out_step_stride) : 0u);
+                    const uint32_t sh = half_e ? 8u : 12u;
                     ob[first] = static_cast<unsigned char>(((both[0] >> sh) & 15u) | (((both[1] >> sh) & 15u) << 4));
                     ob[first + 2u * static_cast<uint32_t>(g.out_step_stride)] =
                         static_cast<unsigned char>(((both[0] >> (sh - 8u)) & 15u) | (((both[1] >> (sh - 8u)) & 15u) << 4));
@@ -913,17 +927,69 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                     }
                 }
             } else {
-                // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then), four
-                // quads per round for all TT timesteps; quad 4 r + e of round r is finished by wave (4 r + e) mod WK of the tile,
-                // which adds the WK partial sums in a fixed order and then runs that quad's timesteps like the unsplit kernel.
+                // Split K: the WK waves of a tile add their partial sums through LDS (the staging regions are dead by then).
                 float* __restrict__ part = reinterpret_cast<float*>(lds + kSpkHeaderBytes);      // [wave][e 0..3][tw][lane][4]
-                for (int r = 0; r < 2; ++r) {
-                    __syncthreads();   // the previous round's sums are consumed (first round: every wave is done with its staging region)
 #define SNNF_SPK_PARK_QUAD(E, F)                                                                                                 \
     _Pragma("unroll") for (int tw = 0; tw < TT; ++tw) {                                                                          \
         const sk_f32x4 four = {acc[tw][F][4 * (E)], acc[tw][F][4 * (E) + 1], acc[tw][F][4 * (E) + 2], acc[tw][F][4 * (E) + 3]};  \
         *reinterpret_cast<sk_f32x4*>(part + (((wave * 4 + (E)) * TT + tw) * 64 + lane) * 4) = four;                             \
     }
+                if (WK == 2) {
+                    // Two waves per tile: wave wk finishes the four quads of fragment wk, which sit in the first half of its
+                    // accumulators (the second wave computes the fragments in swapped places). It hands its sums of the other
+                    // fragment to its partner and adds the partner's sums to its own, which never leave their registers: one exchange.
+                    __syncthreads();   // every wave is done with its staging region
+                    SNNF_SPK_PARK_QUAD(0, 1) SNNF_SPK_PARK_QUAD(1, 1) SNNF_SPK_PARK_QUAD(2, 1) SNNF_SPK_PARK_QUAD(3, 1)
+                    uint32_t rb[TT];
+#pragma unroll
+                    for (int tw = 0; tw < TT; ++tw) rb[tw] = 0u;
+                    if constexpr (FAST) {   // the residual bytes of the first quad travel while the workgroup meets
+                        if (g.res_layout >= 0 && TT > 1) {
+#pragma unroll
+                            for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), oc_e * 8 + 4 * wk);
+                        }
+                    }
+                    __syncthreads();
+                    const int partner = wave ^ 1;
+                    int lane_x = lane;                   // opaque: the addresses below are computed here, not ahead of the matrix loop
+                    asm volatile("" : "+v"(lane_x));
+                    for (int e = 0; e < 4; ++e) {
+                        const int j8 = oc_e * 8 + 4 * wk + e;
+                        sk_f32x4 theirs[TT];
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw)
+                            theirs[tw] = *reinterpret_cast<const sk_f32x4*>(part + (((partner * 4 + e) * TT + tw) * 64 + lane_x) * 4);
+                        float xq[TT][4];
+#define SNNF_SPK_COPY_QUAD(F, Q)                                          \
+    _Pragma("unroll") for (int tw = 0; tw < TT; ++tw)                     \
+        _Pragma("unroll") for (int k = 0; k < 4; ++k) xq[tw][k] = acc[tw][F][4 * (Q) + k]
+                        switch (e) {
+                            case 0: SNNF_SPK_COPY_QUAD(0, 0); break;
+                            case 1: SNNF_SPK_COPY_QUAD(0, 1); break;
+                            case 2: SNNF_SPK_COPY_QUAD(0, 2); break;
+                            default: SNNF_SPK_COPY_QUAD(0, 3); break;
+                        }
+#undef SNNF_SPK_COPY_QUAD
+#pragma unroll
+                        for (int tw = 0; tw < TT; ++tw)
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) xq[tw][k] += theirs[tw][k];   // a sum of two terms: the same in either order
+                        if constexpr (FAST) {
+                            if (e != 0 && g.res_layout >= 0 && TT > 1) {
+#pragma unroll
+                                for (int tw = 0; tw < TT; ++tw) rb[tw] = fast_res(min(tw, t_count - 1), j8);
+                            }
+                            fast_quad(j8, xq, rb, g.res_layout >= 0);
+                        } else {
+                            general_quad(j8, xq);
+                        }
+                    }
+                } else
+                // More waves per tile: four quads per round for all TT timesteps; quad 4 r + e of round r is finished by wave
+                // (4 r + e) mod WK of the tile, which adds the WK partial sums in a fixed order and then runs that quad's timesteps
+                // like the unsplit kernel.
+                for (int r = 0; r < 2; ++r) {
+                    __syncthreads();   // the previous round's sums are consumed (first round: every wave is done with its staging region)
                     if (r == 0) {
                         SNNF_SPK_PARK_QUAD(0, 0) SNNF_SPK_PARK_QUAD(1, 0) SNNF_SPK_PARK_QUAD(2, 0) SNNF_SPK_PARK_QUAD(3, 0)
                     } else {
