@@ -702,15 +702,29 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             auto fast_step4 = [&](const float (&x)[4], int t, float (&S)[4], uint32_t& quiet) __attribute__((always_inline)) {
                 const float c = __uint_as_float(static_cast<uint32_t>(127 + t) << 23);                                   // 2^t
                 const float th2 = __uint_as_float(__float_as_uint(lif.v_threshold) + (static_cast<uint32_t>(t + 1) << 23));   // 2^(t+1) v_th
-#pragma unroll
-                for (int k = 3; k >= 0; --k)
-                    asm("v_fmac_f32 %0, %2, %3\n\t"
-                        "v_cmp_nle_f32 vcc, %4, %0\n\t"
-                        "v_cndmask_b32 %0, 0, %0, vcc\n\t"
-                        "v_addc_co_u32 %1, vcc, %1, %1, vcc"
-                        : "+v"(S[k]), "+v"(quiet)
-                        : "s"(c), "v"(x[k]), "s"(th2)
-                        : "vcc");
+                // Neuron 3 first: the last bit shifted in (neuron 0) lands at the nibble's bit 0. The four comparisons write four
+                // mask registers and every instruction that reads a mask stands at least two instructions behind the one that
+                // wrote it (a vector instruction may not read a scalar register that the previous two vector instructions wrote).
+                uint64_t m0, m1, m2, m3;
+                asm("v_fmac_f32 %0, %9, %13\n\t"
+                    "v_fmac_f32 %1, %9, %12\n\t"
+                    "v_fmac_f32 %2, %9, %11\n\t"
+                    "v_fmac_f32 %3, %9, %10\n\t"
+                    "v_cmp_nle_f32_e64 %5, %14, %0\n\t"
+                    "v_cmp_nle_f32_e64 %6, %14, %1\n\t"
+                    "v_cmp_nle_f32_e64 %7, %14, %2\n\t"
+                    "v_cmp_nle_f32_e64 %8, %14, %3\n\t"
+                    "v_cndmask_b32_e64 %0, 0, %0, %5\n\t"
+                    "v_cndmask_b32_e64 %1, 0, %1, %6\n\t"
+                    "v_cndmask_b32_e64 %2, 0, %2, %7\n\t"
+                    "v_cndmask_b32_e64 %3, 0, %3, %8\n\t"
+                    "v_addc_co_u32_e64 %4, vcc, %4, %4, %5\n\t"
+                    "v_addc_co_u32_e64 %4, vcc, %4, %4, %6\n\t"
+                    "v_addc_co_u32_e64 %4, vcc, %4, %4, %7\n\t"
+                    "v_addc_co_u32_e64 %4, vcc, %4, %4, %8"
+                    : "+v"(S[3]), "+v"(S[2]), "+v"(S[1]), "+v"(S[0]), "+v"(quiet), "=&s"(m3), "=&s"(m2), "=&s"(m1), "=&s"(m0)
+                    : "s"(c), "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "s"(th2)
+                    : "vcc");
             };
             // x += the residual spikes of this half of the byte (bit k of the nibble -> 0.0 / 1.0 through one byte each).
             auto fast_add_res = [&](uint32_t res_byte, float (&x)[4]) __attribute__((always_inline)) {
