@@ -55,11 +55,16 @@ def test_argument_validation_happens_before_any_gpu_work(snnf_lib):
 
 
 def test_packed_weight_size_is_whole_fragments(snnf_lib):
-    # [ceil(Cout/32)][ceil(Cin/CK)][ceil(taps * CK/8 / 2)] fragments of 1 KiB + fp32 bias
-    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 1) == 2 * 2 * 18 * 1024 + 64 * 4
-    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 0) == 2 * 4 * 9 * 1024 + 64 * 4   # fp32 activations: 16-channel chunks
-    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 3, 7, 7, 1) == 2 * 1 * 25 * 1024 + 64 * 4
-    assert snnf_lib.snnf_conv_packed_weight_bytes(70, 40, 1, 1, 2) == 3 * 1 * 4 * 1024 + 96 * 4     # pointwise: one 64-channel chunk
+    # [ceil(Cout/32)][ceil(Cin/CK)][ceil(taps * CK/8 / 2)] fragments of 1 KiB + the fp32 bias, padded with zeros to whole
+    # 64-channel tiles plus one tile (the kernels load a tile's bias without a bounds check)
+    def bias_bytes(cout):
+        nocf = (cout + 31) // 32
+        return (((nocf + 1) // 2) * 64 + 64) * 4
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 1) == 2 * 2 * 18 * 1024 + bias_bytes(64)
+    # fp32 tensors: 16-channel chunks, and three parts of the channel axis (w_hi, w_lo, w_hi: two bf16 terms per operand)
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 64, 3, 3, 0) == 3 * 2 * 4 * 9 * 1024 + bias_bytes(64)
+    assert snnf_lib.snnf_conv_packed_weight_bytes(64, 3, 7, 7, 1) == 2 * 1 * 25 * 1024 + bias_bytes(64)
+    assert snnf_lib.snnf_conv_packed_weight_bytes(70, 40, 1, 1, 2) == 3 * 1 * 4 * 1024 + bias_bytes(70)     # pointwise: one 64-channel chunk
     assert snnf_lib.snnf_lif_pool_linear_workspace_bytes(16, 512) == 16 * 512 * 4
     assert snnf_lib.snnf_conv_packed_weight_bytes(0, 3, 3, 3, 1) == 0
 
@@ -331,3 +336,52 @@ def test_which_16_bit_membrane_calls_run_with_a_float32_working_membrane():
     assert CB._takes_several_launches("depthwise_k3_s1_p1", 17)
     assert CB._takes_several_launches("k3_s1_p1", 4)
     assert CB._takes_several_launches("k1_s1_p0", 2)
+
+
+def _reference_start_membrane(x, v_prev):
+    """The reference's rule for the membrane a step starts from (runtime/snn_custom_ops.py:378-381), restated: a `v_prev`
+    that is no tensor of the shape, device and dtype of `x` is replaced by zeros like `x`."""
+    if not isinstance(v_prev, torch.Tensor) or v_prev.shape != x.shape or v_prev.device != x.device or v_prev.dtype != x.dtype:
+        return torch.zeros_like(x)
+    return v_prev
+
+
+def test_float32_state_next_to_16_bit_activations_both_rules():
+    """Where this package departs from the reference, pinned side by side: a full-shape float32 `v_prev` next to 16-bit
+    activations restarts from zeros (16-bit membrane out) under the reference's rule and is carried in float32 here; every
+    other mismatch (0-dim placeholder, wrong shape, a third dtype) restarts from zeros under both rules (here in float32 when
+    `v_prev` is a float32 tensor on the activations' device), and a state of the activation dtype is carried under both."""
+    g = torch.Generator().manual_seed(5)
+    lif = (1.0, 0.0, 2.0)
+    x = (torch.randn(2, 3, 4, 4, generator=g) * 1.5).to(torch.bfloat16)
+    v32 = torch.randn(2, 3, 4, 4, generator=g) * 0.5
+    # the reference's rule on this input: the float32 state is dropped
+    v_ref = _reference_start_membrane(x, v32)
+    assert v_ref.dtype == torch.bfloat16 and not v_ref.any()
+    s_ref, m_ref = ops._lif_step_torch(x, v_ref, x.dtype, *lif, False)
+    # this package: carried, stepped and returned in float32
+    s_here, m_here = ops.lif_forward_state_torch(x, v32, *lif, False)
+    assert m_here.dtype == torch.float32 and s_here.dtype == torch.bfloat16
+    want_s, want_m = ops._lif_step_torch(x.float(), v32, x.dtype, *lif, False)
+    assert torch.equal(s_here, want_s) and torch.equal(m_here, want_m)
+    assert not torch.equal(m_here.to(torch.bfloat16), m_ref)          # the two rules give different states on this input
+    assert ops._lif_forward_state_meta(x.to("meta"), v32.to("meta"), *lif, False)[1].dtype == torch.float32
+    # mismatches that restart from zeros under both rules. The membrane dtype here follows the dtype and device of `v_prev`
+    # alone (float32 or the activations' dtype on the activations' device, else the activations' dtype), the reference's is
+    # always the activations': a 0-dim float32 zero or a float32 tensor of another shape gives the zero start in float32,
+    # a third dtype gives it in the activation dtype.
+    for v_other, want_dtype in ((torch.tensor(0.0), torch.float32), (torch.zeros(2, 3, 4, 5), torch.float32),
+                                (v32.to(torch.float16), torch.bfloat16), (v32.double(), torch.bfloat16),
+                                (torch.tensor(0.0, dtype=torch.bfloat16), torch.bfloat16)):
+        assert not _reference_start_membrane(x, v_other).any()
+        s_o, m_o = ops.lif_forward_state_torch(x, v_other, *lif, False)
+        want_s, want_m = ops._lif_step_torch(x.to(want_dtype), torch.zeros(x.shape, dtype=want_dtype), x.dtype, *lif, False)
+        assert m_o.dtype == want_dtype and torch.equal(s_o, want_s) and torch.equal(m_o, want_m)
+        if want_dtype == torch.bfloat16:
+            assert torch.equal(s_o, s_ref) and torch.equal(m_o, m_ref)      # exactly the reference's result
+    # a state of the activation dtype is carried under both rules
+    v16 = v32.to(torch.bfloat16)
+    assert _reference_start_membrane(x, v16) is v16
+    s_c, m_c = ops.lif_forward_state_torch(x, v16, *lif, False)
+    want_s, want_m = ops._lif_step_torch(x, v16, x.dtype, *lif, False)
+    assert m_c.dtype == torch.bfloat16 and torch.equal(s_c, want_s) and torch.equal(m_c, want_m)
