@@ -146,8 +146,14 @@ int snnf_pwconv_lif_rowbits(const void* const* xs_bits, int T, int N, int Cin, i
  *   out_sum : [N, K] x_dtype         v_out : [N, C, H, W] v_dtype
  *   workspace : at least snnf_lif_pool_linear_workspace_bytes(N, C) bytes of device memory, 16-byte aligned;
  *               it holds per-(n, c) spike counts between the two launches and needs no initialisation.
+ * Tails as small as those at the end of a network (T * C * H * W of one sample at most 32 Ki, C % 8 == 0 and at most 2048,
+ * C * H * W % 8 == 0, 16-byte aligned operands) run as ONE launch: a workgroup owns a sample and a range of classes, counts the
+ * sample's spikes per channel in LDS and multiplies its weight rows with them; the workspace is then not touched.
+ * snnf_lif_pool_linear_launches() says which of the two forms a shape takes (1 or 2; 0 for invalid extents), assuming
+ * aligned operands.
  */
 size_t snnf_lif_pool_linear_workspace_bytes(int N, int C);
+int snnf_lif_pool_linear_launches(int T, int N, int C, int H, int W, int K);
 int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, int H, int W, int x_dtype,
                          const void* v_init, int v_dtype,
                          const void* fc_weight, const void* fc_bias, int K, int w_dtype,

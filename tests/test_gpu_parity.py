@@ -165,6 +165,34 @@ def test_lif_avgpool_linear_on_batches_with_large_counts(hip_ops, dtype, T, N, C
     _no_fallback(hip_ops, 1)
 
 
+@pytest.mark.parametrize("T,N,C,H,W,K,launches", [(4, 64, 512, 1, 1, 10, 1), (4, 32, 256, 2, 2, 10, 1), (4, 5, 64, 3, 3, 1000, 1),
+                                                   (12, 3, 40, 4, 4, 37, 1), (4, 16, 512, 7, 7, 1000, 2), (4, 6, 36, 3, 3, 10, 2)])
+def test_small_tails_run_as_one_launch_and_equal_the_two_launch_form(snnf_lib, T, N, C, H, W, K, launches):
+    """The backend reports which form a tail took; the one-launch form gives the oracle's results and the membrane of the
+    two-launch form bit for bit (reached here through a weight matrix that is not 16-byte aligned, which the one-launch
+    form does not take; the classifier sums then agree to the output dtype's rounding)."""
+    from triton_snn_fusion_amd.runtime import hip_temporal_lif_avgpool_linear_backend as TB
+    g = gen(380 + C + K)
+    x = q(torch.randn(T, N, C, H, W, generator=g) * 0.75 + 0.15, BF16)
+    w = q(torch.randn(K, C, generator=g) * 0.05, BF16)
+    b = q(torch.randn(K, generator=g) * 0.05, BF16)
+    v0 = torch.rand(N, C, H, W, generator=g) * 0.9
+    ref_out, ref_v, _, _ = O.temporal_lif_avgpool_linear(x, v0, w, b, *LIF)
+    res = TB.run_triton_fused_temporal_lif_avgpool_linear(dev(x, BF16), dev(v0, F32), dev(w, BF16), dev(b, BF16), *LIF, False)
+    assert len(res.kernel_diagnostics["launches"]) == launches == snnf_lib.snnf_lif_pool_linear_launches(T, N, C, H, W, K)
+    assert torch.equal(res.v_next.cpu(), ref_v)
+    assert torch.allclose(res.out_sum.float().cpu(), ref_out, rtol=8e-3, atol=8e-3), (res.out_sum.float().cpu() - ref_out).abs().max()
+    if launches == 1 and C % 8 == 0:
+        # the same call with the weight matrix 2 bytes off a 16-byte boundary: two launches
+        w_store = torch.empty(K * C + 8, device=DEV, dtype=BF16)
+        w_off = w_store[1:1 + K * C].view(K, C)
+        w_off.copy_(dev(w, BF16))
+        assert w_off.data_ptr() % 16 != 0
+        res2 = TB.run_triton_fused_temporal_lif_avgpool_linear(dev(x, BF16), dev(v0, F32), w_off, dev(b, BF16), *LIF, False)
+        assert torch.equal(res2.v_next, res.v_next)
+        assert torch.allclose(res2.out_sum.float(), res.out_sum.float(), rtol=8e-3, atol=8e-3)
+
+
 @pytest.mark.parametrize("N,C,H,W", [(6, 64, 7, 7), (3, 5, 3, 3), (40, 128, 1, 1)])
 def test_lif_avgpool_linear_tensor_v_init(hip_ops, N, C, H, W):
     """A membrane tensor as initial state (vector and element-wise paths of the pooling kernel)."""

@@ -69,6 +69,21 @@ def test_packed_weight_size_is_whole_fragments(snnf_lib):
     assert snnf_lib.snnf_conv_packed_weight_bytes(0, 3, 3, 3, 1) == 0
 
 
+def test_which_tails_run_as_one_launch(snnf_lib):
+    """The tail runs as one launch (a workgroup per sample and class range) when a sample is small, its channels come in whole
+    vectors of 8 and fit the workgroup's counters; otherwise as the pooling launch followed by the classifier launch."""
+    f = snnf_lib.snnf_lif_pool_linear_launches
+    assert f(4, 64, 512, 1, 1, 10) == 1            # VGG-11's tail
+    assert f(4, 4, 512, 2, 2, 1000) == 1
+    assert f(16, 5, 64, 4, 4, 100) == 1
+    assert f(4, 16, 512, 7, 7, 1000) == 2          # ResNet-18's tail: 100 k neuron steps per sample
+    assert f(4, 64, 512, 28, 28, 1000) == 2
+    assert f(4, 3, 30, 7, 7, 10) == 2              # channels no multiple of 8
+    assert f(4, 3, 8, 3, 3, 10) == 1 and f(4, 3, 8, 3, 5, 10) == 1 and f(4, 3, 24, 3, 3, 10) == 1
+    assert f(2, 2, 4096, 1, 1, 10) == 2            # more channels than counters
+    assert f(0, 1, 8, 1, 1, 1) == 0 and f(4, 1, 8, 1, 1, 0) == 0
+
+
 @pytest.mark.parametrize("shape,stride,padding,groups,key", [
     ((8, 4, 1, 1), (1, 1), (0, 0), 1, "k1_s1_p0"),
     ((8, 4, 3, 3), (1, 1), (1, 1), 1, "k3_s1_p1"),

@@ -41,6 +41,7 @@ SIGNATURES = {
     "snnf_rowbits_pack": (_i, [_vp, _vp, _i64, _i, _vp]),
     "snnf_pwconv_lif_rowbits": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i64, _vp, _f, _f, _f, _vp]),
     "snnf_lif_pool_linear_workspace_bytes": (_sz, [_i, _i]),
+    "snnf_lif_pool_linear_launches": (_i, [_i, _i, _i, _i, _i, _i]),
     "snnf_lif_pool_linear": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _sz,
                                   _f, _f, _f, _vp]),
     "snnf_lif_pool_linear_static": (_i, [_pp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _f, _f, _f, _vp]),

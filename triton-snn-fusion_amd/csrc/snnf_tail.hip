@@ -374,6 +374,125 @@ __global__ __launch_bounds__(kThreads) void count_linear_mm_kernel(const int* __
     }
 }
 
+// The whole tail in one launch, for tails as small as those at the end of a network: a workgroup owns one sample and a range
+// of classes. It runs the sample's LIF recurrence (a thread owns 8 consecutive neurons per pass, 16-byte loads, four timesteps
+// in flight), counts the spikes per channel in LDS and multiplies its classes' weight rows with the counts right away: no
+// counts in memory, no second launch. The workgroups of a sample that differ in their class range repeat the recurrence (the
+// sample's activations come from L2 then); the first of them writes the membrane. The products run like
+// count_linear_vec_kernel's (a wave owns kRowsPerWave rows, a lane 8 consecutive channels per trip, shuffle reduction), so the
+// two paths give the same sums bit for bit.
+constexpr int kOneMaxC = 2048;                    // channels of a sample whose counters fit the workgroup's LDS array
+constexpr int64_t kOneMaxSampleWork = 32 * 1024;  // T * C * HW of one sample, at most: 128 LIF steps per thread (larger samples are
+                                                  // better spread over many workgroups by the pooling kernel of the two-launch path)
+
+template <typename XT, typename VT>
+__global__ __launch_bounds__(kThreads) void lif_pool_linear_one_kernel(StepPtrs xs, int T, int C, int HW, int K, int classes_per_block,
+                                                                       const VT* __restrict__ v_init, VT* __restrict__ v_out,
+                                                                       const XT* __restrict__ Wt, const XT* __restrict__ bias,
+                                                                       XT* __restrict__ out, LifParams lif, float inv_hw, float steps) {
+    __shared__ __align__(16) int plane_count[kOneMaxC];
+    const int n = blockIdx.y;
+    const int elems = C * HW;                                    // a multiple of 8 (host)
+    const int64_t base = static_cast<int64_t>(n) * elems;
+    const bool writes_v = blockIdx.x == 0;
+    for (int i = threadIdx.x; i < C; i += kThreads) plane_count[i] = 0;
+    __syncthreads();
+    for (int i0 = threadIdx.x * kVec; i0 < elems; i0 += kThreads * kVec) {
+        float v[kVec];
+        int fired[kVec];
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+            v[j] = 0.0f;
+            fired[j] = 0;
+        }
+        if (v_init != nullptr) {
+            const Pack<VT, kVec> pv = *reinterpret_cast<const Pack<VT, kVec>*>(v_init + base + i0);
+#pragma unroll
+            for (int j = 0; j < kVec; ++j) v[j] = to_float(pv.v[j]);
+        }
+        for (int t0 = 0; t0 < T; t0 += 4) {
+            Pack<XT, kVec> px[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (t0 + u < T) px[u] = *reinterpret_cast<const Pack<XT, kVec>*>(static_cast<const XT*>(xs.p[t0 + u]) + base + i0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (t0 + u < T) {
+#pragma unroll
+                    for (int j = 0; j < kVec; ++j) fired[j] += lif_step(to_float(px[u].v[j]), v[j], lif) ? 1 : 0;
+                }
+            }
+        }
+        if (writes_v) {
+            Pack<VT, kVec> pv;
+#pragma unroll
+            for (int j = 0; j < kVec; ++j) pv.v[j] = from_float<VT>(v[j]);
+            *reinterpret_cast<Pack<VT, kVec>*>(v_out + base + i0) = pv;
+        }
+        // Spikes of consecutive neurons of one channel are summed before they go to that channel's counter.
+        int p = i0 / HW;
+        int rem = i0 - p * HW;
+        int run = 0;
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+            run += fired[j];
+            if (++rem == HW) {
+                if (run != 0) atomicAdd(&plane_count[p], run);
+                run = 0;
+                rem = 0;
+                ++p;
+            }
+        }
+        if (run != 0) atomicAdd(&plane_count[p], run);
+    }
+    __syncthreads();
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int k_begin = blockIdx.x * classes_per_block;
+    const int k_end = min(K, k_begin + classes_per_block);
+    for (int k0 = k_begin + wave * kRowsPerWave; k0 < k_end; k0 += (kThreads / 64) * kRowsPerWave) {
+        float acc[kRowsPerWave];
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
+        for (int c0 = lane * kVec; c0 < C; c0 += 64 * kVec) {
+            const Pack<int, kVec> pc = *reinterpret_cast<const Pack<int, kVec>*>(plane_count + c0);
+            Pack<XT, kVec> pw[kRowsPerWave];
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r) {
+                const int k = min(k0 + r, K - 1);   // rows beyond the range re-read the last one and are not stored
+                pw[r] = *reinterpret_cast<const Pack<XT, kVec>*>(Wt + static_cast<int64_t>(k) * C + c0);
+            }
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+                for (int j = 0; j < kVec; ++j) acc[r] = fmaf(to_float(pw[r].v[j]), static_cast<float>(pc.v[j]), acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc[r] += __shfl_xor(acc[r], off);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r) {
+                const int k = k0 + r;
+                if (k >= k_end) continue;
+                const float bv = bias != nullptr ? steps * to_float(bias[k]) : 0.0f;
+                out[static_cast<int64_t>(n) * K + k] = from_float<XT>(acc[r] * inv_hw + bv);
+            }
+        }
+    }
+}
+
+// Class ranges per sample of the one-launch tail: at least 16 classes each (one pass of the workgroup's four waves), no more
+// workgroups than two per compute unit. 0: the shape takes the two launches.
+int one_launch_class_blocks(int T, int N, int C, int HW, int K) {
+    const int64_t work = static_cast<int64_t>(T) * C * HW;
+    if (C > kOneMaxC || C % kVec != 0 || (static_cast<int64_t>(C) * HW) % kVec != 0 || work > kOneMaxSampleWork) return 0;
+    const int rows_per_pass = (kThreads / 64) * kRowsPerWave;
+    return std::max(1, std::min((K + rows_per_pass - 1) / rows_per_pass, 512 / std::max(1, N)));
+}
+
 template <typename XT, typename VT>
 int run(const StepPtrs& xs, int T, int planes, int HW, const void* v_init, void* v_out, int* counts,
         const LifParams& lif, hipStream_t stream) {
@@ -445,6 +564,13 @@ void run_linear(bool vec, bool matrix, dim3 grid, size_t lds, hipStream_t hs, co
 }  // namespace
 }  // namespace snnf
 
+extern "C" int snnf_lif_pool_linear_launches(int T, int N, int C, int H, int W, int K) {
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1) return 0;
+    const int64_t hw = static_cast<int64_t>(H) * W;
+    if (hw > (1 << 24)) return 2;
+    return snnf::one_launch_class_blocks(T, N, C, static_cast<int>(hw), K) > 0 ? 1 : 2;
+}
+
 extern "C" size_t snnf_lif_pool_linear_workspace_bytes(int N, int C) {
     if (N < 1 || C < 1) return 0;
     return static_cast<size_t>(N) * static_cast<size_t>(C) * sizeof(int);
@@ -484,6 +610,33 @@ int lif_pool_linear_impl(const char* who, const void* const* xs, int T, int N, i
     hipStream_t hs = as_stream(stream);
     const int planes = static_cast<int>(planes64);
     const int HW = static_cast<int>(hw64);
+
+    // Small tails: one launch (a workgroup per sample and class range), when every operand allows 16-byte accesses.
+    {
+        bool aligned = aligned_to(v_out, 16) && (v_init == nullptr || aligned_to(v_init, 16)) && aligned_to(fc_weight, 16);
+        for (int t = 0; t < T; ++t) aligned = aligned && aligned_to(xs[t], 16);
+        const int class_blocks = aligned ? one_launch_class_blocks(T, N, C, HW, K) : 0;
+        if (class_blocks > 0) {
+            const dim3 grid(class_blocks, N);
+            const int per_block = (K + class_blocks - 1) / class_blocks;
+            const float inv_hw = 1.0f / static_cast<float>(HW);
+            const float steps = static_cast<float>(T);
+#define SNNF_TAIL_ONE(XT, VT)                                                                                               \
+    lif_pool_linear_one_kernel<XT, VT><<<grid, kThreads, 0, hs>>>(ptrs, T, C, HW, K, per_block, static_cast<const VT*>(v_init), \
+                                                                  static_cast<VT*>(v_out), static_cast<const XT*>(fc_weight),   \
+                                                                  static_cast<const XT*>(fc_bias), static_cast<XT*>(out_sum), lif, inv_hw, steps)
+            if (x_dtype == SNNF_F32) SNNF_TAIL_ONE(float, float);
+            else if (x_dtype == SNNF_BF16) {
+                if (v_dtype == SNNF_F32) SNNF_TAIL_ONE(bf16_t, float);
+                else SNNF_TAIL_ONE(bf16_t, bf16_t);
+            } else {
+                if (v_dtype == SNNF_F32) SNNF_TAIL_ONE(f16_t, float);
+                else SNNF_TAIL_ONE(f16_t, f16_t);
+            }
+#undef SNNF_TAIL_ONE
+            return check_launch(who);
+        }
+    }
 
     int rc;
     if (x_dtype == SNNF_F32) rc = run<float, float>(ptrs, T, planes, HW, v_init, v_out, counts, lif, hs);

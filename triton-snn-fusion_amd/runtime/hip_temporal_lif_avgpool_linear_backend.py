@@ -136,10 +136,13 @@ def run_triton_fused_temporal_lif_avgpool_linear(x_seq, v_init, fc_weight, fc_bi
         _lib.packed_step_pointers(x), T, N, C, H, W, _lib.dtype_code(x.dtype), _lib.ptr(vi), _lib.dtype_code(v_dtype),
         w.data_ptr(), _lib.ptr(b), K, _lib.dtype_code(w.dtype), out_sum.data_ptr(), v_next.data_ptr(),
         workspace.data_ptr(), ws_bytes, float(v_threshold), float(v_reset), float(tau), _lib.current_stream(x.device)))
+    one_launch = int(lib.snnf_lif_pool_linear_launches(T, N, C, H, W, K)) == 1
     diagnostics = {
         "kernel_kind": "temporal_lif_avgpool_linear",
-        "launches": ["lif_scan_with_spike_counts_per_plane", "classifier_on_summed_counts"],
-        "workspace": f"int32 spike counts [{N}, {C}]",
+        # small tails: a workgroup per sample and class range runs the scan, counts in LDS and applies its classifier rows
+        "launches": (["lif_scan_counts_and_classifier_per_sample"] if one_launch
+                     else ["lif_scan_with_spike_counts_per_plane", "classifier_on_summed_counts"]),
+        "workspace": "unused (counts stay in LDS)" if one_launch else f"int32 spike counts [{N}, {C}]",
         "membrane_dtype": str(v_dtype),
         "accumulator_dtype": "float32",
         "timesteps": T,
