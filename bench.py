@@ -144,10 +144,15 @@ def _time_kernel(fn, steps: int, warmup: int, reps: int = 10, rotate=None):
 COLD_SETS = 4
 
 
-# `roofline.traffic` (HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE) is not measured inside this script: a
-# counter run needs the profiler around the process. The line therefore carries null and names the committed summary of
-# the counter run of this same command.
+# `roofline.traffic` (HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE) cannot be measured inside this script: a
+# counter run needs the profiler around the process. The line carries the figure of the committed counter run of this same
+# command (scaled by the copy probe of that run) for the kernels and the configuration that run covered, null for any other,
+# and names the summary either way.
 TRAFFIC_PROFILE = "profiles/mobilenet_block_hbm_traffic.md"
+MEASURED_TRAFFIC_BYTES = {      # mobilenet_block, bf16, batch 32, fp32 membrane: bytes per launch
+    "layer1_pointwise1x1": 411.8e6,
+    "layer0_depthwise3x3": 257.1e6,
+}
 
 
 class Prepared:
@@ -700,6 +705,8 @@ def main() -> int:
         ai = dominant[1]["flops"] / dominant[1]["algorithmic_bytes"]
         bound = "mfma" if ai > MFMA_BF16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS and dominant[1]["mfma"] is not None else "hbm"
         result["roofline"] = dict(dominant[1][bound], kernel=dominant[0], traffic_measured_in=TRAFFIC_PROFILE)
+        if args.workload == "mobilenet_block" and args.dtype == "bf16" and wl.batch == 32 and bound == "hbm":
+            result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(dominant[0])
     else:
         T, M, fin, fout = wl.T, wl.batch, int(wl.linear_weight.shape[1]), int(wl.linear_weight.shape[0])
         nbytes = (T * M * fin + fout * fin + fout) * prep.esize + T * M * fout * prep.esize + M * fout * 4
