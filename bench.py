@@ -287,6 +287,26 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
                      "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
         total_ms += ms * count
         total_flops += flops * count
+    if internal and which == "resnet18":
+        # The down-sampling blocks: the second convolution with the shortcut convolution in its accumulators is one launch of
+        # the executor; it takes the place of one "+res" layer and of the shortcut layer in the sum.
+        by_name = {r["layer"]: r for r in rows}
+        for name, res_name, sc_name, c, size, sc_c, sc_size in W.RESNET18_SHORTCUT_BLOCKS:
+            bx = B.from_dense(torch.stack([(torch.rand(batch, c, size, size, generator=g) < 0.15).to(dev, dtype) for _ in range(T)]), B.BITS)
+            bs = B.from_dense(torch.stack([(torch.rand(batch, sc_c, sc_size, sc_size, generator=g) < 0.15).to(dev, dtype) for _ in range(T)]), B.BITS)
+            w = (torch.randn(c, c, 3, 3, generator=g) * (2.0 / (c * 9)) ** 0.5).to(dev, dtype)
+            w2 = (torch.randn(c, sc_c, 1, 1, generator=g) * (2.0 / sc_c) ** 0.5).to(dev, dtype)
+            b = (torch.randn(c, generator=g) * 0.1).to(dev, dtype)
+            fn = lambda: B.conv_lif_blocked_shortcut(bx, w, b, [1, 1], bs, w2, b, [2, 2], (1.0, 0.0, 2.0), out_layout=B.BITS)
+            ms, how = _time_kernel(fn, steps, warmup)
+            flops = W.conv_flops(T, batch, c, c, size, size, 3, 3, 1) + W.conv_flops(T, batch, sc_c, c, size, size, 1, 1, 1)
+            internal_bytes = T * batch * (c // 8) * size * size * 2 + T * batch * (sc_c // 8) * sc_size * sc_size + (c * c * 9 + c * sc_c) * esize
+            rows.append({"layer": name, "count": 1, "ms": round(ms, 4), "timed": how, "plan": _plan_summary(), "internal_bytes": internal_bytes,
+                         "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                         "in_place_of": [res_name, sc_name]})
+            total_ms += ms - by_name[res_name]["ms"] - by_name[sc_name]["ms"]
+            by_name[res_name]["count"] -= 1
+            by_name[sc_name]["count"] -= 1
     return {"metric": METRIC, "workload": f"{which}_layers" + ("_internal_layouts" if internal else ""), "dtype": dtype_name, "T": T, "batch": batch,
             "conv_ms_per_forward": round(total_ms, 4), "images_T_per_s_conv_only": round(batch * T / (total_ms * 1e-3), 1),
             "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}

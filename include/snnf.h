@@ -311,6 +311,29 @@ int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const
                           int neuron, float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * The second convolution of a residual block together with the block's projection shortcut: out = LIF(conv(xs) + bias +
+ * conv1x1(shortcut_xs) + shortcut bias), the shortcut's products accumulated as further K steps of the same output
+ * tile. The reference runs the shortcut as a convolution of its own and adds its output through the residual operand of
+ * run_fused_temporal_general_residual (kernels/benchmark_conv_lif_temporal_general.py:1147-1323, as called from
+ * runtime/triton_convlif_backend.py:669-817); here the shortcut's output never exists in memory (and is not rounded to the
+ * activation dtype on the way), and one launch replaces two.
+ *   xs[t]          : N frames [Cin, H, W] in BITS; the main convolution is KH x KW, stride 1, padding (KH-1)/2 x (KW-1)/2
+ *   shortcut_xs[t] : N frames [shortcut_Cin, shortcut_H, shortcut_W] in BITS, convolved 1 x 1 with the given strides and
+ *                    no padding; its output plane must be the main one: (shortcut_H - 1) / shortcut_stride_h + 1 == H
+ *   packed_weight, shortcut_packed_weight : snnf_conv_pack_weight of [Cout, Cin, KH, KW] and [Cout, shortcut_Cin, 1, 1]
+ *                    (each with its own bias) for `x_dtype`
+ *   out, v_init, v_out, neuron, out_layout, out_step_stride : as in snnf_conv_lif_blocked
+ * Cin and shortcut_Cin multiples of 16, 3 <= T <= SNNF_MAX_T_PER_LAUNCH, distinct inputs per timestep;
+ * SNNF_ERR_UNSUPPORTED ("unsupported_shortcut: ...") otherwise: the caller then runs the two convolutions apart.
+ */
+int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void* const* shortcut_xs, int T, int N, int Cin, int H, int W,
+                                   int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int pad_h, int pad_w,
+                                   int shortcut_Cin, int shortcut_H, int shortcut_W, int shortcut_stride_h,
+                                   int shortcut_stride_w, const void* shortcut_packed_weight,
+                                   const void* v_init, void* out, int out_layout, int64_t out_step_stride, void* v_out,
+                                   int neuron, float v_threshold, float v_reset, float tau, void* stream);
+
+/*
  * Registers a measured launch choice for snnf_conv_lif_blocked on one layer shape (the counterpart of the per-kernel-key
  * "best config" the reference's autotuner keeps, kernels/benchmark_conv_lif_temporal_general.py:524-558,1332-1369):
  * columns of a wave's output patch (rows follow: 32 / columns), channel groups of 8 per LDS stage (a power of two) and

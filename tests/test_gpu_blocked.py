@@ -150,6 +150,72 @@ def test_blocked_conv_lif_against_the_oracle(B, Cin, Cout, H, W, k, s, p, dtype,
             assert float(out.data[:, :, c8 - 1, :, :, Cout % 8:].abs().max()) == 0.0
 
 
+SHORTCUT_CASES = [  # main Cin, Cout, H, W, k, shortcut Cin, shortcut stride, T, N, dtype, lif, out layout
+    (128, 128, 8, 8, 3, 64, 2, 4, 2, BF16, (1.0, 0.0, 2.0), "bits"),      # a ResNet downsample block, K shared by waves
+    (32, 64, 12, 12, 3, 32, 2, 4, 2, BF16, (1.0, 0.0, 2.0), "bits"),      # one main stage: a wave per tile
+    (128, 96, 9, 11, 3, 48, 2, 4, 3, BF16, (1.0, -0.5, 3.0), "nchw"),     # ragged planes, odd shortcut plane, general epilogue, dense output
+    (64, 72, 10, 10, 3, 32, 1, 3, 2, BF16, (1.0, 0.0, 2.0), "c8"),        # shortcut of stride 1, 3 of 4 steps, blocked output
+    (64, 64, 14, 14, 3, 64, 2, 6, 2, BF16, (1.0, 0.0, 2.0), "bits"),      # two windows (4 + 2)
+    (64, 128, 8, 8, 5, 32, 2, 4, 2, F16, (1.0, 0.0, 2.0), "bits"),        # 5x5 main kernel, fp16
+    (512, 512, 7, 7, 3, 256, 2, 4, 4, BF16, (1.0, 0.0, 2.0), "bits"),     # the deepest block: K shared by eight waves
+    (256, 256, 4, 4, 3, 128, 2, 4, 6, BF16, (1.0, 0.0, 2.0), "bits"),     # two images per patch
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,Cs,ss,T,N,dtype,lif,outl", SHORTCUT_CASES)
+def test_blocked_conv_with_the_projection_shortcut_in_its_accumulators(B, Cin, Cout, H, W, k, Cs, ss, T, N, dtype, lif, outl):
+    """LIF(conv(x) + conv1x1(shortcut input, stride)) in one launch, against the oracle with the shortcut's output as its
+    (unrounded fp32) residual, and against the same layer run as two launches within the rounding of the shortcut's output."""
+    xs, w, b = _case(3400 + Cin + Cout + H + k + T, T, N, Cin, Cout, H, W, k, dtype)
+    g = gen(3401 + Cs)
+    Hs, Ws = (H - 1) * ss + 1 + (ss - 1) * (H % 2), (W - 1) * ss + 1          # both the smallest and a larger plane that lands on H x W
+    x2 = spikes((T, N, Cs, Hs, Ws), 0.25, g)
+    w2 = q(torch.randn(Cout, Cs, 1, 1, generator=g) * (2.0 / Cs) ** 0.5, dtype)
+    b2 = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    shortcut = [torch.nn.functional.conv2d(x2[t], w2, b2, stride=ss) for t in range(T)]
+    assert tuple(shortcut[0].shape[-2:]) == (H, W)
+    ref = O.temporal_conv_lif([xs[t] for t in range(T)], w, b, torch.tensor(0.0), (1, 1), (k // 2, k // 2), (1, 1), 1, *lif, residuals=shortcut)
+    out_layout = {"nchw": B.NCHW, "c8": B.C8, "bits": B.BITS}[outl]
+    x, xsc = _to_layout(B, xs, "bits", dtype), _to_layout(B, x2, "bits", dtype)
+    print(f"blocked conv {Cin}->{Cout} {H}x{W} k{k} + shortcut {Cs}->{Cout} /{ss} from {Hs}x{Ws} T={T} N={N} -> {outl}", flush=True)
+    out, v = B.conv_lif_blocked_shortcut(x, dev(w, dtype), dev(b, dtype), [k // 2, k // 2], xsc, dev(w2, dtype), dev(b2, dtype), [ss, ss], lif,
+                                         out_layout=out_layout, want_v=True)
+    torch.cuda.synchronize()
+    plan = B.last_conv_plan()
+    assert plan["kernel"] == "blocked" and int(plan["shortcut_stages"]) >= 1, plan
+    assert out.layout == out_layout and out.shape == (T, N, Cout, H, W) and v.dtype == F32
+    rep = check(B.to_dense(out), v, ref, v_threshold=lif[0], what=f"blocked {Cin}->{Cout} k{k} + shortcut {Cs}/{ss} -> {outl}")
+    assert 0.001 < float(ref[0].mean()) < 0.9, float(ref[0].mean())
+    assert rep["neurons_with_matching_history"] >= 0.999 * rep["neurons"]
+    # the two-launch form: the shortcut's sums pass through the activation dtype on their way, the spikes agree but for neurons at the threshold
+    sc_out, _ = B.conv_lif_blocked(xsc, dev(w2, dtype), dev(b2, dtype), [ss, ss], [0, 0], None, out_layout=B.C8)
+    two, _ = B.conv_lif_blocked(x, dev(w, dtype), dev(b, dtype), [1, 1], [k // 2, k // 2], lif, residual=sc_out, out_layout=out_layout)
+    differ = (B.to_dense(two).float() != B.to_dense(out).float()).float().mean()
+    assert float(differ) < 1e-2, float(differ)
+
+
+def test_blocked_conv_shortcut_rejects_what_it_does_not_take(B):
+    T, N = 4, 2
+    xs, w, b = _case(3450, T, N, 64, 64, 8, 8, 3, BF16)
+    x = B.from_dense(dev(xs, BF16), B.BITS)
+    g = gen(3451)
+    def sc(C, H, W, t=T):
+        return B.from_dense(dev(spikes((t, N, C, H, W), 0.2, g), BF16), B.BITS)
+    dw, db = dev(w, BF16), dev(b, BF16)
+    w2 = dev(q(torch.randn(64, 32, 1, 1, generator=g), BF16), BF16)
+    with pytest.raises(RuntimeError, match="unsupported_shortcut"):        # lands on 7x7, not 8x8
+        B.conv_lif_blocked_shortcut(x, dw, db, [1, 1], sc(32, 13, 13), w2, None, [2, 2], LIF)
+    with pytest.raises(RuntimeError, match="unsupported_shortcut"):        # 24 channels: not a multiple of 16
+        B.conv_lif_blocked_shortcut(x, dw, db, [1, 1], sc(24, 15, 15), dev(q(torch.randn(64, 24, 1, 1, generator=g), BF16), BF16), None, [2, 2], LIF)
+    with pytest.raises(RuntimeError, match="unsupported_shortcut"):        # a main convolution that shrinks its plane
+        B.conv_lif_blocked_shortcut(x, dw, db, [0, 0], sc(32, 15, 15), w2, None, [2, 2], LIF)
+    with pytest.raises(RuntimeError, match="unsupported_shortcut"):        # 3x3 shortcut
+        B.conv_lif_blocked_shortcut(x, dw, db, [1, 1], sc(32, 15, 15), dev(q(torch.randn(64, 32, 3, 3, generator=g), BF16), BF16), None, [2, 2], LIF)
+    x2 = B.from_dense(dev(xs[:2], BF16), B.BITS)
+    with pytest.raises(RuntimeError, match="unsupported_shortcut"):        # two timesteps
+        B.conv_lif_blocked_shortcut(x2, dw, db, [1, 1], sc(32, 15, 15, 2), w2, None, [2, 2], LIF)
+
+
 def test_blocked_conv_without_membrane_output_and_chained_windows(B):
     """The final membrane is optional; two calls chained through it equal one call of all steps, bit for bit."""
     T, N, C, H = 4, 2, 64, 12

@@ -281,8 +281,10 @@ def test_fx_layout_propagation_graph_invariants(name):
     calls = [n for n in gm.graph.nodes if n.op == "call_function"]
     targets = [n.target for n in calls]
     n_conv, n_pool = (8, 4) if name == "vgg11" else (20, 1)
-    assert targets.count(R.blocked_conv_lif) == n_conv and targets.count(R.blocked_pool) == n_pool
-    assert stats.internal_layout_nodes == n_conv + n_pool and not stats.skipped
+    n_shortcut = 0 if name == "vgg11" else 3      # 1x1 shortcut convolutions folded into the convolution they are added to
+    assert targets.count(R.blocked_conv_lif) == n_conv - 2 * n_shortcut and targets.count(R.blocked_conv_lif_shortcut) == n_shortcut
+    assert targets.count(R.blocked_pool) == n_pool
+    assert stats.internal_layout_nodes == n_conv - n_shortcut + n_pool and not stats.skipped
     assert targets.count(R.blocked_input) == 1 and targets.count(R.blocked_to_dense) == 1 and targets.count(R.blocked_residual) == 0
     assert targets.count(S.fused_temporal_lif_avgpool_linear) == 1
     dense_ops = (S.fused_temporal_conv_lif_state, S.fused_temporal_conv_add_lif_state, R.pooled_frames, R.conv_bias_frames)
@@ -290,20 +292,25 @@ def test_fx_layout_propagation_graph_invariants(name):
     first = next(n for n in calls if n.target is R.blocked_input)
     assert first.args[0].op == "placeholder" and first.args[1:] == (T, True)          # one shared analog frame
     convs = [n for n in calls if n.target is R.blocked_conv_lif]
-    # layouts: spikes leave bit-packed, LIF-free shortcut sums channel-blocked, the tensor the tail reads dense
+    # layouts: spikes leave bit-packed, the tensor the tail reads dense
     assert [n.args[7] for n in convs if n.args[5] is not None] == [B.BITS] * sum(n.args[5] is not None for n in convs)
     plain = [n for n in convs if n.args[5] is None]
-    assert [n.args[7] for n in plain] == ([B.NCHW] if name == "vgg11" else [B.C8, B.C8, B.C8, B.NCHW])
+    assert [n.args[7] for n in plain] == [B.NCHW]
     assert convs[-1] is plain[-1] and next(iter(convs[-1].users)).target is R.blocked_to_dense
+    produced = (R.blocked_conv_lif, R.blocked_conv_lif_shortcut, R.blocked_pool)
     if name == "resnet18":
-        # residuals: the block input itself (bits) for plain blocks, the shortcut convolution's output for down-sampling ones
+        # residuals: the block input itself (bits) for plain blocks; a down-sampling block's shortcut convolution is part of
+        # the node of its second convolution, which reads the block input (the shortcut's operand) and the first convolution's spikes
         with_res = [n for n in convs if n.args[6] is not None]
-        assert len(with_res) == 8 and all(n.args[6].target in (R.blocked_conv_lif, R.blocked_pool) for n in with_res)
-        assert sum(n.args[6] in plain for n in with_res) == 3
+        assert len(with_res) == 5 and all(n.args[6].target in produced for n in with_res)
         assert plain[-1].args[6] is not None                                            # the pre-tail sum is the convolution's residual
+        for n in (c for c in calls if c.target is R.blocked_conv_lif_shortcut):
+            first_conv = n.args[0]
+            assert first_conv.target is R.blocked_conv_lif and first_conv.args[0] is n.args[5] and n.args[9] == B.BITS
+            assert list(n.args[8]) == [2, 2] and list(first_conv.args[3]) == [2, 2]
     # every operand of a converted node is another converted node (or the input conversion): no dense hop in between
-    for n in convs + [c for c in calls if c.target is R.blocked_pool]:
-        assert n.args[0].target in (R.blocked_conv_lif, R.blocked_pool, R.blocked_input)
+    for n in convs + [c for c in calls if c.target in (R.blocked_pool, R.blocked_conv_lif_shortcut)]:
+        assert n.args[0].target in produced + (R.blocked_input,)
 
 
 def test_fx_layout_propagation_keeps_dense_tensors_around_nodes_it_does_not_know():
@@ -349,6 +356,9 @@ def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
             L = e["layer"]
             xs = [x.float().cpu() for x in e["xs"]]
             rs = None if e["residuals"] is None else [r.float().cpu() for r in e["residuals"]]
+            if e.get("shortcut") is not None:     # a projection shortcut accumulated in the same launch: its sums, unrounded
+                D = e["shortcut"]["layer"]
+                rs = [F.conv2d(x.float().cpu(), D.weight.float().cpu(), D.bias.float().cpu(), D.stride, D.padding) for x in e["shortcut"]["x"]]
             ref = O.temporal_conv_lif(xs, L.weight.float().cpu(), L.bias.float().cpu(), torch.tensor(0.0), tuple(L.stride),
                                       tuple(L.padding), (1, 1), L.groups, *L.lif, residuals=rs)
             check(e["spikes"], e["v"], ref, what=f"{name} {e['name']}")
@@ -514,7 +524,7 @@ def test_fx_graph_on_the_internal_layouts_equals_the_hand_lowered_executor(hip_o
     T = 4
     model, internal = _fused(name, T, internal=True)
     gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16, internal_layouts=True)
-    assert not stats.skipped and stats.internal_layout_nodes == (12 if name == "vgg11" else 21)
+    assert not stats.skipped and stats.internal_layout_nodes == (12 if name == "vgg11" else 18)    # 21 less the three folded shortcuts
     frames = [_frame(name, seed=30 + i).to(DEV, BF16) for i in range(3)]
     hip_ops.reset_fused_op_call_stats()
     with torch.no_grad():

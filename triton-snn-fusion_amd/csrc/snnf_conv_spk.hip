@@ -71,9 +71,25 @@ std::map<TunedKey, TunedPlan>& tuned_plans() {
 
 bool valid_layout(int layout) { return layout == SNNF_LAYOUT_NCHW || layout == SNNF_LAYOUT_C8 || layout == SNNF_LAYOUT_BITS; }
 
+// A projection shortcut whose sums join the main convolution's accumulators: a pointwise convolution (stride s, no padding)
+// of a second bit-packed input with as many output channels and output pixels as the main one.
+struct Shortcut {
+    const void* const* xs;
+    int Cin, H, W, stride_h, stride_w;
+    const void* packed_weight;
+};
+
 }  // namespace
 
 char* conv_plan_buffer();   // the thread's plan text (snnf_conv_igemm.hip), shared with snnf_conv_last_plan()
+
+namespace {
+int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
+                          int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
+                          int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
+                          int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
+                          float v_reset, float tau, void* stream, const Shortcut* sc);
+}  // namespace
 
 }  // namespace snnf
 
@@ -95,8 +111,33 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
                                      int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
                                      int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
                                      float v_reset, float tau, void* stream) {
+    return snnf::conv_lif_blocked_impl("snnf_conv_lif_blocked", xs, x_layout, residuals, res_layout, T, N, Cin, H, W, x_dtype, packed_weight,
+                                       Cout, KH, KW, stride_h, stride_w, pad_h, pad_w, v_init, out, out_layout, out_step_stride, v_out,
+                                       neuron, v_threshold, v_reset, tau, stream, nullptr);
+}
+
+extern "C" int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void* const* shortcut_xs, int T, int N, int Cin, int H, int W,
+                                              int x_dtype, const void* packed_weight, int Cout, int KH, int KW, int pad_h, int pad_w,
+                                              int shortcut_Cin, int shortcut_H, int shortcut_W, int shortcut_stride_h, int shortcut_stride_w,
+                                              const void* shortcut_packed_weight, const void* v_init, void* out, int out_layout,
+                                              int64_t out_step_stride, void* v_out, int neuron, float v_threshold, float v_reset, float tau,
+                                              void* stream) {
     using namespace snnf;
-    const char* who = "snnf_conv_lif_blocked";
+    const char* who = "snnf_conv_lif_blocked_shortcut";
+    if (shortcut_xs == nullptr || shortcut_packed_weight == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: shortcut_xs and shortcut_packed_weight must be non-null", who);
+    const Shortcut sc = {shortcut_xs, shortcut_Cin, shortcut_H, shortcut_W, shortcut_stride_h, shortcut_stride_w, shortcut_packed_weight};
+    return conv_lif_blocked_impl(who, xs, SNNF_LAYOUT_BITS, nullptr, SNNF_LAYOUT_BITS, T, N, Cin, H, W, x_dtype, packed_weight, Cout, KH, KW, 1, 1,
+                                 pad_h, pad_w, v_init, out, out_layout, out_step_stride, v_out, neuron, v_threshold, v_reset, tau, stream, &sc);
+}
+
+namespace snnf {
+namespace {
+int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
+                          int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
+                          int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
+                          int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
+                          float v_reset, float tau, void* stream, const Shortcut* sc) {
     if (xs == nullptr || packed_weight == nullptr || out == nullptr)
         return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs, packed_weight and out must be non-null", who);
     if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0)
@@ -130,6 +171,23 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
         if (residuals != nullptr && (residuals[t] == nullptr || !aligned_to(residuals[t], need_align(res_layout, false))))
             return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: residuals[%d] is null or misaligned for its layout", who, t);
         shared = shared && xs[t] == xs[0];
+    }
+    if (sc != nullptr) {
+        // The shortcut's sums are K steps of the main tile: same output pixels (a main convolution that keeps the plane, the
+        // shortcut's stride taking its own input down to it), whole pairs of channel groups, bit-packed input like the main one.
+        if (sc->Cin < 1 || sc->H < 1 || sc->W < 1 || sc->stride_h < 1 || sc->stride_w < 1)
+            return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: bad shortcut extent (Cin=%d H=%d W=%d s=%dx%d)", who, sc->Cin, sc->H, sc->W, sc->stride_h, sc->stride_w);
+        if (KH != 2 * pad_h + 1 || KW != 2 * pad_w + 1 || (sc->H - 1) / sc->stride_h + 1 != H || (sc->W - 1) / sc->stride_w + 1 != W)
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shortcut: the main convolution must keep its %dx%d plane and the shortcut (%dx%d, stride %dx%d) must land on it",
+                        who, H, W, sc->H, sc->W, sc->stride_h, sc->stride_w);
+        if (sc->Cin % 16 != 0 || Cin % 16 != 0 || shared || T < 3)
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shortcut: needs channel counts that are multiples of 16, at least 3 timesteps and an input per timestep", who);
+        if (!aligned_to(sc->packed_weight, 16))
+            return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: shortcut_packed_weight is misaligned", who);
+        if (static_cast<int64_t>(N) * (sc->Cin / 8) * sc->H * sc->W >= (1LL << 27))
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: shortcut input too large for 32-bit offsets", who);
+        for (int t = 0; t < T; ++t)
+            if (sc->xs[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: shortcut_xs[%d] is null", who, t);
     }
 
     SpkGeom g = {};
@@ -239,6 +297,21 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     g.pair_tap_stride = g.tap_pairs ? 1 : g.gpc / 2;
     if (nst > kSpkMaxSteps)
         return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_kernel: %d matrix steps per stage exceed %d (kernel %dx%d)", who, nst, kSpkMaxSteps, KH, KW);
+    PackGeom pg2 = {};
+    if (sc != nullptr) {
+        pg2 = make_pack_geom(Cout, sc->Cin, 1, 1, false);
+        const int gpc2 = pg2.CK / 8;
+        if (tt != 4 || g.tap_pairs || gpc2 % g.G != 0 || nst + 4 + hg + 4 > kSpkMaxSteps + 4)
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shortcut: this layer's plan (window %d, %d channel groups per stage, %d steps) has no room for a shortcut",
+                        who, tt, g.G, nst);
+        g.sc_C8 = sc->Cin / 8;
+        g.sc_stages = (g.sc_C8 + g.G - 1) / g.G;
+        g.sc_H = sc->H; g.sc_W = sc->W; g.sc_sh = sc->stride_h; g.sc_sw = sc->stride_w;
+        g.sc_gpc_log2 = 0;
+        while ((1 << g.sc_gpc_log2) < gpc2) ++g.sc_gpc_log2;
+        g.sc_npairs = pg2.npairs;
+        g.sc_frag_stride = static_cast<int64_t>(pg2.nchunks) * pg2.npairs * (kFragBytes / 2);
+    }
     g.d_hg = make_fast_div(hg);
     g.d_nst = make_fast_div(nst);
     g.d_KW = make_fast_div(KW);
@@ -247,6 +320,11 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
     for (int t = 0; t < T; ++t) {
         L.xs.p[t] = xs[t];
         if (residuals != nullptr) L.residuals.p[t] = residuals[t];
+        if (sc != nullptr) L.residuals.p[t] = sc->xs[t];   // the second input travels in the residual's place (a shortcut launch has no residual)
+    }
+    if (sc != nullptr) {
+        L.wpacked2 = static_cast<const uint16_t*>(sc->packed_weight);
+        L.bias2 = reinterpret_cast<const float*>(L.wpacked2 + packed_weight_elems(pg2));
     }
     L.g = g;
     L.wpacked = static_cast<const uint16_t*>(packed_weight);
@@ -264,10 +342,14 @@ extern "C" int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const 
                           v_init == nullptr && windows == 1 && Cout % 8 == 0;
     snprintf(snnf::conv_plan_buffer(), 256,
              "kernel=blocked variant=%d window=%d launches=1 tile=%dx%dx%d halo=%dx%d waves=8x1x%d oc_tiles=%d px_tiles=%d "
-             "stage_chunks=%d run=0 lds=%zu grid=%d tuned=%d",
+             "stage_chunks=%d run=0 lds=%zu grid=%d tuned=%d shortcut_stages=%d",
              (wk_log2 > 0 ? 50 : 40) + tt + (fast_epi ? 20 : 0), shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
-             L.lds_bytes, grid, (tuned_patch ? 1 : 0) + (tuned_split ? 2 : 0));
+             L.lds_bytes, grid, (tuned_patch ? 1 : 0) + (tuned_split ? 2 : 0), g.sc_stages);
     L.fast_epilogue = fast_epi;
+    if (sc != nullptr) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_shortcut(L) : launch_conv_spk_f16_shortcut(L);
     if (x_layout == SNNF_LAYOUT_BITS) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_bits(L, tt) : launch_conv_spk_f16_bits(L, tt);
     return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_c8(L, tt) : launch_conv_spk_f16_c8(L, tt);
 }
+
+}  // namespace
+}  // namespace snnf

@@ -70,6 +70,13 @@ struct SpkGeom {
     int64_t out_step_stride;     // bytes between timesteps of `out`
     int lds_wave_bytes;          // private staging region of a wave (a multiple of 16)
     int64_t frag_stride;         // 16-bit elements between consecutive 32-row fragments of the packed weight
+    // A second, pointwise operand pair that shares the accumulators (the projection shortcut of a residual block: its sums
+    // are further K steps of the same output tile). Its input has sc_C8 channel groups on an sc_H x sc_W plane and is
+    // sampled at (sc_sh * ih, sc_sw * iw) for the pixel (ih, iw) of the main input; its stages follow the main ones.
+    int sc_stages;               // 0: none
+    int sc_C8, sc_H, sc_W, sc_sh, sc_sw;
+    int sc_gpc_log2, sc_npairs;  // channel groups (log2) and k-slot pairs per packed chunk of the second weight
+    int64_t sc_frag_stride;
     FastDiv d_ppx, d_PC, d_region, d_rrrc, d_RC, d_n_patches, d_patches_img, d_patches_x, d_gpc, d_hg, d_nst, d_KW;
 };
 
@@ -83,6 +90,8 @@ struct SpkLaunch {
     void* out;
     float* v_out;
     LifParams lif;
+    const uint16_t* wpacked2;   // packed weight and bias of the shortcut (sc_stages > 0), else null
+    const float* bias2;
     int grid;
     size_t lds_bytes;
     hipStream_t stream;
@@ -130,11 +139,11 @@ __device__ __forceinline__ sk_u32x4 sk_expand_bits(uint32_t byte) {
     return d;
 }
 
-template <typename XT, int TT, int IN, bool SK, bool FAST>
+template <typename XT, int TT, int IN, bool SK, bool FAST, bool SC = false>
 __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_eu(TT == 1 ? 4 : 2, TT == 1 ? 4 : 2))) void conv_spk_kernel(
     const StepPtrs xs, const StepPtrs residuals, const SpkGeom g, const uint16_t* __restrict__ wpacked,
     const float* __restrict__ bias, const float* __restrict__ v_init, unsigned char* __restrict__ out,
-    float* __restrict__ v_out, const LifParams lif) {
+    float* __restrict__ v_out, const LifParams lif, const uint16_t* __restrict__ wpacked2, const float* __restrict__ bias2) {
     extern __shared__ __align__(16) unsigned char lds[];
     // ---- every cache line of the kernel arguments is touched once, in one round trip: the compiler loads the arguments
     // where they are used, all over the prologue, and each of those loads then hits the scalar cache instead of waiting
@@ -143,19 +152,20 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         auto ka = __builtin_amdgcn_kernarg_segment_ptr();
         // The explicit arguments are two step tables, the geometry, five pointers and the neuron: the last dword that is
         // touched must lie inside them (what follows is the hidden-argument area, which the compiler may leave out).
-        constexpr size_t kExplicitArgBytes = 2 * sizeof(StepPtrs) + sizeof(SpkGeom) + 5 * sizeof(void*) + sizeof(LifParams);
-        static_assert(0x280 + 4 <= kExplicitArgBytes, "argument prefetch reads past the explicit kernel arguments");
-        static_assert(kExplicitArgBytes <= 0x2c0, "argument prefetch does not cover the last cache line of the arguments");
-        uint32_t d0, d1, d2, d3, d4, d5, d6, d7, d8, d9;
+        constexpr size_t kExplicitArgBytes = 2 * sizeof(StepPtrs) + sizeof(SpkGeom) + 7 * sizeof(void*) + sizeof(LifParams);
+        static_assert(0x2c0 + 4 <= kExplicitArgBytes, "argument prefetch reads past the explicit kernel arguments");
+        static_assert(kExplicitArgBytes <= 0x300, "argument prefetch does not cover the last cache line of the arguments");
+        uint32_t d0, d1, d2, d3, d4, d5, d6, d7, d8, d9, d10;
         asm volatile(
-            "s_load_dword %0, %10, 0x40\n\ts_load_dword %1, %10, 0x80\n\ts_load_dword %2, %10, 0xc0\n\ts_load_dword %3, %10, 0x100\n\t"
-            "s_load_dword %4, %10, 0x140\n\ts_load_dword %5, %10, 0x180\n\ts_load_dword %6, %10, 0x1c0\n\ts_load_dword %7, %10, 0x200\n\t"
-            "s_load_dword %8, %10, 0x240\n\ts_load_dword %9, %10, 0x280\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(d0), "=&s"(d1), "=&s"(d2), "=&s"(d3), "=&s"(d4), "=&s"(d5), "=&s"(d6), "=&s"(d7), "=&s"(d8), "=&s"(d9)
+            "s_load_dword %0, %11, 0x40\n\ts_load_dword %1, %11, 0x80\n\ts_load_dword %2, %11, 0xc0\n\ts_load_dword %3, %11, 0x100\n\t"
+            "s_load_dword %4, %11, 0x140\n\ts_load_dword %5, %11, 0x180\n\ts_load_dword %6, %11, 0x1c0\n\ts_load_dword %7, %11, 0x200\n\t"
+            "s_load_dword %8, %11, 0x240\n\ts_load_dword %9, %11, 0x280\n\ts_load_dword %10, %11, 0x2c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(d0), "=&s"(d1), "=&s"(d2), "=&s"(d3), "=&s"(d4), "=&s"(d5), "=&s"(d6), "=&s"(d7), "=&s"(d8), "=&s"(d9), "=&s"(d10)
             : "s"(ka));
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    static_assert(!SC || (IN == SNNF_LAYOUT_BITS && TT == 4), "the shortcut variants take bit-packed inputs, four timesteps at a time");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr uint32_t ONE = F16 ? 0x3c00u : 0x3f80u;
     constexpr int kResTable = static_cast<int>(sizeof(StepPtrs));
@@ -205,6 +215,21 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             }
             e[2] = e[0];
             table[tid] = e;
+        }
+        if constexpr (SC) {
+            // The shortcut's stages: one tap, the centre of the main kernel (the lane's own pixel), on the same halo; entries
+            // behind the main table's.
+            const int i2 = tid - (nst + 4);
+            if (i2 >= 0 && i2 < hg + 4) {
+                const int gp = min(i2, hg - 1);
+                const int tapoff = (g.ph * g.RC + g.pw) * 16;
+                sk_u32x4 e;
+                e[0] = static_cast<uint32_t>(gp * kFragBytes);
+                e[1] = static_cast<uint32_t>(tapoff + (2 * gp) * region16);
+                e[2] = e[0];
+                e[3] = static_cast<uint32_t>(tapoff + (2 * gp + 1) * region16);
+                table[tid] = e;
+            }
         }
         // ---- staging descriptors of the workgroup: item e of a timestep's stage = (channel group gq, image ii, halo row r, halo
         // column c); its element offset from the stage's first item and the four coordinates, packed. Built once; the staging
@@ -277,8 +302,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
         // With K split over two waves the second one computes the tile's two 32-channel fragments in swapped places: each wave
         // then finishes the fragment in its accumulators' first half (fragment wk) and hands over the second half.
         const int swap_f = (SK && WK == 2) ? wk : 0;
-        const int64_t w_off0 = static_cast<int64_t>(min(ocf0 + swap_f, g.nocf - 1)) * g.frag_stride;
-        const int64_t w_off1 = static_cast<int64_t>(min(ocf0 + 1 - swap_f, g.nocf - 1)) * g.frag_stride;
+        const int64_t w_frag0 = min(ocf0 + swap_f, g.nocf - 1);
+        const int64_t w_frag1 = min(ocf0 + 1 - swap_f, g.nocf - 1);
 
         // ---- this lane's output pixel.
         const int n = n0 + pi;
@@ -304,6 +329,21 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         bias4[f][q] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                         if (ch0 < nbias && (!SK || wk == 0)) bias4[f][q] = *reinterpret_cast<const sk_f32x4*>(bias + ch0);
                     }
+                if constexpr (SC) {
+                    sk_f32x4 more[2][4];
+#pragma unroll
+                    for (int f = 0; f < 2; ++f)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int ch0 = oc_tile * 64 + f * 32 + q * 8 + 4 * half;
+                            more[f][q] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                            if (ch0 < nbias && (!SK || wk == 0)) more[f][q] = *reinterpret_cast<const sk_f32x4*>(bias2 + ch0);
+                        }
+#pragma unroll
+                    for (int f = 0; f < 2; ++f)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) bias4[f][q] += more[f][q];
+                }
             }
 
             // One LDS stage: G channel groups of the patch's halo for TT timesteps, from global memory into this wave's region.
@@ -317,27 +357,37 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             uint32_t pre_ok = 0;
             // Decodes the 4 items of batch jb of stage s from the workgroup's descriptors: their global index (0 when they are
             // padding) and a flag nibble (bit j: real data).
+            // A stage at or beyond g.nstages (SC only) is one of the shortcut's: same halo items, taken from the second input at
+            // the sampled positions.
             auto batch_decode = [&](int s, int jb, int lane_s, int (&idx)[4]) __attribute__((always_inline)) -> uint32_t {
-                const int gg0 = s * g.G;
-                const int base_u = ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
+                const bool second = SC && s >= g.nstages;
+                const int gg0 = (second ? s - g.nstages : s) * g.G;
+                const int c8 = second ? g.sc_C8 : g.C8in;
+                const int base_u = second ? ((n0 * g.sc_C8 + gg0) * g.sc_H + ih_lo * g.sc_sh) * g.sc_W + iw_lo * g.sc_sw
+                                          : ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
                 uint32_t ok_bits = 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const Pack<uint32_t, 2> d = desc[(jb + j) * 64 + lane_s];
                     const int r = static_cast<int>(d.v[1] & 255u), c = static_cast<int>((d.v[1] >> 8) & 255u);
                     const int ii = static_cast<int>((d.v[1] >> 16) & 255u), gq = static_cast<int>(d.v[1] >> 24);
-                    const bool ok = n0 + ii < g.N && gg0 + gq < g.C8in && static_cast<unsigned>(ih_lo + r) < static_cast<unsigned>(g.H) &&
+                    const bool ok = n0 + ii < g.N && gg0 + gq < c8 && static_cast<unsigned>(ih_lo + r) < static_cast<unsigned>(g.H) &&
                                     static_cast<unsigned>(iw_lo + c) < static_cast<unsigned>(g.W);
-                    idx[j] = ok ? base_u + static_cast<int>(d.v[0]) : 0;
+                    int off = static_cast<int>(d.v[0]);
+                    if constexpr (SC) {
+                        if (second) off = ((ii * g.sc_C8 + gq) * g.sc_H + r * g.sc_sh) * g.sc_W + c * g.sc_sw;
+                    }
+                    idx[j] = ok ? base_u + off : 0;
                     ok_bits |= ok ? (1u << j) : 0u;
                 }
                 return ok_bits;
             };
-            auto batch_load_bits = [&](const int (&idx)[4], uint32_t (&raw)[TT][4]) __attribute__((always_inline)) {
+            auto batch_load_bits = [&](int s, const int (&idx)[4], uint32_t (&raw)[TT][4]) __attribute__((always_inline)) {
+                const int ptr_table = SC && s >= g.nstages ? kResTable : 0;
 #pragma unroll
                 for (int t = 0; t < TT; ++t) {
                     const int ts = t0 + t < nsteps_t ? t0 + t : t0;   // steps beyond T repeat the window's first and are never stored
-                    const unsigned char* __restrict__ src = static_cast<const unsigned char*>(sk_kernarg_ptr(0, ts));
+                    const unsigned char* __restrict__ src = static_cast<const unsigned char*>(sk_kernarg_ptr(ptr_table, ts));
 #pragma unroll
                     for (int j = 0; j < 4; ++j) raw[t][j] = src[idx[j]];
                 }
@@ -358,7 +408,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 asm volatile("" : "+v"(lane_s));
                 int idx[4];
                 pre_ok = batch_decode(s, 0, lane_s, idx);
-                batch_load_bits(idx, pre_raw);
+                batch_load_bits(s, idx, pre_raw);
             };
             // One LDS stage: G channel groups of the patch's halo for TT timesteps, from global memory into this wave's region.
             // Item e = slot * 64 + lane of a timestep = (group, image, row, column) of the halo; its LDS address is 16 e. Items
@@ -381,7 +431,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         const uint32_t ok_bits = batch_decode(s, jb, lane_s, idx);
                         if constexpr (IN == SNNF_LAYOUT_BITS) {
                             uint32_t raw[TT][4];
-                            batch_load_bits(idx, raw);
+                            batch_load_bits(s, idx, raw);
                             batch_put_bits(jb, lane_s, ok_bits, raw);
                         } else {
 #pragma unroll
@@ -411,8 +461,9 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             // sets, activation fragments one step ahead through two.
             const int s_first = SK ? wk : 0;
             const int s_step = SK ? WK : 1;
+            const int nstages_all = SC ? g.nstages + g.sc_stages : g.nstages;
             if constexpr (PRE) {
-                if (have && s_first < g.nstages) stage_req(s_first);
+                if (have && s_first < nstages_all) stage_req(s_first);
             }
             // The epilogue's view of the tile's channel block, opaque from here on: the scalar arithmetic that depends on it
             // (per-quad base addresses and store predicates, several hundred scalar instructions that the compiler computes
@@ -437,12 +488,18 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
             if (have) {
                 const uint32_t lane16 = static_cast<uint32_t>(lane) * 16u;
                 const unsigned char* __restrict__ bl = wlds + lane_b;
-                for (int stage = s_first; stage < g.nstages; stage += s_step) {
-                    const int gg0 = stage * g.G;
-                    const int chunk = gg0 >> g.gpc_log2;
-                    const int pbase = chunk * g.npairs + ((gg0 - (chunk << g.gpc_log2)) >> 1);   // pair of (tap 0, the stage's first two groups)
-                    const unsigned char* __restrict__ pa0 = reinterpret_cast<const unsigned char*>(wpacked + w_off0 + static_cast<int64_t>(pbase) * (kFragBytes / 2));
-                    const unsigned char* __restrict__ pa1 = reinterpret_cast<const unsigned char*>(wpacked + w_off1 + static_cast<int64_t>(pbase) * (kFragBytes / 2));
+                for (int stage = s_first; stage < nstages_all; stage += s_step) {
+                    const bool second = SC && stage >= g.nstages;     // a stage of the shortcut
+                    const int gg0 = (second ? stage - g.nstages : stage) * g.G;
+                    const int gpc_l2 = second ? g.sc_gpc_log2 : g.gpc_log2;
+                    const int chunk = gg0 >> gpc_l2;
+                    const int pbase = chunk * (second ? g.sc_npairs : g.npairs) + ((gg0 - (chunk << gpc_l2)) >> 1);   // pair of (tap 0, the stage's first two groups)
+                    const uint16_t* __restrict__ wp = second ? wpacked2 : wpacked;
+                    const int64_t fs = second ? g.sc_frag_stride : g.frag_stride;
+                    const unsigned char* __restrict__ pa0 = reinterpret_cast<const unsigned char*>(wp + w_frag0 * fs + static_cast<int64_t>(pbase) * (kFragBytes / 2));
+                    const unsigned char* __restrict__ pa1 = reinterpret_cast<const unsigned char*>(wp + w_frag1 * fs + static_cast<int64_t>(pbase) * (kFragBytes / 2));
+                    const Pack<uint32_t, 2>* __restrict__ tb = second ? table + 2 * (nst + 4) : table;
+                    const int nst_s = second ? hg : nst;
                     sk_u32x4 wa[4][2];
                     sk_u32x4 wb[2][TT];
                     uint32_t bo[4];
@@ -464,13 +521,13 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                             acc[t][1] = sk_mfma<F16>(wa[sa][1], wb[sb][t], acc[t][1]);
                         }
                     };
-                    req_a(0, table[0]);
-                    req_a(1, table[2]);
-                    req_a(2, table[4]);
-                    Pack<uint32_t, 2> ent = table[6];       // entry of the step whose weights are requested next
+                    req_a(0, tb[0]);
+                    req_a(1, tb[2]);
+                    req_a(2, tb[4]);
+                    Pack<uint32_t, 2> ent = tb[6];       // entry of the step whose weights are requested next
                     stage_in(stage);
                     if constexpr (PRE) {
-                        if (stage + s_step < g.nstages) stage_req(stage + s_step);
+                        if (stage + s_step < nstages_all) stage_req(stage + s_step);
                     }
                     read_b(0, bo[0]);
                     int st = 0;
@@ -506,36 +563,36 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     };
-                    for (; st + 4 <= nst; st += 4) {
+                    for (; st + 4 <= nst_s; st += 4) {
                         req_a(3, ent);
-                        ent = table[2 * (st + 4)];
+                        ent = tb[2 * (st + 4)];
                         read_b(1, bo[1]);
                         mma(0, 0);
                         step_order();
                         req_a(0, ent);
-                        ent = table[2 * (st + 5)];
+                        ent = tb[2 * (st + 5)];
                         read_b(0, bo[2]);
                         mma(1, 1);
                         step_order();
                         req_a(1, ent);
-                        ent = table[2 * (st + 6)];
+                        ent = tb[2 * (st + 6)];
                         read_b(1, bo[3]);
                         mma(2, 0);
                         step_order();
                         req_a(2, ent);
-                        ent = table[2 * (st + 7)];
+                        ent = tb[2 * (st + 7)];
                         read_b(0, bo[0]);
                         mma(3, 1);
                         step_order();
                     }
                     // The last nst % 4 steps: wa[0..2] hold their weight fragments, wb[0] the first one's activations.
-                    if (st < nst) {
-                        if (st + 1 < nst) read_b(1, bo[1]);
+                    if (st < nst_s) {
+                        if (st + 1 < nst_s) read_b(1, bo[1]);
                         mma(0, 0);
-                        if (st + 1 < nst) {
-                            if (st + 2 < nst) read_b(0, bo[2]);
+                        if (st + 1 < nst_s) {
+                            if (st + 2 < nst_s) read_b(0, bo[2]);
                             mma(1, 1);
-                            if (st + 2 < nst) mma(2, 0);
+                            if (st + 2 < nst_s) mma(2, 0);
                         }
                     }
                 }
@@ -1076,11 +1133,25 @@ int launch_conv_spk_variant(const SpkLaunch& L) {
     auto run = [&](auto kernel) -> int {
         if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif_blocked"); rc != SNNF_OK) return rc;
         kernel<<<dim3(L.grid), kSpkWaves * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.g, L.wpacked, L.bias, L.v_init,
-                                                                        static_cast<unsigned char*>(L.out), L.v_out, L.lif);
+                                                                        static_cast<unsigned char*>(L.out), L.v_out, L.lif, L.wpacked2, L.bias2);
         return check_launch("snnf_conv_lif_blocked");
     };
     if (L.fast_epilogue) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true, true>) : run(conv_spk_kernel<XT, TT, IN, false, true>);
     return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true, false>) : run(conv_spk_kernel<XT, TT, IN, false, false>);
+}
+
+// The variants with a projection shortcut in the accumulators: bit-packed inputs, four timesteps side by side.
+template <typename XT>
+int launch_conv_spk_shortcut(const SpkLaunch& L) {
+    auto run = [&](auto kernel) -> int {
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif_blocked_shortcut"); rc != SNNF_OK) return rc;
+        kernel<<<dim3(L.grid), kSpkWaves * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.g, L.wpacked, L.bias, L.v_init,
+                                                                        static_cast<unsigned char*>(L.out), L.v_out, L.lif, L.wpacked2, L.bias2);
+        return check_launch("snnf_conv_lif_blocked_shortcut");
+    };
+    constexpr int B = SNNF_LAYOUT_BITS;
+    if (L.fast_epilogue) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 4, B, true, true, true>) : run(conv_spk_kernel<XT, 4, B, false, true, true>);
+    return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 4, B, true, false, true>) : run(conv_spk_kernel<XT, 4, B, false, false, true>);
 }
 
 template <typename XT, int IN>
@@ -1095,5 +1166,7 @@ int launch_conv_spk_bf16_bits(const SpkLaunch& L, int tt);
 int launch_conv_spk_bf16_c8(const SpkLaunch& L, int tt);
 int launch_conv_spk_f16_bits(const SpkLaunch& L, int tt);
 int launch_conv_spk_f16_c8(const SpkLaunch& L, int tt);
+int launch_conv_spk_bf16_shortcut(const SpkLaunch& L);
+int launch_conv_spk_f16_shortcut(const SpkLaunch& L);
 
 }  // namespace snnf

@@ -774,6 +774,22 @@ def blocked_conv_lif(x, weight, bias, stride, padding, lif, residual, out_layout
     return out
 
 
+def blocked_conv_lif_shortcut(x, weight, bias, padding, lif, shortcut_x, shortcut_weight, shortcut_bias, shortcut_stride, out_layout: int):
+    """The second convolution of a residual block with the block's 1x1 projection shortcut accumulated in the same launch
+    (LIF(conv(x) + conv1x1(shortcut_x))); the two convolutions one after the other where the kernel does not take the pair."""
+    from .runtime import hip_blocked_backend as B
+    try:
+        out, _ = B.conv_lif_blocked_shortcut(x, weight, bias, padding, shortcut_x, shortcut_weight, shortcut_bias, shortcut_stride, lif,
+                                             out_layout=out_layout)
+        return out
+    except RuntimeError as exc:
+        if "unsupported" not in str(exc):
+            raise
+    shortcut, _ = B.conv_lif_blocked_or_dense(shortcut_x, shortcut_weight, shortcut_bias, shortcut_stride, [0, 0], None, out_layout=B.C8)
+    out, _ = B.conv_lif_blocked_or_dense(x, weight, bias, [1, 1], padding, lif, residual=shortcut, out_layout=out_layout)
+    return out
+
+
 def blocked_pool(x, is_max: bool, kernel: int, stride: int, padding: int):
     from .runtime import hip_blocked_backend as B
     try:
@@ -941,6 +957,37 @@ def propagate_internal_layouts(gm: fx.GraphModule) -> int:
                 new = graph.call_function(blocked_pool, (blocked_of[node.args[0]], *node.args[1:]))
             blocked_of[stack] = new
             converted += 1
+    # Projection shortcuts: a LIF-free 1x1 convolution whose only reader is the residual operand of a plane-keeping fused
+    # convolution becomes further K steps of that convolution (one launch, the shortcut's sums never stored).
+    def weight_shape(arg):
+        if isinstance(arg, fx.Node) and arg.op == "get_attr":
+            value = gm
+            for part in arg.target.split("."):
+                value = getattr(value, part)
+            return tuple(value.shape)
+        return None
+
+    for stack, node in list(blocked_of.items()):
+        if node.target is not blocked_conv_lif or node.args[5] is None:
+            continue
+        x_main, w, b, stride, padding, lif, shortcut, out_layout = node.args
+        if not (isinstance(shortcut, fx.Node) and shortcut.target is blocked_conv_lif and shortcut.args[5] is None and shortcut.args[6] is None):
+            continue
+        sc_stack = next((s for s, n in blocked_of.items() if n is shortcut), None)
+        shape, sc_shape = weight_shape(w), weight_shape(shortcut.args[1])
+        if (sc_stack is None or shape is None or sc_shape is None or len(shortcut.users) != 1 or reads_blocked(sc_stack)[1]
+                or sc_shape[2:] != (1, 1) or list(shortcut.args[4]) != [0, 0] or list(stride) != [1, 1]
+                or [2 * p + 1 for p in padding] != list(shape[2:]) or shape[1] % 16 or sc_shape[1] % 16):
+            continue
+        with graph.inserting_before(node):
+            fused = graph.call_function(blocked_conv_lif_shortcut, (x_main, w, b, list(padding), lif, shortcut.args[0], shortcut.args[1],
+                                                                    shortcut.args[2], list(shortcut.args[3]), out_layout))
+        node.replace_all_uses_with(fused)
+        blocked_of[stack] = fused
+        del blocked_of[sc_stack]
+        graph.erase_node(node)
+        graph.erase_node(shortcut)
+        converted -= 1
     # Phase 2: whoever still reads a converted stack as a tensor gets it converted back (a no-op for dense outputs).
     for stack, new in blocked_of.items():
         with graph.inserting_after(new):

@@ -393,6 +393,27 @@ class _FusedNetwork(nn.Module):
                           y=B.to_dense(out), native=True, blocked=True)
         return out
 
+    def conv_lif_shortcut_b(self, name: str, x, layer: _FusedLayer, shortcut_x, shortcut: _FusedLayer, out_layout=None):
+        """The second convolution of a down-sampling block with the block's LIF-free 1x1 shortcut in its accumulators (one
+        launch); None when the kernel does not take the pair in this form (the caller then runs the two apart)."""
+        from .runtime import hip_blocked_backend as B
+        if out_layout is None:
+            out_layout = B.BITS if layer.lif is not None else B.C8
+        if layer.stride != [1, 1] or shortcut.padding != [0, 0] or tuple(shortcut.weight.shape[2:]) != (1, 1):
+            return None
+        try:
+            out, v = B.conv_lif_blocked_shortcut(x, layer.weight, layer.bias, layer.padding, shortcut_x, shortcut.weight, shortcut.bias,
+                                                 shortcut.stride, layer.lif, out_layout=out_layout,
+                                                 want_v=self.keep_membranes or self.record is not None)
+        except RuntimeError as exc:
+            if "unsupported" not in str(exc):
+                raise
+            return None
+        if self.record is not None:
+            self._log(kind="conv_lif", name=name, xs=list(B.to_dense(x).unbind(0)), residuals=None, layer=layer, spikes=B.to_dense(out), v=v,
+                      blocked=True, shortcut=dict(x=B.to_dense(shortcut_x), layer=shortcut))
+        return out
+
     def pooled_b(self, name: str, x, pool: nn.Module):
         from .runtime import hip_blocked_backend as B
         from .runtime.hip_pool_backend import pool_config
@@ -518,16 +539,22 @@ class FusedSpikingResNet18(_FusedNetwork):
         return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
 
     def run_blocked(self, x):
-        """Stem on the channel-blocked frame, everything after it on bit-packed spikes; the LIF-free shortcuts produce
-        blocked analog residuals; the last block's sum is written dense for the tail."""
+        """Stem on the channel-blocked frame, everything after it on bit-packed spikes; a LIF-free shortcut convolution is
+        accumulated inside the block's second convolution (or, where that kernel does not take the pair, produces a blocked
+        analog residual); the last block's sum is written dense for the tail."""
         from .runtime import hip_blocked_backend as B
         frame = B.from_dense(x, B.C8, shared=True)
         frame.T = self.T
         seq = self.conv_lif_b("stem", frame, self.stem)
         seq = self.pooled_b("maxpool", seq, self.maxpool)
         for i, (conv1, conv2, down) in enumerate(self.block_layers):
-            identity = seq if down is None else self.conv_lif_b(f"blocks.{i}.downsample", seq, down)
             hidden = self.conv_lif_b(f"blocks.{i}.conv1", seq, conv1)
+            if down is not None and conv2.lif is not None:
+                fused = self.conv_lif_shortcut_b(f"blocks.{i}.conv2", hidden, conv2, seq, down)
+                if fused is not None:
+                    seq = fused
+                    continue
+            identity = seq if down is None else self.conv_lif_b(f"blocks.{i}.downsample", seq, down)
             if conv2.lif is not None:
                 seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity)
             else:   # last block: its neuron is the tail's

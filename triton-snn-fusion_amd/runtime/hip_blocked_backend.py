@@ -222,6 +222,47 @@ def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tens
     return out, v_out
 
 
+def conv_lif_blocked_shortcut(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], padding,
+                              shortcut_x: Blocked, shortcut_weight: torch.Tensor, shortcut_bias: Optional[torch.Tensor], shortcut_stride,
+                              lif: Optional[Sequence[float]], out_layout: int = BITS, want_v: bool = False):
+    """The second convolution of a residual block with the block's projection shortcut in the same accumulators:
+    LIF(conv(x) + bias + conv1x1(shortcut_x, stride) + shortcut bias), both inputs bit-packed, the main convolution keeping
+    its plane (stride 1, "same" padding). One launch instead of two, and the shortcut's output never exists in memory.
+    Raises RuntimeError("unsupported_shortcut: ...") for layers the kernel does not take in this form (the caller then
+    runs the shortcut as a convolution of its own and hands its output to conv_lif_blocked as the residual).
+    Returns (Blocked output, final membrane or None)."""
+    if x.layout != BITS or shortcut_x.layout != BITS:
+        raise RuntimeError("unsupported_shortcut: both inputs must be bit-packed")
+    if weight.dim() != 4 or shortcut_weight.dim() != 4 or int(weight.shape[1]) != x.C or int(shortcut_weight.shape[1]) != shortcut_x.C or \
+            tuple(shortcut_weight.shape[2:]) != (1, 1) or int(shortcut_weight.shape[0]) != int(weight.shape[0]):
+        raise RuntimeError(f"unsupported_shortcut: weights {tuple(weight.shape)} / {tuple(shortcut_weight.shape)} do not match the inputs")
+    if weight.dtype != x.dtype or shortcut_weight.dtype != x.dtype or shortcut_x.dtype != x.dtype:
+        raise RuntimeError("unsupported_dtype: weight dtypes must be the activation dtype")
+    if (shortcut_x.T, shortcut_x.N) != (x.T, x.N) or x.shared or shortcut_x.shared:
+        raise RuntimeError("unsupported_shortcut: the two inputs must have the same timesteps and batch, one frame per timestep")
+    cout, _, kh, kw = (int(d) for d in weight.shape)
+    ph, pw = _as_pair(padding)
+    ssh, ssw = _as_pair(shortcut_stride)
+    dev = x.data.device
+    if bias is None:
+        bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    if shortcut_bias is None:
+        shortcut_bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    if _TUNED is None:
+        load_tuned_plans()
+    packed = _packed_weight(weight, bias, x.dtype)
+    packed_sc = _packed_weight(shortcut_weight, shortcut_bias, x.dtype)
+    out = empty_blocked(out_layout, x.T, x.N, cout, x.H, x.W, x.dtype, dev)
+    neuron = lif is not None
+    v_out = torch.empty((x.N, cout, x.H, x.W), dtype=torch.float32, device=dev) if neuron and (want_v or x.T > 4) else None
+    v_th, v_reset, tau = (float(lif[0]), float(lif[1]), float(lif[2])) if neuron else (1.0, 0.0, 2.0)
+    _lib.check("snnf_conv_lif_blocked_shortcut", _lib.lib().snnf_conv_lif_blocked_shortcut(
+        x.step_pointers(), shortcut_x.step_pointers(), x.T, x.N, x.C, x.H, x.W, _lib.dtype_code(x.dtype), packed.data_ptr(), cout, kh, kw,
+        ph, pw, shortcut_x.C, shortcut_x.H, shortcut_x.W, ssh, ssw, packed_sc.data_ptr(), None, out.data.data_ptr(), out_layout,
+        out.step_stride_bytes(), _lib.ptr(v_out), 1 if neuron else 0, v_th, v_reset, tau, _lib.current_stream(dev)))
+    return out, v_out
+
+
 def conv_lif_dense_on_blocked(x: Blocked, weight: torch.Tensor, bias: torch.Tensor, stride, padding, lif: Optional[Sequence[float]],
                               residual: Optional[Blocked] = None, out_layout: int = BITS):
     """The same layer through the dense entry points on unpacked tensors, for a layer the internal-layout kernel refuses

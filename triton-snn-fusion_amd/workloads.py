@@ -147,6 +147,14 @@ RESNET18_LAYERS = [
     ("3x3/2 256->512 @14", 256, 512, 14, 3, 2, 1, False, False, 1), ("1x1/2 256->512 @14", 256, 512, 14, 1, 2, 0, False, False, 1),
     ("3x3 512->512 @7", 512, 512, 7, 3, 1, 1, False, False, 1), ("3x3 512->512 @7 +res", 512, 512, 7, 3, 1, 1, True, False, 2),
 ]
+# The down-sampling blocks of the ResNet-18 configuration as the internal-layout executor runs them: the block's second
+# convolution with the 1x1 stride-2 shortcut accumulated in the same launch, in place of one "+res" layer and the shortcut layer.
+# (name, the "+res" layer it stands for, the shortcut layer it absorbs, channels, plane size, shortcut channels, shortcut plane size)
+RESNET18_SHORTCUT_BLOCKS = [
+    ("3x3 128->128 @28 + 1x1/2 64->128 @56", "3x3 128->128 @28 +res", "1x1/2 64->128 @56", 128, 28, 64, 56),
+    ("3x3 256->256 @14 + 1x1/2 128->256 @28", "3x3 256->256 @14 +res", "1x1/2 128->256 @28", 256, 14, 128, 28),
+    ("3x3 512->512 @7 + 1x1/2 256->512 @14", "3x3 512->512 @7 +res", "1x1/2 256->512 @14", 512, 7, 256, 14),
+]
 VGG11_LAYERS = [
     ("3x3 3->64 @32", 3, 64, 32, 3, 1, 1, False, True, 1), ("3x3 64->128 @16", 64, 128, 16, 3, 1, 1, False, False, 1),
     ("3x3 128->256 @8", 128, 256, 8, 3, 1, 1, False, False, 1), ("3x3 256->256 @8", 256, 256, 8, 3, 1, 1, False, False, 1),
