@@ -334,6 +334,24 @@ int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void* const* sho
                                    int neuron, float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * Convolution + bias + LIF followed by a 2 x 2 / stride 2 average pool of the spikes, in one launch: the four lanes that
+ * hold a pooling window add their spikes in registers and the kernel writes the quarters (0, 1/4, ..., 1: exact in 16 bits)
+ * channel-blocked at half the plane; the spikes themselves are never stored. The reference runs the pool as a layer of its
+ * own between two fused operators (its rewrite leaves nn.AvgPool2d in the graph, compiler/fx_lif_temporal_rewrite.py:
+ * 2214-2333); results are identical to snnf_conv_lif_blocked followed by snnf_pool2d_blocked, bit for bit.
+ *   xs, x_layout, packed_weight, geometry, LIF parameters : as in snnf_conv_lif_blocked (no residual, zero initial membrane)
+ *   out   : T x N frames [Cout, Ho / 2, Wo / 2] in C8, `out_step_stride` BYTES between timesteps
+ *   v_out : [N, Cout, Ho, Wo] fp32 NCHW (the membrane of the unpooled neurons) or NULL
+ * T == 4 (distinct inputs, or one shared frame), Ho and Wo even, Cout a multiple of 8, tau == 2 with v_reset == 0;
+ * SNNF_ERR_UNSUPPORTED ("unsupported_pool: ...") otherwise: the caller then runs the pool as a launch of its own.
+ */
+int snnf_conv_lif_blocked_avgpool(const void* const* xs, int x_layout, int T, int N, int Cin, int H, int W, int x_dtype,
+                                  const void* packed_weight, int Cout, int KH, int KW,
+                                  int stride_h, int stride_w, int pad_h, int pad_w,
+                                  void* out, int64_t out_step_stride, void* v_out,
+                                  float v_threshold, float v_reset, float tau, void* stream);
+
+/*
  * Registers a measured launch choice for snnf_conv_lif_blocked on one layer shape (the counterpart of the per-kernel-key
  * "best config" the reference's autotuner keeps, kernels/benchmark_conv_lif_temporal_general.py:524-558,1332-1369):
  * columns of a wave's output patch (rows follow: 32 / columns), channel groups of 8 per LDS stage (a power of two) and

@@ -216,6 +216,64 @@ def test_blocked_conv_shortcut_rejects_what_it_does_not_take(B):
         B.conv_lif_blocked_shortcut(x2, dw, db, [1, 1], sc(32, 15, 15, 2), w2, None, [2, 2], LIF)
 
 
+POOLED_CASES = [  # Cin, Cout, H, W, k, s, p, N, dtype, input: "bits" | "c8" | "frame" (one analog frame for the four steps)
+    (64, 128, 16, 16, 3, 1, 1, 4, BF16, "bits"),      # VGG-11's second layer
+    (3, 64, 32, 32, 3, 1, 1, 2, BF16, "frame"),       # its first: one frame, four LIF steps
+    (256, 256, 8, 8, 3, 1, 1, 4, BF16, "c8"),         # analog blocked input (the layer behind a pool), K shared by waves
+    (512, 512, 4, 4, 3, 1, 1, 6, BF16, "c8"),         # 4x4 planes: two images per patch
+    (128, 64, 2, 2, 3, 1, 1, 20, BF16, "bits"),       # 2x2 planes: eight images per patch, one window each
+    (64, 72, 12, 20, 3, 1, 1, 3, F16, "bits"),        # fp16, 72 channels, a plane that is no multiple of the patch
+    (64, 64, 16, 24, 3, 2, 1, 2, BF16, "bits"),       # stride 2 onto an 8x12 plane
+    (32, 64, 20, 12, 5, 1, 2, 2, BF16, "bits"),       # 5x5
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,W,k,s,p,N,dtype,inl", POOLED_CASES)
+def test_blocked_conv_with_its_average_pool_in_the_same_launch(B, Cin, Cout, H, W, k, s, p, N, dtype, inl):
+    """conv + LIF + 2x2 average pool in one launch: bit for bit the two launches, and the unpooled neurons' membrane and the
+    pooled spikes against the oracle."""
+    T = 4
+    xs, w, b = _case(3500 + Cin + Cout + H + k, T, N, Cin, Cout, H, W, k, dtype, analog=inl != "bits", shared=inl == "frame")
+    frames = [xs[0]] * T if inl == "frame" else [xs[t] for t in range(T)]
+    ref = O.temporal_conv_lif(frames, w, b, torch.tensor(0.0), (s, s), (p, p), (1, 1), 1, *LIF)
+    if inl == "frame":
+        x = B.from_dense(dev(xs[0], dtype), B.C8, shared=True)
+        x.T = T
+    else:
+        x = _to_layout(B, xs, inl, dtype)
+    dw, db = dev(w, dtype), dev(b, dtype)
+    print(f"blocked conv + pool {Cin}->{Cout} {H}x{W} k{k} N={N} {inl}", flush=True)
+    pooled, v = B.conv_lif_blocked_avgpool(x, dw, db, [s, s], [p, p], LIF, want_v=True)
+    torch.cuda.synchronize()
+    Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    assert pooled.layout == B.C8 and pooled.shape == (T, N, Cout, Ho // 2, Wo // 2)
+    spikes_out, v2 = B.conv_lif_blocked(x, dw, db, [s, s], [p, p], LIF, want_v=True)
+    two = B.pool_blocked(spikes_out, False, 2, 2, 0)
+    assert torch.equal(pooled.data, two.data) and torch.equal(v, v2)
+    rep = check(B.to_dense(spikes_out), v, ref, what=f"blocked {Cin}->{Cout} k{k} + pool")
+    assert 0.001 < float(ref[0].mean()) < 0.9, float(ref[0].mean())
+    got = B.to_dense(pooled).float().cpu()
+    want = torch.nn.functional.avg_pool2d(ref[0].flatten(0, 1), 2).reshape(got.shape)
+    assert float((got != want).float().mean()) <= 4 * (1.0 - rep["neurons_with_matching_history"] / rep["neurons"]) + 1e-9
+    if Cout % 8:
+        assert float(pooled.data[:, :, -1, :, :, Cout % 8:].abs().max()) == 0.0
+
+
+def test_blocked_conv_with_pool_rejects_what_it_does_not_take(B):
+    xs, w, b = _case(3550, 4, 2, 64, 64, 17, 17, 3, BF16)
+    x = B.from_dense(dev(xs, BF16), B.BITS)
+    dw, db = dev(w, BF16), dev(b, BF16)
+    with pytest.raises(RuntimeError, match="unsupported_pool"):       # 17 -> 9: odd plane
+        B.conv_lif_blocked_avgpool(x, dw, db, [2, 2], [1, 1], LIF)
+    xs2, w2, b2 = _case(3551, 4, 2, 64, 64, 8, 8, 3, BF16)
+    x2 = B.from_dense(dev(xs2, BF16), B.BITS)
+    with pytest.raises(RuntimeError, match="unsupported_pool"):       # tau 3: not the straight-line epilogue
+        B.conv_lif_blocked_avgpool(x2, dev(w2, BF16), dev(b2, BF16), [1, 1], [1, 1], (1.0, 0.0, 3.0))
+    x3 = B.from_dense(dev(xs2[:3], BF16), B.BITS)
+    with pytest.raises(RuntimeError, match="unsupported_pool"):       # three timesteps
+        B.conv_lif_blocked_avgpool(x3, dev(w2, BF16), dev(b2, BF16), [1, 1], [1, 1], LIF)
+
+
 def test_blocked_conv_without_membrane_output_and_chained_windows(B):
     """The final membrane is optional; two calls chained through it equal one call of all steps, bit for bit."""
     T, N, C, H = 4, 2, 64, 12

@@ -21,11 +21,12 @@ struct SpkPlan {
 // Patch of a wave (PR x PC output pixels of one image, or PI whole planes when a plane has at most 32 pixels) and the
 // channel groups per LDS stage G: the patch with the most useful matrix lanes and the smallest halo whose stage fits the
 // wave's LDS region and its staging slots; the largest such G (fewer, longer stages).
-bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best, int only_pc = 0, int only_g = 0) {
+bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best, int only_pc = 0, int only_g = 0, bool even = false) {
     best.score = -1.0;
     for (int pc = 1; pc <= 32 && pc <= g0.Wo; ++pc) {
         if (only_pc > 0 && pc != only_pc) continue;
         const int pr = std::min(32 / pc, g0.Ho);
+        if (even && ((pc & 1) || (pr & 1))) continue;   // 2x2 windows of the output must lie inside a patch
         const bool whole = pr == g0.Ho && pc == g0.Wo;
         const int pi = whole ? std::max(1, std::min(g0.N, 32 / (pr * pc))) : 1;
         const int rr = (pr - 1) * g0.sh + g0.KH;
@@ -88,7 +89,7 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
                           int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
                           int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
                           int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
-                          float v_reset, float tau, void* stream, const Shortcut* sc);
+                          float v_reset, float tau, void* stream, const Shortcut* sc, bool pool2 = false);
 }  // namespace
 
 }  // namespace snnf
@@ -131,13 +132,22 @@ extern "C" int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void*
                                  pad_h, pad_w, v_init, out, out_layout, out_step_stride, v_out, neuron, v_threshold, v_reset, tau, stream, &sc);
 }
 
+extern "C" int snnf_conv_lif_blocked_avgpool(const void* const* xs, int x_layout, int T, int N, int Cin, int H, int W, int x_dtype,
+                                             const void* packed_weight, int Cout, int KH, int KW, int stride_h, int stride_w, int pad_h,
+                                             int pad_w, void* out, int64_t out_step_stride, void* v_out, float v_threshold, float v_reset,
+                                             float tau, void* stream) {
+    return snnf::conv_lif_blocked_impl("snnf_conv_lif_blocked_avgpool", xs, x_layout, nullptr, 0, T, N, Cin, H, W, x_dtype, packed_weight, Cout, KH,
+                                       KW, stride_h, stride_w, pad_h, pad_w, nullptr, out, SNNF_LAYOUT_C8, out_step_stride, v_out, 1, v_threshold,
+                                       v_reset, tau, stream, nullptr, true);
+}
+
 namespace snnf {
 namespace {
 int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, const void* const* residuals, int res_layout, int T,
                           int N, int Cin, int H, int W, int x_dtype, const void* packed_weight, int Cout, int KH,
                           int KW, int stride_h, int stride_w, int pad_h, int pad_w, const void* v_init, void* out,
                           int out_layout, int64_t out_step_stride, void* v_out, int neuron, float v_threshold,
-                          float v_reset, float tau, void* stream, const Shortcut* sc) {
+                          float v_reset, float tau, void* stream, const Shortcut* sc, bool pool2) {
     if (xs == nullptr || packed_weight == nullptr || out == nullptr)
         return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: xs, packed_weight and out must be non-null", who);
     if (T < 1 || N < 1 || Cin < 1 || H < 1 || W < 1 || Cout < 1 || KH < 1 || KW < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0)
@@ -228,11 +238,15 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
         if (it != tuned_plans().end()) tuned = it->second;
     }
     SpkPlan pl = {};
-    bool planned = (tuned.patch_cols > 0 || tuned.stage_groups > 0) && plan_spk(g, tt, pl, tuned.patch_cols, tuned.stage_groups);
+    if (pool2 && (!neuron || T != 4 || (g.Ho & 1) || (g.Wo & 1) || residuals != nullptr || v_init != nullptr || Cout % 8 != 0))
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_pool: needs four timesteps, a neuron from the zero membrane, no residual, an even %dx%d output plane and whole channel groups",
+                    who, g.Ho, g.Wo);
+    bool planned = (tuned.patch_cols > 0 || tuned.stage_groups > 0) && plan_spk(g, tt, pl, tuned.patch_cols, tuned.stage_groups, pool2);
     const bool tuned_patch = planned;
     for (; !planned && tt >= 1; tt >>= 1) {
-        planned = plan_spk(g, tt, pl);
+        planned = plan_spk(g, tt, pl, 0, 0, pool2);
         if (planned) break;
+        if (pool2) break;   // the pooled store covers the four steps of one window
     }
     if (!planned)
         return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: no patch of this layer fits a wave's LDS region (kernel %dx%d, stride %dx%d)",
@@ -336,7 +350,7 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
     L.grid = grid;
     L.lds_bytes = lds_bytes;
     L.stream = as_stream(stream);
-    const bool fast_epi = neuron && out_layout == SNNF_LAYOUT_BITS && (residuals == nullptr || res_layout == SNNF_LAYOUT_BITS) &&
+    const bool fast_epi = neuron && (out_layout == SNNF_LAYOUT_BITS || pool2) && (residuals == nullptr || res_layout == SNNF_LAYOUT_BITS) &&
                           L.lif.charge_mode == CHARGE_SCALE && L.lif.inv_tau == 0.5f && L.lif.v_reset == 0.0f &&
                           L.lif.v_threshold >= 1e-30f && L.lif.v_threshold <= 1e30f &&   // its multiples by 2^t stay normal numbers
                           v_init == nullptr && windows == 1 && Cout % 8 == 0;
@@ -346,6 +360,12 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
              (wk_log2 > 0 ? 50 : 40) + tt + (fast_epi ? 20 : 0), shared ? T : tt, g.PI, g.PR, g.PC, g.RR, g.RC, 1 << wk_log2, oc_tiles, g.n_patches, g.G,
              L.lds_bytes, grid, (tuned_patch ? 1 : 0) + (tuned_split ? 2 : 0), g.sc_stages);
     L.fast_epilogue = fast_epi;
+    if (pool2) {
+        if (!fast_epi || windows != 1 || (tt != 4 && !shared))
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_pool: the pooled output needs the usual neuron (tau 2, hard reset to 0) and the four steps in one window", who);
+        L.g.pool2 = 1;
+        return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_pooled(L, tt) : launch_conv_spk_f16_pooled(L, tt);
+    }
     if (sc != nullptr) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_shortcut(L) : launch_conv_spk_f16_shortcut(L);
     if (x_layout == SNNF_LAYOUT_BITS) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_bits(L, tt) : launch_conv_spk_f16_bits(L, tt);
     return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_c8(L, tt) : launch_conv_spk_f16_c8(L, tt);

@@ -67,6 +67,7 @@ struct SpkGeom {
     int n_items, iters;          // (patch, 64-channel tile) pairs; loop trips per wave
     int in_layout, res_layout, out_layout;   // snnf_layout codes; res_layout < 0: no residual
     int analog_out;              // no neuron: the sums themselves are written (C8 or NCHW)
+    int pool2;                   // the POOL variants: the spikes leave as their 2x2 averages (quarters, C8, half the plane)
     int64_t out_step_stride;     // bytes between timesteps of `out`
     int lds_wave_bytes;          // private staging region of a wave (a multiple of 16)
     int64_t frag_stride;         // 16-bit elements between consecutive 32-row fragments of the packed weight
@@ -139,7 +140,7 @@ __device__ __forceinline__ sk_u32x4 sk_expand_bits(uint32_t byte) {
     return d;
 }
 
-template <typename XT, int TT, int IN, bool SK, bool FAST, bool SC = false>
+template <typename XT, int TT, int IN, bool SK, bool FAST, bool SC = false, bool POOL = false>
 __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_eu(TT == 1 ? 4 : 2, TT == 1 ? 4 : 2))) void conv_spk_kernel(
     const StepPtrs xs, const StepPtrs residuals, const SpkGeom g, const uint16_t* __restrict__ wpacked,
     const float* __restrict__ bias, const float* __restrict__ v_init, unsigned char* __restrict__ out,
@@ -166,6 +167,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
     __builtin_amdgcn_sched_barrier(0);
 
     static_assert(!SC || (IN == SNNF_LAYOUT_BITS && TT == 4), "the shortcut variants take bit-packed inputs, four timesteps at a time");
+    static_assert(!POOL || (FAST && (TT == 4 || TT == 1)), "the pooled output belongs to the straight-line epilogue of four steps");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr uint32_t ONE = F16 ? 0x3c00u : 0x3f80u;
     constexpr int kResTable = static_cast<int>(sizeof(StepPtrs));
@@ -830,6 +832,39 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         static_cast<unsigned char>(((both[0] >> (sh - 8u)) & 15u) | (((both[1] >> (sh - 8u)) & 15u) << 4));
                 }
             };
+            // The four steps 0..3 as 2x2 average pools of the spikes (POOL): the four lanes of a window (patches have even
+            // extents, so a window lies inside one wave half) hold one byte-wide count per channel and step, add them in a
+            // reduce-scatter of two exchanges (first with the horizontal neighbour, two steps each way; then with the vertical
+            // one, one step each way), and the lane at window position (row r, column c) ends up with step 2 c + r, whose
+            // four quarters it stores as 16-bit values of the pooled, channel-blocked tensor.
+            auto fast_store4_pooled = [&](int j8, uint32_t quiet) __attribute__((always_inline)) {
+                const uint32_t fired = ~quiet;
+                uint32_t w[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) w[t] = __umul24((fired >> (4 * (3 - t))) & 15u, 0x00204081u) & 0x01010101u;
+                int lane_e = lane;
+                asm volatile("" : "+v"(lane_e));
+                const uint32_t pos = reinterpret_cast<const uint32_t*>(lds + kSpkTableBytes + kSpkDescBytes)[lane_e & 31];
+                const int pi_e = static_cast<int>(pos & 255u), prow_e = static_cast<int>((pos >> 8) & 255u), pcol_e = static_cast<int>(pos >> 16);
+                const bool odd_col = (pcol_e & 1) != 0, odd_row = (prow_e & 1) != 0;
+                uint32_t keep0 = odd_col ? w[2] : w[0], keep1 = odd_col ? w[3] : w[1];
+                const uint32_t give0 = odd_col ? w[0] : w[2], give1 = odd_col ? w[1] : w[3];
+                const int side = (lane_e ^ 1) * 4;
+                keep0 += static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(side, static_cast<int>(give0)));
+                keep1 += static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(side, static_cast<int>(give1)));
+                uint32_t keep = odd_row ? keep1 : keep0;
+                const uint32_t give = odd_row ? keep0 : keep1;
+                keep += static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((lane_e + (odd_row ? -g.PC : g.PC)) * 4, static_cast<int>(give)));
+                if (j8 < g.C8out && px_ok) {
+                    const int step = (odd_col ? 2 : 0) + (odd_row ? 1 : 0);
+                    const int hp = g.Ho >> 1, wp = g.Wo >> 1;
+                    const uint32_t off = static_cast<uint32_t>(((((n0 + pi_e) * g.C8out + j8) * hp + ((oh0 + prow_e) >> 1)) * wp + ((ow0 + pcol_e) >> 1)) * 8 + 4 * half_e);
+                    Pack<XT, 4> q4;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) q4.v[k] = from_float<XT>(static_cast<float>((keep >> (8 * k)) & 255u) * 0.25f);
+                    *reinterpret_cast<Pack<XT, 4>*>(out + static_cast<int64_t>(step) * g.out_step_stride + static_cast<int64_t>(off) * 2) = q4;
+                }
+            };
             // All steps of one quad whose sums are xq[tw][k]: residual, LIF, bit-packed store, optional membrane store.
             auto fast_quad = [&](int j8, const float (&xq)[TT][4], const uint32_t (&rb)[TT], bool with_res) __attribute__((always_inline)) {
                 float S[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -839,7 +874,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                         uint32_t quiet = 0;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) fast_step4(xq[0], i, S, quiet);
-                        fast_store4(j8, quiet);
+                        if constexpr (POOL) fast_store4_pooled(j8, quiet);
+                        else fast_store4(j8, quiet);
                     } else {
                         for (int ta0 = 0; ta0 < t_count; ta0 += 8) {
                             const int cnt = min(8, t_count - ta0);
@@ -871,8 +907,12 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 #pragma unroll
                             for (int tw = 0; tw < TT; ++tw) fast_step4(xq[tw], tw, S, quiet);
                         }
-                        if constexpr (TT == 4) fast_store4(j8, quiet);
-                        else fast_store(0, TT, j8, quiet);
+                        if constexpr (TT == 4) {
+                            if constexpr (POOL) fast_store4_pooled(j8, quiet);
+                            else fast_store4(j8, quiet);
+                        } else {
+                            fast_store(0, TT, j8, quiet);
+                        }
                     } else {
 #pragma unroll
                         for (int tw = 0; tw < TT; ++tw) {
@@ -1140,6 +1180,19 @@ int launch_conv_spk_variant(const SpkLaunch& L) {
     return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, TT, IN, true, false>) : run(conv_spk_kernel<XT, TT, IN, false, false>);
 }
 
+// The variants whose spikes leave as 2x2 average pools: straight-line epilogue, four steps (side by side, or of one frame).
+template <typename XT, int IN>
+int launch_conv_spk_pooled(const SpkLaunch& L, int tt) {
+    auto run = [&](auto kernel) -> int {
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif_blocked_avgpool"); rc != SNNF_OK) return rc;
+        kernel<<<dim3(L.grid), kSpkWaves * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.g, L.wpacked, L.bias, L.v_init,
+                                                                        static_cast<unsigned char*>(L.out), L.v_out, L.lif, L.wpacked2, L.bias2);
+        return check_launch("snnf_conv_lif_blocked_avgpool");
+    };
+    if (tt == 4) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 4, IN, true, true, false, true>) : run(conv_spk_kernel<XT, 4, IN, false, true, false, true>);
+    return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 1, IN, true, true, false, true>) : run(conv_spk_kernel<XT, 1, IN, false, true, false, true>);
+}
+
 // The variants with a projection shortcut in the accumulators: bit-packed inputs, four timesteps side by side.
 template <typename XT>
 int launch_conv_spk_shortcut(const SpkLaunch& L) {
@@ -1168,5 +1221,7 @@ int launch_conv_spk_f16_bits(const SpkLaunch& L, int tt);
 int launch_conv_spk_f16_c8(const SpkLaunch& L, int tt);
 int launch_conv_spk_bf16_shortcut(const SpkLaunch& L);
 int launch_conv_spk_f16_shortcut(const SpkLaunch& L);
+int launch_conv_spk_bf16_pooled(const SpkLaunch& L, int tt);
+int launch_conv_spk_f16_pooled(const SpkLaunch& L, int tt);
 
 }  // namespace snnf

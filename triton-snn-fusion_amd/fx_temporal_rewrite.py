@@ -790,6 +790,19 @@ def blocked_conv_lif_shortcut(x, weight, bias, padding, lif, shortcut_x, shortcu
     return out
 
 
+def blocked_conv_lif_avgpool(x, weight, bias, stride, padding, lif):
+    """Conv + folded BN + LIF and the 2x2 / 2 average pool of its spikes in one launch; the two one after the other where the
+    kernel does not take the layer in that form."""
+    from .runtime import hip_blocked_backend as B
+    try:
+        out, _ = B.conv_lif_blocked_avgpool(x, weight, bias, stride, padding, lif)
+        return out
+    except RuntimeError as exc:
+        if "unsupported" not in str(exc):
+            raise
+    return blocked_pool(blocked_conv_lif(x, weight, bias, stride, padding, lif, None, B.BITS), False, 2, 2, 0)
+
+
 def blocked_pool(x, is_max: bool, kernel: int, stride: int, padding: int):
     from .runtime import hip_blocked_backend as B
     try:
@@ -987,6 +1000,23 @@ def propagate_internal_layouts(gm: fx.GraphModule) -> int:
         del blocked_of[sc_stack]
         graph.erase_node(node)
         graph.erase_node(shortcut)
+        converted -= 1
+    # A 2x2 average pool that is the only reader of a fused convolution's spikes runs inside that convolution's launch.
+    for stack, node in list(blocked_of.items()):
+        if node.target is not blocked_pool or tuple(node.args[1:]) != (False, 2, 2, 0):
+            continue
+        conv = node.args[0]
+        conv_stack = next((s for s, n in blocked_of.items() if n is conv), None)
+        if (not isinstance(conv, fx.Node) or conv.target is not blocked_conv_lif or conv.args[5] is None or conv.args[6] is not None
+                or conv.args[7] != B.BITS or len(conv.users) != 1 or conv_stack is None or reads_blocked(conv_stack)[1]):
+            continue
+        with graph.inserting_before(node):
+            fused = graph.call_function(blocked_conv_lif_avgpool, tuple(conv.args[:6]))
+        node.replace_all_uses_with(fused)
+        blocked_of[stack] = fused
+        del blocked_of[conv_stack]
+        graph.erase_node(node)
+        graph.erase_node(conv)
         converted -= 1
     # Phase 2: whoever still reads a converted stack as a tensor gets it converted back (a no-op for dense outputs).
     for stack, new in blocked_of.items():

@@ -414,6 +414,27 @@ class _FusedNetwork(nn.Module):
                       blocked=True, shortcut=dict(x=B.to_dense(shortcut_x), layer=shortcut))
         return out
 
+    def conv_lif_pool_b(self, name: str, x, layer: _FusedLayer, pool_name: str, pool: nn.Module):
+        """Conv + folded BN + LIF and the 2x2 average pool behind it in one launch (the spikes are never stored); None when
+        the pool is another one or the kernel does not take the layer in this form (the caller then runs the two apart)."""
+        from .runtime import hip_blocked_backend as B
+        from .runtime.hip_pool_backend import pool_config
+        if layer.lif is None or pool_config(pool) != (False, 2, 2, 0):
+            return None
+        try:
+            y, v = B.conv_lif_blocked_avgpool(x, layer.weight, layer.bias, layer.stride, layer.padding, layer.lif,
+                                              want_v=self.keep_membranes or self.record is not None)
+        except RuntimeError as exc:
+            if "unsupported" not in str(exc):
+                raise
+            return None
+        if self.record is not None:      # the spikes for the record come from the unpooled launch; the pooled tensor is the fused launch's
+            spikes, _ = B.conv_lif_blocked(x, layer.weight, layer.bias, layer.stride, layer.padding, layer.lif)
+            xs = list(B.to_dense(x).unbind(0)) if not x.shared else [B.to_dense(x)[0]] * x.T
+            self._log(kind="conv_lif", name=name, xs=xs, residuals=None, layer=layer, spikes=B.to_dense(spikes), v=v, blocked=True)
+            self._log(kind="pool", name=pool_name, x=B.to_dense(spikes), pool=pool, y=B.to_dense(y), native=True, blocked=True)
+        return y
+
     def pooled_b(self, name: str, x, pool: nn.Module):
         from .runtime import hip_blocked_backend as B
         from .runtime.hip_pool_backend import pool_config
@@ -496,13 +517,23 @@ class FusedSpikingVGG11(_FusedNetwork):
         return self.tail(seq, self.tail_lif, self.fc_weight, self.fc_bias)
 
     def run_blocked(self, x):
-        """The same layer sequence with the frame channel-blocked, every spike tensor bit-packed (2x2 average pools turn
-        bits into blocked quarters) and only the last, neuron-free convolution writing the dense tensor the tail reads."""
+        """The same layer sequence with the frame channel-blocked, every spike tensor bit-packed (a 2x2 average pool runs inside
+        the convolution in front of it, which then writes blocked quarters instead of bits) and only the last, neuron-free
+        convolution writing the dense tensor the tail reads."""
         from .runtime import hip_blocked_backend as B
         seq = B.from_dense(x, B.C8, shared=True)
         seq.T = self.T
+        skip = False
         for i, (kind, item) in enumerate(self.steps):
+            if skip:            # this pool ran inside the convolution in front of it
+                skip = False
+                continue
             if kind == "conv":
+                if i + 1 < len(self.steps) and self.steps[i + 1][0] == "pool":
+                    fused = self.conv_lif_pool_b(f"features.{i}", seq, item, f"features.{i + 1}", self.steps[i + 1][1])
+                    if fused is not None:
+                        seq, skip = fused, True
+                        continue
                 seq = self.conv_lif_b(f"features.{i}", seq, item)
             elif kind == "pool":
                 seq = self.pooled_b(f"features.{i}", seq, item)

@@ -263,6 +263,38 @@ def conv_lif_blocked_shortcut(x: Blocked, weight: torch.Tensor, bias: Optional[t
     return out, v_out
 
 
+def conv_lif_blocked_avgpool(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding, lif: Sequence[float],
+                             want_v: bool = False):
+    """Convolution + bias + LIF and the 2x2 / stride 2 average pool of its spikes in one launch: returns (the pooled tensor,
+    channel-blocked quarters at half the plane; final membrane of the unpooled neurons or None). Bit for bit
+    `pool_blocked(conv_lif_blocked(...), False, 2, 2, 0)` without the spikes ever being stored. Raises
+    RuntimeError("unsupported_pool: ...") where the kernel does not take the layer in this form."""
+    if x.layout not in (C8, BITS):
+        raise RuntimeError("unsupported_layout: conv_lif_blocked_avgpool takes inputs in C8 or BITS layout")
+    if weight.dim() != 4 or int(weight.shape[1]) != x.C:
+        raise RuntimeError(f"unsupported_groups: weight {tuple(weight.shape)} does not match {x.C} input channels (dense convolutions only)")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise RuntimeError("unsupported_dtype: weight / bias dtype must be the activation dtype")
+    cout, _, kh, kw = (int(d) for d in weight.shape)
+    sh, sw = _as_pair(stride)
+    ph, pw = _as_pair(padding)
+    ho, wo = (x.H + 2 * ph - kh) // sh + 1, (x.W + 2 * pw - kw) // sw + 1
+    if ho % 2 or wo % 2:
+        raise RuntimeError(f"unsupported_pool: the {ho}x{wo} output plane is not even")
+    dev = x.data.device
+    if bias is None:
+        bias = torch.zeros(cout, dtype=weight.dtype, device=weight.device)
+    if _TUNED is None:
+        load_tuned_plans()
+    packed = _packed_weight(weight, bias, x.dtype)
+    out = empty_blocked(C8, x.T, x.N, cout, ho // 2, wo // 2, x.dtype, dev)
+    v_out = torch.empty((x.N, cout, ho, wo), dtype=torch.float32, device=dev) if want_v else None
+    _lib.check("snnf_conv_lif_blocked_avgpool", _lib.lib().snnf_conv_lif_blocked_avgpool(
+        x.step_pointers(), x.layout, x.T, x.N, x.C, x.H, x.W, _lib.dtype_code(x.dtype), packed.data_ptr(), cout, kh, kw, sh, sw, ph, pw,
+        out.data.data_ptr(), out.step_stride_bytes(), _lib.ptr(v_out), float(lif[0]), float(lif[1]), float(lif[2]), _lib.current_stream(dev)))
+    return out, v_out
+
+
 def conv_lif_dense_on_blocked(x: Blocked, weight: torch.Tensor, bias: torch.Tensor, stride, padding, lif: Optional[Sequence[float]],
                               residual: Optional[Blocked] = None, out_layout: int = BITS):
     """The same layer through the dense entry points on unpacked tensors, for a layer the internal-layout kernel refuses
