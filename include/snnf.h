@@ -352,6 +352,20 @@ int snnf_conv_lif_blocked_avgpool(const void* const* xs, int x_layout, int T, in
                                   float v_threshold, float v_reset, float tau, void* stream);
 
 /*
+ * Global average pool and classifier on bit-packed spikes, summed over T and scaled:
+ *   out[n, k] = out_scale * sum_t ( fc_weight[k, :] . mean_hw(s_t[n, :, :, :]) + fc_bias[k] )
+ * The network's last neuron then fires inside the convolution in front of it (snnf_conv_lif_blocked with a bit-packed
+ * output) instead of inside snnf_lif_pool_linear, and this entry point is what remains of the tail: the pooling and the
+ * classifier that the reference keeps as nn.AdaptiveAvgPool2d / nn.Linear modules behind its last fused convolution
+ * when the convolution pattern claims that neuron (compiler/fx_lif_temporal_rewrite.py:2214-2333), and the mean over
+ * the timesteps of its loop wrapper (out_scale = 1 / T). One launch: a workgroup per sample and class range.
+ *   spikes[t] : N frames [C, H, W] in BITS     fc_weight : [K, C], fc_bias : [K] or NULL, out : [N, K], all w_dtype
+ * C a multiple of 8 and at most 2048, w_dtype SNNF_BF16 or SNNF_F16, T <= SNNF_MAX_T_PER_LAUNCH.
+ */
+int snnf_spike_pool_linear(const void* const* spikes, int T, int N, int C, int H, int W, const void* fc_weight,
+                           const void* fc_bias, int K, int w_dtype, void* out, float out_scale, void* stream);
+
+/*
  * Registers a measured launch choice for snnf_conv_lif_blocked on one layer shape (the counterpart of the per-kernel-key
  * "best config" the reference's autotuner keeps, kernels/benchmark_conv_lif_temporal_general.py:524-558,1332-1369):
  * columns of a wave's output patch (rows follow: 32 / columns), channel groups of 8 per LDS stage (a power of two) and

@@ -274,6 +274,33 @@ def test_blocked_conv_with_pool_rejects_what_it_does_not_take(B):
         B.conv_lif_blocked_avgpool(x3, dev(w2, BF16), dev(b2, BF16), [1, 1], [1, 1], LIF)
 
 
+@pytest.mark.parametrize("T,N,C,H,W,K,dtype,scale", [
+    (4, 16, 512, 7, 7, 1000, BF16, 0.25),      # ResNet-18's tail
+    (4, 64, 512, 1, 1, 10, BF16, 0.25),        # VGG-11's
+    (3, 5, 24, 5, 3, 7, F16, 1.0),             # odd everything, the plain sum over T
+    (16, 2, 64, 20, 20, 33, BF16, 1.0 / 16),   # 6400 spikes per channel at most: the byte counters are flushed on the way
+    (1, 3, 2048, 2, 2, 130, BF16, 1.0),        # the widest layer
+])
+def test_pool_and_classifier_on_bit_packed_spikes(B, T, N, C, H, W, K, dtype, scale):
+    """Exact spike counts, fp32 dot products: the result equals scale * (W . sum_t mean_hw(s_t) + T b) computed in float64,
+    to the rounding of the output dtype."""
+    g = gen(3600 + C + K)
+    s = spikes((T, N, C, H, W), 0.3, g)
+    s[:, :, 0] = 1.0                                    # one channel that always fires: the largest count
+    w = q(torch.randn(K, C, generator=g) * 0.05, dtype)
+    b = q(torch.randn(K, generator=g) * 0.05, dtype)
+    x = B.from_dense(dev(s, dtype), B.BITS)
+    got = B.spike_pool_linear(x, dev(w, dtype), dev(b, dtype), scale)
+    torch.cuda.synchronize()
+    counts = s.double().sum((0, 3, 4))                  # [N, C]
+    want = scale * (counts @ w.double().t() / (H * W) + T * b.double())
+    assert got.shape == (N, K) and got.dtype == dtype
+    eps = 2.0 ** -8 if dtype == BF16 else 2.0 ** -11
+    assert torch.allclose(got.double().cpu(), want, rtol=eps, atol=1e-4), float((got.double().cpu() - want).abs().max())
+    no_bias = B.spike_pool_linear(x, dev(w, dtype), None, scale)
+    assert torch.allclose(no_bias.double().cpu(), want - scale * T * b.double(), rtol=eps, atol=1e-4)
+
+
 def test_blocked_conv_without_membrane_output_and_chained_windows(B):
     """The final membrane is optional; two calls chained through it equal one call of all steps, bit for bit."""
     T, N, C, H = 4, 2, 64, 12

@@ -385,6 +385,50 @@ constexpr int kOneMaxC = 2048;                    // channels of a sample whose 
 constexpr int64_t kOneMaxSampleWork = 32 * 1024;  // T * C * HW of one sample, at most: 128 LIF steps per thread (larger samples are
                                                   // better spread over many workgroups by the pooling kernel of the two-launch path)
 
+// out[n, k] = (Wt[k, :] . counts / HW + steps * bias[k]) * out_scale for the classes of this workgroup's range, from the
+// per-channel spike counts of sample n in LDS: kRowsPerWave rows per wave and pass, a lane takes 8 channels at a time.
+template <typename XT>
+__device__ __forceinline__ void classify_counts(const int* plane_count, int n, int C, int K, int classes_per_block, const XT* __restrict__ Wt,
+                                                const XT* __restrict__ bias, XT* __restrict__ out, float inv_hw, float steps, float out_scale) {
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int k_begin = blockIdx.x * classes_per_block;
+    const int k_end = min(K, k_begin + classes_per_block);
+    for (int k0 = k_begin + wave * kRowsPerWave; k0 < k_end; k0 += (kThreads / 64) * kRowsPerWave) {
+        float acc[kRowsPerWave];
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
+        for (int c0 = lane * kVec; c0 < C; c0 += 64 * kVec) {
+            const Pack<int, kVec> pc = *reinterpret_cast<const Pack<int, kVec>*>(plane_count + c0);
+            Pack<XT, kVec> pw[kRowsPerWave];
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r) {
+                const int k = min(k0 + r, K - 1);   // rows beyond the range re-read the last one and are not stored
+                pw[r] = *reinterpret_cast<const Pack<XT, kVec>*>(Wt + static_cast<int64_t>(k) * C + c0);
+            }
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r)
+#pragma unroll
+                for (int j = 0; j < kVec; ++j) acc[r] = fmaf(to_float(pw[r].v[j]), static_cast<float>(pc.v[j]), acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < kRowsPerWave; ++r) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc[r] += __shfl_xor(acc[r], off);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r) {
+                const int k = k0 + r;
+                if (k >= k_end) continue;
+                const float bv = bias != nullptr ? steps * to_float(bias[k]) : 0.0f;
+                const float sum = acc[r] * inv_hw + bv;
+                out[static_cast<int64_t>(n) * K + k] = from_float<XT>(out_scale == 1.0f ? sum : sum * out_scale);
+            }
+        }
+    }
+}
+
 template <typename XT, typename VT>
 __global__ __launch_bounds__(kThreads) void lif_pool_linear_one_kernel(StepPtrs xs, int T, int C, int HW, int K, int classes_per_block,
                                                                        const VT* __restrict__ v_init, VT* __restrict__ v_out,
@@ -446,42 +490,53 @@ __global__ __launch_bounds__(kThreads) void lif_pool_linear_one_kernel(StepPtrs 
         if (run != 0) atomicAdd(&plane_count[p], run);
     }
     __syncthreads();
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int k_begin = blockIdx.x * classes_per_block;
-    const int k_end = min(K, k_begin + classes_per_block);
-    for (int k0 = k_begin + wave * kRowsPerWave; k0 < k_end; k0 += (kThreads / 64) * kRowsPerWave) {
-        float acc[kRowsPerWave];
+    classify_counts<XT>(plane_count, n, C, K, classes_per_block, Wt, bias, out, inv_hw, steps, 1.0f);
+}
+
+// Average pool and classifier on bit-packed spikes (one byte = 8 channels of a pixel), summed over T: the workgroup of a
+// sample and a class range counts the sample's spikes per channel (a thread walks the bytes of one channel group and a
+// share of its pixels, with one byte-wide counter per channel in two registers) and applies its weight rows.
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void spike_pool_linear_kernel(StepPtrs spikes, int T, int C8, int HW, int parts, int K,
+                                                                    int classes_per_block, const XT* __restrict__ Wt,
+                                                                    const XT* __restrict__ bias, XT* __restrict__ out, float inv_hw,
+                                                                    float steps, float out_scale) {
+    __shared__ __align__(16) int plane_count[kOneMaxC];
+    const int n = blockIdx.y;
+    const int C = C8 * 8;
+    for (int i = threadIdx.x; i < C; i += kThreads) plane_count[i] = 0;
+    __syncthreads();
+    const int per_part = (HW + parts - 1) / parts;
+    for (int u = threadIdx.x; u < C8 * parts; u += kThreads) {
+        const int c8 = u / parts;
+        const int part = u - c8 * parts;
+        const int p_begin = part * per_part, p_end = min(HW, p_begin + per_part);
+        const int64_t base = (static_cast<int64_t>(n) * C8 + c8) * HW;
+        uint32_t lo = 0, hi = 0;
+        int pending = 0;
+        auto flush = [&]() {
 #pragma unroll
-        for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
-        for (int c0 = lane * kVec; c0 < C; c0 += 64 * kVec) {
-            const Pack<int, kVec> pc = *reinterpret_cast<const Pack<int, kVec>*>(plane_count + c0);
-            Pack<XT, kVec> pw[kRowsPerWave];
-#pragma unroll
-            for (int r = 0; r < kRowsPerWave; ++r) {
-                const int k = min(k0 + r, K - 1);   // rows beyond the range re-read the last one and are not stored
-                pw[r] = *reinterpret_cast<const Pack<XT, kVec>*>(Wt + static_cast<int64_t>(k) * C + c0);
+            for (int j = 0; j < 4; ++j) {
+                const int a = static_cast<int>((lo >> (8 * j)) & 255u), b = static_cast<int>((hi >> (8 * j)) & 255u);
+                if (a != 0) atomicAdd(&plane_count[c8 * 8 + j], a);
+                if (b != 0) atomicAdd(&plane_count[c8 * 8 + 4 + j], b);
             }
-#pragma unroll
-            for (int r = 0; r < kRowsPerWave; ++r)
-#pragma unroll
-                for (int j = 0; j < kVec; ++j) acc[r] = fmaf(to_float(pw[r].v[j]), static_cast<float>(pc.v[j]), acc[r]);
-        }
-#pragma unroll
-        for (int r = 0; r < kRowsPerWave; ++r) {
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) acc[r] += __shfl_xor(acc[r], off);
-        }
-        if (lane == 0) {
-#pragma unroll
-            for (int r = 0; r < kRowsPerWave; ++r) {
-                const int k = k0 + r;
-                if (k >= k_end) continue;
-                const float bv = bias != nullptr ? steps * to_float(bias[k]) : 0.0f;
-                out[static_cast<int64_t>(n) * K + k] = from_float<XT>(acc[r] * inv_hw + bv);
+            lo = hi = 0;
+            pending = 0;
+        };
+        for (int t = 0; t < T; ++t) {
+            const unsigned char* __restrict__ src = static_cast<const unsigned char*>(spikes.p[t]) + base;
+            for (int p = p_begin; p < p_end; ++p) {
+                const uint32_t byte = src[p];
+                lo += __umul24(byte & 15u, 0x00204081u) & 0x01010101u;
+                hi += __umul24(byte >> 4, 0x00204081u) & 0x01010101u;
+                if (++pending == 255) flush();
             }
         }
+        flush();
     }
+    __syncthreads();
+    classify_counts<XT>(plane_count, n, C, K, classes_per_block, Wt, bias, out, inv_hw, steps, out_scale);
 }
 
 // Class ranges per sample of the one-launch tail: at least 16 classes each (one pass of the workgroup's four waves), no more
@@ -678,6 +733,47 @@ extern "C" int snnf_lif_pool_linear(const void* const* xs, int T, int N, int C, 
                     snnf_lif_pool_linear_workspace_bytes(N, C));
     return lif_pool_linear_impl("snnf_lif_pool_linear", xs, T, N, C, H, W, x_dtype, v_init, v_dtype, fc_weight, fc_bias, K, w_dtype,
                                 out_sum, v_out, static_cast<int*>(workspace), v_threshold, v_reset, tau, stream);
+}
+
+extern "C" int snnf_spike_pool_linear(const void* const* spikes, int T, int N, int C, int H, int W, const void* fc_weight,
+                                      const void* fc_bias, int K, int w_dtype, void* out, float out_scale, void* stream) {
+    using namespace snnf;
+    const char* who = "snnf_spike_pool_linear";
+    if (spikes == nullptr || fc_weight == nullptr || out == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: spikes, fc_weight and out must be non-null", who);
+    if (T < 1 || N < 1 || C < 1 || H < 1 || W < 1 || K < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: T=%d N=%d C=%d H=%d W=%d K=%d", who, T, N, C, H, W, K);
+    if (T > SNNF_MAX_T_PER_LAUNCH)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_temporal_length: T=%d exceeds %d", who, T, SNNF_MAX_T_PER_LAUNCH);
+    if (w_dtype != SNNF_BF16 && w_dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: bfloat16 or float16 classifier (the dtype of the result)", who);
+    if (C % 8 != 0 || C > kOneMaxC || N > 65535)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: %d channels (whole groups of 8, at most %d) of %d samples (at most 65535)", who, C, kOneMaxC, N);
+    if (!aligned_to(fc_weight, 16) || !aligned_to(out, 2) || (fc_bias != nullptr && !aligned_to(fc_bias, 2)))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: fc_weight must be 16-byte aligned, fc_bias and out element aligned", who);
+    StepPtrs ptrs = {};
+    for (int t = 0; t < T; ++t) {
+        if (spikes[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: spikes[%d] is null", who, t);
+        ptrs.p[t] = spikes[t];
+    }
+    const int HW = H * W;
+    const int C8 = C / 8;
+    const int parts = std::max(1, std::min(HW, kThreads / std::max(1, C8)));   // threads that share a channel group's pixels
+    const int rows_per_pass = (kThreads / 64) * kRowsPerWave;
+    const int class_blocks = std::max(1, std::min((K + rows_per_pass - 1) / rows_per_pass, 1024 / std::max(1, N)));
+    const int per_block = (K + class_blocks - 1) / class_blocks;
+    const dim3 grid(class_blocks, N);
+    const float inv_hw = 1.0f / static_cast<float>(HW);
+    hipStream_t hs = as_stream(stream);
+    if (w_dtype == SNNF_BF16)
+        spike_pool_linear_kernel<bf16_t><<<grid, kThreads, 0, hs>>>(ptrs, T, C8, HW, parts, K, per_block, static_cast<const bf16_t*>(fc_weight),
+                                                                    static_cast<const bf16_t*>(fc_bias), static_cast<bf16_t*>(out), inv_hw,
+                                                                    static_cast<float>(T), out_scale);
+    else
+        spike_pool_linear_kernel<f16_t><<<grid, kThreads, 0, hs>>>(ptrs, T, C8, HW, parts, K, per_block, static_cast<const f16_t*>(fc_weight),
+                                                                   static_cast<const f16_t*>(fc_bias), static_cast<f16_t*>(out), inv_hw,
+                                                                   static_cast<float>(T), out_scale);
+    return check_launch(who);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

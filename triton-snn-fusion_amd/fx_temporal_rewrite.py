@@ -803,6 +803,23 @@ def blocked_conv_lif_avgpool(x, weight, bias, stride, padding, lif):
     return blocked_pool(blocked_conv_lif(x, weight, bias, stride, padding, lif, None, B.BITS), False, 2, 2, 0)
 
 
+def blocked_conv_lif_pool_linear(x, weight, bias, stride, padding, lif, residual, fc_weight, fc_bias, scale: float):
+    """The network's last convolution with the tail's neuron in its epilogue (bit-packed spikes out), then average pool and
+    classifier on those spikes, summed over T and scaled (1 / T: the mean over the timesteps): [N, K]. Where a kernel does
+    not take the layer in this form, the convolution writes its sums dense and the LIF -> pool -> Linear operator follows."""
+    from .runtime import hip_blocked_backend as B
+    try:
+        spikes, _ = B.conv_lif_blocked(x, weight, bias, stride, padding, lif, residual=residual, out_layout=B.BITS)
+        return B.spike_pool_linear(spikes, fc_weight, fc_bias, scale)
+    except RuntimeError as exc:
+        if "unsupported" not in str(exc):
+            raise
+    sums, _ = B.conv_lif_blocked_or_dense(x, weight, bias, stride, padding, None, residual=residual, out_layout=B.NCHW)
+    zero = torch.zeros((), dtype=torch.float32, device=sums.data.device)
+    out_sum, _ = torch.ops.snn_custom.fused_temporal_lif_avgpool_linear(B.to_dense(sums), zero, fc_weight, fc_bias, *lif, False)
+    return out_sum * scale
+
+
 def blocked_pool(x, is_max: bool, kernel: int, stride: int, padding: int):
     from .runtime import hip_blocked_backend as B
     try:
@@ -1018,6 +1035,32 @@ def propagate_internal_layouts(gm: fx.GraphModule) -> int:
         graph.erase_node(node)
         graph.erase_node(conv)
         converted -= 1
+    # The tail: a LIF -> average pool -> Linear operator from the zero membrane whose only operand is a LIF-free convolution
+    # that nobody else reads, and whose membrane nobody reads: the neuron fires in that convolution's epilogue and the pool
+    # and the classifier run on the bit-packed spikes; a division of the logits by a constant (the mean over T) is folded in.
+    tail_ops = (S.fused_temporal_lif_avgpool_linear, S.fused_temporal_lif_avgpool_linear.default)
+    for tail in [n for n in graph.nodes if n.op == "call_function" and n.target in tail_ops]:
+        if tail.kwargs or len(tail.args) != 8:
+            continue
+        stack, v0, fc_w, fc_b, v_th, v_reset, tau, detach = tail.args
+        conv = blocked_of.get(stack) if isinstance(stack, fx.Node) else None
+        items = find_tuple_getitems(tail)
+        if (conv is None or conv.target is not blocked_conv_lif or conv.args[5] is not None or conv.args[7] != B.NCHW
+                or not _scalar_zero_node(gm, v0) or len(stack.users) != 1 or len(tail.users) != 1 or 0 not in items):
+            continue
+        logits = items[0]
+        scale, last = 1.0, logits
+        if len(logits.users) == 1:
+            user = next(iter(logits.users))
+            if (user.op == "call_function" and user.target in (operator.truediv, torch.div) and user.args[0] is logits
+                    and isinstance(user.args[1], (int, float)) and not user.kwargs and user.args[1] != 0):
+                scale, last = 1.0 / float(user.args[1]), user
+        with graph.inserting_before(tail):
+            fused = graph.call_function(blocked_conv_lif_pool_linear, (*conv.args[:5], (v_th, v_reset, tau), conv.args[6], fc_w, fc_b, scale))
+        last.replace_all_uses_with(fused)
+        del blocked_of[stack]
+        for dead in ([last] if last is not logits else []) + [logits, tail, conv]:
+            graph.erase_node(dead)
     # Phase 2: whoever still reads a converted stack as a tensor gets it converted back (a no-op for dense outputs).
     for stack, new in blocked_of.items():
         with graph.inserting_after(new):

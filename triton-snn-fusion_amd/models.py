@@ -435,6 +435,26 @@ class _FusedNetwork(nn.Module):
             self._log(kind="pool", name=pool_name, x=B.to_dense(spikes), pool=pool, y=B.to_dense(y), native=True, blocked=True)
         return y
 
+    def last_conv_and_tail_b(self, name: str, x, layer: _FusedLayer, lif, fc_weight, fc_bias, residual=None) -> torch.Tensor:
+        """The network's last, neuron-free convolution (+ residual) and the LIF -> average pool -> Linear tail behind it: the
+        tail's neuron fires in the convolution's epilogue (bit-packed spikes out), the pool and the classifier run on the
+        bits and yield the mean over T. Where a kernel does not take the layer in that form the convolution writes its sums
+        dense and the tail operator follows."""
+        from .runtime import hip_blocked_backend as B
+        with_neuron = copy.copy(layer)
+        with_neuron.lif = tuple(lif)
+        try:
+            spikes = self.conv_lif_b(name, x, with_neuron, residual=residual, out_layout=B.BITS)
+            logits = B.spike_pool_linear(spikes, fc_weight, fc_bias, 1.0 / self.T)
+        except RuntimeError as exc:
+            if "unsupported" not in str(exc):
+                raise
+            sums = self.conv_lif_b(name, x, layer, residual=residual, out_layout=B.NCHW)
+            return self.tail(B.to_dense(sums), lif, fc_weight, fc_bias)
+        if self.record is not None:
+            self._log(kind="spike_pool_linear", name="tail", x=B.to_dense(spikes), fc_weight=fc_weight, fc_bias=fc_bias, out=logits)
+        return logits
+
     def pooled_b(self, name: str, x, pool: nn.Module):
         from .runtime import hip_blocked_backend as B
         from .runtime.hip_pool_backend import pool_config
@@ -518,8 +538,8 @@ class FusedSpikingVGG11(_FusedNetwork):
 
     def run_blocked(self, x):
         """The same layer sequence with the frame channel-blocked, every spike tensor bit-packed (a 2x2 average pool runs inside
-        the convolution in front of it, which then writes blocked quarters instead of bits) and only the last, neuron-free
-        convolution writing the dense tensor the tail reads."""
+        the convolution in front of it, which then writes blocked quarters instead of bits); the tail's neuron fires in the
+        last convolution, and the pool and the classifier read its bit-packed spikes."""
         from .runtime import hip_blocked_backend as B
         seq = B.from_dense(x, B.C8, shared=True)
         seq.T = self.T
@@ -537,8 +557,10 @@ class FusedSpikingVGG11(_FusedNetwork):
                 seq = self.conv_lif_b(f"features.{i}", seq, item)
             elif kind == "pool":
                 seq = self.pooled_b(f"features.{i}", seq, item)
+            elif i == len(self.steps) - 1:      # the last convolution: the tail's neuron fires in it
+                return self.last_conv_and_tail_b(f"features.{i}", seq, item, self.tail_lif, self.fc_weight, self.fc_bias)
             else:
-                seq = self.conv_lif_b(f"features.{i}", seq, item, out_layout=B.NCHW)
+                seq = self.conv_lif_b(f"features.{i}", seq, item, out_layout=B.C8)
         return self.tail(B.to_dense(seq), self.tail_lif, self.fc_weight, self.fc_bias)
 
 
@@ -572,7 +594,8 @@ class FusedSpikingResNet18(_FusedNetwork):
     def run_blocked(self, x):
         """Stem on the channel-blocked frame, everything after it on bit-packed spikes; a LIF-free shortcut convolution is
         accumulated inside the block's second convolution (or, where that kernel does not take the pair, produces a blocked
-        analog residual); the last block's sum is written dense for the tail."""
+        analog residual); the tail's neuron fires in the last block's second convolution, and the pool and the classifier read
+        its bit-packed spikes."""
         from .runtime import hip_blocked_backend as B
         frame = B.from_dense(x, B.C8, shared=True)
         frame.T = self.T
@@ -588,8 +611,10 @@ class FusedSpikingResNet18(_FusedNetwork):
             identity = seq if down is None else self.conv_lif_b(f"blocks.{i}.downsample", seq, down)
             if conv2.lif is not None:
                 seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity)
-            else:   # last block: its neuron is the tail's
-                seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity, out_layout=B.NCHW)
+            elif i == len(self.block_layers) - 1:   # last block: its neuron is the tail's and fires in this convolution
+                return self.last_conv_and_tail_b(f"blocks.{i}.conv2", hidden, conv2, self.tail_lif, self.fc_weight, self.fc_bias, residual=identity)
+            else:
+                seq = self.conv_lif_b(f"blocks.{i}.conv2", hidden, conv2, residual=identity, out_layout=B.C8)
         return self.tail(B.to_dense(seq), self.tail_lif, self.fc_weight, self.fc_bias)
 
 

@@ -295,6 +295,22 @@ def conv_lif_blocked_avgpool(x: Blocked, weight: torch.Tensor, bias: Optional[to
     return out, v_out
 
 
+def spike_pool_linear(x: Blocked, fc_weight: torch.Tensor, fc_bias: Optional[torch.Tensor], scale: float = 1.0) -> torch.Tensor:
+    """scale * sum_t (fc_weight . mean_hw(spikes_t) + fc_bias) of bit-packed spikes: [N, K] in the activation dtype. What is
+    left of the LIF -> average pool -> Linear tail when the network's last neuron has fired inside the convolution in front of
+    it; `scale = 1 / T` gives the mean over the timesteps."""
+    if x.layout != BITS or x.shared:
+        raise RuntimeError("unsupported_layout: spike_pool_linear takes bit-packed spikes, one frame per timestep")
+    if fc_weight.dim() != 2 or int(fc_weight.shape[1]) != x.C or fc_weight.dtype != x.dtype or (fc_bias is not None and fc_bias.dtype != x.dtype):
+        raise RuntimeError(f"unsupported_shape: classifier {tuple(fc_weight.shape)} {fc_weight.dtype} does not match {x.C} channels of {x.dtype}")
+    w = fc_weight if fc_weight.is_contiguous() else fc_weight.contiguous()
+    out = torch.empty((x.N, int(w.shape[0])), dtype=x.dtype, device=x.data.device)
+    _lib.check("snnf_spike_pool_linear", _lib.lib().snnf_spike_pool_linear(
+        x.step_pointers(), x.T, x.N, x.C, x.H, x.W, w.data_ptr(), _lib.ptr(fc_bias), int(w.shape[0]), _lib.dtype_code(x.dtype),
+        out.data_ptr(), float(scale), _lib.current_stream(x.data.device)))
+    return out
+
+
 def conv_lif_dense_on_blocked(x: Blocked, weight: torch.Tensor, bias: torch.Tensor, stride, padding, lif: Optional[Sequence[float]],
                               residual: Optional[Blocked] = None, out_layout: int = BITS):
     """The same layer through the dense entry points on unpacked tensors, for a layer the internal-layout kernel refuses
