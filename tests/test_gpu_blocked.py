@@ -319,6 +319,9 @@ def test_blocked_conv_without_membrane_output_and_chained_windows(B):
 
 SHARED_CASES = [  # Cin, Cout, H, W, k, s, p, T, N
     (3, 64, 32, 32, 7, 2, 3, 4, 2),      # ResNet stem: one analog frame, taps paired inside a single channel group
+    (3, 64, 32, 32, 3, 1, 1, 4, 3),      # VGG stem at its own size
+    (8, 32, 9, 13, 3, 1, 1, 4, 2),       # a whole channel group, ragged plane
+    (1, 16, 12, 12, 5, 1, 2, 2, 2),      # one channel
     (3, 64, 16, 16, 3, 1, 1, 16, 2),     # VGG stem, 16 LIF steps on one convolution
     (64, 64, 8, 8, 3, 1, 1, 5, 2),       # whole channel groups
 ]
@@ -335,6 +338,30 @@ def test_blocked_conv_with_one_analog_frame_for_all_timesteps(B, Cin, Cout, H, W
     assert plan["kernel"] == "blocked" and plan["window"] == T
     check(B.to_dense(out), v, ref, what=f"blocked shared frame {Cin}->{Cout} k{k}")
     assert 0.001 < float(ref[0].mean()) < 0.9
+    if Cin <= 8:
+        # The frame as it is (dense, no conversion launch): same matrix operands, bit for bit the same result.
+        frame = B.input_frame(dev(xs[0], BF16), T)
+        assert frame.layout == B.NCHW and frame.shared
+        out2, v2 = B.conv_lif_blocked(frame, dev(w, BF16), dev(b, BF16), [s, s], [p, p], LIF, want_v=True)
+        assert B.last_conv_plan()["kernel"] == "blocked"
+        assert torch.equal(out2.data, out.data) and torch.equal(v2, v)
+        if T == 4 and out.H % 2 == 0 and out.W % 2 == 0:
+            pooled, _ = B.conv_lif_blocked_avgpool(frame, dev(w, BF16), dev(b, BF16), [s, s], [p, p], LIF)
+            assert torch.equal(pooled.data, B.pool_blocked(out, False, 2, 2, 0).data)
+    else:
+        assert B.input_frame(dev(xs[0], BF16), T).layout == B.C8
+
+
+def test_blocked_conv_takes_a_dense_input_only_as_one_small_frame(B):
+    xs, w, b = _case(3460, 4, 2, 3, 16, 8, 8, 3, BF16, analog=True)
+    per_step = B.from_dense(dev(xs, BF16), B.NCHW)                      # a frame per timestep: not the shared input
+    with pytest.raises(RuntimeError, match="unsupported_layout"):
+        B.conv_lif_blocked(per_step, dev(w, BF16), dev(b, BF16), [1, 1], [1, 1], LIF)
+    xs16, w16, b16 = _case(3461, 4, 2, 16, 16, 8, 8, 3, BF16, analog=True, shared=True)
+    wide = B.from_dense(dev(xs16[0], BF16), B.NCHW, shared=True)         # 16 channels
+    wide.T = 4
+    with pytest.raises(RuntimeError, match="unsupported_layout"):
+        B.conv_lif_blocked(wide, dev(w16, BF16), dev(b16, BF16), [1, 1], [1, 1], LIF)
 
 
 CONV_BIAS_CASES = [  # Cin, Cout, H, W, k, s, p, T, N, residual layout, out layout

@@ -157,8 +157,8 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
         return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_temporal_length: T=%d exceeds %d", who, T, SNNF_MAX_T_PER_LAUNCH);
     if (x_dtype != SNNF_BF16 && x_dtype != SNNF_F16)
         return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_dtype: the internal layouts hold bf16 or fp16 activations", who);
-    if (x_layout != SNNF_LAYOUT_C8 && x_layout != SNNF_LAYOUT_BITS)
-        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: inputs must be in C8 or BITS layout", who);
+    if (x_layout != SNNF_LAYOUT_C8 && x_layout != SNNF_LAYOUT_BITS && x_layout != SNNF_LAYOUT_NCHW)
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: inputs must be in C8 or BITS layout (or one dense frame of at most 8 channels)", who);
     if (!valid_layout(out_layout) || (residuals != nullptr && !valid_layout(res_layout)))
         return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: unknown layout code", who);
     if (!neuron && out_layout == SNNF_LAYOUT_BITS)
@@ -182,6 +182,8 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
             return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: residuals[%d] is null or misaligned for its layout", who, t);
         shared = shared && xs[t] == xs[0];
     }
+    if (x_layout == SNNF_LAYOUT_NCHW && (!shared || Cin > 8))
+        return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: a dense input must be one frame of at most 8 channels shared by all timesteps (Cin=%d)", who, Cin);
     if (sc != nullptr) {
         // The shortcut's sums are K steps of the main tile: same output pixels (a main convolution that keeps the plane, the
         // shortcut's stride taking its own input down to it), whole pairs of channel groups, bit-packed input like the main one.
@@ -364,9 +366,11 @@ int conv_lif_blocked_impl(const char* who, const void* const* xs, int x_layout, 
         if (!fast_epi || windows != 1 || (tt != 4 && !shared))
             return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_pool: the pooled output needs the usual neuron (tau 2, hard reset to 0) and the four steps in one window", who);
         L.g.pool2 = 1;
+        if (x_layout == SNNF_LAYOUT_NCHW) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_frame(L, true) : launch_conv_spk_f16_frame(L, true);
         return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_pooled(L, tt) : launch_conv_spk_f16_pooled(L, tt);
     }
     if (sc != nullptr) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_shortcut(L) : launch_conv_spk_f16_shortcut(L);
+    if (x_layout == SNNF_LAYOUT_NCHW) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_frame(L, false) : launch_conv_spk_f16_frame(L, false);
     if (x_layout == SNNF_LAYOUT_BITS) return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_bits(L, tt) : launch_conv_spk_f16_bits(L, tt);
     return x_dtype == SNNF_BF16 ? launch_conv_spk_bf16_c8(L, tt) : launch_conv_spk_f16_c8(L, tt);
 }

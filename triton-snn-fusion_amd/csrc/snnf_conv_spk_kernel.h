@@ -168,6 +168,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
 
     static_assert(!SC || (IN == SNNF_LAYOUT_BITS && TT == 4), "the shortcut variants take bit-packed inputs, four timesteps at a time");
     static_assert(!POOL || (FAST && (TT == 4 || TT == 1)), "the pooled output belongs to the straight-line epilogue of four steps");
+    static_assert(IN != SNNF_LAYOUT_NCHW || TT == 1, "a dense input is one frame for all timesteps");
     constexpr bool F16 = dtype_of<XT>::value == SNNF_F16;
     constexpr uint32_t ONE = F16 ? 0x3c00u : 0x3f80u;
     constexpr int kResTable = static_cast<int>(sizeof(StepPtrs));
@@ -249,7 +250,8 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const int rem2 = rem - ii * (g.RR * g.RC);
                 const int r = sk_div(rem2, g.d_RC);
                 const int c = rem2 - r * g.RC;
-                d.v[0] = static_cast<uint32_t>(((ii * g.C8in + gq) * g.H + r) * g.W + c);
+                if constexpr (IN == SNNF_LAYOUT_NCHW) d.v[0] = static_cast<uint32_t>(((ii * g.Cin + gq * 8) * g.H + r) * g.W + c);   // elements of a dense frame
+                else d.v[0] = static_cast<uint32_t>(((ii * g.C8in + gq) * g.H + r) * g.W + c);
                 d.v[1] = static_cast<uint32_t>(r) | (static_cast<uint32_t>(c) << 8) | (static_cast<uint32_t>(ii) << 16) | (static_cast<uint32_t>(gq) << 24);
             }
             desc_w[e] = d;
@@ -366,6 +368,7 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                 const int gg0 = (second ? s - g.nstages : s) * g.G;
                 const int c8 = second ? g.sc_C8 : g.C8in;
                 const int base_u = second ? ((n0 * g.sc_C8 + gg0) * g.sc_H + ih_lo * g.sc_sh) * g.sc_W + iw_lo * g.sc_sw
+                                   : IN == SNNF_LAYOUT_NCHW ? ((n0 * g.Cin + gg0 * 8) * g.H + ih_lo) * g.W + iw_lo
                                           : ((n0 * g.C8in + gg0) * g.H + ih_lo) * g.W + iw_lo;   // may be negative; only added to in-image items
                 uint32_t ok_bits = 0;
 #pragma unroll
@@ -435,6 +438,32 @@ __global__ __launch_bounds__(kSpkWaves * 64, 1) __attribute__((amdgpu_waves_per_
                             uint32_t raw[TT][4];
                             batch_load_bits(s, idx, raw);
                             batch_put_bits(jb, lane_s, ok_bits, raw);
+                        } else if constexpr (IN == SNNF_LAYOUT_NCHW) {
+                            // A dense frame of at most 8 channels (the network's input): one 16-bit load per channel and item.
+                            const int plane = g.H * g.W;
+#pragma unroll
+                            for (int t = 0; t < TT; ++t) {
+                                const int ts = t0 + t < nsteps_t ? t0 + t : t0;
+                                const uint16_t* __restrict__ src = static_cast<const uint16_t*>(sk_kernarg_ptr(0, ts));
+                                uint32_t h[4][8];
+#pragma unroll
+                                for (int k = 0; k < 8; ++k) {
+                                    if (k < g.Cin) {
+#pragma unroll
+                                        for (int j = 0; j < 4; ++j) h[j][k] = src[idx[j] + k * plane];
+                                    } else {
+#pragma unroll
+                                        for (int j = 0; j < 4; ++j) h[j][k] = 0u;
+                                    }
+                                }
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    sk_u32x4 d;
+#pragma unroll
+                                    for (int k = 0; k < 4; ++k) d[k] = ((ok_bits >> j) & 1u) ? (h[j][2 * k] | (h[j][2 * k + 1] << 16)) : 0u;
+                                    *reinterpret_cast<sk_u32x4*>(wlds + t * tile_t + min((jb + j) * 64 + lane_s, g.IT) * 16) = d;
+                                }
+                            }
                         } else {
 #pragma unroll
                             for (int t = 0; t < TT; ++t) {
@@ -1193,6 +1222,21 @@ int launch_conv_spk_pooled(const SpkLaunch& L, int tt) {
     return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 1, IN, true, true, false, true>) : run(conv_spk_kernel<XT, 1, IN, false, true, false, true>);
 }
 
+// The variants that read the network's input as it is: one dense frame of at most 8 channels for all timesteps.
+template <typename XT>
+int launch_conv_spk_frame(const SpkLaunch& L, bool pooled) {
+    auto run = [&](auto kernel) -> int {
+        if (const int rc = reserve_lds(reinterpret_cast<const void*>(kernel), L.lds_bytes, "snnf_conv_lif_blocked"); rc != SNNF_OK) return rc;
+        kernel<<<dim3(L.grid), kSpkWaves * 64, L.lds_bytes, L.stream>>>(L.xs, L.residuals, L.g, L.wpacked, L.bias, L.v_init,
+                                                                        static_cast<unsigned char*>(L.out), L.v_out, L.lif, L.wpacked2, L.bias2);
+        return check_launch("snnf_conv_lif_blocked");
+    };
+    constexpr int D = SNNF_LAYOUT_NCHW;
+    if (pooled) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 1, D, true, true, false, true>) : run(conv_spk_kernel<XT, 1, D, false, true, false, true>);
+    if (L.fast_epilogue) return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 1, D, true, true>) : run(conv_spk_kernel<XT, 1, D, false, true>);
+    return L.g.wk_log2 > 0 ? run(conv_spk_kernel<XT, 1, D, true, false>) : run(conv_spk_kernel<XT, 1, D, false, false>);
+}
+
 // The variants with a projection shortcut in the accumulators: bit-packed inputs, four timesteps side by side.
 template <typename XT>
 int launch_conv_spk_shortcut(const SpkLaunch& L) {
@@ -1223,5 +1267,7 @@ int launch_conv_spk_bf16_shortcut(const SpkLaunch& L);
 int launch_conv_spk_f16_shortcut(const SpkLaunch& L);
 int launch_conv_spk_bf16_pooled(const SpkLaunch& L, int tt);
 int launch_conv_spk_f16_pooled(const SpkLaunch& L, int tt);
+int launch_conv_spk_bf16_frame(const SpkLaunch& L, bool pooled);
+int launch_conv_spk_f16_frame(const SpkLaunch& L, bool pooled);
 
 }  // namespace snnf

@@ -746,13 +746,11 @@ def batch_timestep_calls(gm: fx.GraphModule) -> int:
 # (runtime/hip_blocked_backend.py); dense tensors remain at the graph's inputs and outputs and in front of every node the
 # pass does not know. The graph functions below are the targets of the new nodes.
 def blocked_input(frames, T: int, shared: bool):
-    """Graph input side: one analog frame [N, C, H, W] shared by all T steps, or a dense [T, N, C, H, W] tensor (or the
-    list of its T steps), into the channel-blocked layout."""
+    """Graph input side: one analog frame [N, C, H, W] shared by all T steps (read as it is when it has at most 8 channels),
+    or a dense [T, N, C, H, W] tensor (or the list of its T steps), into the channel-blocked layout."""
     from .runtime import hip_blocked_backend as B
     if shared:
-        x = B.from_dense(frames.contiguous(), B.C8, shared=True)
-        x.T = int(T)
-        return x
+        return B.input_frame(frames, T)
     if isinstance(frames, (list, tuple)):
         frames = torch.stack(list(frames))
     return B.from_dense(frames, B.C8)

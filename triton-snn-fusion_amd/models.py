@@ -541,8 +541,7 @@ class FusedSpikingVGG11(_FusedNetwork):
         the convolution in front of it, which then writes blocked quarters instead of bits); the tail's neuron fires in the
         last convolution, and the pool and the classifier read its bit-packed spikes."""
         from .runtime import hip_blocked_backend as B
-        seq = B.from_dense(x, B.C8, shared=True)
-        seq.T = self.T
+        seq = B.input_frame(x, self.T)
         skip = False
         for i, (kind, item) in enumerate(self.steps):
             if skip:            # this pool ran inside the convolution in front of it
@@ -597,8 +596,7 @@ class FusedSpikingResNet18(_FusedNetwork):
         analog residual); the tail's neuron fires in the last block's second convolution, and the pool and the classifier read
         its bit-packed spikes."""
         from .runtime import hip_blocked_backend as B
-        frame = B.from_dense(x, B.C8, shared=True)
-        frame.T = self.T
+        frame = B.input_frame(x, self.T)
         seq = self.conv_lif_b("stem", frame, self.stem)
         seq = self.pooled_b("maxpool", seq, self.maxpool)
         for i, (conv1, conv2, down) in enumerate(self.block_layers):

@@ -169,14 +169,30 @@ def get_autotune_best_config(T, N, Cin, H, W, weight_shape, stride, padding, sha
 _NEEDS_MEMBRANE_BUFFER: set = set()
 
 
+def _is_input_frame(x: Blocked) -> bool:
+    """One dense frame of at most 8 channels for all timesteps (a network's input): the convolution kernel reads it as it is."""
+    return x.layout == NCHW and x.shared and x.C <= 8
+
+
+def input_frame(frame: torch.Tensor, T: int) -> Blocked:
+    """A network's analog input [N, C, H, W], the same for all T timesteps, as the operand of the first convolution: dense
+    as it is when it has at most 8 channels, channel-blocked otherwise."""
+    _check_dtype(frame.dtype)
+    if frame.dim() != 4 or not frame.is_cuda:
+        raise RuntimeError("unsupported_rank: input_frame takes an [N, C, H, W] tensor on the GPU")
+    x = from_dense(frame.contiguous(), NCHW if int(frame.shape[1]) <= 8 else C8, shared=True)
+    x.T = int(T)
+    return x
+
+
 def conv_lif_blocked(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding,
                      lif: Optional[Sequence[float]], residual: Optional[Blocked] = None, out_layout: int = BITS,
                      v_init: Optional[torch.Tensor] = None, want_v: bool = False):
     """Dense convolution + bias (+ residual) + LIF over the T steps of `x` (C8 or BITS), or without a neuron when `lif` is
     None (output C8 or NCHW). Returns (Blocked output, final membrane [N, Cout, Ho, Wo] fp32 or None). The membrane is
     only written when asked for (`want_v`) or when the timesteps take more than one window of the kernel."""
-    if x.layout not in (C8, BITS):
-        raise RuntimeError("unsupported_layout: conv_lif_blocked takes inputs in C8 or BITS layout")
+    if x.layout not in (C8, BITS) and not _is_input_frame(x):
+        raise RuntimeError("unsupported_layout: conv_lif_blocked takes inputs in C8 or BITS layout (or one dense frame of at most 8 channels)")
     if weight.dim() != 4 or int(weight.shape[1]) != x.C:
         raise RuntimeError(f"unsupported_groups: weight {tuple(weight.shape)} does not match {x.C} input channels (dense convolutions only)")
     if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
@@ -269,8 +285,8 @@ def conv_lif_blocked_avgpool(x: Blocked, weight: torch.Tensor, bias: Optional[to
     channel-blocked quarters at half the plane; final membrane of the unpooled neurons or None). Bit for bit
     `pool_blocked(conv_lif_blocked(...), False, 2, 2, 0)` without the spikes ever being stored. Raises
     RuntimeError("unsupported_pool: ...") where the kernel does not take the layer in this form."""
-    if x.layout not in (C8, BITS):
-        raise RuntimeError("unsupported_layout: conv_lif_blocked_avgpool takes inputs in C8 or BITS layout")
+    if x.layout not in (C8, BITS) and not _is_input_frame(x):
+        raise RuntimeError("unsupported_layout: conv_lif_blocked_avgpool takes inputs in C8 or BITS layout (or one dense frame of at most 8 channels)")
     if weight.dim() != 4 or int(weight.shape[1]) != x.C:
         raise RuntimeError(f"unsupported_groups: weight {tuple(weight.shape)} does not match {x.C} input channels (dense convolutions only)")
     if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
