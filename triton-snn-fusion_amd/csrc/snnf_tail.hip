@@ -496,15 +496,30 @@ __global__ __launch_bounds__(kThreads) void lif_pool_linear_one_kernel(StepPtrs 
 // Average pool and classifier on bit-packed spikes (one byte = 8 channels of a pixel), summed over T: the workgroup of a
 // sample and a class range counts the sample's spikes per channel (a thread walks the bytes of one channel group and a
 // share of its pixels, with one byte-wide counter per channel in two registers) and applies its weight rows.
-template <typename XT>
-__global__ __launch_bounds__(kThreads) void spike_pool_linear_kernel(StepPtrs spikes, int T, int C8, int HW, int parts, int K,
-                                                                    int classes_per_block, const XT* __restrict__ Wt,
-                                                                    const XT* __restrict__ bias, XT* __restrict__ out, float inv_hw,
-                                                                    float steps, float out_scale) {
+constexpr int kSpikeStageBytes = 32 * 1024;   // a sample's bit-packed spikes of all timesteps, staged in LDS when they fit
+
+template <typename XT, bool STAGED>
+__global__ __launch_bounds__(kThreads) void spike_pool_linear_kernel(const unsigned char* __restrict__ spikes, int64_t step_stride, int T, int C8,
+                                                                    int HW, int parts, int K, int classes_per_block,
+                                                                    const XT* __restrict__ Wt, const XT* __restrict__ bias,
+                                                                    XT* __restrict__ out, float inv_hw, float steps, float out_scale) {
     __shared__ __align__(16) int plane_count[kOneMaxC];
+    __shared__ __align__(16) unsigned char staged[STAGED ? kSpikeStageBytes : 16];
     const int n = blockIdx.y;
     const int C = C8 * 8;
     for (int i = threadIdx.x; i < C; i += kThreads) plane_count[i] = 0;
+    const int sample_bytes = C8 * HW;
+    if constexpr (STAGED) {
+        // The sample's bytes of every timestep are contiguous: coalesced 16-byte loads bring them into LDS (a multiple of 16
+        // bytes at a 16-byte aligned address, checked on the host), and the counting below reads single bytes from there.
+        const int vecs = sample_bytes / 16;
+        for (int i = threadIdx.x; i < T * vecs; i += kThreads) {
+            const int t = i / vecs;
+            const int v = i - t * vecs;
+            *reinterpret_cast<uint4*>(staged + t * sample_bytes + v * 16) =
+                *reinterpret_cast<const uint4*>(spikes + static_cast<int64_t>(t) * step_stride + static_cast<int64_t>(n) * sample_bytes + v * 16);
+        }
+    }
     __syncthreads();
     const int per_part = (HW + parts - 1) / parts;
     for (int u = threadIdx.x; u < C8 * parts; u += kThreads) {
@@ -524,13 +539,33 @@ __global__ __launch_bounds__(kThreads) void spike_pool_linear_kernel(StepPtrs sp
             lo = hi = 0;
             pending = 0;
         };
-        for (int t = 0; t < T; ++t) {
-            const unsigned char* __restrict__ src = static_cast<const unsigned char*>(spikes.p[t]) + base;
-            for (int p = p_begin; p < p_end; ++p) {
-                const uint32_t byte = src[p];
-                lo += __umul24(byte & 15u, 0x00204081u) & 0x01010101u;
-                hi += __umul24(byte >> 4, 0x00204081u) & 0x01010101u;
-                if (++pending == 255) flush();
+        // 8 pixels x 4 timesteps per trip, all 32 loads in flight together (positions beyond the range re-read its last byte
+        // and count as zero: no branch around a load).
+        for (int p0 = p_begin; p0 < p_end; p0 += 8) {
+            for (int t0 = 0; t0 < T; t0 += 4) {
+                uint32_t byte[4][8];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if constexpr (STAGED) {
+                        const unsigned char* src = staged + min(t0 + u, T - 1) * sample_bytes + c8 * HW;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) byte[u][j] = src[min(p0 + j, p_end - 1)];
+                    } else {
+                        const unsigned char* __restrict__ src = spikes + static_cast<int64_t>(min(t0 + u, T - 1)) * step_stride + base;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) byte[u][j] = src[min(p0 + j, p_end - 1)];
+                    }
+                }
+                if (pending > 255 - 32) flush();
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t b = (t0 + u < T && p0 + j < p_end) ? byte[u][j] : 0u;
+                        lo += __umul24(b & 15u, 0x00204081u) & 0x01010101u;
+                        hi += __umul24(b >> 4, 0x00204081u) & 0x01010101u;
+                    }
+                pending += 32;
             }
         }
         flush();
@@ -751,11 +786,14 @@ extern "C" int snnf_spike_pool_linear(const void* const* spikes, int T, int N, i
         return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_shape: %d channels (whole groups of 8, at most %d) of %d samples (at most 65535)", who, C, kOneMaxC, N);
     if (!aligned_to(fc_weight, 16) || !aligned_to(out, 2) || (fc_bias != nullptr && !aligned_to(fc_bias, 2)))
         return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: fc_weight must be 16-byte aligned, fc_bias and out element aligned", who);
-    StepPtrs ptrs = {};
-    for (int t = 0; t < T; ++t) {
+    for (int t = 0; t < T; ++t)
         if (spikes[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "%s: spikes[%d] is null", who, t);
-        ptrs.p[t] = spikes[t];
-    }
+    // The timesteps of a bit-packed tensor lie at equal distances (one allocation): the kernel walks them by a stride.
+    const int64_t step_stride = T > 1 ? static_cast<const unsigned char*>(spikes[1]) - static_cast<const unsigned char*>(spikes[0]) : 0;
+    for (int t = 1; t < T; ++t)
+        if (static_cast<const unsigned char*>(spikes[t]) - static_cast<const unsigned char*>(spikes[t - 1]) != step_stride)
+            return fail(SNNF_ERR_UNSUPPORTED, "%s: unsupported_layout: the timesteps must lie at equal distances in memory", who);
+    const unsigned char* base = static_cast<const unsigned char*>(spikes[0]);
     const int HW = H * W;
     const int C8 = C / 8;
     const int parts = std::max(1, std::min(HW, kThreads / std::max(1, C8)));   // threads that share a channel group's pixels
@@ -765,14 +803,20 @@ extern "C" int snnf_spike_pool_linear(const void* const* spikes, int T, int N, i
     const dim3 grid(class_blocks, N);
     const float inv_hw = 1.0f / static_cast<float>(HW);
     hipStream_t hs = as_stream(stream);
-    if (w_dtype == SNNF_BF16)
-        spike_pool_linear_kernel<bf16_t><<<grid, kThreads, 0, hs>>>(ptrs, T, C8, HW, parts, K, per_block, static_cast<const bf16_t*>(fc_weight),
-                                                                    static_cast<const bf16_t*>(fc_bias), static_cast<bf16_t*>(out), inv_hw,
-                                                                    static_cast<float>(T), out_scale);
-    else
-        spike_pool_linear_kernel<f16_t><<<grid, kThreads, 0, hs>>>(ptrs, T, C8, HW, parts, K, per_block, static_cast<const f16_t*>(fc_weight),
-                                                                   static_cast<const f16_t*>(fc_bias), static_cast<f16_t*>(out), inv_hw,
-                                                                   static_cast<float>(T), out_scale);
+    const int64_t sample_bytes = static_cast<int64_t>(C8) * HW;
+    const bool staged = sample_bytes % 16 == 0 && T * sample_bytes <= kSpikeStageBytes && aligned_to(base, 16) && step_stride % 16 == 0;
+#define SNNF_SPIKE_TAIL(XT, STAGED)                                                                                                         \
+    spike_pool_linear_kernel<XT, STAGED><<<grid, kThreads, 0, hs>>>(base, step_stride, T, C8, HW, parts, K, per_block, static_cast<const XT*>(fc_weight), \
+                                                                    static_cast<const XT*>(fc_bias), static_cast<XT*>(out), inv_hw,          \
+                                                                    static_cast<float>(T), out_scale)
+    if (w_dtype == SNNF_BF16) {
+        if (staged) SNNF_SPIKE_TAIL(bf16_t, true);
+        else SNNF_SPIKE_TAIL(bf16_t, false);
+    } else {
+        if (staged) SNNF_SPIKE_TAIL(f16_t, true);
+        else SNNF_SPIKE_TAIL(f16_t, false);
+    }
+#undef SNNF_SPIKE_TAIL
     return check_launch(who);
 }
 
