@@ -351,7 +351,7 @@ def _fused(name, T=4, gain=5.0, internal=False):
 def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
     """Every recorded operator call of one forward against the oracle on that call's own operands (teacher forcing)."""
     kinds = [e["kind"] for e in fused.record]
-    if internal and name != "mobilenet":     # the tail's neuron fires in the last convolution; pool and classifier read its bits
+    if internal:     # the tail's neuron fires in the last convolution; pool and classifier read its bits
         assert kinds.count("conv_lif") == NEURONS[name] and kinds.count("spike_pool_linear") == 1 and kinds.count("tail") == 0
     else:
         assert kinds.count("conv_lif") == NEURONS[name] - 1 and kinds.count("tail") == 1
@@ -393,11 +393,12 @@ def _check_recorded_operators(hip_ops, name, fused, out, T, internal):
     assert active >= 5, "the test network is nearly silent"
     stats = hip_ops.get_fused_op_call_stats()
     if internal and name == "mobilenet":
-        # row-packed spikes between the stride-1 depthwise and the pointwise layers; the stem (analog frame), the two stride-2
-        # depthwise layers and the tail go through the dense operator layer, the LIF-free last convolution through snnf_conv_bias
+        # row-packed spikes between the stride-1 depthwise and the pointwise layers; the stem (analog frame) and the two stride-2
+        # depthwise layers go through the dense operator layer; the last convolution (with the tail's neuron) runs on
+        # channel-packed bits
         packed = [e["name"] for e in fused.record if e.get("blocked")]
-        assert packed == ["features.1", "features.2", "features.4", "features.5", "features.6"], packed
-        assert stats["fallback"] == 0 and stats["triton"] == 4, stats
+        assert packed == ["features.1", "features.2", "features.4", "features.5", "features.6", "features.8"], packed
+        assert stats["fallback"] == 0 and stats["triton"] == 3, stats
     elif internal:      # nothing goes through the dense operator layer
         assert all(e.get("blocked") for e in fused.record if e["kind"] != "spike_pool_linear")
         assert stats["fallback"] == 0 and stats["triton"] == 0, stats
@@ -483,8 +484,14 @@ def test_internal_layouts_track_the_dense_executor(hip_ops, name):
     cos = float(F.cosine_similarity(got.flatten(), want.flatten(), dim=0))
     print(f"{name}: internal layouts vs dense executor, cosine similarity of the logits {cos:.5f}")
     assert cos > 0.8, cos
-    if name == "mobilenet":     # the row-packed entry points are the dense kernels with another fetch / store: the same bits
-        assert torch.equal(got, want)
+    if name == "mobilenet":
+        # The row-packed entry points are the dense kernels with another fetch / store: every spike tensor up to the last
+        # convolution is the same, bit for bit (the last convolution and the tail differ: its sums meet the tail's neuron
+        # unrounded on the internal layouts).
+        same = [(d["name"], torch.equal(d["spikes"], i["spikes"])) for d, i in zip(dense.record, internal.record)
+                if d["kind"] == "conv_lif" and i["kind"] == "conv_lif" and d["name"] == i["name"] and d["name"] != "features.8"]
+        assert len(same) == 8 and all(ok for _, ok in same), same
+        assert cos > 0.9999, cos
 
 
 @pytest.mark.gpu

@@ -677,6 +677,10 @@ class FusedSpikingMobileNet(_FusedNetwork):
                 bits = None
             if layer.lif is not None:
                 dense = self.conv_lif(name, list(dense.unbind(0)), layer)
+            elif i == len(self.layers) - 1:
+                # The last, neuron-free convolution: on channel-packed bits, with the tail's neuron in its epilogue, and the pool
+                # and the classifier on its bits.
+                return self.last_conv_and_tail_b(name, B.from_dense(dense, B.BITS), layer, self.tail_lif, self.fc_weight, self.fc_bias)
             else:
                 dense = self.plain_conv(name, dense, layer)
         if dense is None:
