@@ -232,3 +232,94 @@ def test_random_row_packed_depthwise_and_pointwise_cases(hip_ops, seed, cases):
             assert (sp != sp_d).float().mean().item() < 2e-3, what
         pointwise_cases += 1
     assert pointwise_cases >= cases // 8
+
+
+@pytest.mark.parametrize("seed,cases", [(19, 600)])
+def test_random_fused_blocked_cases(snnf_lib, seed, cases):
+    """The forms that take a neighbour into a convolution's launch: a projection shortcut in the accumulators (against the oracle
+    with the shortcut's unrounded sums as its residual), the 2x2 average pool of the spikes (bit for bit the two launches, and
+    the oracle), pool + classifier on bit-packed spikes (exact counts, float64 dot products)."""
+    from triton_snn_fusion_amd import _lib
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B, hip_convlif_backend as CB
+    rnd = random.Random(seed)
+    lay = {"nchw": B.NCHW, "c8": B.C8, "bits": B.BITS}
+    ran = collections.Counter()
+    for case in range(cases):
+        kind = rnd.choice(["shortcut", "shortcut", "pool", "tail"])
+        dtype = rnd.choice([BF16, BF16, F16])
+        g = gen(seed * 100000 + case)
+        CB.clear_packed_weight_cache()
+        if kind == "shortcut":
+            Cin, Cs = rnd.choice([16, 32, 48, 64, 128, 256]), rnd.choice([16, 32, 64, 96, 128])
+            Cout = rnd.choice([8, 24, 32, 64, 72, 128, 192, 256])
+            k, ss = rnd.choice([1, 3, 3, 3, 5]), rnd.choice([1, 2, 2, 3])
+            H, W = rnd.randint(1, 20), rnd.randint(1, 20)
+            T, N = rnd.choice([3, 4, 4, 4, 5, 8]), rnd.randint(1, 6)
+            lif, outl, want_v = rnd.choice(LIFS), rnd.choice(["bits", "bits", "c8", "nchw"]), rnd.random() < 0.6
+            Hs, Ws = (H - 1) * ss + 1 + rnd.randint(0, ss - 1), (W - 1) * ss + 1 + rnd.randint(0, ss - 1)
+            per_image = T * Cout * H * W * (Cin * k * k + Cs)
+            N = max(1, min(N, int(MAX_MACS / per_image)))
+            what = f"case {case}: {Cin}->{Cout} {H}x{W} k{k} + shortcut {Cs}->{Cout} /{ss} from {Hs}x{Ws} T={T} N={N} {dtype} -> {outl} lif={lif} membrane out={want_v}"
+            print(what, flush=True)
+            xs, x2 = spikes((T, N, Cin, H, W), 0.25, g), spikes((T, N, Cs, Hs, Ws), 0.25, g)
+            w = q(torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * k * k)) ** 0.5 * 2.0, dtype)
+            w2 = q(torch.randn(Cout, Cs, 1, 1, generator=g) * (2.0 / Cs) ** 0.5, dtype)
+            b, b2 = q(torch.randn(Cout, generator=g) * 0.1, dtype), q(torch.randn(Cout, generator=g) * 0.1, dtype)
+            shortcut = [torch.nn.functional.conv2d(x2[t], w2, b2, stride=ss) for t in range(T)]
+            ref = O.temporal_conv_lif([xs[t] for t in range(T)], w, b, torch.tensor(0.0), (1, 1), (k // 2, k // 2), (1, 1), 1, *lif, residuals=shortcut)
+            try:
+                out, v = B.conv_lif_blocked_shortcut(B.from_dense(dev(xs, dtype), B.BITS), dev(w, dtype), dev(b, dtype), [k // 2, k // 2],
+                                                     B.from_dense(dev(x2, dtype), B.BITS), dev(w2, dtype), dev(b2, dtype), [ss, ss], lif,
+                                                     out_layout=lay[outl], want_v=want_v)
+            except _lib.SnnfError as e:      # plans without room for the shortcut's stages are refused, not miscomputed
+                assert "unsupported" in str(e), str(e)
+                continue
+            if v is None:
+                v = dev(ref[1], F32)
+            check(B.to_dense(out), v, ref, v_threshold=lif[0], what=what, max_rate=2e-4)
+        elif kind == "pool":
+            Cin, Cout = rnd.choice([3, 8, 16, 32, 64, 128, 256]), rnd.choice([8, 16, 32, 64, 72, 128, 256])
+            k, s = rnd.choice([1, 3, 3, 3, 5]), rnd.choice([1, 1, 2])
+            p = k // 2
+            Ho, Wo = 2 * rnd.randint(1, 10), 2 * rnd.randint(1, 10)
+            H, W = (Ho - 1) * s + 1, (Wo - 1) * s + 1                 # (H + 2 p - k) // s + 1 == Ho with p = k // 2
+            N = rnd.randint(1, 8)
+            inl = "frame" if Cin == 3 else rnd.choice(["bits", "bits", "c8"])
+            T = 4
+            per_image = T * Cout * Ho * Wo * Cin * k * k
+            N = max(1, min(N, int(MAX_MACS / per_image)))
+            what = f"case {case}: {Cin}->{Cout} {H}x{W} k{k} s{s} + 2x2 average pool N={N} {dtype} {inl}"
+            print(what, flush=True)
+            if inl == "frame":
+                frame = q(torch.randn(N, Cin, H, W, generator=g), dtype)
+                frames, x = [frame] * T, B.input_frame(dev(frame, dtype), T)
+            else:
+                xs = q(torch.randn(T, N, Cin, H, W, generator=g), dtype) if inl == "c8" else spikes((T, N, Cin, H, W), 0.25, g)
+                frames, x = [xs[t] for t in range(T)], B.from_dense(dev(xs, dtype), lay[inl])
+            w = q(torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * k * k)) ** 0.5 * 2.0, dtype)
+            b = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+            lif = (1.0, 0.0, 2.0)
+            ref = O.temporal_conv_lif(frames, w, b, torch.tensor(0.0), (s, s), (p, p), (1, 1), 1, *lif)
+            try:
+                pooled, v = B.conv_lif_blocked_avgpool(x, dev(w, dtype), dev(b, dtype), [s, s], [p, p], lif, want_v=True)
+            except _lib.SnnfError as e:
+                assert "unsupported" in str(e), str(e)
+                continue
+            sp, v2 = B.conv_lif_blocked(x, dev(w, dtype), dev(b, dtype), [s, s], [p, p], lif, want_v=True)
+            assert torch.equal(pooled.data, B.pool_blocked(sp, False, 2, 2, 0).data) and torch.equal(v, v2), what
+            check(B.to_dense(sp), v, ref, what=what, max_rate=2e-4)
+        else:
+            T, N, C = rnd.choice([1, 2, 3, 4, 4, 8, 16]), rnd.randint(1, 20), 8 * rnd.choice([1, 2, 3, 8, 16, 40, 64, 256])
+            H, W, K = rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 3, 10, 17, 64, 70, 100, 1000])
+            scale = rnd.choice([1.0, 1.0 / T])
+            what = f"case {case}: pool + classifier on bits T={T} N={N} C={C} {H}x{W} K={K} {dtype} scale={scale}"
+            print(what, flush=True)
+            s_ = spikes((T, N, C, H, W), rnd.choice([0.1, 0.5, 1.0]), g)
+            w = q(torch.randn(K, C, generator=g) * 0.05, dtype)
+            b = q(torch.randn(K, generator=g) * 0.05, dtype) if rnd.random() < 0.8 else None
+            got = B.spike_pool_linear(B.from_dense(dev(s_, dtype), B.BITS), dev(w, dtype), None if b is None else dev(b, dtype), scale)
+            want = scale * (s_.double().sum((0, 3, 4)) @ w.double().t() / (H * W) + (0.0 if b is None else T * b.double()))
+            eps = 2.0 ** -8 if dtype == BF16 else 2.0 ** -11
+            assert torch.allclose(got.double().cpu(), want, rtol=eps, atol=2e-4), (what, float((got.double().cpu() - want).abs().max()))
+        ran[kind] += 1
+    assert ran["shortcut"] > 0.25 * cases and ran["pool"] > 0.12 * cases and ran["tail"] > 0.12 * cases, ran
