@@ -23,12 +23,19 @@ struct SpkPlan {
 // wave's LDS region and its staging slots; the largest such G (fewer, longer stages).
 bool plan_spk(const SpkGeom& g0, int tt, SpkPlan& best, int only_pc = 0, int only_g = 0, bool even = false) {
     best.score = -1.0;
+    const int cus = compute_units();
     for (int pc = 1; pc <= 32 && pc <= g0.Wo; ++pc) {
         if (only_pc > 0 && pc != only_pc) continue;
         const int pr = std::min(32 / pc, g0.Ho);
         if (even && ((pc & 1) || (pr & 1))) continue;   // 2x2 windows of the output must lie inside a patch
         const bool whole = pr == g0.Ho && pc == g0.Wo;
-        const int pi = whole ? std::max(1, std::min(g0.N, 32 / (pr * pc))) : 1;
+        int pi = whole ? std::max(1, std::min(g0.N, 32 / (pr * pc))) : 1;
+        // Whole planes of several images per patch: half as many images (idle matrix lanes) when the layer would otherwise have
+        // fewer tiles than half the compute units; a tile's K is shared by the eight waves of a workgroup at that size, so tiles
+        // are workgroups (512 -> 512 on 2 x 2 planes at batch 64: 64 workgroups of 8 images 24.1 us, 128 of 4 images 21.3 us,
+        // 256 of 2 images 22.6 us, single images 34.7 us).
+        const int oc_tiles = (g0.Cout + 63) / 64;
+        if (pi > 1 && ((g0.N + pi - 1) / pi) * oc_tiles * 2 < cus) pi >>= 1;
         const int rr = (pr - 1) * g0.sh + g0.KH;
         const int rc = (pc - 1) * g0.sw + g0.KW;
         if (rr > 255 || rc > 255) continue;
