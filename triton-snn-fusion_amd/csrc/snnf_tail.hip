@@ -798,7 +798,7 @@ extern "C" int snnf_spike_pool_linear(const void* const* spikes, int T, int N, i
     const int C8 = C / 8;
     const int parts = std::max(1, std::min(HW, kThreads / std::max(1, C8)));   // threads that share a channel group's pixels
     const int rows_per_pass = (kThreads / 64) * kRowsPerWave;
-    const int class_blocks = std::max(1, std::min((K + rows_per_pass - 1) / rows_per_pass, 1024 / std::max(1, N)));
+    const int class_blocks = std::max(1, std::min((K + rows_per_pass - 1) / rows_per_pass, 512 / std::max(1, N)));
     const int per_block = (K + class_blocks - 1) / class_blocks;
     const dim3 grid(class_blocks, N);
     const float inv_hw = 1.0f / static_cast<float>(HW);
