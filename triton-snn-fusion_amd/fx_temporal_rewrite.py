@@ -745,15 +745,16 @@ def batch_timestep_calls(gm: fx.GraphModule) -> int:
 # channel-blocked (analog values) as a `Blocked` value and the nodes call the internal-layout entry points
 # (runtime/hip_blocked_backend.py); dense tensors remain at the graph's inputs and outputs and in front of every node the
 # pass does not know. The graph functions below are the targets of the new nodes.
-def blocked_input(frames, T: int, shared: bool):
+def blocked_input(frames, T: int, shared: bool, spikes: bool = False):
     """Graph input side: one analog frame [N, C, H, W] shared by all T steps (read as it is when it has at most 8 channels),
-    or a dense [T, N, C, H, W] tensor (or the list of its T steps), into the channel-blocked layout."""
+    or a dense [T, N, C, H, W] tensor (or the list of its T steps), into the channel-blocked layout; `spikes`: the tensor is
+    the spike output of a fused operator (zeros and ones) and goes into the bit-packed layout."""
     from .runtime import hip_blocked_backend as B
     if shared:
         return B.input_frame(frames, T)
     if isinstance(frames, (list, tuple)):
         frames = torch.stack(list(frames))
-    return B.from_dense(frames, B.C8)
+    return B.from_dense(frames, B.BITS if spikes else B.C8)
 
 
 def blocked_residual(frames):
@@ -935,6 +936,14 @@ def propagate_internal_layouts(gm: fx.GraphModule) -> int:
     inputs: Dict[Tuple, fx.Node] = {}
     converted = 0
 
+    def is_spike_stack(node) -> bool:
+        """The stack is element 0 of a fused temporal operator that returns (spikes, membrane): zeros and ones."""
+        if not (isinstance(node, fx.Node) and node.op == "call_function" and node.target is operator.getitem and node.args[1] == 0):
+            return False
+        producer = node.args[0]
+        name = getattr(getattr(producer, "target", None), "__name__", "") or str(getattr(producer, "target", ""))
+        return isinstance(producer, fx.Node) and producer.op == "call_function" and "fused_temporal" in name and "lif_state" in name
+
     def as_blocked(arg, residual: bool, T_hint=None) -> fx.Node:
         kind, src, T = _sequence_source(arg, T_hint)
         if kind == "stack" and src in blocked_of:
@@ -943,6 +952,8 @@ def propagate_internal_layouts(gm: fx.GraphModule) -> int:
         if key not in inputs:
             if residual:
                 inputs[key] = graph.call_function(blocked_residual, (src if kind != "list" else list(src),))
+            elif kind == "stack" and is_spike_stack(src):
+                inputs[key] = graph.call_function(blocked_input, (src, T, False, True))
             else:
                 inputs[key] = graph.call_function(blocked_input, (src if kind != "list" else list(src), T, kind == "shared"))
         return inputs[key]
