@@ -314,8 +314,8 @@ int snnf_conv_lif_blocked(const void* const* xs, int x_layout, const void* const
  * The second convolution of a residual block together with the block's projection shortcut: out = LIF(conv(xs) + bias +
  * conv1x1(shortcut_xs) + shortcut bias), the shortcut's products accumulated as further K steps of the same output
  * tile. The reference runs the shortcut as a convolution of its own and adds its output through the residual operand of
- * run_fused_temporal_general_residual (kernels/benchmark_conv_lif_temporal_general.py:1147-1323, as called from
- * runtime/triton_convlif_backend.py:669-817); here the shortcut's output never exists in memory (and is not rounded to the
+ * run_fused_temporal_general_residual (kernels/benchmark_conv_lif_temporal_general.py:1097-1323, as called from
+ * runtime/triton_convlif_backend.py:689-817); here the shortcut's output never exists in memory (and is not rounded to the
  * activation dtype on the way), and one launch replaces two.
  *   xs[t]          : N frames [Cin, H, W] in BITS; the main convolution is KH x KW, stride 1, padding (KH-1)/2 x (KW-1)/2
  *   shortcut_xs[t] : N frames [shortcut_Cin, shortcut_H, shortcut_W] in BITS, convolved 1 x 1 with the given strides and
@@ -337,8 +337,9 @@ int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void* const* sho
  * Convolution + bias + LIF followed by a 2 x 2 / stride 2 average pool of the spikes, in one launch: the four lanes that
  * hold a pooling window add their spikes in registers and the kernel writes the quarters (0, 1/4, ..., 1: exact in 16 bits)
  * channel-blocked at half the plane; the spikes themselves are never stored. The reference runs the pool as a layer of its
- * own between two fused operators (its rewrite leaves nn.AvgPool2d in the graph, compiler/fx_lif_temporal_rewrite.py:
- * 2214-2333); results are identical to snnf_conv_lif_blocked followed by snnf_pool2d_blocked, bit for bit.
+ * own between two fused operators (its rewrites replace Conv-BN-LIF chains only, compiler/fx_lif_temporal_rewrite.py:
+ * 2037-2113, and leave pooling modules in the graph); results are identical to snnf_conv_lif_blocked followed by
+ * snnf_pool2d_blocked, bit for bit.
  *   xs, x_layout, packed_weight, geometry, LIF parameters : as in snnf_conv_lif_blocked (no residual, zero initial membrane)
  *   out   : T x N frames [Cout, Ho / 2, Wo / 2] in C8, `out_step_stride` BYTES between timesteps
  *   v_out : [N, Cout, Ho, Wo] fp32 NCHW (the membrane of the unpooled neurons) or NULL
@@ -357,8 +358,9 @@ int snnf_conv_lif_blocked_avgpool(const void* const* xs, int x_layout, int T, in
  * The network's last neuron then fires inside the convolution in front of it (snnf_conv_lif_blocked with a bit-packed
  * output) instead of inside snnf_lif_pool_linear, and this entry point is what remains of the tail: the pooling and the
  * classifier that the reference keeps as nn.AdaptiveAvgPool2d / nn.Linear modules behind its last fused convolution
- * when the convolution pattern claims that neuron (compiler/fx_lif_temporal_rewrite.py:2214-2333), and the mean over
- * the timesteps of its loop wrapper (out_scale = 1 / T). One launch: a workgroup per sample and class range.
+ * when the convolution patterns have claimed that neuron (the tail pattern only sees the neurons they left over:
+ * `excluded_lif_nodes`, compiler/fx_lif_temporal_rewrite.py:791-799), and the mean over the timesteps of its loop
+ * wrapper (out_scale = 1 / T). One launch: a workgroup per sample and class range.
  *   spikes[t] : N frames [C, H, W] in BITS     fc_weight : [K, C], fc_bias : [K] or NULL, out : [N, K], all w_dtype
  * C a multiple of 8 and at most 2048, w_dtype SNNF_BF16 or SNNF_F16, T <= SNNF_MAX_T_PER_LAUNCH.
  */
