@@ -571,6 +571,42 @@ def test_fx_graph_on_the_internal_layouts_equals_the_hand_lowered_executor(hip_o
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("T", [3, 6])
+@pytest.mark.parametrize("name", ["vgg11", "resnet18"])
+def test_internal_layouts_with_other_step_counts_take_the_unfused_forms_where_needed(hip_ops, name, T):
+    """Three timesteps (one short window) and six (two windows): the convolution + average pool launch only takes four, so the
+    graph's nodes run convolution and pool apart; the shortcut and the bit-packed tail take both. Graph == hand-lowered
+    executor bit for bit, every recorded operator against the oracle, no eager fallback."""
+    model, internal = _fused(name, T, internal=True)
+    gm, stats = R.compile_temporal(M.SingleStepModeLoopWrapper(model, T), tail_first=True, device=DEV, dtype=BF16, internal_layouts=True)
+    assert not stats.skipped
+    x = _frame(name, seed=40 + T)
+    hip_ops.reset_fused_op_call_stats()
+    with torch.no_grad():
+        got = gm(x.to(DEV, BF16))
+    internal.record = []
+    want = internal(x)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert hip_ops.get_fused_op_call_stats()["fallback"] == 0
+    kinds = [e["kind"] for e in internal.record]
+    assert kinds.count("conv_lif") == NEURONS[name] and kinds.count("spike_pool_linear") == 1
+    if name == "vgg11":
+        assert kinds.count("pool") == 4          # as launches of their own (recorded by the pooling call, not by a fused launch)
+    for e in internal.record:
+        if e["kind"] != "conv_lif":
+            continue
+        L = e["layer"]
+        rs = None if e["residuals"] is None else [r.float().cpu() for r in e["residuals"]]
+        if e.get("shortcut") is not None:
+            D = e["shortcut"]["layer"]
+            rs = [F.conv2d(f.float().cpu(), D.weight.float().cpu(), D.bias.float().cpu(), D.stride, D.padding) for f in e["shortcut"]["x"]]
+        ref = O.temporal_conv_lif([f.float().cpu() for f in e["xs"]], L.weight.float().cpu(), L.bias.float().cpu(), torch.tensor(0.0),
+                                  tuple(L.stride), tuple(L.padding), (1, 1), L.groups, *L.lif, residuals=rs)
+        check(e["spikes"], e["v"], ref, what=f"{name} T={T} {e['name']}")
+
+
+@pytest.mark.gpu
 def test_fx_graph_with_an_unknown_layer_between_fused_layers_on_the_gpu(hip_ops):
     """Dense hand-overs around a node the layout pass does not know: same logits as the dense rewritten graph up to
     near-threshold flips (both graphs run the same arithmetic on different kernels)."""
