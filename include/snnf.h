@@ -338,8 +338,9 @@ int snnf_conv_lif_blocked_shortcut(const void* const* xs, const void* const* sho
  * hold a pooling window add their spikes in registers and the kernel writes the quarters (0, 1/4, ..., 1: exact in 16 bits)
  * channel-blocked at half the plane; the spikes themselves are never stored. The reference runs the pool as a layer of its
  * own between two fused operators (its rewrites replace Conv-BN-LIF chains only, compiler/fx_lif_temporal_rewrite.py:
- * 2037-2113, and leave pooling modules in the graph); results are identical to snnf_conv_lif_blocked followed by
- * snnf_pool2d_blocked, bit for bit.
+ * 2037-2113, and leave pooling modules in the graph); results are those of snnf_conv_lif_blocked followed by
+ * snnf_pool2d_blocked: bit for bit where both launches share K among waves in the same way, to the summation order
+ * otherwise (this form plans patches of even extents, which can change that partition).
  *   xs, x_layout, packed_weight, geometry, LIF parameters : as in snnf_conv_lif_blocked (no residual, zero initial membrane)
  *   out   : T x N frames [Cout, Ho / 2, Wo / 2] in C8, `out_step_stride` BYTES between timesteps
  *   v_out : [N, Cout, Ho, Wo] fp32 NCHW (the membrane of the unpooled neurons) or NULL

@@ -247,8 +247,12 @@ def test_blocked_conv_with_its_average_pool_in_the_same_launch(B, Cin, Cout, H, 
     torch.cuda.synchronize()
     Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
     assert pooled.layout == B.C8 and pooled.shape == (T, N, Cout, Ho // 2, Wo // 2)
+    plan = B.last_conv_plan()
     spikes_out, v2 = B.conv_lif_blocked(x, dw, db, [s, s], [p, p], LIF, want_v=True)
+    plan2 = B.last_conv_plan()
     two = B.pool_blocked(spikes_out, False, 2, 2, 0)
+    # the same partition of K over waves and stages (true for these shapes): the same sums, bit for bit
+    assert (plan["waves"], plan["stage_chunks"]) == (plan2["waves"], plan2["stage_chunks"]), (plan, plan2)
     assert torch.equal(pooled.data, two.data) and torch.equal(v, v2)
     rep = check(B.to_dense(spikes_out), v, ref, what=f"blocked {Cin}->{Cout} k{k} + pool")
     assert 0.001 < float(ref[0].mean()) < 0.9, float(ref[0].mean())

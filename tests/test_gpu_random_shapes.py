@@ -305,9 +305,21 @@ def test_random_fused_blocked_cases(snnf_lib, seed, cases):
             except _lib.SnnfError as e:
                 assert "unsupported" in str(e), str(e)
                 continue
+            plan = B.last_conv_plan()
             sp, v2 = B.conv_lif_blocked(x, dev(w, dtype), dev(b, dtype), [s, s], [p, p], lif, want_v=True)
-            assert torch.equal(pooled.data, B.pool_blocked(sp, False, 2, 2, 0).data) and torch.equal(v, v2), what
-            check(B.to_dense(sp), v, ref, what=what, max_rate=2e-4)
+            plan2 = B.last_conv_plan()
+            two = B.pool_blocked(sp, False, 2, 2, 0)
+            if (plan["waves"], plan["stage_chunks"]) == (plan2["waves"], plan2["stage_chunks"]):
+                # the same partition of K over waves and stages: the same sums, bit for bit
+                assert torch.equal(pooled.data, two.data) and torch.equal(v, v2), what
+            else:
+                # even patches changed how K is shared: another summation order, spikes equal but for neurons at the threshold
+                assert float((pooled.data != two.data).float().mean()) < 2e-3, what
+            rep_ = check(B.to_dense(sp), v, ref, what=what, max_rate=2e-4)
+            check(B.to_dense(sp), v2, ref, what=what, max_rate=2e-4)
+            got = B.to_dense(pooled).float().cpu()
+            want = torch.nn.functional.avg_pool2d(ref[0].flatten(0, 1), 2).reshape(got.shape)
+            assert float((got != want).float().mean()) <= 4 * (1.0 - rep_["neurons_with_matching_history"] / rep_["neurons"]) + 2e-3, what
         else:
             T, N, C = rnd.choice([1, 2, 3, 4, 4, 8, 16]), rnd.randint(1, 20), 8 * rnd.choice([1, 2, 3, 8, 16, 40, 64, 256])
             H, W, K = rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 2, 3, 4, 5, 7, 14, 25]), rnd.choice([1, 3, 10, 17, 64, 70, 100, 1000])

@@ -282,8 +282,9 @@ def conv_lif_blocked_shortcut(x: Blocked, weight: torch.Tensor, bias: Optional[t
 def conv_lif_blocked_avgpool(x: Blocked, weight: torch.Tensor, bias: Optional[torch.Tensor], stride, padding, lif: Sequence[float],
                              want_v: bool = False):
     """Convolution + bias + LIF and the 2x2 / stride 2 average pool of its spikes in one launch: returns (the pooled tensor,
-    channel-blocked quarters at half the plane; final membrane of the unpooled neurons or None). Bit for bit
-    `pool_blocked(conv_lif_blocked(...), False, 2, 2, 0)` without the spikes ever being stored. Raises
+    channel-blocked quarters at half the plane; final membrane of the unpooled neurons or None). The result of
+    `pool_blocked(conv_lif_blocked(...), False, 2, 2, 0)` without the spikes ever being stored (bit for bit where both launches
+    share K among waves in the same way; this form plans patches of even extents, which can change the summation order). Raises
     RuntimeError("unsupported_pool: ...") where the kernel does not take the layer in this form."""
     if x.layout not in (C8, BITS) and not _is_input_frame(x):
         raise RuntimeError("unsupported_layout: conv_lif_blocked_avgpool takes inputs in C8 or BITS layout (or one dense frame of at most 8 channels)")
