@@ -13,7 +13,10 @@
 //   * spikes leave as bits: the accumulator layout gives a lane 4 consecutive channels of its pixel, the two halves of
 //     a wave exchange their nibbles with one cross-lane move and store bytes; the membrane is fp32 NCHW and optional;
 //   * deep layers with few pixels split K over WK waves of a workgroup (whole LDS stages each) and add their partial
-//     sums through LDS in a fixed order, one timestep per round.
+//     sums through LDS in a fixed order, one timestep per round;
+//   * neighbours of a convolution that fit its tile join its launch: the 1x1 projection shortcut of a residual block as
+//     further K steps on a second input (SC), the 2x2 average pool of the spikes as a reduce-scatter between the four
+//     lanes of a window (POOL), and a network's dense input frame of at most 8 channels read as it is (IN = NCHW).
 #pragma once
 
 #include <type_traits>
