@@ -226,7 +226,10 @@ def _linear_case(seed, T, M, Fin, Fout, dtype, bias=True, p=0.1):
 @pytest.mark.parametrize("T,M,Fin,Fout,bias", [(8, 64, 256, 128, True), (3, 5, 100, 37, True), (16, 1, 512, 512, False),
                                                 (4, 16, 1000, 48, True), (20, 3, 64, 16, True), (2, 33, 96, 130, True),
                                                 (4, 64, 512, 1024, True), (16, 64, 256, 1024, True), (5, 40, 200, 64, True),
-                                                (12, 17, 264, 96, False)])
+                                                (12, 17, 264, 96, False),
+                                                # wide tiles of 8 rows: ragged last row tile, K % 128 = 8, at most 8 rows, a K of two slabs and 8
+                                                (8, 20, 1032, 2048, True), (8, 7, 520, 4096, False), (5, 9, 136, 2048, True),
+                                                (3, 12, 264, 2048, True), (16, 24, 392, 1024, True)])
 def test_linear_lif_packed(hip_ops, dtype, vdtype, T, M, Fin, Fout, bias):
     x, w_dev, b_dev, w_ref, b_ref = _linear_case(400 + Fin, T, M, Fin, Fout, dtype, bias)
     ref = O.temporal_linear_lif(x, w_ref, b_ref, torch.tensor(0.0), *LIF)

@@ -263,40 +263,54 @@ constexpr int kStagedWaves = 8;
 constexpr int kSlabK = 128;                       // K elements per slab = 4 matrix K steps (wider slabs measured no faster once
                                                   // several slabs are in flight; they cost LDS and registers)
 
-template <int TT, int OCF, int SLABK> struct StagedShape {
-    static constexpr int TPW = TT >= 8 ? 4 : 2;                 // timesteps per wave: its weight fragments serve all of them (LDS reads per
+// TM rows of the batch per workgroup: 16, or 8 where 16-row tiles would leave half of the compute units idle (a fragment
+// of 16 activation rows then holds two timesteps of the 8 rows; the tile stages half the activations per weight row).
+template <int TT, int OCF, int SLABK, int TM> struct StagedShape {
+    static_assert(TM == 8 || TM == 16, "8 or 16 batch rows per tile");
+    static constexpr int FRAGS = TT * TM / 16;                   // activation fragments (16 rows: TM rows of 16 / TM timesteps) per K step
+    static constexpr int TPW = FRAGS >= 8 ? 4 : 2;               // fragments per wave: its weight fragments serve all of them (LDS reads per
                                                                  // matrix instruction fall with the size of a wave's register tile)
-    static constexpr int TG = TT / TPW;                          // wave groups along time
+    static constexpr int TG = FRAGS / TPW;                       // wave groups along time
     static constexpr int KSPLIT = kStagedWaves / TG;             // waves sharing the K steps of a slab
-    static constexpr int ROWS = TT * kTileM + OCF * kTileOC;     // operand rows per slab
+    static_assert(SLABK / 32 >= KSPLIT, "a slab has a K step for every wave of a group");
+    static constexpr int ROWS = TT * TM + OCF * kTileOC;         // operand rows per slab
     static constexpr int PITCH_B = SLABK * 2 + 16;               // bytes per operand row in LDS (the 16-byte reads of 8 consecutive rows fall into distinct banks)
     static constexpr int ITEMS = (ROWS * (SLABK / 8) + kStagedWaves * 64 - 1) / (kStagedWaves * 64);   // octets per thread
     static constexpr int RING = ITEMS <= 3 ? 4 : 2;              // slabs in flight per thread (even; ITEMS x 4 registers each, 8 for fp32 storage)
     static constexpr int PITCH = OCF * kTileOC + 4;              // floats per row of an accumulator tile in LDS
     static constexpr size_t slab_bytes = static_cast<size_t>(ROWS) * PITCH_B;
-    static constexpr size_t acc_bytes = static_cast<size_t>(KSPLIT) * TT * kTileM * PITCH * sizeof(float);
+    static constexpr size_t acc_bytes = static_cast<size_t>(KSPLIT) * TT * TM * PITCH * sizeof(float);
     static constexpr size_t lds_bytes = slab_bytes > acc_bytes ? slab_bytes : acc_bytes;
 };
 
-template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK>
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM>
 __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
                                                                               const XT* __restrict__ bias,
                                                                               const VT* __restrict__ v_init, XT* __restrict__ spikes,
                                                                               VT* __restrict__ v_out, LifParams lif,
                                                                               float* __restrict__ ws_partial, int* __restrict__ ws_count,
                                                                               int slabs_per_part) {
-    using SH = StagedShape<TT, OCF, SLABK>;
+    using SH = StagedShape<TT, OCF, SLABK, TM>;
     constexpr int kSlabOctets = SLABK / 8;            // 16-byte staging items per operand row
     constexpr int kSlabPitch = SH::PITCH_B;
     constexpr int NT = kStagedWaves * 64;
     constexpr int TILE_OC = OCF * kTileOC;
-    constexpr int OUTS = TILE_OC * kTileM;
+    constexpr int OUTS = TILE_OC * TM;
     extern __shared__ __align__(16) unsigned char staged_lds[];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int oc0 = blockIdx.x * TILE_OC;
-    const int m0 = blockIdx.y * kTileM;
+    const int m0 = blockIdx.y * TM;
+
+    // The output of this thread in the recurrence at the end (a tile has at most as many as the workgroup has threads):
+    // its bias and its membrane are fetched here, so that the recurrence does not begin with a trip to memory.
+    static_assert(OUTS <= NT, "one output per thread");
+    const int out_m = m0 + tid / TILE_OC, out_oc = oc0 + tid % TILE_OC;
+    const bool out_live = tid < OUTS && out_m < g.M && out_oc < g.Fout;
+    const int64_t out_index = static_cast<int64_t>(out_live ? out_m : 0) * g.Fout + (out_live ? out_oc : 0);
+    const float bv = bias != nullptr ? to_float(bias[out_live ? out_oc : 0]) : 0.0f;
+    const float v_first = v_init != nullptr ? to_float(v_init[out_index]) : 0.0f;
 
     // Staging items of this thread: item i = tid + j * NT is octet i % 16 of operand row i / 16 (NT is a multiple of 16, so
     // the octet is the same for all of a thread's items). Rows beyond M / Fout re-read the last real row; what they produce
@@ -312,17 +326,17 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         item_live[j] = row < SH::ROWS;
         const int r = item_live[j] ? row : 0;
         const XT* ptr;
-        if (r < TT * kTileM) {
-            const int t = r / kTileM;
+        if (r < TT * TM) {
+            const int t = r / TM;
             const void* base = xs.p[0];
 #pragma unroll
             for (int u = 1; u < TT; ++u) base = t == u ? xs.p[u] : base;
-            ptr = static_cast<const XT*>(base) + static_cast<int64_t>(min(m0 + r % kTileM, g.M - 1)) * g.x_row_stride;
+            ptr = static_cast<const XT*>(base) + static_cast<int64_t>(min(m0 + r % TM, g.M - 1)) * g.x_row_stride;
         } else {
-            ptr = W + static_cast<int64_t>(min(oc0 + r - TT * kTileM, g.Fout - 1)) * g.Fin;
+            ptr = W + static_cast<int64_t>(min(oc0 + r - TT * TM, g.Fout - 1)) * g.Fin;
         }
         item_row[j] = ptr;
-        item_is_w[j] = r >= TT * kTileM;
+        item_is_w[j] = r >= TT * TM;
         item_dst[j] = static_cast<uint32_t>(r * kSlabPitch + octet * 16);
     }
 
@@ -370,58 +384,69 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         fetch(slab0 + r, r);
         __builtin_amdgcn_sched_barrier(0);      // oldest slab first, as in the loop: its wait then leaves the others in flight
     }
+    // A slab parked in LDS from the ring, and this wave's K steps of a parked slab (every KSPLIT-th), four at a time: their
+    // operand reads go out together.
+    auto park = [&](int r, unsigned char* buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < SH::ITEMS; ++j)
+            if (item_live[j])
+                *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r], pre_part[r] == (item_is_w[j] ? 1 : 2));
+    };
+    auto multiply = [&](const unsigned char* buf) __attribute__((always_inline)) {
+        constexpr int OWN = SLABK / 32 / SH::KSPLIT;
+        const unsigned char* own = buf + frag_off + (kp % SH::KSPLIT) * 64;
+#pragma unroll
+        for (int i0 = 0; i0 < OWN; i0 += 4) {
+            u32x4 a[4][OCF], b[4][SH::TPW];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (i0 + i < OWN) {
+                    const int off = (i0 + i) * SH::KSPLIT * 64;
+#pragma unroll
+                    for (int f = 0; f < OCF; ++f) a[i][f] = *reinterpret_cast<const u32x4*>(own + (TT * TM + f * kTileOC) * kSlabPitch + off);
+#pragma unroll
+                    for (int u = 0; u < SH::TPW; ++u) b[i][u] = *reinterpret_cast<const u32x4*>(own + (tg * SH::TPW + u) * 16 * kSlabPitch + off);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (i0 + i < OWN) {
+#pragma unroll
+                    for (int u = 0; u < SH::TPW; ++u)
+#pragma unroll
+                        for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[i][f], b[i][u], acc[f][u]);
+                }
+            }
+        }
+    };
+    // Parking slab s + 1 (in the other buffer) ahead of the multiplication of slab s, so that a slab's barrier does not wait
+    // for its writes, measured slower (64 rows x 8 timesteps 2048 -> 1024: 10.0 -> 10.4 us, 16 rows 25088 -> 4096: 63 -> 76):
+    // the wait for the loads of s + 1 then stands before the work on s.
     for (int round = 0; round < rounds; ++round) {
 #pragma unroll
         for (int r = 0; r < RING; ++r) {
             const int slab = slab0 + round * RING + r;
             unsigned char* buf = staged_lds + (DB ? (r & 1) * SH::slab_bytes : 0);      // RING is even
-#pragma unroll
-            for (int j = 0; j < SH::ITEMS; ++j)
-                if (item_live[j])
-                    *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r], pre_part[r] == (item_is_w[j] ? 1 : 2));
+            park(r, buf);
             __syncthreads();
             fetch(slab + RING, r);
-            // This wave's K steps of the slab (every KSPLIT-th), four at a time: their operand reads go out together.
-            constexpr int OWN = SLABK / 32 / SH::KSPLIT;
-            const unsigned char* own = buf + frag_off + (kp % SH::KSPLIT) * 64;
-#pragma unroll
-            for (int i0 = 0; i0 < OWN; i0 += 4) {
-                u32x4 a[4][OCF], b[4][SH::TPW];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (i0 + i < OWN) {
-                        const int off = (i0 + i) * SH::KSPLIT * 64;
-#pragma unroll
-                        for (int f = 0; f < OCF; ++f) a[i][f] = *reinterpret_cast<const u32x4*>(own + (TT * kTileM + f * kTileOC) * kSlabPitch + off);
-#pragma unroll
-                        for (int u = 0; u < SH::TPW; ++u) b[i][u] = *reinterpret_cast<const u32x4*>(own + (tg * SH::TPW + u) * kTileM * kSlabPitch + off);
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (i0 + i < OWN) {
-#pragma unroll
-                        for (int u = 0; u < SH::TPW; ++u)
-#pragma unroll
-                            for (int f = 0; f < OCF; ++f) acc[f][u] = mfma16<XT>(a[i][f], b[i][u], acc[f][u]);
-                    }
-                }
-            }
+            multiply(buf);
             if (!DB) __syncthreads();
         }
     }
     if (DB) __syncthreads();
 
-    // Accumulators -> LDS as [K part][t][m][PITCH]; D[i = oc][j = m]: lane holds column j = lane % 16, rows 4 (lane / 16) + r.
+    // Accumulators -> LDS as [K part][t][m][PITCH] (row t * TM + m is row (t * TM + m) % 16 of fragment (t * TM + m) / 16);
+    // D[i = oc][j = row]: lane holds column j = lane % 16, rows 4 (lane / 16) + r.
     float* partial = reinterpret_cast<float*>(staged_lds);
-    constexpr int SLAB_F = kTileM * SH::PITCH;
+    constexpr int SLAB_F = TM * SH::PITCH;
 #pragma unroll
     for (int u = 0; u < SH::TPW; ++u)
 #pragma unroll
         for (int f = 0; f < OCF; ++f)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                partial[(kp * TT + tg * SH::TPW + u) * SLAB_F + (lane & 15) * SH::PITCH + f * kTileOC + (lane >> 4) * 4 + r] = acc[f][u][r];
+                partial[((kp * SH::FRAGS + tg * SH::TPW + u) * 16 + (lane & 15)) * SH::PITCH + f * kTileOC + (lane >> 4) * 4 + r] = acc[f][u][r];
     __syncthreads();
 
     // K split over workgroups: every workgroup of a tile leaves its sums in the workspace and counts itself in; the one
@@ -459,14 +484,10 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         if (!arrived_last) return;
     }
 
-    for (int e = tid; e < OUTS; e += NT) {
+    if (out_live) {
+        const int e = tid;
         const int slot = (e / TILE_OC) * SH::PITCH + e % TILE_OC;
-        const int m = m0 + e / TILE_OC;
-        const int oc = oc0 + e % TILE_OC;
-        if (m >= g.M || oc >= g.Fout) continue;
-        const float bv = bias != nullptr ? to_float(bias[oc]) : 0.0f;
-        const int64_t o = static_cast<int64_t>(m) * g.Fout + oc;
-        float v = v_init != nullptr ? to_float(v_init[o]) : 0.0f;
+        float v = v_first;
         const float* __restrict__ all = ws_partial + static_cast<int64_t>(tile) * parts * (TT * OUTS) + e;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
@@ -479,10 +500,10 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
                     for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
                 }
                 const float cur = sum + bv;
-                spikes[t * g.spike_step_stride + o] = spike_value<XT>(lif_step(cur, v, lif));
+                spikes[t * g.spike_step_stride + out_index] = spike_value<XT>(lif_step(cur, v, lif));
             }
         }
-        v_out[o] = from_float<VT>(v);
+        v_out[out_index] = from_float<VT>(v);
     }
 }
 
@@ -492,14 +513,15 @@ struct LinWorkspace {
     size_t bytes;
 };
 constexpr size_t kLinCounterBytes = 64 * 1024;     // 16384 tiles
+constexpr int kLinLongK = 96;                      // K slabs from which two K parts of 16-row tiles beat 8-row tiles (see linear_half_row_tiles)
 
-template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK>
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM>
 int launch_staged_db(dim3 grid, int slabs_per_part, const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias,
                      const void* v_init, void* spikes, void* v_out, const LifParams& lif, hipStream_t stream) {
-    using SH = StagedShape<TT, OCF, SLABK>;
+    using SH = StagedShape<TT, OCF, SLABK, TM>;
     constexpr size_t lds = DB ? 2 * SH::slab_bytes : SH::lds_bytes;
     static_assert(lds <= 160 * 1024 && SH::acc_bytes <= lds, "slabs exceed LDS");
-    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB, SLABK>;
+    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB, SLABK, TM>;
     if (lds > 64 * 1024) {
         static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -523,44 +545,72 @@ inline int linear_split_parts(int64_t tiles, int unit_slabs, size_t part_bytes, 
     return 2;
 }
 
-template <typename XT, typename VT, int TT, int OCF>
+template <typename XT, typename VT, int TT, int OCF, int TM = kTileM, int SLABK = kSlabK>
 int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
                   void* v_out, const LifParams& lif, hipStream_t stream) {
-    dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + kTileM - 1) / kTileM);
+    dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + TM - 1) / TM);
     if (grid.y > 65535) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif: M=%d too large", g.M);
-    const int unit_slabs = g.kparts * ((g.Fin + kSlabK - 1) / kSlabK);        // all K parts of an fp32 tensor
+    const int unit_slabs = g.kparts * ((g.Fin + SLABK - 1) / SLABK);          // all K parts of an fp32 tensor
     const int64_t tiles = static_cast<int64_t>(grid.x) * grid.y;
-    const size_t part_bytes = static_cast<size_t>(TT) * OCF * kTileOC * kTileM * sizeof(float);
-    int parts = ws.base != nullptr ? linear_split_parts(tiles, unit_slabs, part_bytes, ws.bytes) : 1;
+    const size_t part_bytes = static_cast<size_t>(TT) * OCF * kTileOC * TM * sizeof(float);
+    int parts = ws.base != nullptr ? linear_split_parts(tiles, unit_slabs * (SLABK / kSlabK), part_bytes, ws.bytes) : 1;
     const int unit_slabs_per_part = (unit_slabs + parts - 1) / parts;
-    using SH = StagedShape<TT, OCF, kSlabK>;
+    using SH = StagedShape<TT, OCF, SLABK, TM>;
     parts = (unit_slabs + unit_slabs_per_part - 1) / unit_slabs_per_part;      // no empty part
     grid.z = parts;
     // Two slab buffers where a CU gets one workgroup anyway (they would cost occupancy otherwise) and both fit LDS.
     constexpr bool can_double = 2 * SH::slab_bytes <= 160 * 1024;
     if constexpr (can_double) {
         if (tiles * parts <= compute_units())
-            return launch_staged_db<XT, VT, TT, OCF, true, kSlabK>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            return launch_staged_db<XT, VT, TT, OCF, true, SLABK, TM>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     }
-    return launch_staged_db<XT, VT, TT, OCF, false, kSlabK>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_staged_db<XT, VT, TT, OCF, false, SLABK, TM>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+}
+
+// Tiles of 8 batch rows instead of 16 (a workgroup then stages 8 x T activation rows per slab for its 32 weight rows):
+// for batches of up to 8 rows, whose tiles of 16 would stage every row twice, and where tiles of 16 rows give workgroups
+// to at most half of the compute units. Measured at 8 timesteps, 16-bit tensors (16 -> 8 rows): 64 rows 2048 -> 1024
+// 13.5 -> 10.5 us (16 timesteps: 24.8 -> 16.8), 24 rows 1024 -> 2048 9.1 -> 7.4, 16 rows 4096 -> 4096 20.0 -> 16.8 (against
+// 16-row tiles with K split in two), 1 row 25088 -> 4096 61.9 -> 43.5; slower where 16-row tiles fill the chip (128 rows
+// 2048 -> 1024 15.3 -> 18.7) and for the longest K, where two K parts of 16-row tiles read every weight once and two
+// 8-row tiles read it twice (16 rows 25088 -> 4096: 65 -> 71 with a workspace).
+inline bool linear_half_row_tiles(const LinWorkspace& ws, const LinGeom& g) {
+    if (g.M <= 8) return true;
+    const int64_t m_tiles = (g.M + kTileM - 1) / kTileM;
+    const int64_t tiles16 = g.Fout % (2 * kTileOC) == 0 ? g.Fout / (2 * kTileOC) * m_tiles : (g.Fout + kTileOC - 1) / kTileOC * m_tiles;
+    if (tiles16 * 2 > compute_units()) return false;
+    const int unit_slabs = g.kparts * ((g.Fin + kSlabK - 1) / kSlabK);
+    return ws.base == nullptr || unit_slabs < kLinLongK;
+}
+
+template <typename XT, typename VT, int OCF, int TM>
+int launch_staged_tt(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+                     void* v_out, const LifParams& lif, hipStream_t stream) {
+    // 4 timesteps of 8 rows are two fragments: their eight waves split a slab of 8 K steps. Narrow tiles of 8 rows take
+    // slabs of 8 K steps too: with one weight fragment a wave has too little to do per barrier otherwise (8 timesteps,
+    // 16 rows, 2048 -> 1024: 8.9 -> 7.9 us; 8 rows 25088 -> 1000: 39.5 -> 33.6); wide tiles are slower that way (64 rows
+    // 2048 -> 1024: 10.1 -> 11.0 us).
+    constexpr int kWide = (TM == 8 && OCF == 1) ? 2 * kSlabK : kSlabK;
+    if (g.T <= 4) return launch_staged<XT, VT, 4, OCF, TM, TM == 8 ? 2 * kSlabK : kSlabK>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    if (g.T <= 8) return launch_staged<XT, VT, 8, OCF, TM, kWide>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_staged<XT, VT, 16, OCF, TM, kWide>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 template <typename XT, typename VT, bool FAST>
 int launch_tt(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
               void* v_out, const LifParams& lif, hipStream_t stream) {
-    // Two feature fragments per workgroup (half the activation traffic) when that still leaves at least 128 workgroups.
-    const bool wide = g.Fout % (2 * kTileOC) == 0 &&
-                      static_cast<int64_t>(g.Fout / (2 * kTileOC)) * ((g.M + kTileM - 1) / kTileM) >= 128;
     if constexpr (FAST) {
         if (g.T > 2) {
-            if (wide) {
-                if (g.T <= 4) return launch_staged<XT, VT, 4, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-                if (g.T <= 8) return launch_staged<XT, VT, 8, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-                return launch_staged<XT, VT, 16, 2>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            // Two feature fragments per workgroup (half the activation traffic) when that still leaves at least 128 workgroups.
+            const bool half_rows = linear_half_row_tiles(ws, g);
+            const int tm = half_rows ? 8 : kTileM;
+            const bool wide = g.Fout % (2 * kTileOC) == 0 && static_cast<int64_t>(g.Fout / (2 * kTileOC)) * ((g.M + tm - 1) / tm) >= 128;
+            if (half_rows) {
+                if (wide) return launch_staged_tt<XT, VT, 2, 8>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+                return launch_staged_tt<XT, VT, 1, 8>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
             }
-            if (g.T <= 4) return launch_staged<XT, VT, 4, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-            if (g.T <= 8) return launch_staged<XT, VT, 8, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
-            return launch_staged<XT, VT, 16, 1>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            if (wide) return launch_staged_tt<XT, VT, 2, kTileM>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            return launch_staged_tt<XT, VT, 1, kTileM>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
         }
     }
     if (g.T <= 1) return launch_one<XT, VT, 1, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
