@@ -253,10 +253,11 @@ int launch_one(const StepPtrs& xs, const LinGeom& g, const void* W, const void* 
 // Staged variant (4 timesteps or more, 16-byte aligned rows, Fin % 8 == 0). Operand fragments fetched straight from
 // global memory put the 16 rows of a fragment in 16 adjacent lanes, i.e. 16 different cache lines per 256 bytes
 // fetched, and the texture path then delivers about 16 bytes per clock and CU. Here a K slab of 128 elements of every
-// operand row (the 16 x TT activation rows and the 16 x OCF weight rows of the tile) is fetched with adjacent lanes on
+// operand row (the TM x TT activation rows and the 16 x OCF weight rows of the tile) is fetched with adjacent lanes on
 // adjacent 16 bytes, parked in LDS (row pitch 272 bytes: the 16-byte reads of 8 consecutive rows fall into distinct
-// banks), and the waves read their fragments from there. Wave w owns timesteps (w % TG) * TPW ... and, when fewer than 8
-// timesteps leave waves to spare, every KSPLIT-th K step of the slab. The next slab's loads are in flight while the
+// banks), and the waves read their fragments from there. Wave w owns activation fragments (w % TG) * TPW ... (a fragment
+// is one timestep of 16 rows or two timesteps of 8) and, when fewer than 8 fragment groups leave waves to spare, every
+// KSPLIT-th K step of the slab. The next slab's loads are in flight while the
 // current one multiplies. The accumulators meet in LDS (aliasing the slab) for the LIF recurrence.
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kStagedWaves = 8;
@@ -576,11 +577,14 @@ int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, 
 // 8-row tiles read it twice (16 rows 25088 -> 4096: 65 -> 71 with a workspace).
 inline bool linear_half_row_tiles(const LinWorkspace& ws, const LinGeom& g) {
     if (g.M <= 8) return true;
-    const int64_t m_tiles = (g.M + kTileM - 1) / kTileM;
-    const int64_t tiles16 = g.Fout % (2 * kTileOC) == 0 ? g.Fout / (2 * kTileOC) * m_tiles : (g.Fout + kTileOC - 1) / kTileOC * m_tiles;
-    if (tiles16 * 2 > compute_units()) return false;
+    const int64_t oc_tiles = g.Fout % (2 * kTileOC) == 0 ? g.Fout / (2 * kTileOC) : (g.Fout + kTileOC - 1) / kTileOC;
+    if (oc_tiles * ((g.M + kTileM - 1) / kTileM) * 2 > compute_units()) return false;
     const int unit_slabs = g.kparts * ((g.Fin + kSlabK - 1) / kSlabK);
-    return ws.base == nullptr || unit_slabs < kLinLongK;
+    if (ws.base == nullptr || unit_slabs < 32) return true;                  // K is not split either way
+    if (oc_tiles * ((g.M + 7) / 8) * 2 <= compute_units()) return true;      // tiles of 8 rows split K as well
+    // 16-row tiles in two K parts or 8-row tiles unsplit: up to 4 timesteps the split wins (16 rows 4096 -> 4096: 13.6
+    // against 14.0 us), beyond that only for the longest K.
+    return g.T > 4 && unit_slabs < kLinLongK;
 }
 
 template <typename XT, typename VT, int OCF, int TM>
