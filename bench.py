@@ -39,6 +39,8 @@ def _parse():
     ap.add_argument("--layers", default=None, choices=["resnet18", "vgg11"],
                     help="instead of a workload: time every fused conv layer shape of the spiking ResNet-18 (T=4, B=16, "
                          "224x224) or VGG-11 (T=4, B=64, 32x32) configuration on its own, synthetic spike inputs")
+    ap.add_argument("--batch", type=int, default=None,
+                    help="with --layers: time the layer shapes at this batch instead of the configuration's (16 for ResNet-18, 64 for VGG-11)")
     ap.add_argument("--internal", action="store_true",
                     help="with --layers: time the layers as the network executor runs them, on the bit-packed / channel-blocked internal layouts")
     ap.add_argument("--model", default=None, choices=["resnet18", "vgg11", "mobilenet"],
@@ -234,7 +236,7 @@ def _roofline(bound: str, work: float, ms: float, traffic=None):
             "frac": round(achieved / peak, 4), "traffic": traffic}
 
 
-def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, internal: bool = False):
+def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, internal: bool = False, batch_override=None):
     """Times every fused conv(+residual)+LIF layer shape of a network configuration on its own (graph replay, HIP events).
     `internal`: the layer as it runs inside the network executor, spikes bit-packed on both sides (an analog frame
     channel-blocked), final membrane not written; otherwise through the dense operator (NCHW in and out, fp32 membrane)."""
@@ -243,6 +245,8 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
     from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
     ops = torch.ops.snn_custom
     layers, batch = (W.RESNET18_LAYERS, W.RESNET18_BATCH) if which == "resnet18" else (W.VGG11_LAYERS, W.VGG11_BATCH)
+    if batch_override is not None:
+        batch = batch_override      # not the configuration's batch: how the kernels behave with more rounds of waves per launch
     T, dev = 4, torch.device("cuda:0")
     esize = torch.empty((), dtype=dtype).element_size()
     g = torch.Generator(device="cpu")
@@ -587,7 +591,7 @@ def main() -> int:
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
 
     if args.layers is not None:
-        sweep = _layer_sweep(args.layers, dtype, args.dtype, args.steps, args.warmup, internal=args.internal)
+        sweep = _layer_sweep(args.layers, dtype, args.dtype, args.steps, args.warmup, internal=args.internal, batch_override=args.batch)
         stats = ops.get_fused_op_call_stats()
         sweep["native_calls"], sweep["fallback_calls"] = stats["triton"], stats["fallback"]
         print(json.dumps(sweep))
