@@ -317,9 +317,9 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
 
 
 def _plan_summary() -> str:
-    from triton_snn_fusion_amd.runtime.hip_convlif_backend import last_conv_plan
+    from triton_snn_fusion_amd.runtime.hip_blocked_backend import last_conv_plan
     plan = last_conv_plan()
-    keys = ("kernel", "variant", "window", "tile", "waves", "stage_chunks", "grid")
+    keys = ("kernel", "variant", "window", "tile", "waves", "stage_chunks", "grid", "rows", "features_in", "features_out", "x")
     return " ".join(f"{k}={plan[k]}" for k in keys if k in plan)
 
 

@@ -369,6 +369,27 @@ int snnf_spike_pool_linear(const void* const* spikes, int T, int N, int C, int H
                            const void* fc_bias, int K, int w_dtype, void* out, float out_scale, void* stream);
 
 /*
+ * Temporal Linear + LIF on the internal layouts: the operator of snnf_linear_lif_ws with its spikes leaving as bits and its
+ * activation rows arriving as 16-bit elements or as bits, for a network executor that owns both tensors. Its use: a
+ * convolution + LIF on a plane of a few pixels (the last stage of a VGG on 32 x 32 inputs works on 2 x 2 planes) is a
+ * matrix product of a sample's whole frame, [Cin x H x W] -> [Cout x H x W], with a weight matrix that holds every tap at
+ * the pair of pixels it connects and no padding; with the frame's features in the order (channel / 8, pixel, channel % 8)
+ * a C8 frame is such a row of elements, a BITS frame such a row of bits, and the spike bits written here are a BITS frame.
+ * Same launcher as snnf_linear_lif (kernels/generated_temporal_linear_lif_kernel.py:205-363); the reference runs such a
+ * layer through its convolution kernel (kernels/benchmark_conv_lif_temporal_general.py:629-676) and has no counterpart.
+ *   xs[t]     : [M, Fin] elements of `dtype`, row stride `x_row_stride` elements (x_bits == 0), or [M, Fin / 8] bytes, bit j
+ *               of byte b = feature 8 b + j, row stride `x_row_stride` bytes (x_bits != 0)
+ *   weight    : [Fout, Fin] `dtype`, bias : [Fout] `dtype` or NULL     v_init : [M, Fout] fp32 or NULL (zero)
+ *   spike_bits: [T, M, Fout / 8] bytes, `spike_step_stride` bytes between timesteps     v_out : [M, Fout] fp32 or NULL
+ *   workspace : as in snnf_linear_lif_ws, or NULL
+ * 3 <= T <= 8, Fin a multiple of 8, Fout of 32, dtype SNNF_BF16 or SNNF_F16; SNNF_ERR_UNSUPPORTED otherwise.
+ */
+int snnf_linear_lif_bits(const void* const* xs, int x_bits, int T, int M, int Fin, int64_t x_row_stride, int dtype,
+                         const void* weight, const void* bias, int Fout, const void* v_init, void* spike_bits,
+                         int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Registers a measured launch choice for snnf_conv_lif_blocked on one layer shape (the counterpart of the per-kernel-key
  * "best config" the reference's autotuner keeps, kernels/benchmark_conv_lif_temporal_general.py:524-558,1332-1369):
  * columns of a wave's output patch (rows follow: 32 / columns), channel groups of 8 per LDS stage (a power of two) and

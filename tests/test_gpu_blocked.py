@@ -611,3 +611,94 @@ def test_two_blocks_chained_on_row_packed_spikes(B):
     assert torch.equal(B.unpack_rowbits(p1, dtype), s1)
     assert torch.equal(B.unpack_rowbits(p2, dtype), s2)
     assert torch.equal(B.unpack_rowbits(p3, dtype), s3) and torch.equal(pv3, v3)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Convolutions on planes of a few pixels run as one matrix product per frame on the Linear + LIF kernel
+# (snnf_linear_lif_bits: activation rows as C8 elements or as bits, spikes out as bits)
+# ---------------------------------------------------------------------------------------------------------------
+PLANE_CASES = [  # T, N, Cin, Cout, H, W, k, dtype
+    (4, 64, 128, 128, 2, 2, 3, BF16), (4, 7, 64, 72, 2, 2, 3, F16), (6, 20, 32, 64, 1, 1, 3, BF16), (3, 5, 16, 16, 2, 1, 3, BF16),
+    (8, 33, 256, 128, 1, 2, 1, F16), (5, 9, 24, 40, 2, 2, 5, BF16), (4, 1, 512, 512, 2, 2, 3, BF16), (4, 16, 1024, 256, 2, 2, 3, BF16),
+]
+
+
+@pytest.mark.parametrize("source", ["bits", "quarters"])
+@pytest.mark.parametrize("T,N,Cin,Cout,H,W,k,dtype", PLANE_CASES)
+def test_small_plane_convolutions_as_matrix_products(B, T, N, Cin, Cout, H, W, k, dtype, source):
+    import torch.nn.functional as F
+    g = gen(9100 + Cin + Cout + T + N)
+    if source == "bits":
+        x = spikes((T, N, Cin, H, W), 0.2, g)
+        bx = B.from_dense(dev(x, dtype), B.BITS)
+    else:       # what an average pool in front of the layer leaves: quarters, channel-blocked
+        x = F.avg_pool2d(spikes((T * N, Cin, 2 * H, 2 * W), 0.3, g), 2).reshape(T, N, Cin, H, W)
+        bx = B.from_dense(dev(x, dtype), B.C8)
+    w = q(torch.randn(Cout, Cin, k, k, generator=g) * (2.0 / (Cin * min(k * k, H * W))) ** 0.5 * 2.5, dtype)
+    b = q(torch.randn(Cout, generator=g) * 0.1, dtype)
+    ref = O.temporal_conv_lif([x[t] for t in range(T)], w, b, torch.tensor(0.0), (1, 1), (k // 2, k // 2), (1, 1), 1, *LIF)
+    dw, db = dev(w, dtype), dev(b, dtype)
+    out, v = B.conv_lif_blocked(bx, dw, db, 1, k // 2, LIF, out_layout=B.BITS)
+    plan = B.last_conv_plan()
+    assert v is None and plan["kernel"] == "plane_matrix" and plan["x"] == ("bits" if source == "bits" else "c8"), plan
+    assert out.layout == B.BITS and out.shape == (T, N, Cout, H, W)
+    rep = check(B.to_dense(out), ref[1], ref, what=f"plane matrix {Cin}->{Cout} {H}x{W} k{k} {source}")      # spikes only
+    assert 0.001 < float(ref[0].mean()) < 0.9
+    assert rep["neurons_with_matching_history"] >= 0.999 * rep["neurons"], rep
+    # the same layer with a membrane output stays on the convolution kernel and agrees up to flips at the threshold
+    out_c, v_c = B.conv_lif_blocked(bx, dw, db, 1, k // 2, LIF, out_layout=B.BITS, want_v=True)
+    assert B.last_conv_plan()["kernel"] != "plane_matrix"
+    check(B.to_dense(out_c), v_c, ref, what="the same layer on the convolution kernel")
+    assert (B.to_dense(out_c) != B.to_dense(out)).float().mean().item() < 2e-3
+    # a second call finds the expanded matrix in the cache and writes the same bits
+    out_again, _ = B.conv_lif_blocked(bx, dw, db, 1, k // 2, LIF, out_layout=B.BITS)
+    assert torch.equal(out_again.data, out.data)
+
+
+def test_linear_lif_on_bits_through_the_c_abi(snnf_lib):
+    """snnf_linear_lif_bits against the oracle's Linear + LIF: rows of elements and rows of bits, an initial membrane, the
+    final membrane, ragged rows, a K long enough for the split over workgroups; and what it refuses."""
+    from triton_snn_fusion_amd import _lib
+    for seed, (T, M, Fin, Fout, x_bits, dtype, tensor_v) in enumerate([(4, 40, 264, 96, 1, BF16, True), (8, 5, 4096, 64, 0, F16, False),
+                                                                        (3, 64, 2048, 2048, 1, BF16, False), (5, 16, 4104, 32, 1, BF16, True)]):
+        g = gen(9200 + seed)
+        x = spikes((T, M, Fin), 0.2, g) if x_bits else q(torch.rand(T, M, Fin, generator=g) * spikes((T, M, Fin), 0.3, g), dtype)
+        w = q(torch.randn(Fout, Fin, generator=g) * (3.0 / Fin ** 0.5), dtype)
+        b = q(torch.randn(Fout, generator=g) * 0.1, dtype)
+        v0 = torch.rand(M, Fout, generator=g) * 0.8 if tensor_v else None
+        ref = O.temporal_linear_lif(x, w, b, v0 if tensor_v else torch.tensor(0.0), *LIF)
+        if x_bits:
+            weights = (2 ** torch.arange(8, dtype=torch.int32))
+            dx = (x.reshape(T, M, Fin // 8, 8).to(torch.int32) * weights).sum(-1).to(torch.uint8).to(DEV)
+            stride = Fin // 8
+        else:
+            dx = x.to(DEV, dtype)
+            stride = Fin
+        dw, db = w.to(DEV, dtype), b.to(DEV, dtype)
+        dv0 = v0.to(DEV) if tensor_v else None
+        bits = torch.full((T, M, Fout // 8), 0xA5, dtype=torch.uint8, device=DEV)
+        v = torch.full((M, Fout), 7.0, device=DEV)
+        need = int(snnf_lib.snnf_linear_lif_workspace_bytes(T, M, Fin, Fout))
+        ws = torch.zeros(need, dtype=torch.uint8, device=DEV) if need else None
+        print(f"linear on bits: T={T} M={M} {Fin}->{Fout} x_bits={x_bits} {dtype} workspace {need}", flush=True)
+        rc = snnf_lib.snnf_linear_lif_bits(_lib.packed_step_pointers(dx), x_bits, T, M, Fin, stride, _lib.dtype_code(dtype), dw.data_ptr(),
+                                           db.data_ptr(), Fout, _lib.ptr(dv0), bits.data_ptr(), M * (Fout // 8), v.data_ptr(), *LIF,
+                                           _lib.ptr(ws), need, _lib.current_stream(dx.device))
+        assert rc == 0, snnf_lib.snnf_last_error()
+        torch.cuda.synchronize()
+        got = ((bits.cpu().to(torch.int32).unsqueeze(-1) >> torch.arange(8, dtype=torch.int32)) & 1).reshape(T, M, Fout).float()
+        check(got, v, ref, what=f"linear on bits {Fin}->{Fout}")
+        assert 0.001 < float(ref[0].mean()) < 0.9
+        if ws is not None:
+            assert int(ws[: 64 * 1024].view(torch.int32).abs().sum()) == 0
+    x = torch.zeros(4, 8, 64, dtype=BF16, device=DEV)
+    w = torch.zeros(32, 64, dtype=BF16, device=DEV)
+    out = torch.zeros(4, 8, 4, dtype=torch.uint8, device=DEV)
+    def call(T=4, Fin=64, Fout=32, stride=64, dtype=BF16, step=32):
+        return snnf_lib.snnf_linear_lif_bits(_lib.packed_step_pointers(x), 0, T, 8, Fin, stride, _lib.dtype_code(dtype), w.data_ptr(), None, Fout,
+                                             None, out.data_ptr(), step, None, *LIF, None, 0, _lib.current_stream(x.device))
+    assert call() == 0
+    for bad, reason in ((dict(T=2), b"unsupported_window"), (dict(Fout=24), b"unsupported_shape"), (dict(Fin=60), b"unsupported_shape"),
+                        (dict(dtype=F32), b"unsupported_dtype"), (dict(stride=60), b"x_row_stride"), (dict(step=16), b"spike_step_stride")):
+        assert call(**bad) != 0 and reason in snnf_lib.snnf_last_error(), (bad, snnf_lib.snnf_last_error())
+    torch.cuda.synchronize()

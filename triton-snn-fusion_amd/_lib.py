@@ -62,6 +62,7 @@ SIGNATURES = {
                                             _vp, _vp, _i, _i64, _vp, _i, _f, _f, _f, _vp]),
     "snnf_conv_lif_blocked_avgpool": (_i, [_pp, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _f, _f, _f, _vp]),
     "snnf_spike_pool_linear": (_i, [_pp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp, _f, _vp]),
+    "snnf_linear_lif_bits": (_i, [_pp, _i, _i, _i, _i, _i64, _i, _vp, _vp, _i, _vp, _vp, _i64, _vp, _f, _f, _f, _vp, _sz, _vp]),
     "snnf_pool2d": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "snnf_conv_bias": (_i, [_pp, _pp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
 }

@@ -117,6 +117,17 @@ __device__ __forceinline__ u32x4 finish_octet(const RawOctet<XT>& r, bool inside
     return out;
 }
 
+// Eight features at one bit each (bit j = feature j) as a matrix operand of zeros and ones.
+template <typename XT>
+__device__ __forceinline__ u32x4 expand_bit_octet(uint32_t bits, bool inside) {
+    constexpr uint32_t kOne = dtype_of<XT>::value == SNNF_F16 ? 0x3C00u : 0x3F80u;
+    bits = inside ? bits : 0u;
+    u32x4 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = ((bits >> (2 * j)) & 1u) * kOne | ((bits >> (2 * j + 1)) & 1u) * (kOne << 16);
+    return out;
+}
+
 template <typename XT>
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     using F = typename Frag<XT>::type;
@@ -284,7 +295,11 @@ template <int TT, int OCF, int SLABK, int TM> struct StagedShape {
     static constexpr size_t lds_bytes = slab_bytes > acc_bytes ? slab_bytes : acc_bytes;
 };
 
-template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM>
+// XBITS: the activation rows are rows of bits (byte b of a row = features 8 b ... 8 b + 7, bit j = feature 8 b + j; the row
+// stride is in bytes), expanded to 0 / 1 operands where a slab is parked. SBITS: the spikes leave as bits in the same form
+// ([T][M][Fout / 8] bytes, the step stride in bytes) instead of elements. Both are the internal layouts of a network executor
+// (a convolution on a plane of a few pixels is this matrix product, see snnf_linear_lif_bits).
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM, bool XBITS = false, bool SBITS = false>
 __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(StepPtrs xs, LinGeom g, const XT* __restrict__ W,
                                                                               const XT* __restrict__ bias,
                                                                               const VT* __restrict__ v_init, XT* __restrict__ spikes,
@@ -317,6 +332,8 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     // the octet is the same for all of a thread's items). Rows beyond M / Fout re-read the last real row; what they produce
     // is never stored.
     const int octet = tid % kSlabOctets;
+    constexpr int kRowsPerPass = NT / kSlabOctets;      // operand rows one pass of the workgroup's threads covers
+    static_assert(!XBITS || ((TT * TM) % kRowsPerPass == 0 && sizeof(XT) == 2), "a pass holds activation rows or weight rows, not both");
     const XT* item_row[SH::ITEMS];
     uint32_t item_dst[SH::ITEMS];
     bool item_live[SH::ITEMS];
@@ -332,7 +349,10 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
             const void* base = xs.p[0];
 #pragma unroll
             for (int u = 1; u < TT; ++u) base = t == u ? xs.p[u] : base;
-            ptr = static_cast<const XT*>(base) + static_cast<int64_t>(min(m0 + r % TM, g.M - 1)) * g.x_row_stride;
+            if constexpr (XBITS)       // a byte pointer kept in the array of element pointers
+                ptr = reinterpret_cast<const XT*>(static_cast<const unsigned char*>(base) + static_cast<int64_t>(min(m0 + r % TM, g.M - 1)) * g.x_row_stride);
+            else
+                ptr = static_cast<const XT*>(base) + static_cast<int64_t>(min(m0 + r % TM, g.M - 1)) * g.x_row_stride;
         } else {
             ptr = W + static_cast<int64_t>(min(oc0 + r - TT * TM, g.Fout - 1)) * g.Fin;
         }
@@ -376,7 +396,12 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         pre_inside[r] = slab < slab_end && k < g.Fin;
         const int ks = pre_inside[r] ? k : 0;
 #pragma unroll
-        for (int j = 0; j < SH::ITEMS; ++j) pre[r][j] = load_raw_octet<XT>(item_row[j] + ks);   // items beyond the rows re-read row 0
+        for (int j = 0; j < SH::ITEMS; ++j) {
+            if (XBITS && j * kRowsPerPass < TT * TM)       // one byte = the octet's eight features
+                pre[r][j].lo[0] = reinterpret_cast<const unsigned char*>(item_row[j])[ks >> 3];
+            else
+                pre[r][j] = load_raw_octet<XT>(item_row[j] + ks);   // items beyond the rows re-read row 0
+        }
     };
     // Fragment addresses in the slab: lane = 16 q + r reads K elements 8 q .. 8 q + 7 of row r of its fragment.
     const uint32_t frag_off = static_cast<uint32_t>((lane & 15) * kSlabPitch + (lane >> 4) * 16);
@@ -390,8 +415,12 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
     auto park = [&](int r, unsigned char* buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < SH::ITEMS; ++j)
-            if (item_live[j])
-                *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r], pre_part[r] == (item_is_w[j] ? 1 : 2));
+            if (item_live[j]) {
+                if (XBITS && j * kRowsPerPass < TT * TM)
+                    *reinterpret_cast<u32x4*>(buf + item_dst[j]) = expand_bit_octet<XT>(pre[r][j].lo[0], pre_inside[r]);
+                else
+                    *reinterpret_cast<u32x4*>(buf + item_dst[j]) = finish_octet<XT>(pre[r][j], pre_inside[r], pre_part[r] == (item_is_w[j] ? 1 : 2));
+            }
     };
     auto multiply = [&](const unsigned char* buf) __attribute__((always_inline)) {
         constexpr int OWN = SLABK / 32 / SH::KSPLIT;
@@ -485,7 +514,7 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
         if (!arrived_last) return;
     }
 
-    if (out_live) {
+    if (SBITS ? tid < OUTS : out_live) {      // SBITS: whole waves, for the ballot (OUTS is a multiple of 64)
         const int e = tid;
         const int slot = (e / TILE_OC) * SH::PITCH + e % TILE_OC;
         float v = v_first;
@@ -501,10 +530,19 @@ __global__ __launch_bounds__(kStagedWaves * 64) void linear_lif_staged_kernel(St
                     for (int w = 0; w < SH::KSPLIT; ++w) sum += partial[(w * TT + t) * SLAB_F + slot];
                 }
                 const float cur = sum + bv;
-                spikes[t * g.spike_step_stride + out_index] = spike_value<XT>(lif_step(cur, v, lif));
+                const bool fired = lif_step(cur, v, lif);
+                if constexpr (SBITS) {
+                    // Lane l of the wave holds feature oc0 + l % TILE_OC (a multiple of 8 apart from l % 8): byte l / 8 of the ballot.
+                    const uint64_t fired_lanes = __ballot(fired && out_live);
+                    if ((lane & 7) == 0 && out_live)
+                        reinterpret_cast<unsigned char*>(spikes)[t * g.spike_step_stride + static_cast<int64_t>(out_m) * (g.Fout >> 3) + (out_oc >> 3)] =
+                            static_cast<unsigned char>(fired_lanes >> lane);
+                } else {
+                    spikes[t * g.spike_step_stride + out_index] = spike_value<XT>(fired);
+                }
             }
         }
-        v_out[out_index] = from_float<VT>(v);
+        if (v_out != nullptr && out_live) v_out[out_index] = from_float<VT>(v);
     }
 }
 
@@ -516,13 +554,13 @@ struct LinWorkspace {
 constexpr size_t kLinCounterBytes = 64 * 1024;     // 16384 tiles
 constexpr int kLinLongK = 96;                      // K slabs from which two K parts of 16-row tiles beat 8-row tiles (see linear_half_row_tiles)
 
-template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM>
+template <typename XT, typename VT, int TT, int OCF, bool DB, int SLABK, int TM, bool XBITS = false, bool SBITS = false>
 int launch_staged_db(dim3 grid, int slabs_per_part, const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias,
                      const void* v_init, void* spikes, void* v_out, const LifParams& lif, hipStream_t stream) {
     using SH = StagedShape<TT, OCF, SLABK, TM>;
     constexpr size_t lds = DB ? 2 * SH::slab_bytes : SH::lds_bytes;
     static_assert(lds <= 160 * 1024 && SH::acc_bytes <= lds, "slabs exceed LDS");
-    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB, SLABK, TM>;
+    auto kernel = linear_lif_staged_kernel<XT, VT, TT, OCF, DB, SLABK, TM, XBITS, SBITS>;
     if (lds > 64 * 1024) {
         static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -546,7 +584,7 @@ inline int linear_split_parts(int64_t tiles, int unit_slabs, size_t part_bytes, 
     return 2;
 }
 
-template <typename XT, typename VT, int TT, int OCF, int TM = kTileM, int SLABK = kSlabK>
+template <typename XT, typename VT, int TT, int OCF, int TM = kTileM, int SLABK = kSlabK, bool XBITS = false, bool SBITS = false>
 int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
                   void* v_out, const LifParams& lif, hipStream_t stream) {
     dim3 grid((g.Fout + OCF * kTileOC - 1) / (OCF * kTileOC), (g.M + TM - 1) / TM);
@@ -563,9 +601,9 @@ int launch_staged(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, 
     constexpr bool can_double = 2 * SH::slab_bytes <= 160 * 1024;
     if constexpr (can_double) {
         if (tiles * parts <= compute_units())
-            return launch_staged_db<XT, VT, TT, OCF, true, SLABK, TM>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+            return launch_staged_db<XT, VT, TT, OCF, true, SLABK, TM, XBITS, SBITS>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     }
-    return launch_staged_db<XT, VT, TT, OCF, false, SLABK, TM>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_staged_db<XT, VT, TT, OCF, false, SLABK, TM, XBITS, SBITS>(grid, unit_slabs_per_part, ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 // Tiles of 8 batch rows instead of 16 (a workgroup then stages 8 x T activation rows per slab for its 32 weight rows):
@@ -622,6 +660,19 @@ int launch_tt(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, cons
     if (g.T <= 4) return launch_one<XT, VT, 4, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     if (g.T <= 8) return launch_one<XT, VT, 8, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
     return launch_one<XT, VT, 16, FAST, 1>(xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+}
+
+// The internal-layout forms: spikes out as bits, activation rows as elements or as bits; wide tiles (Fout % 32 == 0), 3 to 8
+// timesteps, fp32 membrane.
+template <typename XT, bool XBITS>
+int launch_bits(const LinWorkspace& ws, const StepPtrs& xs, const LinGeom& g, const void* W, const void* bias, const void* v_init, void* spikes,
+                void* v_out, const LifParams& lif, hipStream_t stream) {
+    if (linear_half_row_tiles(ws, g)) {
+        if (g.T <= 4) return launch_staged<XT, float, 4, 2, 8, 2 * kSlabK, XBITS, true>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+        return launch_staged<XT, float, 8, 2, 8, kSlabK, XBITS, true>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    }
+    if (g.T <= 4) return launch_staged<XT, float, 4, 2, kTileM, kSlabK, XBITS, true>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
+    return launch_staged<XT, float, 8, 2, kTileM, kSlabK, XBITS, true>(ws, xs, g, W, bias, v_init, spikes, v_out, lif, stream);
 }
 
 template <typename XT, typename VT>
@@ -732,4 +783,54 @@ static int linear_lif_impl(const char* who, const void* const* xs, int T, int M,
         if (rc != SNNF_OK) return rc;
     }
     return SNNF_OK;
+}
+
+extern "C" int snnf_linear_lif_bits(const void* const* xs, int x_bits, int T, int M, int Fin, int64_t x_row_stride, int dtype,
+                                    const void* weight, const void* bias, int Fout, const void* v_init, void* spike_bits,
+                                    int64_t spike_step_stride, void* v_out, float v_threshold, float v_reset, float tau,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace snnf;
+    if (xs == nullptr || weight == nullptr || spike_bits == nullptr)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: xs, weight and spike_bits must be non-null");
+    if (T < 1 || M < 1 || Fin < 1 || Fout < 1)
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: T=%d M=%d Fin=%d Fout=%d", T, M, Fin, Fout);
+    if (dtype != SNNF_BF16 && dtype != SNNF_F16)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif_bits: unsupported_dtype: bfloat16 or float16 weights (and activation elements)");
+    if (T < 3 || T > 8)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif_bits: unsupported_window: 3 to 8 timesteps per call, got %d", T);
+    if (Fin % 8 != 0 || Fout % 32 != 0)
+        return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif_bits: unsupported_shape: Fin %% 8 and Fout %% 32 must be 0, got %d -> %d", Fin, Fout);
+    if (x_row_stride < (x_bits ? Fin / 8 : Fin) || (!x_bits && x_row_stride % 8 != 0))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: x_row_stride=%lld (bytes for rows of bits, elements in multiples of 8 otherwise)",
+                    (long long)x_row_stride);
+    if (spike_step_stride < static_cast<int64_t>(M) * (Fout / 8))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: spike_step_stride=%lld bytes is less than a step's M * Fout / 8", (long long)spike_step_stride);
+    if (!aligned_to(weight, 16)) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: weight must be 16-byte aligned");
+    if (workspace != nullptr && !aligned_to(workspace, 256))
+        return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: workspace must be 256-byte aligned");
+    if (!(tau != 0.0f)) return fail(SNNF_ERR_UNSUPPORTED, "snnf_linear_lif_bits: unsupported_tau: tau must be nonzero");
+    const int tt = T <= 4 ? 4 : 8;
+    StepPtrs ptrs = {};
+    for (int t = 0; t < tt; ++t) {
+        ptrs.p[t] = xs[t < T ? t : 0];      // padded steps re-read step 0 and are never stored
+        if (ptrs.p[t] == nullptr) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: xs[%d] is null", t);
+        if (!x_bits && !aligned_to(ptrs.p[t], 16)) return fail(SNNF_ERR_INVALID_ARGUMENT, "snnf_linear_lif_bits: xs[%d] must be 16-byte aligned", t);
+    }
+    LinGeom g;
+    g.T = T;
+    g.M = M;
+    g.Fin = Fin;
+    g.Fout = Fout;
+    g.x_row_stride = x_row_stride;
+    g.spike_step_stride = spike_step_stride;
+    g.ksteps = (Fin + 31) / 32;
+    g.kparts = 1;
+    const LinWorkspace ws = {workspace, workspace != nullptr ? workspace_bytes : 0};
+    const LifParams lif = make_lif_params(v_threshold, v_reset, tau);
+    hipStream_t hs = as_stream(stream);
+    if (dtype == SNNF_BF16)
+        return x_bits ? launch_bits<bf16_t, true>(ws, ptrs, g, weight, bias, v_init, spike_bits, v_out, lif, hs)
+                      : launch_bits<bf16_t, false>(ws, ptrs, g, weight, bias, v_init, spike_bits, v_out, lif, hs);
+    return x_bits ? launch_bits<f16_t, true>(ws, ptrs, g, weight, bias, v_init, spike_bits, v_out, lif, hs)
+                  : launch_bits<f16_t, false>(ws, ptrs, g, weight, bias, v_init, spike_bits, v_out, lif, hs);
 }

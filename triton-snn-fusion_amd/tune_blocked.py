@@ -76,6 +76,10 @@ def main() -> int:
             _time_us(fn, torch)                           # warm-up: clocks and caches settle before anything is compared
             base = _time_us(fn, torch)
             base_plan = B.last_conv_plan()
+            if base_plan.get("kernel") == "plane_matrix":
+                B.register_tuned_plan(key, 0, 0, 0)
+                print(f"{net} {name}: {base:.2f} us as a matrix product per frame on the Linear + LIF kernel, nothing to choose", flush=True)
+                continue
             wo = (size + 2 * pad - k) // stride + 1
             seen = {(base_plan.get("tile"), base_plan.get("stage_chunks"), base_plan.get("waves"))}
             best = (base, 0, 0, 0, base_plan)
