@@ -124,7 +124,7 @@ __device__ __forceinline__ u32x4 expand_bit_octet(uint32_t bits, bool inside) {
     bits = inside ? bits : 0u;
     u32x4 out;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) out[j] = ((bits >> (2 * j)) & 1u) * kOne | ((bits >> (2 * j + 1)) & 1u) * (kOne << 16);
+    for (int j = 0; j < 4; ++j) out[j] = ((((bits >> (2 * j)) & 3u) * 0x8001u) & 0x10001u) * kOne;      // bit 0 -> low half, bit 1 -> high half
     return out;
 }
 
