@@ -252,7 +252,7 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
     g = torch.Generator(device="cpu")
     g.manual_seed(0)
     v0 = torch.zeros((), dtype=torch.float32, device=dev)
-    rows, total_ms, total_flops = [], 0.0, 0
+    rows, total_ms, total_flops, total_executed = [], 0.0, 0, 0
     for name, cin, cout, size, k, stride, pad, residual, analog, count in layers:
         if analog:
             frame = torch.randn(batch, cin, size, size, generator=g).to(dev, dtype)
@@ -289,8 +289,11 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
                      **({"internal_bytes": internal_bytes} if internal else {}),
                      "tflops": round(flops / (ms * 1e-3) / 1e12, 1), "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+        if analog:      # one frame for all T: the kernels convolve it once, the step-by-step network T times (what `flops` counts)
+            rows[-1]["mfma_frac_of_executed_flops"] = round(flops / T / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         total_ms += ms * count
         total_flops += flops * count
+        total_executed += (flops // T if analog else flops) * count
     if internal and which == "resnet18":
         # The down-sampling blocks: the second convolution with the shortcut convolution in its accumulators is one launch of
         # the executor; it takes the place of one "+res" layer and of the shortcut layer in the sum.
@@ -313,7 +316,8 @@ def _layer_sweep(which: str, dtype, dtype_name: str, steps: int, warmup: int, in
             by_name[sc_name]["count"] -= 1
     return {"metric": METRIC, "workload": f"{which}_layers" + ("_internal_layouts" if internal else ""), "dtype": dtype_name, "T": T, "batch": batch,
             "conv_ms_per_forward": round(total_ms, 4), "images_T_per_s_conv_only": round(batch * T / (total_ms * 1e-3), 1),
-            "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
+            "mfma_frac_overall": round(total_flops / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "mfma_frac_overall_of_executed_flops": round(total_executed / (total_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "layers": rows}
 
 
 def _plan_summary() -> str:
@@ -374,15 +378,20 @@ MODEL_CONFIGS = {"resnet18": dict(batch=16, size=224, T=4), "vgg11": dict(batch=
                  "mobilenet": dict(batch=32, size=64, T=4)}
 
 
-def _conv_flops_of(model, size: int, T: int, batch: int) -> int:
-    """2 * MACs of every Conv2d of `model` over T steps of a batch, from one CPU forward of a single frame (output shapes by hook)."""
+def _conv_flops_of(model, size: int, T: int, batch: int):
+    """2 * MACs of every Conv2d of `model` over T steps of a batch, from one CPU forward of a single frame (output shapes by
+    hook): (as the step-by-step network computes them, as the fused forward executes them). The two differ by the first
+    convolution, whose input frame is the same at every step: the fused operators convolve it once."""
     import torch
     from triton_snn_fusion_amd import models as M
     total = [0]
+    first = []
 
     def hook(mod, _inputs, out):
         cout, cin_g, kh, kw = (int(d) for d in mod.weight.shape)
-        total[0] += 2 * int(out.shape[2]) * int(out.shape[3]) * cout * cin_g * kh * kw
+        flops = 2 * int(out.shape[2]) * int(out.shape[3]) * cout * cin_g * kh * kw
+        total[0] += flops
+        first.append(flops)
 
     handles = [m.register_forward_hook(hook) for m in model.modules() if isinstance(m, torch.nn.Conv2d)]
     try:
@@ -393,7 +402,7 @@ def _conv_flops_of(model, size: int, T: int, batch: int) -> int:
     finally:
         for h in handles:
             h.remove()
-    return total[0] * T * batch
+    return total[0] * T * batch, (total[0] * T - first[0] * (T - 1)) * batch
 
 
 def _model_forward(name: str, dtype, steps: int, warmup: int):
@@ -475,8 +484,9 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
         best = min(best, ms_ig)
     except Exception as exc:  # pragma: no cover - reported, the dense executor's numbers stand
         out.setdefault("internal_layouts", {})["error"] = str(exc)[:300]
-    conv_flops = _conv_flops_of(M.build_network(name, seed=0), cfg["size"], cfg["T"], cfg["batch"])
-    out["conv_flops_per_forward"] = conv_flops
+    conv_flops, conv_flops_executed = _conv_flops_of(M.build_network(name, seed=0), cfg["size"], cfg["T"], cfg["batch"])
+    out["conv_flops_per_forward"] = conv_flops                        # the network's: T steps of every convolution
+    out["conv_flops_executed_per_forward"] = conv_flops_executed      # the shared input frame is convolved once for all T
     # Headline of the entry: the FX-rewritten graph on the internal layouts when it ran (the hand-lowered executor of the
     # same operator sequence is reported beside it under "internal_layouts"), otherwise the best of the executors.
     if ms_fx_internal is not None and name in ("resnet18", "vgg11"):
@@ -498,6 +508,7 @@ def _model_forward(name: str, dtype, steps: int, warmup: int):
         else:
             out["ms_per_forward_of"] = "eager launches"
     out["roofline"] = _roofline("mfma", conv_flops, best)
+    out["roofline"]["frac_of_executed_flops"] = round(conv_flops_executed / (best * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
     out["ms_per_forward"] = round(best, 4)
     out["images_T_per_s"] = round(cfg["batch"] * cfg["T"] / (best * 1e-3), 1)
     out["images_per_s"] = round(cfg["batch"] / (best * 1e-3), 1)
