@@ -335,3 +335,47 @@ def test_random_fused_blocked_cases(snnf_lib, seed, cases):
             assert torch.allclose(got.double().cpu(), want, rtol=eps, atol=2e-4), (what, float((got.double().cpu() - want).abs().max()))
         ran[kind] += 1
     assert ran["shortcut"] > 0.25 * cases and ran["pool"] > 0.12 * cases and ran["tail"] > 0.12 * cases, ran
+
+
+@pytest.mark.parametrize("seed,cases", [(23, 120)])
+def test_random_small_plane_cases(snnf_lib, seed, cases):
+    """Convolution + LIF on planes of one to four pixels with a bit-packed output and no membrane output: one matrix product
+    per frame on the Linear + LIF kernel, from bits or from channel-blocked elements, all neuron settings, kernels larger than
+    the plane, batches that leave row tiles ragged, matrices long enough for the K split over workgroups."""
+    import torch.nn.functional as F
+    from triton_snn_fusion_amd.runtime import hip_blocked_backend as B
+    rnd = random.Random(seed)
+    ran = collections.Counter()
+    for case in range(cases):
+        dtype = rnd.choice([BF16, BF16, F16])
+        g = gen(seed * 100000 + case)
+        H, W = rnd.choice([(1, 1), (1, 2), (2, 1), (2, 2), (2, 2), (2, 2), (1, 3), (4, 1)])
+        Cin, Cout = 8 * rnd.choice([1, 2, 3, 8, 16, 33, 64, 128]), 8 * rnd.choice([1, 2, 4, 5, 16, 32, 64])
+        kh, kw = rnd.choice([1, 3, 3, 3, 5]), rnd.choice([1, 3, 3, 3, 5])
+        T, N = rnd.choice([3, 4, 4, 4, 5, 6, 8]), rnd.choice([1, 2, 5, 8, 9, 16, 17, 40, 64])
+        lif = rnd.choice(LIFS)
+        source = rnd.choice(["bits", "bits", "quarters", "analog"])
+        if (Cout * H * W) % 32 != 0 or Cin * H * W * Cout * H * W > B.PLANE_MATRIX_MAX_ELEMENTS:
+            continue
+        what = f"case {case}: {Cin}->{Cout} {H}x{W} k{kh}x{kw} T={T} N={N} {dtype} {source} lif={lif}"
+        print(what, flush=True)
+        if source == "bits":
+            x = spikes((T, N, Cin, H, W), rnd.choice([0.1, 0.3]), g)
+            bx = B.from_dense(dev(x, dtype), B.BITS)
+        elif source == "quarters":
+            x = F.avg_pool2d(spikes((T * N, Cin, 2 * H, 2 * W), 0.3, g), 2).reshape(T, N, Cin, H, W)
+            bx = B.from_dense(dev(x, dtype), B.C8)
+        else:
+            x = q(torch.randn(T, N, Cin, H, W, generator=g) * 0.4, dtype)
+            bx = B.from_dense(dev(x, dtype), B.C8)
+        taps = min(kh, 2 * H - 1) * min(kw, 2 * W - 1)
+        w = q(torch.randn(Cout, Cin, kh, kw, generator=g) * (2.0 / (Cin * min(taps, H * W))) ** 0.5 * 2.5, dtype)
+        b = q(torch.randn(Cout, generator=g) * 0.1, dtype) if rnd.random() < 0.8 else None
+        ref = O.temporal_conv_lif([x[t] for t in range(T)], w, b, torch.tensor(0.0), (1, 1), (kh // 2, kw // 2), (1, 1), 1, *lif)
+        out, v = B.conv_lif_blocked(bx, dev(w, dtype), None if b is None else dev(b, dtype), 1, [kh // 2, kw // 2], lif, out_layout=B.BITS)
+        plan = B.last_conv_plan()
+        assert v is None and plan["kernel"] == "plane_matrix", (what, plan)
+        check(B.to_dense(out), ref[1], ref, v_threshold=lif[0], what=what, max_rate=2e-4)      # spikes only: the oracle's membrane stands in
+        ran[source] += 1
+    print(dict(ran))
+    assert min(ran[s] for s in ("bits", "quarters", "analog")) >= 10, ran
